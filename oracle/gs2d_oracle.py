@@ -1,0 +1,344 @@
+"""CPU restatement of the reference's 2-D Gaussian splatting (TEST INFRASTRUCTURE ONLY).
+
+This file is the checker that the HIP path is compared with.  It is never imported by the
+product package; the product fails loudly when its HIP library is missing instead of
+falling back to anything in here.
+
+Every function cites the reference lines it restates (paths relative to the reference
+checkout).  All functions are dtype-generic torch code: call them with float64 tensors to
+obtain the fp64 truth and with float32 tensors for the "naive PyTorch fp32" comparison.
+
+Pins (see tests/test_oracle.py): a scalar brute-force triple loop in plain C
+(oracle/gs2d_bruteforce.c) and in Python, the N=1 closed form, colour-constancy,
+permutation/zero-alpha/translation/rotation invariants, matrix-route vs closed-form
+covariance inverse, finite-difference gradcheck of the analytic backward, Euler and
+translation identities of the gradients.  The reference ships no golden vectors or tests
+for this path, so parity with the reference's *runtime* output is unpinned by the
+reference itself; these mathematical pins replace it.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+
+Tensor = torch.Tensor
+
+
+# --------------------------------------------------------------------------------------
+# covariance inverse
+# --------------------------------------------------------------------------------------
+def cov_inverse_matrix(scales: Tensor, rotations: Tensor, eps: float = 1e-6):
+    """(R S S^T R^T + eps I)^-1 by the matrix route; follows src/igs/gs2d.py:548-580.
+
+    The reference builds ``scale_matrices`` and ``eye`` without a dtype (:561, :572), so
+    it cannot run in fp64; this restatement creates them in the input dtype.
+    Returns (cov_inv_00, cov_inv_01, cov_inv_11), each [B, N, 1, 1].
+    """
+    b, ng, _ = scales.shape
+    c, s = torch.cos(rotations), torch.sin(rotations)
+    rot = torch.stack([torch.stack([c, -s], dim=2), torch.stack([s, c], dim=2)], dim=2)
+    sm = torch.zeros(b, ng, 2, 2, dtype=scales.dtype, device=scales.device)
+    sm = sm + torch.diag_embed(scales)
+    rs = torch.bmm(rot.flatten(0, 1), sm.flatten(0, 1))
+    cov = torch.bmm(rs, rs.transpose(-2, -1)).unflatten(0, (b, ng))
+    eye = torch.eye(2, dtype=cov.dtype, device=cov.device).expand(b, ng, -1, -1)
+    inv = torch.inverse(cov + eps * eye)
+    return (
+        inv[..., 0, 0, None, None],
+        inv[..., 0, 1, None, None],
+        inv[..., 1, 1, None, None],
+    )
+
+
+def cov_inverse_closed(scales: Tensor, rotations: Tensor, eps: float = 1e-6):
+    """Closed form of the same inverse: Sigma + eps I = R diag(s0^2+eps, s1^2+eps) R^T.
+
+    A = c^2 i0 + s^2 i1, B = c s (i0 - i1), D = s^2 i0 + c^2 i1, i_k = 1/(s_k^2 + eps).
+    Equivalent to src/igs/gs2d.py:548-580.  Returns three [B, N, 1, 1] tensors.
+    """
+    c, s = torch.cos(rotations), torch.sin(rotations)
+    i0 = 1.0 / (scales[..., 0] ** 2 + eps)
+    i1 = 1.0 / (scales[..., 1] ** 2 + eps)
+    a = c * c * i0 + s * s * i1
+    b = c * s * (i0 - i1)
+    d = s * s * i0 + c * c * i1
+    return a[..., None, None], b[..., None, None], d[..., None, None]
+
+
+# --------------------------------------------------------------------------------------
+# forward
+# --------------------------------------------------------------------------------------
+def naive_gaussian_2d(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors,
+                      eps: float = 1e-6) -> Tensor:
+    """Normative expression; follows src/igs/gs2d.py:24-44 (README.md:66-103).
+
+    x, y [B,1,H,W]; position [B,N,2]; cov_inv_* [B,N,1,1]; alphas [B,N]; colors [B,N,C].
+    Materialises the [B,N,H,W] weight, so only for sizes where that fits.
+    """
+    dx = x - position[..., 0, None, None]
+    dy = y - position[..., 1, None, None]
+    q = dx * dx * cov_inv_00 + 2 * dx * dy * cov_inv_01 + dy * dy * cov_inv_11
+    weight = torch.exp(-0.5 * q) * alphas[..., None, None]
+    weight_sum = weight.sum(dim=1, keepdim=True)
+    b, ng, h, w = weight.shape
+    nw = (weight / (weight_sum + eps)).permute(0, 2, 3, 1).flatten(1, 2)
+    result = torch.bmm(nw, colors)
+    return result.unflatten(1, (h, w)).permute(0, 3, 1, 2)
+
+
+def render_naive(positions, colors, scales, rotations, alphas, x_grid, y_grid,
+                 eps: float = 1e-6, closed_form: bool = False) -> Tensor:
+    """`render(..., fused=False)`; follows src/igs/gs2d.py:524-609."""
+    f = cov_inverse_closed if closed_form else cov_inverse_matrix
+    a, b, d = f(scales, rotations, eps)
+    return naive_gaussian_2d(x_grid, y_grid, positions, a, b, d, alphas, colors, eps)
+
+
+def _as4(g: Tensor, b: int) -> Tensor:
+    if g.dim() == 3:
+        g = g[:, None]
+    if g.shape[0] == 1 and b > 1:
+        g = g.expand(b, -1, -1, -1)
+    return g
+
+
+def forward_strips(x, y, position, a, b_, d, alphas, colors, eps=1e-6, rows=8):
+    """Same expression evaluated per image and per strip of rows (pixels are independent),
+    so that large shapes fit.  Returns (out [B,C,H,W], den [B,H,W])."""
+    B, N, C = colors.shape
+    x, y = _as4(x, B), _as4(y, B)
+    H, W = x.shape[-2:]
+    out = torch.empty(B, C, H, W, dtype=x.dtype, device=x.device)
+    den = torch.empty(B, H, W, dtype=x.dtype, device=x.device)
+    for ib in range(B):
+        for r0 in range(0, H, rows):
+            xs, ys = x[ib, :, r0:r0 + rows], y[ib, :, r0:r0 + rows]   # [1,r,W]
+            dx = xs - position[ib, :, 0, None, None]
+            dy = ys - position[ib, :, 1, None, None]
+            q = dx * dx * a[ib] + 2 * dx * dy * b_[ib] + dy * dy * d[ib]
+            wgt = torch.exp(-0.5 * q) * alphas[ib, :, None, None]        # [N,r,W]
+            s = wgt.sum(0)
+            num = torch.einsum("nhw,nc->chw", wgt, colors[ib])
+            den[ib, r0:r0 + rows] = s
+            out[ib, :, r0:r0 + rows] = num / (s + eps)
+    return out, den
+
+
+# --------------------------------------------------------------------------------------
+# backward, analytic (closed form); pinned by autograd of the naive expression and by
+# finite differences in tests/test_oracle.py
+# --------------------------------------------------------------------------------------
+def backward_strips(x, y, position, a, b_, d, alphas, colors, grad_out, eps=1e-6, rows=8,
+                    grid_grads: bool = False) -> Dict[str, Tensor]:
+    """Gradients of sum(out * grad_out) w.r.t. the operator inputs.
+
+    With g^ = g/(den+eps), s = <g^, out>, G_n = <g^, c_n> - s, w_n = alpha_n e_n:
+      d alpha_n = sum_px G e        d color_nc = sum_px g^_c w
+      d px = sum G w (A dx + B dy)  d py = sum G w (B dx + D dy)
+      d A = sum -1/2 G w dx^2       d B = sum -G w dx dy      d D = sum -1/2 G w dy^2
+      d x_px = -sum_n G w (A dx + B dy), d y_px likewise.
+    (The hand-written backward in src/igs/gs2d.py:176,370 uses grad*grad for the d/d den
+    term and is not followed; the naive expression under autograd is the reference.)
+    """
+    B, N, C = colors.shape
+    x, y = _as4(x, B), _as4(y, B)
+    H, W = x.shape[-2:]
+    dt, dev = x.dtype, x.device
+    g = dict(
+        position=torch.zeros(B, N, 2, dtype=dt, device=dev),
+        cov_inv_00=torch.zeros(B, N, dtype=dt, device=dev),
+        cov_inv_01=torch.zeros(B, N, dtype=dt, device=dev),
+        cov_inv_11=torch.zeros(B, N, dtype=dt, device=dev),
+        alphas=torch.zeros(B, N, dtype=dt, device=dev),
+        colors=torch.zeros(B, N, C, dtype=dt, device=dev),
+    )
+    if grid_grads:
+        g["x"] = torch.zeros(B, 1, H, W, dtype=dt, device=dev)
+        g["y"] = torch.zeros(B, 1, H, W, dtype=dt, device=dev)
+    for ib in range(B):
+        A, Bc, D = a[ib].reshape(N, 1, 1), b_[ib].reshape(N, 1, 1), d[ib].reshape(N, 1, 1)
+        for r0 in range(0, H, rows):
+            xs, ys = x[ib, :, r0:r0 + rows], y[ib, :, r0:r0 + rows]
+            dx = xs - position[ib, :, 0, None, None]
+            dy = ys - position[ib, :, 1, None, None]
+            e = torch.exp(-0.5 * (dx * dx * A + 2 * dx * dy * Bc + dy * dy * D))
+            wgt = e * alphas[ib, :, None, None]
+            den = wgt.sum(0) + eps
+            out = torch.einsum("nhw,nc->chw", wgt, colors[ib]) / den
+            gh = grad_out[ib, :, r0:r0 + rows] / den                      # [C,r,W]
+            s = (gh * out).sum(0)
+            G = torch.einsum("chw,nc->nhw", gh, colors[ib]) - s
+            Gw = G * wgt
+            lx = A * dx + Bc * dy
+            ly = Bc * dx + D * dy
+            g["alphas"][ib] += (G * e).sum((1, 2))
+            g["colors"][ib] += torch.einsum("chw,nhw->nc", gh, wgt)
+            g["position"][ib, :, 0] += (Gw * lx).sum((1, 2))
+            g["position"][ib, :, 1] += (Gw * ly).sum((1, 2))
+            g["cov_inv_00"][ib] += (-0.5 * Gw * dx * dx).sum((1, 2))
+            g["cov_inv_01"][ib] += (-Gw * dx * dy).sum((1, 2))
+            g["cov_inv_11"][ib] += (-0.5 * Gw * dy * dy).sum((1, 2))
+            if grid_grads:
+                g["x"][ib, 0, r0:r0 + rows] = -(Gw * lx).sum(0)
+                g["y"][ib, 0, r0:r0 + rows] = -(Gw * ly).sum(0)
+    return g
+
+
+def chain_to_scale_rotation(scales, rotations, gA, gB, gD, eps=1e-6):
+    """Chain rule from (dA, dB, dD) to (d scales [B,N,2], d rotations [B,N]) through the
+    closed form of cov_inverse_closed."""
+    c, s = torch.cos(rotations), torch.sin(rotations)
+    i0 = 1.0 / (scales[..., 0] ** 2 + eps)
+    i1 = 1.0 / (scales[..., 1] ** 2 + eps)
+    gi0 = gA * c * c + gB * c * s + gD * s * s
+    gi1 = gA * s * s - gB * c * s + gD * c * c
+    gs = torch.stack([gi0 * (-2 * scales[..., 0] * i0 * i0),
+                      gi1 * (-2 * scales[..., 1] * i1 * i1)], dim=-1)
+    Bv = c * s * (i0 - i1)
+    gth = (gD - gA) * 2 * Bv + gB * (c * c - s * s) * (i0 - i1)
+    return gs, gth
+
+
+def render_backward_strips(positions, colors, scales, rotations, alphas, x_grid, y_grid,
+                           grad_out, eps=1e-6, rows=8) -> Dict[str, Tensor]:
+    """Gradients w.r.t. the function-level inputs (positions, colors, scales, rotations,
+    alphas), evaluated in strips."""
+    a, b_, d = cov_inverse_closed(scales, rotations, eps)
+    g = backward_strips(x_grid, y_grid, positions, a, b_, d, alphas, colors, grad_out, eps, rows)
+    gs, gth = chain_to_scale_rotation(scales, rotations, g["cov_inv_00"], g["cov_inv_01"],
+                                      g["cov_inv_11"], eps)
+    return dict(positions=g["position"], colors=g["colors"], scales=gs, rotations=gth,
+                alphas=g["alphas"])
+
+
+def render_autograd(positions, colors, scales, rotations, alphas, x_grid, y_grid, grad_out,
+                    eps=1e-6, closed_form=False) -> Tuple[Tensor, Dict[str, Tensor]]:
+    """Naive expression under torch autograd (the stated gradient oracle when run in
+    fp64).  Returns (out, grads)."""
+    leaves = dict(positions=positions, colors=colors, scales=scales, rotations=rotations,
+                  alphas=alphas)
+    leaves = {k: v.detach().clone().requires_grad_(True) for k, v in leaves.items()}
+    out = render_naive(leaves["positions"], leaves["colors"], leaves["scales"],
+                       leaves["rotations"], leaves["alphas"], x_grid, y_grid, eps, closed_form)
+    gr = torch.autograd.grad(out, list(leaves.values()), grad_out)
+    return out.detach(), dict(zip(leaves.keys(), gr))
+
+
+def operator_autograd(x, y, position, a, b_, d, alphas, colors, grad_out, eps=1e-6):
+    """Naive operator-level expression under autograd, all 8 tensor inputs as leaves."""
+    names = ["x", "y", "position", "cov_inv_00", "cov_inv_01", "cov_inv_11", "alphas", "colors"]
+    leaves = [t.detach().clone().requires_grad_(True) for t in (x, y, position, a, b_, d, alphas, colors)]
+    out = naive_gaussian_2d(*leaves, eps)
+    gr = torch.autograd.grad(out, leaves, grad_out)
+    return out.detach(), dict(zip(names, gr))
+
+
+# --------------------------------------------------------------------------------------
+# scalar brute force (tiny inputs only) -- an independent pin for the vectorised code
+# --------------------------------------------------------------------------------------
+def brute_force_forward(x, y, position, a, b_, d, alphas, colors, eps=1e-6):
+    """Plain Python triple loop over (image, pixel, gaussian) in Python floats (fp64)."""
+    B, N, C = colors.shape
+    x, y = _as4(x, B), _as4(y, B)
+    H, W = x.shape[-2:]
+    out = torch.zeros(B, C, H, W, dtype=torch.float64)
+    for ib in range(B):
+        for i in range(H):
+            for j in range(W):
+                xv, yv = float(x[ib, 0, i, j]), float(y[ib, 0, i, j])
+                den, num = 0.0, [0.0] * C
+                for n in range(N):
+                    dx = xv - float(position[ib, n, 0])
+                    dy = yv - float(position[ib, n, 1])
+                    q = (float(a.reshape(B, N)[ib, n]) * dx * dx
+                         + 2.0 * float(b_.reshape(B, N)[ib, n]) * dx * dy
+                         + float(d.reshape(B, N)[ib, n]) * dy * dy)
+                    wv = math.exp(-0.5 * q) * float(alphas[ib, n])
+                    den += wv
+                    for c in range(C):
+                        num[c] += wv * float(colors[ib, n, c])
+                for c in range(C):
+                    out[ib, c, i, j] = num[c] / (den + eps)
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# grids, module head
+# --------------------------------------------------------------------------------------
+def xy_grid(size, dtype=torch.float32):
+    """Follows src/igs/gs2d.py:503-522: x in +-sqrt(w/h), y in +-sqrt(h/w), each [1,h,w]."""
+    h, w = size
+    ar = h / w
+    hr, wr = ar ** 0.5, 1 / ar ** 0.5
+    xg = torch.linspace(-wr, wr, w, dtype=dtype).view(1, 1, w).expand(1, h, w)
+    yg = torch.linspace(-hr, hr, h, dtype=dtype).view(1, h, 1).expand(1, h, w)
+    return xg, yg
+
+
+def module_forward(weight, bias, feature, size, num_gaussians_per_emb, output_dim=3,
+                   eps=1e-6):
+    """Module head + render; follows src/igs/gs2d.py:611-689 for grid=None,
+    pos_map_offset=False.  Returns (image, gs_feature)."""
+    gs_feature = torch.nn.functional.linear(feature, weight, bias)
+    gs_feature = gs_feature.unflatten(-1, (-1, 6 + output_dim)).flatten(1, 2)
+    b = gs_feature.shape[0]
+    positions, log_scales, rotations, logit_opacity, colors = gs_feature.split(
+        [2, 2, 1, 1, output_dim], dim=-1)
+    xg, yg = xy_grid(size, dtype=feature.dtype)
+    xg = xg[None].repeat(b, 1, 1, 1)
+    yg = yg[None].repeat(b, 1, 1, 1)
+    alphas = torch.ones_like(logit_opacity[..., 0])
+    scales = torch.exp(log_scales) + eps
+    img = render_naive(positions, colors, scales, rotations[..., 0], alphas, xg, yg, eps)
+    return img, gs_feature
+
+
+# --------------------------------------------------------------------------------------
+# seeded synthetic inputs for the benchmark configurations
+# --------------------------------------------------------------------------------------
+CONFIGS = {
+    # name: B, N, H, W, C, scale range, colour law
+    "c0": dict(B=1, N=2048, H=256, W=256, C=3, smin=0.25, smax=0.75, colors="uniform"),
+    "c1": dict(B=16, N=8192, H=256, W=256, C=3, smin=0.02, smax=0.3, colors="uniform"),
+    "c2": dict(B=1, N=16384, H=512, W=512, C=3, smin=0.01, smax=0.1, colors="uniform"),
+    "c4": dict(B=4, N=32768, H=384, W=640, C=16, smin=0.005, smax=0.05, colors="normal"),
+}
+
+
+def make_inputs(B, N, H, W, C, smin, smax, colors="uniform", seed=0, dtype=torch.float32,
+                x_extent: Optional[float] = None, expand_grids=True):
+    """Seeded inputs in the draw order positions, colors, scales, rotations, alphas,
+    grad_out (CPU generator).  Grids: x = linspace(-xe, xe, W), y = linspace(-1, 1, H)
+    with xe = W/H unless given (1 for square images)."""
+    g = torch.Generator().manual_seed(seed)
+    xe = (W / H) if x_extent is None else x_extent
+    pos = torch.rand(B, N, 2, generator=g, dtype=torch.float64) * 2 - 1
+    pos[..., 0] *= xe
+    if colors == "uniform":
+        col = torch.rand(B, N, C, generator=g, dtype=torch.float64)
+    else:
+        col = torch.randn(B, N, C, generator=g, dtype=torch.float64)
+    sc = torch.rand(B, N, 2, generator=g, dtype=torch.float64) * (smax - smin) + smin
+    rot = torch.rand(B, N, generator=g, dtype=torch.float64) * (2 * math.pi)
+    al = torch.rand(B, N, generator=g, dtype=torch.float64)
+    go = torch.randn(B, C, H, W, generator=g, dtype=torch.float64)
+    # everything is rounded to fp32 first so that the fp64 truth and the fp32 kernels see
+    # the same numbers
+    t = lambda v: v.to(torch.float32).to(dtype)
+    xg = torch.linspace(-xe, xe, W, dtype=torch.float32).to(dtype)
+    yg = torch.linspace(-1, 1, H, dtype=torch.float32).to(dtype)
+    xg = xg.view(1, 1, 1, W).expand(B, 1, H, W)     # stride 0 over B and H
+    yg = yg.view(1, 1, H, 1).expand(B, 1, H, W)     # stride 0 over B and W
+    if not expand_grids:
+        xg, yg = xg.contiguous(), yg.contiguous()
+    return dict(positions=t(pos), colors=t(col), scales=t(sc), rotations=t(rot), alphas=t(al),
+                x_grid=xg, y_grid=yg, grad_out=t(go))
+
+
+def make_config_inputs(name: str, dtype=torch.float32, **override):
+    cfg = dict(CONFIGS[name])
+    cfg.update(override)
+    seed = 1000 + int(name[1:])
+    return make_inputs(seed=seed, dtype=dtype, **cfg)

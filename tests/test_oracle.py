@@ -1,0 +1,248 @@
+"""Pins for the CPU oracle (no GPU).  The reference ships no golden vectors for this
+path, so the oracle is pinned by independent restatements and by what the mathematics
+fixes; each test is chosen so that a plausible slip (dropped term, wrong sign/index,
+transposed operand) fails it."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gs2d_oracle as O
+from oracle.chunked_cpu import ChunkedCPUSplat
+
+torch.manual_seed(0)
+F64 = torch.float64
+
+
+def tiny(B=2, N=5, H=3, W=4, C=3, seed=0, dtype=F64):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.rand(*s, generator=g, dtype=dtype)
+    x = r(B, 1, H, W) * 2 - 1
+    y = r(B, 1, H, W) * 2 - 1
+    pos = r(B, N, 2) * 2 - 1
+    sc = r(B, N, 2) * 0.5 + 0.2
+    rot = r(B, N) * 2 * math.pi
+    al = r(B, N)
+    col = torch.randn(B, N, C, generator=g, dtype=dtype)
+    go = torch.randn(B, C, H, W, generator=g, dtype=dtype)
+    return x, y, pos, sc, rot, al, col, go
+
+
+def _p(t):
+    return np.ascontiguousarray(t.detach().numpy(), dtype=np.float64)
+
+
+def c_forward(lib, x, y, pos, a, b, d, al, col, eps):
+    B, N, C = col.shape
+    H, W = x.shape[-2:]
+    arrs = [_p(x.reshape(B, H, W)), _p(y.reshape(B, H, W)), _p(pos), _p(a.reshape(B, N)),
+            _p(b.reshape(B, N)), _p(d.reshape(B, N)), _p(al), _p(col)]
+    out = np.zeros((B, C, H, W))
+    den = np.zeros((B, H, W))
+    dp = ctypes.POINTER(ctypes.c_double)
+    lib.gs2d_bf_forward.restype = None
+    lib.gs2d_bf_forward(*[v.ctypes.data_as(dp) for v in arrs], B, N, H, W, C,
+                        ctypes.c_double(eps), out.ctypes.data_as(dp), den.ctypes.data_as(dp))
+    return arrs, out, den
+
+
+def c_backward(lib, arrs, out, den, go, B, N, H, W, C, eps):
+    dp = ctypes.POINTER(ctypes.c_double)
+    g = dict(position=np.zeros((B, N, 2)), cov_inv_00=np.zeros((B, N)), cov_inv_01=np.zeros((B, N)),
+             cov_inv_11=np.zeros((B, N)), alphas=np.zeros((B, N)), colors=np.zeros((B, N, C)),
+             x=np.zeros((B, 1, H, W)), y=np.zeros((B, 1, H, W)))
+    gon = _p(go)
+    lib.gs2d_bf_backward.restype = None
+    lib.gs2d_bf_backward(*[v.ctypes.data_as(dp) for v in arrs], out.ctypes.data_as(dp),
+                         den.ctypes.data_as(dp), gon.ctypes.data_as(dp), B, N, H, W, C,
+                         ctypes.c_double(eps),
+                         *[g[k].ctypes.data_as(dp) for k in
+                           ("position", "cov_inv_00", "cov_inv_01", "cov_inv_11", "alphas", "colors", "x", "y")])
+    return g
+
+
+# ---------------------------------------------------------------- covariance inverse
+def test_cov_inverse_closed_equals_matrix_route():
+    _, _, _, sc, rot, *_ = tiny(N=64)
+    for eps in (1e-6, 1e-2):
+        m = O.cov_inverse_matrix(sc, rot, eps)
+        c = O.cov_inverse_closed(sc, rot, eps)
+        for u, v in zip(m, c):
+            assert torch.allclose(u, v, rtol=1e-12, atol=1e-12)
+
+
+def test_cov_inverse_is_inverse_of_sigma():
+    # (A,B;B,D) times R diag(s^2+eps) R^T must be the identity (catches a transposed R).
+    _, _, _, sc, rot, *_ = tiny(N=16)
+    eps = 1e-3
+    a, b, d = [t.reshape(-1) for t in O.cov_inverse_closed(sc, rot, eps)]
+    c, s = torch.cos(rot).reshape(-1), torch.sin(rot).reshape(-1)
+    l0, l1 = (sc[..., 0] ** 2 + eps).reshape(-1), (sc[..., 1] ** 2 + eps).reshape(-1)
+    s00 = c * c * l0 + s * s * l1
+    s01 = c * s * (l0 - l1)
+    s11 = s * s * l0 + c * c * l1
+    assert torch.allclose(a * s00 + b * s01, torch.ones_like(a), atol=1e-10)
+    assert torch.allclose(a * s01 + b * s11, torch.zeros_like(a), atol=1e-10)
+    assert torch.allclose(b * s01 + d * s11, torch.ones_like(a), atol=1e-10)
+    # axis-aligned special case: theta = 0 -> A = 1/(s0^2+eps), B = 0, D = 1/(s1^2+eps)
+    a0, b0, d0 = O.cov_inverse_closed(sc, torch.zeros_like(rot), eps)
+    assert torch.allclose(a0.reshape(-1), 1 / l0) and torch.all(b0 == 0)
+    assert torch.allclose(d0.reshape(-1), 1 / l1)
+
+
+# ---------------------------------------------------------------- forward
+@pytest.mark.parametrize("C", [1, 3, 4])
+def test_forward_vs_bruteforce_python_and_c(bruteforce_lib, C):
+    x, y, pos, sc, rot, al, col, go = tiny(C=C, seed=C)
+    a, b, d = O.cov_inverse_closed(sc, rot)
+    ref = O.naive_gaussian_2d(x, y, pos, a, b, d, al, col)
+    bf = O.brute_force_forward(x, y, pos, a, b, d, al, col)
+    assert torch.allclose(ref, bf, rtol=1e-12, atol=1e-14)
+    _, cout, cden = c_forward(bruteforce_lib, x, y, pos, a, b, d, al, col, 1e-6)
+    assert np.allclose(ref.numpy(), cout, rtol=1e-12, atol=1e-14)
+    out_s, den_s = O.forward_strips(x, y, pos, a, b, d, al, col, rows=2)
+    assert torch.allclose(out_s, ref, rtol=1e-12, atol=1e-14)
+    assert np.allclose(den_s.numpy(), cden, rtol=1e-12)
+
+
+def test_forward_single_gaussian_closed_form():
+    x, y, pos, sc, rot, al, col, _ = tiny(B=1, N=1, C=3)
+    eps = 1e-6
+    out = O.render_naive(pos, col, sc, rot, al, x, y, eps)
+    # isotropic-free closed form: rotate the offset into the Gaussian's frame.
+    c, s = math.cos(float(rot[0, 0])), math.sin(float(rot[0, 0]))
+    dx, dy = x[0, 0] - pos[0, 0, 0], y[0, 0] - pos[0, 0, 1]
+    u, v = c * dx + s * dy, -s * dx + c * dy
+    q = u * u / (sc[0, 0, 0] ** 2 + eps) + v * v / (sc[0, 0, 1] ** 2 + eps)
+    w = al[0, 0] * torch.exp(-0.5 * q)
+    expect = col[0, 0, :, None, None] * (w / (w + eps))
+    assert torch.allclose(out[0], expect, rtol=1e-10, atol=1e-14)
+
+
+def test_forward_invariants():
+    x, y, pos, sc, rot, al, col, _ = tiny(N=7)
+    base = O.render_naive(pos, col, sc, rot, al, x, y)
+    # constant colour k -> k * den/(den+eps)
+    a, b, d = O.cov_inverse_closed(sc, rot)
+    _, den = O.forward_strips(x, y, pos, a, b, d, al, col)
+    k = 0.37
+    outk = O.render_naive(pos, torch.full_like(col, k), sc, rot, al, x, y)
+    assert torch.allclose(outk, (k * den / (den + 1e-6))[:, None].expand_as(outk), rtol=1e-12)
+    # permutation of the Gaussians
+    perm = torch.randperm(7)
+    outp = O.render_naive(pos[:, perm], col[:, perm], sc[:, perm], rot[:, perm], al[:, perm], x, y)
+    assert torch.allclose(outp, base, rtol=1e-12, atol=1e-15)
+    # appending alpha = 0 Gaussians
+    z = lambda t: torch.cat([t, t[:, :2]], 1)
+    al0 = torch.cat([al, torch.zeros_like(al[:, :2])], 1)
+    out0 = O.render_naive(z(pos), z(col), z(sc), z(rot), al0, x, y)
+    assert torch.allclose(out0, base, rtol=1e-13, atol=1e-15)
+    # joint translation of grid and positions
+    t = torch.tensor([0.3, -0.2], dtype=F64)
+    outt = O.render_naive(pos + t, col, sc, rot, al, x + t[0], y + t[1])
+    assert torch.allclose(outt, base, rtol=1e-10, atol=1e-13)
+    # theta -> theta + pi; (s0, s1, theta) -> (s1, s0, theta + pi/2)
+    assert torch.allclose(O.render_naive(pos, col, sc, rot + math.pi, al, x, y), base, rtol=1e-10)
+    assert torch.allclose(O.render_naive(pos, col, sc.flip(-1), rot + math.pi / 2, al, x, y), base, rtol=1e-10)
+    # convexity: alphas >= 0 -> min_c <= out <= max_c per channel
+    assert (base <= col.amax(1)[:, :, None, None] + 1e-12).all()
+    assert (base >= torch.minimum(col.amin(1), torch.zeros(1, dtype=F64))[:, :, None, None] - 1e-12).all()
+
+
+# ---------------------------------------------------------------- backward
+def test_backward_analytic_vs_autograd_and_c(bruteforce_lib):
+    x, y, pos, sc, rot, al, col, go = tiny(N=6, H=4, W=5)
+    a, b, d = O.cov_inverse_closed(sc, rot)
+    out, ga = O.operator_autograd(x, y, pos, a, b, d, al, col, go)
+    gs = O.backward_strips(x, y, pos, a, b, d, al, col, go, rows=3, grid_grads=True)
+    B, N, C = col.shape
+    H, W = x.shape[-2:]
+    arrs, cout, cden = c_forward(bruteforce_lib, x, y, pos, a, b, d, al, col, 1e-6)
+    gc = c_backward(bruteforce_lib, arrs, cout, cden, go, B, N, H, W, C, 1e-6)
+    for k in ("x", "y", "position", "cov_inv_00", "cov_inv_01", "cov_inv_11", "alphas", "colors"):
+        ref = ga[k].reshape(gs[k].shape)
+        assert torch.allclose(gs[k], ref, rtol=1e-9, atol=1e-12), k
+        assert np.allclose(gc[k], ref.numpy().reshape(gc[k].shape), rtol=1e-9, atol=1e-12), k
+
+
+def test_backward_function_level_vs_autograd_both_cov_routes():
+    x, y, pos, sc, rot, al, col, go = tiny(N=6, H=4, W=5, seed=3)
+    g = O.render_backward_strips(pos, col, sc, rot, al, x, y, go)
+    for closed in (False, True):
+        _, ga = O.render_autograd(pos, col, sc, rot, al, x, y, go, closed_form=closed)
+        for k in g:
+            assert torch.allclose(g[k], ga[k], rtol=1e-8, atol=1e-11), (k, closed)
+
+
+def test_backward_finite_differences():
+    # central differences on the scalar L = sum(out * go), independent of autograd.
+    x, y, pos, sc, rot, al, col, go = tiny(B=1, N=3, H=3, W=3, seed=5)
+    g = O.render_backward_strips(pos, col, sc, rot, al, x, y, go)
+    L = lambda **kw: float((O.render_naive(kw.get("pos", pos), kw.get("col", col), kw.get("sc", sc),
+                                          kw.get("rot", rot), kw.get("al", al), x, y) * go).sum())
+    h = 1e-6
+    for name, key, t in (("pos", "positions", pos), ("col", "colors", col), ("sc", "scales", sc),
+                         ("rot", "rotations", rot), ("al", "alphas", al)):
+        flat = t.reshape(-1)
+        for i in range(flat.numel()):
+            tp, tm = flat.clone(), flat.clone()
+            tp[i] += h
+            tm[i] -= h
+            fd = (L(**{name: tp.view_as(t)}) - L(**{name: tm.view_as(t)})) / (2 * h)
+            an = float(g[key].reshape(-1)[i])
+            assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), (name, i, fd, an)
+
+
+def test_backward_identities():
+    x, y, pos, sc, rot, al, col, go = tiny(N=9, H=5, W=4, seed=7)
+    eps = 1e-6
+    a, b, d = O.cov_inverse_closed(sc, rot, eps)
+    g = O.backward_strips(x, y, pos, a, b, d, al, col, go, eps, grid_grads=True)
+    # translation: sum_n dL/dpos_n = - sum_px (dL/dx, dL/dy)
+    assert torch.allclose(g["position"][..., 0].sum(1), -g["x"].sum((1, 2, 3)), rtol=1e-9, atol=1e-12)
+    assert torch.allclose(g["position"][..., 1].sum(1), -g["y"].sum((1, 2, 3)), rtol=1e-9, atol=1e-12)
+    # Euler (degree-0 homogeneity in alphas up to eps): sum alpha dL/dalpha = eps sum <g,out>/(den+eps)
+    out, den = O.forward_strips(x, y, pos, a, b, d, al, col, eps)
+    rhs = eps * ((go * out).sum(1) / (den + eps)).sum((1, 2))
+    assert torch.allclose((al * g["alphas"]).sum(1), rhs, rtol=1e-6, atol=1e-13)
+    # isotropic Gaussians: dL/dtheta = 0
+    iso = sc[..., :1].expand(-1, -1, 2)
+    gi = O.render_backward_strips(pos, col, iso, rot, al, x, y, go)
+    assert gi["rotations"].abs().max() < 1e-9 * max(1.0, float(gi["positions"].abs().max()))
+    # linearity in grad_out
+    g2 = O.backward_strips(x, y, pos, a, b, d, al, col, 2.5 * go, eps)
+    assert torch.allclose(g2["alphas"], 2.5 * g["alphas"], rtol=1e-12)
+
+
+# ---------------------------------------------------------------- CPU baseline + helpers
+def test_chunked_cpu_baseline_matches_oracle():
+    x, y, pos, sc, rot, al, col, go = tiny(B=2, N=70, H=6, W=7, seed=11)  # N not a multiple of 32
+    a, b, d = O.cov_inverse_closed(sc, rot)
+    out, ga = O.operator_autograd(x, y, pos, a, b, d, al, col, go)
+    leaves = [t.clone().requires_grad_(True) for t in (x, y, pos, a, b, d, al, col)]
+    o2 = ChunkedCPUSplat.apply(*leaves, 1e-6)
+    o2.backward(go)
+    assert torch.allclose(o2, out, rtol=1e-11, atol=1e-14)
+    for t, k in zip(leaves, ("x", "y", "position", "cov_inv_00", "cov_inv_01", "cov_inv_11", "alphas", "colors")):
+        assert torch.allclose(t.grad, ga[k], rtol=1e-9, atol=1e-12), k
+
+
+def test_xy_grid_ranges():
+    xg, yg = O.xy_grid((384, 640))
+    assert xg.shape == (1, 384, 640) and yg.shape == (1, 384, 640)
+    assert xg.stride(1) == 0 and yg.stride(2) == 0
+    assert math.isclose(float(xg[0, 0, -1]), math.sqrt(640 / 384), rel_tol=1e-6)
+    assert math.isclose(float(yg[0, -1, 0]), math.sqrt(384 / 640), rel_tol=1e-6)
+    assert math.isclose(float(xg[0, 0, -1]) * float(yg[0, -1, 0]), 1.0, rel_tol=1e-6)
+
+
+def test_make_inputs_is_seeded_and_shaped():
+    a = O.make_config_inputs("c0", N=16, H=8, W=8)
+    b = O.make_config_inputs("c0", N=16, H=8, W=8)
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    assert a["x_grid"].shape == (1, 1, 8, 8) and a["x_grid"].stride(2) == 0
+    assert a["scales"].min() >= 0.25 and a["scales"].max() <= 0.75
+    c4 = O.make_config_inputs("c4", B=1, N=8, H=12, W=20)
+    assert math.isclose(float(c4["x_grid"].max()), 20 / 12, rel_tol=1e-6)
