@@ -1,0 +1,26 @@
+"""igs_amd -- MI355X-native 2-D Gaussian splatting (forward + backward) behind the
+KohakuBlueleaf/IGS function / autograd.Function / module interface.
+
+`from igs_amd import GaussianSplatting2D, gaussian_splatting_2d` mirrors
+`from igs.gs2d import GaussianSplatting2D, gaussian_splatting_2d` of the reference
+(src/igs/__init__.py:1, README.md:19).
+"""
+from .gs2d import (  # noqa: F401
+    GaussianSplatting2D,
+    GaussianSplatting2DChunkedKernel,
+    GaussianSplatting2DKernel,
+    TorchGaussianSplatting2DChunked,
+    TorchGaussianSplatting2DKernel,
+    gaussian_splatting_2d,
+    naive_gaussian_2d,
+)
+
+__all__ = [
+    "GaussianSplatting2D",
+    "gaussian_splatting_2d",
+    "naive_gaussian_2d",
+    "GaussianSplatting2DKernel",
+    "TorchGaussianSplatting2DKernel",
+    "TorchGaussianSplatting2DChunked",
+    "GaussianSplatting2DChunkedKernel",
+]

@@ -1,0 +1,966 @@
+// igs_gs2d.hip -- hand-written gfx950 (CDNA4) kernels and the C ABI for the 2-D Gaussian
+// splatting forward/backward.
+//
+// Math (reference src/igs/gs2d.py:24-44): q = A dx^2 + 2 B dx dy + D dy^2,
+// e = exp(-q/2), w = alpha e, out_c = sum_n w c_nc / (sum_n w + eps).
+//
+// Design in one paragraph.  The path is bound by fp32 VALU + transcendental issue, not by
+// HBM (a few tens of MB per call) and not by MFMA (colour contraction has C = 3), so the
+// kernels are organised to need no cross-lane reduction at all and the fewest VALU
+// instructions per (Gaussian, pixel) pair:
+//   * forward  : a lane owns pixels, the Gaussian record is wave-uniform and arrives
+//                through the scalar data path (s_load -> SGPR operands); den and the C
+//                numerators stay in VGPRs for the whole Gaussian loop.
+//   * backward : a lane owns Gaussians, the pixel record (g^ = g/(den+eps), -s = -<g^,out>)
+//                is wave-uniform (SGPRs); the lane accumulates the six moments of G e and
+//                the C colour sums over its pixel tile in VGPRs.  Per-tile partials go to a
+//                [B,T,6+C,N] buffer which a finalize kernel sums in a fixed order (no
+//                float atomics anywhere, bit-reproducible).
+//   * separable grids (x independent of the row, y independent of the column: every
+//     linspace grid) let both kernels hoist the row/column part of the quadratic form and
+//     of the moment sums: 3 VALU ops per pair for q instead of 7, 5 instead of 9 for the
+//     moments.
+// exp() is one v_exp_f32: A, 2B, D are pre-multiplied by -0.5 log2(e) when packed.
+// Streams of uniform records are software-pipelined by hand: the next group of records is
+// requested right after the wait for the current one, so the scalar-load latency is
+// covered by the current group's VALU work.  Record arrays are zero-padded (alpha = 0 /
+// g^ = 0 records contribute exactly 0) so the hot loops have no tails.
+//
+// Build flags disable packed-fp32 instruction selection (-packed-fp32-ops), so every VALU
+// op below is a scalar-per-lane fp32 op.
+
+#include <hip/hip_runtime.h>
+
+#include <stdint.h>
+
+#include "igs_hip.h"
+
+namespace {
+
+constexpr float kNegHalfLog2e = -0.72134752044448170368f;  // -0.5 * log2(e)
+constexpr int kThreads = 256;
+constexpr int kFwdSepP = 8;  // rows per lane, separable forward
+constexpr int kFwdGenP = 4;  // pixels per lane, general forward
+constexpr int kBwdG = 2;     // Gaussians per lane, backward
+
+__host__ __device__ constexpr int rec_stride_of(int C) { return (6 + C + 3) & ~3; }
+__host__ __device__ constexpr int pix_stride_sep(int C) { return (C + 1 + 3) & ~3; }
+__host__ __device__ constexpr int pix_stride_gen(int C) { return (C + 3 + 3) & ~3; }
+
+__device__ __forceinline__ float hw_exp2(float v) { return __builtin_amdgcn_exp2f(v); }
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Map the linear
+// block id so that every XCD walks one contiguous range of tiles (same image -> the same
+// packed Gaussian records stay hot in that XCD's L2).  Launch 8*ceil(total/8) blocks and
+// skip results >= total.
+__device__ __forceinline__ int xcd_contiguous(int linear, int total) {
+    const int per = (total + 7) >> 3;
+    return (linear & 7) * per + (linear >> 3);
+}
+
+// ----------------------------------------------------------------------------- pack
+// One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
+// with A' = k A, B2' = 2 k B, D' = k D, k = -0.5 log2 e.  Records N..Np-1 are zero.
+template <bool kScaleRot>
+__global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ position,
+                                                   const float* __restrict__ p0,  // cov00 | scales
+                                                   const float* __restrict__ p1,  // cov01 | rotations
+                                                   const float* __restrict__ p2,  // cov11 | unused
+                                                   const float* __restrict__ alphas,
+                                                   const float* __restrict__ colors, int N,
+                                                   int Np, int C, int RS, float eps,
+                                                   float* __restrict__ packed) {
+    const int n = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (n >= Np) return;
+    float* r = packed + ((size_t)b * Np + n) * RS;
+    if (n >= N) {  // padding: alpha = 0 and e = exp2(0) = 1, so it contributes exactly 0
+        for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        return;
+    }
+    const size_t i = (size_t)b * N + n;
+    float A, Bc, D;
+    if (kScaleRot) {
+        const float s0 = p0[2 * i], s1 = p0[2 * i + 1];
+        float sn, cs;
+        sincosf(p1[i], &sn, &cs);
+        const float i0 = 1.0f / (s0 * s0 + eps), i1 = 1.0f / (s1 * s1 + eps);
+        A = cs * cs * i0 + sn * sn * i1;
+        Bc = cs * sn * (i0 - i1);
+        D = sn * sn * i0 + cs * cs * i1;
+    } else {
+        A = p0[i];
+        Bc = p1[i];
+        D = p2[i];
+    }
+    const float al = alphas[i];
+    r[0] = position[2 * i];
+    r[1] = position[2 * i + 1];
+    r[2] = kNegHalfLog2e * A;
+    r[3] = 2.0f * kNegHalfLog2e * Bc;
+    r[4] = kNegHalfLog2e * D;
+    r[5] = al;
+    for (int c = 0; c < C; ++c) r[6 + c] = al * colors[i * C + c];
+    for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
+}
+
+// ----------------------------------------------------------------------------- forward
+struct FwdArgs {
+    const float* packed;  // [B][Np][RS]
+    const float* x;
+    const float* y;
+    long sxb, sxh, sxw, syb, syh, syw;
+    int B, Np, H, W;
+    int n_per_split, S;  // n_per_split % 4 == 0
+    int tiles_x, tiles_y, total_tiles, wx;
+    float eps;
+    float* out;
+    float* den;
+    float* part;  // [S][B][C+1][HW] when S > 1
+};
+
+template <int C>
+struct GRec {
+    float px, py, A, B2, D, al;
+    float ac[C];
+};
+
+template <int C>
+__device__ __forceinline__ GRec<C> load_grec(const float* __restrict__ r) {
+    GRec<C> g;
+    g.px = r[0];
+    g.py = r[1];
+    g.A = r[2];
+    g.B2 = r[3];
+    g.D = r[4];
+    g.al = r[5];
+#pragma unroll
+    for (int c = 0; c < C; ++c) g.ac[c] = r[6 + c];
+    return g;
+}
+
+// Walks `groups` groups of 4 consecutive records starting at rec, two records in flight
+// ahead of the two being consumed.  f(const GRec<C>&) is the per-Gaussian body.
+template <int C, class F>
+__device__ __forceinline__ void stream_gaussians(const float* __restrict__ rec, int groups, F&& f) {
+    constexpr int RS = rec_stride_of(C);
+    GRec<C> a0 = load_grec<C>(rec), a1 = load_grec<C>(rec + RS);
+    for (int i = 0; i < groups; ++i) {
+        const GRec<C> b0 = load_grec<C>(rec + 2 * RS), b1 = load_grec<C>(rec + 3 * RS);
+        f(a0);
+        f(a1);
+        const float* nxt = (i + 1 < groups) ? rec + 4 * RS : rec;  // last: harmless re-read
+        a0 = load_grec<C>(nxt);
+        a1 = load_grec<C>(nxt + RS);
+        f(b0);
+        f(b1);
+        rec = nxt;
+    }
+}
+
+template <int C>
+__device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p, float dsum,
+                                          const float (&num)[C]) {
+    const size_t HW = (size_t)a.H * a.W;
+    if (a.S == 1) {
+        const float inv = 1.0f / (dsum + a.eps);
+        a.den[(size_t)b * HW + p] = dsum;
+#pragma unroll
+        for (int c = 0; c < C; ++c) a.out[((size_t)b * C + c) * HW + p] = num[c] * inv;
+    } else {
+        float* dst = a.part + ((size_t)s * a.B + b) * (C + 1) * HW + p;
+#pragma unroll
+        for (int c = 0; c < C; ++c) dst[(size_t)c * HW] = num[c];
+        dst[(size_t)C * HW] = dsum;
+    }
+}
+
+// Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows;
+// workgroup = wx x (4/wx) waves.  Per Gaussian and lane: dx, A'dx^2, B2'dx once, then per
+// pixel dy, 2 fma, exp2, 1 + C fma.
+template <int C, int P>
+__global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
+    constexpr int RS = rec_stride_of(C);
+    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
+    if (tile >= a.total_tiles) return;
+    const int per_img = a.tiles_x * a.tiles_y;
+    const int b = tile / per_img;
+    const int tl = tile - b * per_img;
+    const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int wxi = wave % a.wx, wyi = wave / a.wx;
+    const int col0 = (tx * a.wx + wxi) * 64;
+    const int row0 = (ty * (4 / a.wx) + wyi) * P;
+    if (row0 >= a.H || col0 >= a.W) return;  // wave-uniform
+    const int col = col0 + lane;
+    const float xv = a.x[b * a.sxb + (long)min(col, a.W - 1) * a.sxw];
+    float yv[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) yv[p] = a.y[b * a.syb + (long)min(row0 + p, a.H - 1) * a.syh];
+
+    float dsum[P], num[P][C];
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        dsum[p] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) num[p][c] = 0.0f;
+    }
+    const int s = blockIdx.y;
+    const int n0 = s * a.n_per_split;
+    const int n1 = min(a.Np, n0 + a.n_per_split);
+    stream_gaussians<C>(a.packed + ((size_t)b * a.Np + n0) * RS, (n1 - n0) >> 2,
+                        [&](const GRec<C>& g) {
+                            const float dx = xv - g.px;
+                            const float adx = g.A * dx;
+                            const float c0 = adx * dx;
+                            const float c1 = g.B2 * dx;
+#pragma unroll
+                            for (int p = 0; p < P; ++p) {
+                                const float dy = yv[p] - g.py;
+                                const float t = fmaf(g.D, dy, c1);
+                                const float q = fmaf(t, dy, c0);
+                                const float e = hw_exp2(q);
+                                dsum[p] = fmaf(e, g.al, dsum[p]);
+#pragma unroll
+                                for (int c = 0; c < C; ++c) num[p][c] = fmaf(e, g.ac[c], num[p][c]);
+                            }
+                        });
+    if (col < a.W) {
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+            if (row0 + p < a.H) fwd_store<C>(a, b, s, (row0 + p) * a.W + col, dsum[p], num[p]);
+    }
+}
+
+// General grid: lane = P pixels of a flat 256*P pixel tile.
+template <int C, int P>
+__global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
+    constexpr int RS = rec_stride_of(C);
+    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
+    if (tile >= a.total_tiles) return;
+    const int per_img = a.tiles_x;
+    const int b = tile / per_img;
+    const int tl = tile - b * per_img;
+    const int HW = a.H * a.W;
+    float xv[P], yv[P];
+    int pix[P];
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+        pix[j] = tl * (kThreads * P) + j * kThreads + threadIdx.x;
+        const int pc = min(pix[j], HW - 1);
+        const int h = pc / a.W, w = pc - h * a.W;
+        xv[j] = a.x[b * a.sxb + h * a.sxh + w * a.sxw];
+        yv[j] = a.y[b * a.syb + h * a.syh + w * a.syw];
+    }
+    float dsum[P], num[P][C];
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+        dsum[j] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) num[j][c] = 0.0f;
+    }
+    const int s = blockIdx.y;
+    const int n0 = s * a.n_per_split;
+    const int n1 = min(a.Np, n0 + a.n_per_split);
+    stream_gaussians<C>(a.packed + ((size_t)b * a.Np + n0) * RS, (n1 - n0) >> 2,
+                        [&](const GRec<C>& g) {
+#pragma unroll
+                            for (int j = 0; j < P; ++j) {
+                                const float dx = xv[j] - g.px;
+                                const float dy = yv[j] - g.py;
+                                float t = g.A * dx;
+                                t = fmaf(g.B2, dy, t);
+                                const float v = g.D * dy;
+                                float q = t * dx;
+                                q = fmaf(v, dy, q);
+                                const float e = hw_exp2(q);
+                                dsum[j] = fmaf(e, g.al, dsum[j]);
+#pragma unroll
+                                for (int c = 0; c < C; ++c) num[j][c] = fmaf(e, g.ac[c], num[j][c]);
+                            }
+                        });
+#pragma unroll
+    for (int j = 0; j < P; ++j)
+        if (pix[j] < HW) fwd_store<C>(a, b, s, pix[j], dsum[j], num[j]);
+}
+
+// Split-N combine: fixed-order sum over the S partial images, then normalise.
+__global__ __launch_bounds__(kThreads) void k_fwd_combine(const float* __restrict__ part, int S,
+                                                          int B, int C, int HW, float eps,
+                                                          float* __restrict__ out,
+                                                          float* __restrict__ den) {
+    const int p = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (p >= HW) return;
+    float d = 0.0f;
+    for (int s = 0; s < S; ++s) d += part[(((size_t)s * B + b) * (C + 1) + C) * HW + p];
+    den[(size_t)b * HW + p] = d;
+    const float inv = 1.0f / (d + eps);
+    for (int c = 0; c < C; ++c) {
+        float v = 0.0f;
+        for (int s = 0; s < S; ++s) v += part[(((size_t)s * B + b) * (C + 1) + c) * HW + p];
+        out[((size_t)b * C + c) * HW + p] = v * inv;
+    }
+}
+
+// ----------------------------------------------------------------------------- backward
+// Prologue, one thread per (padded) pixel: g^_c = g_c / (den + eps), s = <g^, out>.
+//   separable: records [B][H][Wp][CP] = g^_0..g^_{C-1}, -s, 0..; columns W..Wp-1 are zero
+//              records; followed by the compact column coordinates xs [B][Wp]
+//              (padding columns repeat x of column W-1).
+//   general  : records [B][HWp][CP] = x, y, g^.., -s, 0..; padding pixels are zero records
+//              carrying the coordinates of the last pixel.
+template <int C, bool kSep>
+__global__ __launch_bounds__(kThreads) void k_bwd_pix(const float* __restrict__ out,
+                                                      const float* __restrict__ den,
+                                                      const float* __restrict__ gout,
+                                                      const float* __restrict__ x,
+                                                      const float* __restrict__ y, long sxb,
+                                                      long sxh, long sxw, long syb, long syh,
+                                                      long syw, int B, int H, int W, int Wp,
+                                                      int HWp, float eps,
+                                                      float* __restrict__ pixrec) {
+    constexpr int CP = kSep ? pix_stride_sep(C) : pix_stride_gen(C);
+    constexpr int OFF = kSep ? 0 : 2;
+    const int HW = H * W;
+    const int i = blockIdx.x * kThreads + threadIdx.x;  // padded pixel index
+    const int b = blockIdx.y;
+    int h, w;
+    bool valid;
+    if (kSep) {
+        if (i >= H * Wp) return;
+        h = i / Wp;
+        w = i - h * Wp;
+        valid = w < W;
+        if (h == 0) {
+            float* xs = pixrec + (size_t)B * H * Wp * CP;
+            xs[(size_t)b * Wp + w] = x[b * sxb + (long)min(w, W - 1) * sxw];
+        }
+    } else {
+        if (i >= HWp) return;
+        valid = i < HW;
+        const int pc = min(i, HW - 1);
+        h = pc / W;
+        w = pc - h * W;
+    }
+    float r[CP];
+#pragma unroll
+    for (int k = 0; k < CP; ++k) r[k] = 0.0f;
+    if (valid) {
+        const int p = h * W + w;
+        const float inv = 1.0f / (den[(size_t)b * HW + p] + eps);
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const float gh = gout[((size_t)b * C + c) * HW + p] * inv;
+            s = fmaf(gh, out[((size_t)b * C + c) * HW + p], s);
+            r[OFF + c] = gh;
+        }
+        r[OFF + C] = -s;
+    }
+    if (!kSep) {
+        r[0] = x[b * sxb + h * sxh + w * sxw];
+        r[1] = y[b * syb + h * syh + w * syw];
+    }
+    const size_t rec = kSep ? ((size_t)b * H * Wp + i) : ((size_t)b * HWp + i);
+    float4* dst = reinterpret_cast<float4*>(pixrec + rec * CP);
+#pragma unroll
+    for (int k = 0; k < CP / 4; ++k)
+        dst[k] = make_float4(r[4 * k], r[4 * k + 1], r[4 * k + 2], r[4 * k + 3]);
+}
+
+struct BwdArgs {
+    const float* packed;  // [B][Np][RS]
+    const float* colors;  // [B][N][C]
+    const float* pixrec;
+    const float* xs;      // separable: [B][Wp]
+    const float* y;
+    long syb, syh;
+    int N, Np, H, W, Wp, HWp;
+    int per_tile;  // rows (separable) or pixels (general, multiple of 256) per tile
+    int T;
+    float* partial;  // [B][T][6+C][N]
+};
+
+// Partial field order: 0 M0 = sum G e, 1 Mx = sum G e dx, 2 My, 3 Mxx, 4 Mxy, 5 Myy,
+// 6+c = sum e g^_c.
+template <int C, int G>
+__device__ __forceinline__ void bwd_store(const BwdArgs& a, int b, int t, const int (&n)[G],
+                                          const float (&M)[G][6], const float (&CG)[G][C]) {
+    constexpr int NF = 6 + C;
+    float* base = a.partial + ((size_t)b * a.T + t) * NF * a.N;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        if (n[g] < a.N) {
+#pragma unroll
+            for (int f = 0; f < 6; ++f) base[(size_t)f * a.N + n[g]] = M[g][f];
+#pragma unroll
+            for (int c = 0; c < C; ++c) base[(size_t)(6 + c) * a.N + n[g]] = CG[g][c];
+        }
+    }
+}
+
+template <int C, int G>
+__device__ __forceinline__ void bwd_load_gaussians(const BwdArgs& a, int b, int (&n)[G],
+                                                   float (&px)[G], float (&py)[G], float (&A)[G],
+                                                   float (&B2)[G], float (&D)[G],
+                                                   float (&col)[G][C]) {
+    constexpr int RS = rec_stride_of(C);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        n[g] = (blockIdx.x * G + g) * kThreads + threadIdx.x;
+        const int nc = min(n[g], a.N - 1);
+        const float* r = a.packed + ((size_t)b * a.Np + nc) * RS;
+        px[g] = r[0];
+        py[g] = r[1];
+        A[g] = r[2];
+        B2[g] = r[3];
+        D[g] = r[4];
+#pragma unroll
+        for (int c = 0; c < C; ++c) col[g][c] = a.colors[((size_t)b * a.N + nc) * C + c];
+    }
+}
+
+// Four consecutive pixel records (uniform -> SGPRs).
+template <int CP>
+struct PixQuad {
+    float v[4][CP];
+};
+
+template <int CP>
+__device__ __forceinline__ PixQuad<CP> load_quad(const float* __restrict__ p) {
+    PixQuad<CP> q;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int k = 0; k < CP; ++k) q.v[j][k] = p[j * CP + k];
+    return q;
+}
+
+// Separable grid: lane = G Gaussians; the tile is a range of full rows.  Per row the dy
+// part of q is hoisted, and row sums R0 = sum G e, R1 = sum G e dx, R2 = sum G e dx^2 (and
+// the colour sums) are folded into the totals once per row.
+template <int C, int G>
+__global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
+    constexpr int CP = pix_stride_sep(C);
+    const int b = blockIdx.z, t = blockIdx.y;
+    int n[G];
+    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
+    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+    float M[G][6], CG[G][C];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int f = 0; f < 6; ++f) M[g][f] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
+    }
+    const int r0 = t * a.per_tile, r1 = min(a.H, r0 + a.per_tile);
+    const float* xrow = a.xs + (size_t)b * a.Wp;
+    const int octs = a.Wp >> 3;  // Wp % 8 == 0
+    for (int r = r0; r < r1; ++r) {
+        const float yv = a.y[b * a.syb + (long)r * a.syh];
+        float dy[G], cyy[G], bdy[G], R0[G], R1[G], R2[G], RC[G][C];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            dy[g] = yv - py[g];
+            const float ddy = D[g] * dy[g];
+            cyy[g] = ddy * dy[g];
+            bdy[g] = B2[g] * dy[g];
+            R0[g] = R1[g] = R2[g] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
+        }
+        auto body = [&](const PixQuad<CP>& pq, const float (&xq)[4]) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const float dx = xq[j] - px[g];
+                    const float tt = fmaf(A[g], dx, bdy[g]);
+                    const float q = fmaf(tt, dx, cyy[g]);
+                    const float e = hw_exp2(q);
+                    float Gv = pq.v[j][0] * col[g][0];
+#pragma unroll
+                    for (int c = 1; c < C; ++c) Gv = fmaf(pq.v[j][c], col[g][c], Gv);
+                    Gv += pq.v[j][C];
+                    const float ge = Gv * e;
+                    R0[g] += ge;
+                    const float t1 = ge * dx;
+                    R1[g] += t1;
+                    R2[g] = fmaf(t1, dx, R2[g]);
+#pragma unroll
+                    for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pq.v[j][c], RC[g][c]);
+                }
+            }
+        };
+        const float* prow = a.pixrec + ((size_t)b * a.H + r) * a.Wp * CP;
+        const float* xp = xrow;
+        PixQuad<CP> qa = load_quad<CP>(prow);
+        float xa[4] = {xp[0], xp[1], xp[2], xp[3]};
+        for (int o = 0; o < octs; ++o) {
+            const PixQuad<CP> qb = load_quad<CP>(prow + 4 * CP);
+            const float xb[4] = {xp[4], xp[5], xp[6], xp[7]};
+            body(qa, xa);
+            const bool more = o + 1 < octs;
+            const float* pn = more ? prow + 8 * CP : prow;  // last: harmless re-read
+            const float* xn = more ? xp + 8 : xp;
+            qa = load_quad<CP>(pn);
+            xa[0] = xn[0]; xa[1] = xn[1]; xa[2] = xn[2]; xa[3] = xn[3];
+            body(qb, xb);
+            prow = pn;
+            xp = xn;
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            M[g][0] += R0[g];
+            M[g][1] += R1[g];
+            M[g][3] += R2[g];
+            M[g][2] = fmaf(dy[g], R0[g], M[g][2]);
+            M[g][4] = fmaf(dy[g], R1[g], M[g][4]);
+            M[g][5] = fmaf(dy[g] * dy[g], R0[g], M[g][5]);
+#pragma unroll
+            for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+        }
+    }
+    bwd_store<C, G>(a, b, t, n, M, CG);
+}
+
+// General grid: the tile is a flat pixel range (multiple of 256); x and y come with the
+// pixel record.  Sums are flushed into the totals every 256 pixels (two-level summation).
+template <int C, int G>
+__global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
+    constexpr int CP = pix_stride_gen(C);
+    const int b = blockIdx.z, t = blockIdx.y;
+    int n[G];
+    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
+    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+    float M[G][6], CG[G][C];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int f = 0; f < 6; ++f) M[g][f] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
+    }
+    const int p0 = t * a.per_tile, p1 = min(a.HWp, p0 + a.per_tile);  // HWp % 4 == 0
+    for (int pc = p0; pc < p1; pc += 256) {
+        const int pe = min(p1, pc + 256);
+        float R[G][6], RC[G][C];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int f = 0; f < 6; ++f) R[g][f] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
+        }
+        const float* prec = a.pixrec + ((size_t)b * a.HWp + pc) * CP;
+        for (int p = pc; p < pe; p += 4, prec += 4 * CP) {
+            const PixQuad<CP> pq = load_quad<CP>(prec);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const float dx = pq.v[j][0] - px[g];
+                    const float dy = pq.v[j][1] - py[g];
+                    float tt = A[g] * dx;
+                    tt = fmaf(B2[g], dy, tt);
+                    const float v = D[g] * dy;
+                    float q = tt * dx;
+                    q = fmaf(v, dy, q);
+                    const float e = hw_exp2(q);
+                    float Gv = pq.v[j][2] * col[g][0];
+#pragma unroll
+                    for (int c = 1; c < C; ++c) Gv = fmaf(pq.v[j][2 + c], col[g][c], Gv);
+                    Gv += pq.v[j][2 + C];
+                    const float ge = Gv * e;
+                    R[g][0] += ge;
+                    const float t1 = ge * dx, t2 = ge * dy;
+                    R[g][1] += t1;
+                    R[g][2] += t2;
+                    R[g][3] = fmaf(t1, dx, R[g][3]);
+                    R[g][4] = fmaf(t1, dy, R[g][4]);
+                    R[g][5] = fmaf(t2, dy, R[g][5]);
+#pragma unroll
+                    for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pq.v[j][2 + c], RC[g][c]);
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int f = 0; f < 6; ++f) M[g][f] += R[g][f];
+#pragma unroll
+            for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+        }
+    }
+    bwd_store<C, G>(a, b, t, n, M, CG);
+}
+
+// Finalize: one thread per Gaussian; sums the T tile partials in order and applies
+//   d alpha = M0, d color_c = alpha CG_c, d px = alpha (A Mx + B My), d py = alpha (B Mx + D My),
+//   dA = -1/2 alpha Mxx, dB = -alpha Mxy, dD = -1/2 alpha Myy,
+// and (function level) the chain rule through A = c^2 i0 + s^2 i1, B = c s (i0 - i1),
+// D = s^2 i0 + c^2 i1, i_k = 1/(s_k^2 + eps).
+template <bool kScaleRot>
+__global__ __launch_bounds__(kThreads) void k_bwd_finalize(
+    const float* __restrict__ partial, int T, const float* __restrict__ p0,
+    const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ alphas,
+    int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
+    float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
+    float* __restrict__ g_col) {
+    const int n = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (n >= N) return;
+    const int NF = 6 + C;
+    const size_t i = (size_t)b * N + n;
+    const float* base = partial + (size_t)b * T * NF * N + n;
+    float M[6];
+#pragma unroll
+    for (int f = 0; f < 6; ++f) {
+        float s = 0.0f;
+        for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + f) * N];
+        M[f] = s;
+    }
+    const float al = alphas[i];
+    float A, Bc, D, cs = 0.f, sn = 0.f, i0 = 0.f, i1 = 0.f, s0 = 0.f, s1 = 0.f;
+    if (kScaleRot) {
+        s0 = p0[2 * i];
+        s1 = p0[2 * i + 1];
+        sincosf(p1[i], &sn, &cs);
+        i0 = 1.0f / (s0 * s0 + eps);
+        i1 = 1.0f / (s1 * s1 + eps);
+        A = cs * cs * i0 + sn * sn * i1;
+        Bc = cs * sn * (i0 - i1);
+        D = sn * sn * i0 + cs * cs * i1;
+    } else {
+        A = p0[i];
+        Bc = p1[i];
+        D = p2[i];
+    }
+    if (g_alpha) g_alpha[i] = M[0];
+    if (g_pos) {
+        g_pos[2 * i] = al * (A * M[1] + Bc * M[2]);
+        g_pos[2 * i + 1] = al * (Bc * M[1] + D * M[2]);
+    }
+    const float gA = -0.5f * al * M[3], gB = -al * M[4], gD = -0.5f * al * M[5];
+    if (kScaleRot) {
+        if (g0) {  // scales [B,N,2]
+            const float gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
+            const float gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
+            g0[2 * i] = gi0 * (-2.0f * s0 * i0 * i0);
+            g0[2 * i + 1] = gi1 * (-2.0f * s1 * i1 * i1);
+        }
+        if (g1) g1[i] = (gD - gA) * 2.0f * Bc + gB * (cs * cs - sn * sn) * (i0 - i1);
+    } else {
+        if (g0) g0[i] = gA;
+        if (g1) g1[i] = gB;
+        if (g2) g2[i] = gD;
+    }
+    if (g_col) {
+        for (int c = 0; c < C; ++c) {
+            float s = 0.0f;
+            for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + 6 + c) * N];
+            g_col[i * C + c] = al * s;
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------- host side
+int g_cached_cus = 0;
+
+int device_cus() {
+    if (g_cached_cus > 0) return g_cached_cus;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    g_cached_cus = cus;
+    return cus;
+}
+
+inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
+
+bool shape_ok(int B, int N, int H, int W) {
+    if (B <= 0 || N <= 0 || H <= 0 || W <= 0) return false;
+    if (B > 65535) return false;
+    if ((long)H * W > (1L << 28) || (long)B * N > (1L << 28)) return false;
+    return true;
+}
+
+struct FwdGeometry {
+    int wx, tiles_x, tiles_y, total_tiles;
+};
+
+FwdGeometry fwd_geometry(int B, int H, int W, bool sep) {
+    FwdGeometry g;
+    if (sep) {
+        // choose the wave arrangement (wx waves along the columns) that wastes the fewest lanes
+        long best = -1;
+        g.wx = 4;
+        for (int wx = 4; wx >= 1; wx >>= 1) {
+            const long cols = (long)ceil_div(W, 64 * wx) * 64 * wx;
+            const long rows = (long)ceil_div(H, kFwdSepP * (4 / wx)) * kFwdSepP * (4 / wx);
+            const long area = cols * rows;
+            if (best < 0 || area < best) {
+                best = area;
+                g.wx = wx;
+            }
+        }
+        g.tiles_x = ceil_div(W, 64 * g.wx);
+        g.tiles_y = ceil_div(H, kFwdSepP * (4 / g.wx));
+    } else {
+        g.wx = 4;
+        g.tiles_x = ceil_div((long)H * W, kThreads * kFwdGenP);
+        g.tiles_y = 1;
+    }
+    g.total_tiles = B * g.tiles_x * g.tiles_y;
+    return g;
+}
+
+int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
+    if (!p) return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, N, H, W)) return IGS_ERR_BAD_SHAPE;
+    if (C < 1 || C > IGS_MAX_CHANNELS) return IGS_ERR_BAD_CHANNELS;
+    if (grid_mode != IGS_GRID_GENERAL && grid_mode != IGS_GRID_SEPARABLE) return IGS_ERR_BAD_MODE;
+    const bool sep = grid_mode == IGS_GRID_SEPARABLE;
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    const long target_waves = (long)cus * 4 * 4;  // 4 waves per SIMD
+    p->B = B; p->N = N; p->H = H; p->W = W; p->C = C;
+    p->rec_stride = rec_stride_of(C);
+    p->n_padded = (N + 3) & ~3;
+    p->w_padded = sep ? (W + 7) & ~7 : W;
+    p->hw_padded = (H * W + 3) & ~3;
+    const FwdGeometry fg = fwd_geometry(B, H, W, sep);
+    long S = (target_waves + (long)fg.total_tiles * 4 - 1) / ((long)fg.total_tiles * 4);
+    const long maxS = N / 64 > 0 ? N / 64 : 1;  // keep >= 64 Gaussians per split
+    if (S > maxS) S = maxS;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    // Gaussians per split: a multiple of 4; drop splits that would be empty
+    const int nps = (ceil_div(p->n_padded, S) + 3) & ~3;
+    S = ceil_div(p->n_padded, nps);
+    p->fwd_split = (int)S;
+    p->fwd_n_per_split = nps;
+    const long groups = (long)B * ceil_div(N, kThreads * kBwdG) * 4;  // waves per tile
+    long T = (target_waves * 2 + groups - 1) / groups;                   // 8 waves per SIMD
+    const long maxT = sep ? H : ceil_div(p->hw_padded, 256);
+    if (T > maxT) T = maxT;
+    if (T < 1) T = 1;
+    if (sep) {
+        p->bwd_per_tile = ceil_div(H, T);
+    } else {
+        p->bwd_per_tile = (ceil_div(p->hw_padded, T) + 255) & ~255;
+    }
+    T = ceil_div(sep ? H : p->hw_padded, p->bwd_per_tile);
+    p->bwd_tiles = (int)T;
+    p->pix_stride = sep ? pix_stride_sep(C) : pix_stride_gen(C);
+    p->packed_bytes = (uint64_t)B * p->n_padded * p->rec_stride * sizeof(float);
+    p->fwd_ws_bytes = S > 1 ? (uint64_t)S * B * (C + 1) * H * W * sizeof(float) : 0;
+    p->pix_bytes = sep ? ((uint64_t)B * H * p->w_padded * p->pix_stride + (uint64_t)B * p->w_padded) * sizeof(float)
+                       : (uint64_t)B * p->hw_padded * p->pix_stride * sizeof(float);
+    p->partial_bytes = (uint64_t)B * T * (6 + C) * N * sizeof(float);
+    return IGS_OK;
+}
+
+inline int launch_status() {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? IGS_OK : (int)e;
+}
+
+template <int C>
+int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
+    const int blocks = ((a.total_tiles + 7) / 8) * 8;
+    const dim3 grid(blocks, a.S, 1);
+    if (sep)
+        hipLaunchKernelGGL((k_fwd_sep<C, kFwdSepP>), grid, dim3(kThreads), 0, st, a);
+    else
+        hipLaunchKernelGGL((k_fwd_gen<C, kFwdGenP>), grid, dim3(kThreads), 0, st, a);
+    return launch_status();
+}
+
+template <int C>
+int launch_backward(const BwdArgs& a, int B, bool sep, const float* out, const float* den,
+                    const float* gout, const float* x, const float* y, const int64_t* gs,
+                    float eps, float* pixrec, hipStream_t st) {
+    const int padded = sep ? a.H * a.Wp : a.HWp;
+    const dim3 pgrid(ceil_div(padded, kThreads), B, 1);
+    if (sep)
+        hipLaunchKernelGGL((k_bwd_pix<C, true>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
+                           gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
+                           pixrec);
+    else
+        hipLaunchKernelGGL((k_bwd_pix<C, false>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
+                           gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
+                           pixrec);
+    int rc = launch_status();
+    if (rc) return rc;
+    const dim3 grid(ceil_div(a.N, kThreads * kBwdG), a.T, B);
+    if (sep)
+        hipLaunchKernelGGL((k_bwd_sep<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
+    else
+        hipLaunchKernelGGL((k_bwd_gen<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
+    return launch_status();
+}
+
+// Channel counts with a compiled specialisation; other C <= 16 are rejected by the ABI
+// (the host wrapper zero-pads colours / grad_out up to the next one, which is exact).
+#define IGS_DISPATCH_C(C, CALL)                          \
+    switch (C) {                                         \
+        case 1: { constexpr int kC = 1; CALL; } break;   \
+        case 2: { constexpr int kC = 2; CALL; } break;   \
+        case 3: { constexpr int kC = 3; CALL; } break;   \
+        case 4: { constexpr int kC = 4; CALL; } break;   \
+        case 8: { constexpr int kC = 8; CALL; } break;   \
+        case 16: { constexpr int kC = 16; CALL; } break; \
+        default: return IGS_ERR_BAD_CHANNELS;            \
+    }
+
+bool channels_compiled(int C) { return C == 1 || C == 2 || C == 3 || C == 4 || C == 8 || C == 16; }
+
+}  // namespace
+
+// ============================================================================= C ABI
+extern "C" {
+
+int igs_abi_version(void) { return IGS_ABI_VERSION; }
+
+const char* igs_status_string(int status) {
+    switch (status) {
+        case IGS_OK: return "ok";
+        case IGS_ERR_NULL_POINTER: return "null pointer argument";
+        case IGS_ERR_BAD_SHAPE: return "bad shape (dimension <= 0 or too large)";
+        case IGS_ERR_BAD_CHANNELS: return "unsupported channel count (compiled: 1, 2, 3, 4, 8, 16)";
+        case IGS_ERR_WORKSPACE: return "workspace smaller than igs_gs2d_plan requires";
+        case IGS_ERR_BAD_MODE: return "unknown grid mode";
+        case IGS_ERR_NO_DEVICE: return "no usable HIP device";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "unknown igs status";
+}
+
+int igs_gs2d_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* plan) {
+    const int rc = make_plan(B, N, H, W, C, grid_mode, plan);
+    if (rc) return rc;
+    return channels_compiled(C) ? IGS_OK : IGS_ERR_BAD_CHANNELS;
+}
+
+int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const float* cov_inv_01,
+                         const float* cov_inv_11, const float* alphas, const float* colors, int B,
+                         int N, int C, float* packed, igs_stream_t stream) {
+    if (!position || !cov_inv_00 || !cov_inv_01 || !cov_inv_11 || !alphas || !colors || !packed)
+        return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
+    if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    const int Np = (N + 3) & ~3;
+    hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
+                       (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
+                       colors, N, Np, C, rec_stride_of(C), 0.0f, packed);
+    return launch_status();
+}
+
+int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const float* rotations,
+                            const float* alphas, const float* colors, int B, int N, int C, float eps,
+                            float* packed, igs_stream_t stream) {
+    if (!positions || !scales || !rotations || !alphas || !colors || !packed)
+        return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
+    if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    const int Np = (N + 3) & ~3;
+    hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
+                       (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
+                       alphas, colors, N, Np, C, rec_stride_of(C), eps, packed);
+    return launch_status();
+}
+
+int igs_gs2d_forward(const float* packed, const float* x, const float* y,
+                     const int64_t grid_strides[6], int grid_mode, int B, int N, int H, int W, int C,
+                     float eps, float* out, float* den, void* ws, size_t ws_bytes,
+                     igs_stream_t stream) {
+    if (!packed || !x || !y || !grid_strides || !out || !den) return IGS_ERR_NULL_POINTER;
+    igs_gs2d_plan_t plan;
+    int rc = make_plan(B, N, H, W, C, grid_mode, &plan);
+    if (rc) return rc;
+    if (plan.fwd_ws_bytes > 0 && (!ws || ws_bytes < plan.fwd_ws_bytes)) return IGS_ERR_WORKSPACE;
+    const bool sep = grid_mode == IGS_GRID_SEPARABLE;
+    const FwdGeometry fg = fwd_geometry(B, H, W, sep);
+    FwdArgs a;
+    a.packed = packed; a.x = x; a.y = y;
+    a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
+    a.syb = grid_strides[3]; a.syh = grid_strides[4]; a.syw = grid_strides[5];
+    a.B = B; a.Np = plan.n_padded; a.H = H; a.W = W;
+    a.S = plan.fwd_split;
+    a.n_per_split = plan.fwd_n_per_split;
+    a.tiles_x = fg.tiles_x; a.tiles_y = fg.tiles_y; a.total_tiles = fg.total_tiles; a.wx = fg.wx;
+    a.eps = eps; a.out = out; a.den = den; a.part = (float*)ws;
+    hipStream_t st = (hipStream_t)stream;
+    IGS_DISPATCH_C(C, rc = launch_forward<kC>(a, sep, st));
+    if (rc) return rc;
+    if (a.S > 1) {
+        hipLaunchKernelGGL(k_fwd_combine, dim3(ceil_div((long)H * W, kThreads), B), dim3(kThreads), 0,
+                           st, (const float*)ws, a.S, B, C, H * W, eps, out, den);
+        rc = launch_status();
+    }
+    return rc;
+}
+
+int igs_gs2d_backward(const float* packed, const float* colors, const float* x, const float* y,
+                      const int64_t grid_strides[6], int grid_mode, const float* out,
+                      const float* den, const float* grad_out, int B, int N, int H, int W, int C,
+                      float eps, float* pix_ws, size_t pix_bytes, float* partial,
+                      size_t partial_bytes, igs_stream_t stream) {
+    if (!packed || !colors || !x || !y || !grid_strides || !out || !den || !grad_out || !pix_ws ||
+        !partial)
+        return IGS_ERR_NULL_POINTER;
+    igs_gs2d_plan_t plan;
+    int rc = make_plan(B, N, H, W, C, grid_mode, &plan);
+    if (rc) return rc;
+    if (pix_bytes < plan.pix_bytes || partial_bytes < plan.partial_bytes) return IGS_ERR_WORKSPACE;
+    const bool sep = grid_mode == IGS_GRID_SEPARABLE;
+    BwdArgs a;
+    a.packed = packed; a.colors = colors; a.pixrec = pix_ws;
+    a.xs = sep ? pix_ws + (size_t)B * H * plan.w_padded * plan.pix_stride : nullptr;
+    a.y = y;
+    a.syb = grid_strides[3]; a.syh = grid_strides[4];
+    a.N = N; a.Np = plan.n_padded; a.H = H; a.W = W; a.Wp = plan.w_padded; a.HWp = plan.hw_padded;
+    a.T = plan.bwd_tiles;
+    a.per_tile = plan.bwd_per_tile;
+    a.partial = partial;
+    hipStream_t st = (hipStream_t)stream;
+    IGS_DISPATCH_C(C, rc = launch_backward<kC>(a, B, sep, out, den, grad_out, x, y, grid_strides, eps, pix_ws, st));
+    return rc;
+}
+
+int igs_gs2d_finalize_covinv(const float* partial, int T, const float* cov_inv_00,
+                             const float* cov_inv_01, const float* cov_inv_11, const float* alphas,
+                             int B, int N, int C, float* g_position, float* g_cov_inv_00,
+                             float* g_cov_inv_01, float* g_cov_inv_11, float* g_alphas,
+                             float* g_colors, igs_stream_t stream) {
+    if (!partial || !cov_inv_00 || !cov_inv_01 || !cov_inv_11 || !alphas) return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, N, 1, 1) || T < 1) return IGS_ERR_BAD_SHAPE;
+    if (C < 1 || C > IGS_MAX_CHANNELS) return IGS_ERR_BAD_CHANNELS;
+    hipLaunchKernelGGL((k_bwd_finalize<false>), dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
+                       (hipStream_t)stream, partial, T, cov_inv_00, cov_inv_01, cov_inv_11, alphas, N,
+                       C, 0.0f, g_position, g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas,
+                       g_colors);
+    return launch_status();
+}
+
+int igs_gs2d_finalize_scale_rot(const float* partial, int T, const float* scales,
+                                const float* rotations, const float* alphas, int B, int N, int C,
+                                float eps, float* g_positions, float* g_scales, float* g_rotations,
+                                float* g_alphas, float* g_colors, igs_stream_t stream) {
+    if (!partial || !scales || !rotations || !alphas) return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, N, 1, 1) || T < 1) return IGS_ERR_BAD_SHAPE;
+    if (C < 1 || C > IGS_MAX_CHANNELS) return IGS_ERR_BAD_CHANNELS;
+    hipLaunchKernelGGL((k_bwd_finalize<true>), dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
+                       (hipStream_t)stream, partial, T, scales, rotations, (const float*)nullptr,
+                       alphas, N, C, eps, g_positions, g_scales, g_rotations, (float*)nullptr,
+                       g_alphas, g_colors);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,134 @@
+/* igs_hip.h -- C ABI of libigs_hip.so: 2-D Gaussian splatting forward/backward for
+ * AMD MI355X (gfx950).
+ *
+ * This is the boundary a host framework binds (ctypes / cffi / pybind / dlopen).  Every
+ * entry point takes plain device pointers and sizes; the library never allocates, frees or
+ * keeps a pointer, never synchronises the device, and launches on the stream it is given.
+ * All tensors are fp32 and dense/contiguous unless a stride argument says otherwise.
+ * Return value: 0 on success, a negative igs_status for a rejected argument, or a positive
+ * hipError_t if a launch failed.  No C++ exception crosses this boundary.
+ *
+ * Reference interfaces replaced (paths relative to the KohakuBlueleaf/IGS checkout):
+ *   - the `.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps)`
+ *     operator, forward + backward: src/igs/gs2d.py:47-262, :265-465,
+ *     src/igs/gs_triton.py:408-640, src/igs/gs_triton_chunked.py:543-924;
+ *   - the covariance-inverse preamble of `render`: src/igs/gs2d.py:548-580.
+ */
+#ifndef IGS_HIP_H
+#define IGS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IGS_ABI_VERSION 1
+#define IGS_MAX_CHANNELS 16
+
+typedef void *igs_stream_t; /* a hipStream_t */
+
+typedef enum igs_status {
+    IGS_OK = 0,
+    IGS_ERR_NULL_POINTER = -1,
+    IGS_ERR_BAD_SHAPE = -2,      /* a dimension <= 0 or too large for 32-bit indexing */
+    IGS_ERR_BAD_CHANNELS = -3,   /* C outside 1..IGS_MAX_CHANNELS */
+    IGS_ERR_WORKSPACE = -4,      /* a workspace is smaller than igs_gs2d_plan says */
+    IGS_ERR_BAD_MODE = -5,       /* unknown grid mode */
+    IGS_ERR_NO_DEVICE = -6       /* no usable HIP device */
+} igs_status;
+
+/* How the pixel coordinates are described.
+ * x(b,h,w) = x[b*sxb + h*sxh + w*sxw], y likewise with (syb, syh, syw); strides are in
+ * elements and may be 0 (expanded tensors).
+ *   IGS_GRID_GENERAL   : arbitrary per-pixel coordinates (what the reference operator
+ *                        accepts, src/igs/gs2d.py:82-83).
+ *   IGS_GRID_SEPARABLE : the caller guarantees x does not depend on h and y does not
+ *                        depend on w (every linspace/meshgrid grid, e.g. xy_grid,
+ *                        src/igs/gs2d.py:503-522).  sxh and syw are then ignored and the
+ *                        kernels factor the quadratic form by rows/columns.
+ */
+typedef enum igs_grid_mode { IGS_GRID_GENERAL = 0, IGS_GRID_SEPARABLE = 1 } igs_grid_mode;
+
+/* Launch plan and workspace sizes for one problem shape (filled by igs_gs2d_plan). */
+typedef struct igs_gs2d_plan_t {
+    int32_t B, N, H, W, C;
+    int32_t rec_stride;      /* floats per packed Gaussian record                          */
+    int32_t n_padded;        /* records per image in the packed buffer (N rounded up to 4) */
+    int32_t w_padded;        /* separable: pixel-record columns per row (W rounded up to 8)*/
+    int32_t hw_padded;       /* general: pixel records per image (H*W rounded up to 4)     */
+    int32_t fwd_split;       /* number of Gaussian-range splits of the forward (>= 1)      */
+    int32_t fwd_n_per_split; /* records per split (multiple of 4)                          */
+    int32_t bwd_tiles;       /* number of pixel tiles T of the backward partial buffer     */
+    int32_t bwd_per_tile;    /* rows (separable) or pixels (general) per backward tile     */
+    int32_t pix_stride;      /* floats per pixel record of the backward prologue           */
+    uint64_t packed_bytes;   /* packed Gaussian buffer: B*n_padded*rec_stride*4            */
+    uint64_t fwd_ws_bytes;   /* forward split workspace (0 when fwd_split == 1)            */
+    uint64_t pix_bytes;      /* backward per-pixel buffer                                  */
+    uint64_t partial_bytes;  /* backward partial sums: B*T*(6+C)*N*4                       */
+} igs_gs2d_plan_t;
+
+int igs_abi_version(void);
+const char *igs_status_string(int status);
+
+/* Shape -> launch plan + workspace sizes.  Pure host arithmetic apart from a cached
+ * query of the current device's compute-unit count.  grid_mode is an igs_grid_mode. */
+int igs_gs2d_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t *plan);
+
+/* Pack per-Gaussian parameters for the kernels (operator level: the caller already has
+ * the inverse covariance).  position [B,N,2]; cov_inv_00/01/11 [B,N]; alphas [B,N];
+ * colors [B,N,C]; packed: plan.packed_bytes.  Replaces nothing in the reference (its
+ * kernels read the tensors directly); it exists so the hot loops read one record. */
+int igs_gs2d_pack_covinv(const float *position, const float *cov_inv_00, const float *cov_inv_01,
+                         const float *cov_inv_11, const float *alphas, const float *colors,
+                         int B, int N, int C, float *packed, igs_stream_t stream);
+
+/* Same, from scales [B,N,2] and rotations [B,N]: closed form of
+ * (R S S^T R^T + eps I)^-1, replacing src/igs/gs2d.py:548-580. */
+int igs_gs2d_pack_scale_rot(const float *positions, const float *scales, const float *rotations,
+                            const float *alphas, const float *colors, int B, int N, int C,
+                            float eps, float *packed, igs_stream_t stream);
+
+/* Forward: out [B,C,H,W] = sum_n w_n c_n / (sum_n w_n + eps), den [B,H,W] = sum_n w_n.
+ * Replaces the forward of src/igs/gs2d.py:68-144 / src/igs/gs_triton_chunked.py:551-680.
+ * grid_strides = {sxb, sxh, sxw, syb, syh, syw}.  ws: plan.fwd_ws_bytes (may be NULL when
+ * that is 0). */
+int igs_gs2d_forward(const float *packed, const float *x, const float *y,
+                     const int64_t grid_strides[6], int grid_mode, int B, int N, int H, int W,
+                     int C, float eps, float *out, float *den, void *ws, size_t ws_bytes,
+                     igs_stream_t stream);
+
+/* Backward, stage 1 and 2: per-pixel prologue (g^ = grad_out/(den+eps), s = <g^, out>)
+ * and the recomputing per-Gaussian reduction over pixel tiles into `partial`.
+ * Replaces the backward of src/igs/gs2d.py:146-262 / src/igs/gs_triton.py:159-405.
+ * colors [B,N,C]; out, grad_out [B,C,H,W]; den [B,H,W]; pix_ws: plan.pix_bytes;
+ * partial: plan.partial_bytes.  Neither grad_out nor out/den are modified. */
+int igs_gs2d_backward(const float *packed, const float *colors, const float *x, const float *y,
+                      const int64_t grid_strides[6], int grid_mode, const float *out,
+                      const float *den, const float *grad_out, int B, int N, int H, int W, int C,
+                      float eps, float *pix_ws, size_t pix_bytes, float *partial,
+                      size_t partial_bytes, igs_stream_t stream);
+
+/* Backward, stage 3 (operator level): fixed-order sum of the tile partials and the
+ * gradients of the operator inputs.  Any output pointer may be NULL (not wanted).
+ * g_position [B,N,2]; g_cov_inv_* [B,N]; g_alphas [B,N]; g_colors [B,N,C]. */
+int igs_gs2d_finalize_covinv(const float *partial, int T, const float *cov_inv_00,
+                             const float *cov_inv_01, const float *cov_inv_11,
+                             const float *alphas, int B, int N, int C, float *g_position,
+                             float *g_cov_inv_00, float *g_cov_inv_01, float *g_cov_inv_11,
+                             float *g_alphas, float *g_colors, igs_stream_t stream);
+
+/* Backward, stage 3 (function level): as above plus the chain rule through the closed-form
+ * covariance inverse to scales [B,N,2] and rotations [B,N] (the autograd of
+ * src/igs/gs2d.py:548-580). */
+int igs_gs2d_finalize_scale_rot(const float *partial, int T, const float *scales,
+                                const float *rotations, const float *alphas, int B, int N, int C,
+                                float eps, float *g_positions, float *g_scales,
+                                float *g_rotations, float *g_alphas, float *g_colors,
+                                igs_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IGS_HIP_H */
