@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Benchmark of the 2-D Gaussian-splatting hot path on one MI355X.
+
+A "step" is one forward + one backward of `gaussian_splatting_2d` over one batch of
+synthetic inputs (already resident in HBM) at the headline configuration
+B=16, N=8192, 256x256, C=3, fp32.  Prints ONE JSON line:
+
+  metric/value : Gaussian-pixel evaluations per second, forward+backward = B*N*H*W / t_step
+  roofline     : the dominant kernel (backward per-Gaussian reduction), algorithmic FLOPs per
+                 launch / its HIP-event-timed launch duration, against the fp32 vector peak
+  cpu_baseline : the chunked torch autograd path of the reference restated on the CPU
+                 (oracle/chunked_cpu.py), timed on this box's host cores on a bounded sample.
+
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) peak
+
+
+def flops_per_pair(C: int):
+    """Algorithmic FLOPs per Gaussian-pixel pair (FMA = 2, exp = 1)."""
+    return 12 + 2 * C, 30 + 4 * C
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c4"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards over the batch with no "
+              "exchange; no multi-GPU run is part of it). Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import igs_amd
+    from igs_amd import _lib
+    from igs_amd.gs2d import _Grid, _Splat, _ptr, _stream
+    from oracle import gs2d_oracle as O
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    d = {k: v.to(dev) for k, v in O.make_config_inputs(args.config).items()}
+    B, N, C = d["colors"].shape
+    H, W = d["x_grid"].shape[-2:]
+    # the configuration's grids are linspaces *expanded* to [B,1,H,W]; .to(device) materialises
+    # them, so restore the stride-0 form on the device
+    d["x_grid"] = d["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+    d["y_grid"] = d["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+    pairs = B * N * H * W
+    names = ("positions", "colors", "scales", "rotations", "alphas")
+    leaves = {k: d[k].clone().requires_grad_(True) for k in names}
+
+    def forward():
+        return igs_amd.gaussian_splatting_2d(leaves["positions"], leaves["colors"], leaves["scales"],
+                                             leaves["rotations"], leaves["alphas"], d["x_grid"], d["y_grid"])
+
+    def step():
+        out = forward()
+        out.backward(d["grad_out"])
+        for v in leaves.values():
+            v.grad = None
+
+    # ---- whole step: W warm-ups, then exactly K steps between two synchronisations
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t_step = (time.perf_counter() - t0) / args.steps
+
+    # ---- forward only (reported next to it)
+    with torch.no_grad():
+        for _ in range(3):
+            forward()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            forward()
+        torch.cuda.synchronize()
+        t_fwd = (time.perf_counter() - t0) / args.steps
+
+    # ---- dominant kernel alone, HIP events on the stream it is launched on
+    grid = _Grid(d["x_grid"], d["y_grid"], B)
+    op = _Splat(B, N, C, grid, 1e-6, dev)
+    f32 = lambda t: t.detach().float().contiguous()
+    col = f32(d["colors"])
+    packed = op.pack_scale_rot(f32(d["positions"]), f32(d["scales"]), f32(d["rotations"]), f32(d["alphas"]), col)
+    out, den = op.forward(packed)
+    pix = op._empty(op.plan.pix_bytes)
+    partial = op._empty(op.plan.partial_bytes)
+    lib = _lib.load()
+    st = _stream(dev)
+    _lib.check(lib.igs_gs2d_backward_prologue(_ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode, _ptr(grid.flag),
+                                              _ptr(out),
+                                              _ptr(den), _ptr(f32(d["grad_out"])), B, N, H, W, C, 1e-6, _ptr(pix),
+                                              int(op.plan.pix_bytes), st), "prologue")
+
+    def reduce_kernel():
+        _lib.check(lib.igs_gs2d_backward_reduce(_ptr(packed), _ptr(col), _ptr(grid.y), grid.strides, grid.mode,
+                                                _ptr(grid.flag), B, N,
+                                                H, W, C, _ptr(pix), int(op.plan.pix_bytes), _ptr(partial),
+                                                int(op.plan.partial_bytes), st), "reduce")
+
+    def fwd_kernel():
+        op.forward(packed)
+
+    def event_time(fn, reps):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(torch.cuda.current_stream(dev))
+        for _ in range(reps):
+            fn()
+        e1.record(torch.cuda.current_stream(dev))
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    t_bwd_kernel = event_time(reduce_kernel, args.steps)
+    t_fwd_kernel = event_time(fwd_kernel, args.steps)
+    f_fwd, f_bwd = flops_per_pair(C)
+    achieved = pairs * f_bwd / t_bwd_kernel / 1e12
+
+    result = {
+        "metric": "gaussian_pixel_evals_per_sec_fwd_bwd",
+        "value": pairs / t_step,
+        "unit": "pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": t_step * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{args.config}: gaussian_splatting_2d fwd+bwd, B={B} N={N} {H}x{W} C={C} fp32, "
+                               "linspace grids, seeded U/N inputs", "B": B, "N": N, "H": H, "W": W, "C": C},
+        "fwd_pairs_per_s": pairs / t_fwd,
+        "fwd_ms": t_fwd * 1e3,
+        "step_tflops": pairs * (f_fwd + f_bwd) / t_step / 1e12,
+        "step_frac_of_fp32_vector_peak": pairs * (f_fwd + f_bwd) / t_step / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+        "roofline": {
+            "bound": "valu",
+            "kernel": "k_bwd_sep<3,2> (backward per-Gaussian reduction)" if C == 3 else f"k_bwd_sep<{C},2>",
+            "achieved": achieved,
+            "peak": FP32_VECTOR_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / FP32_VECTOR_PEAK_TFLOPS,
+            "flops_per_pair": f_bwd,
+            "pairs_per_launch": pairs,
+            "launch_ms": t_bwd_kernel * 1e3,
+            "traffic": None,
+            "forward_kernel": {"launch_ms": t_fwd_kernel * 1e3, "flops_per_pair": f_fwd,
+                               "achieved": pairs * f_fwd / t_fwd_kernel / 1e12,
+                               "frac": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS},
+            "note": "peak = published fp32 vector peak (packed FMA); this build compiles with packed-fp32 "
+                    "instruction selection disabled, so its own issue ceiling is half of it",
+        },
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(args.config, O)
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+def cpu_baseline(config: str, O):
+    """Chunked torch autograd path on the host cores, one image of the same workload."""
+    import torch
+
+    from oracle.chunked_cpu import render_chunked_cpu
+
+    threads = torch.get_num_threads()
+    d = O.make_config_inputs(config, B=1)
+    B, N, C = d["colors"].shape
+    H, W = d["x_grid"].shape[-2:]
+    if config == "c4":
+        d = O.make_config_inputs(config, B=1, N=N // 8)
+        N = N // 8
+    names = ("positions", "colors", "scales", "rotations", "alphas")
+    leaves = {k: d[k].clone().requires_grad_(True) for k in names}
+    xg, yg = d["x_grid"].contiguous(), d["y_grid"].contiguous()
+
+    def run():
+        out = render_chunked_cpu(leaves["positions"], leaves["colors"], leaves["scales"], leaves["rotations"],
+                                 leaves["alphas"], xg, yg)
+        out.backward(d["grad_out"])
+        for v in leaves.values():
+            v.grad = None
+
+    # warm-up on a 1/16 slice of the Gaussians, then one timed pass
+    small = {k: v[:, : max(N // 16, 32)].detach().clone().requires_grad_(True) for k, v in leaves.items()}
+    o = render_chunked_cpu(small["positions"], small["colors"], small["scales"], small["rotations"], small["alphas"], xg, yg)
+    o.backward(d["grad_out"])
+    t0 = time.perf_counter()
+    run()
+    t = time.perf_counter() - t0
+    pairs = B * N * H * W
+    return {"value": pairs / t, "unit": "pairs/s", "cores": threads, "kind": "port",
+            "sample": f"one image of {config} (B=1, N={N}, {H}x{W}, C={C}), fwd+bwd once, {t:.1f} s, "
+                      f"eager torch fp32 with {threads} threads"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

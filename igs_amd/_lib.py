@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libigs_hip.
 
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1
+IGS_GRID_AUTO = 2
 IGS_MAX_CHANNELS = 16
 COMPILED_CHANNELS = (1, 2, 3, 4, 8, 16)
 
@@ -48,14 +49,19 @@ SIGNATURES = {
     "igs_gs2d_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, POINTER(Plan)]),
     "igs_gs2d_pack_covinv": (c_int, [_FP, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, _FP, c_void_p]),
     "igs_gs2d_pack_scale_rot": (c_int, [_FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, _FP, c_void_p]),
-    "igs_gs2d_forward": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, c_int, c_int, c_int, c_int, c_int,
+    "igs_gs2d_grid_classify": (c_int, [_FP, _FP, _STRIDES, c_int, c_int, c_int, _FP, c_void_p]),
+    "igs_gs2d_forward": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
                                  c_float, _FP, _FP, c_void_p, c_size_t, c_void_p]),
-    "igs_gs2d_backward": (c_int, [_FP, _FP, _FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, c_int, c_int,
+    "igs_gs2d_backward_prologue": (c_int, [_FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int,
+                                           c_int, c_int, c_float, _FP, c_size_t, c_void_p]),
+    "igs_gs2d_backward_reduce": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
+                                         _FP, c_size_t, _FP, c_size_t, c_void_p]),
+    "igs_gs2d_backward": (c_int, [_FP, _FP, _FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int,
                                   c_int, c_int, c_int, c_float, _FP, c_size_t, _FP, c_size_t, c_void_p]),
-    "igs_gs2d_finalize_covinv": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int,
+    "igs_gs2d_finalize_covinv": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                          _FP, _FP, _FP, _FP, _FP, _FP, c_void_p]),
-    "igs_gs2d_finalize_scale_rot": (c_int, [_FP, c_int, _FP, _FP, _FP, c_int, c_int, c_int, c_float,
-                                            _FP, _FP, _FP, _FP, _FP, c_void_p]),
+    "igs_gs2d_finalize_scale_rot": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
+                                            c_float, _FP, _FP, _FP, _FP, _FP, c_void_p]),
 }
 
 _lib = None

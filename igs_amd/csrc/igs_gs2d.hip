@@ -117,7 +117,14 @@ struct FwdArgs {
     float* out;
     float* den;
     float* part;  // [S][B][C+1][HW] when S > 1
+    const int* flag;  // AUTO grid mode: run only if *flag == want (nullptr: always run)
+    int want;
 };
+
+// AUTO grid mode launches both the separable and the general variant of a kernel; the
+// device-side classification flag (1 = separable) decides which one does the work.
+#define IGS_GATE(a) \
+    if ((a).flag != nullptr && *(a).flag != (a).want) return
 
 template <int C>
 struct GRec {
@@ -181,6 +188,7 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 template <int C, int P>
 __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     constexpr int RS = rec_stride_of(C);
+    IGS_GATE(a);
     const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
     if (tile >= a.total_tiles) return;
     const int per_img = a.tiles_x * a.tiles_y;
@@ -237,6 +245,7 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
 template <int C, int P>
 __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
     constexpr int RS = rec_stride_of(C);
+    IGS_GATE(a);
     const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
     if (tile >= a.total_tiles) return;
     const int per_img = a.tiles_x;
@@ -289,7 +298,9 @@ __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
 __global__ __launch_bounds__(kThreads) void k_fwd_combine(const float* __restrict__ part, int S,
                                                           int B, int C, int HW, float eps,
                                                           float* __restrict__ out,
-                                                          float* __restrict__ den) {
+                                                          float* __restrict__ den,
+                                                          const int* __restrict__ flag, int want) {
+    if (flag != nullptr && *flag != want) return;
     const int p = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (p >= HW) return;
@@ -320,9 +331,11 @@ __global__ __launch_bounds__(kThreads) void k_bwd_pix(const float* __restrict__ 
                                                       long sxh, long sxw, long syb, long syh,
                                                       long syw, int B, int H, int W, int Wp,
                                                       int HWp, float eps,
-                                                      float* __restrict__ pixrec) {
+                                                      float* __restrict__ pixrec,
+                                                      const int* __restrict__ flag, int want) {
     constexpr int CP = kSep ? pix_stride_sep(C) : pix_stride_gen(C);
     constexpr int OFF = kSep ? 0 : 2;
+    if (flag != nullptr && *flag != want) return;
     const int HW = H * W;
     const int i = blockIdx.x * kThreads + threadIdx.x;  // padded pixel index
     const int b = blockIdx.y;
@@ -381,6 +394,8 @@ struct BwdArgs {
     int per_tile;  // rows (separable) or pixels (general, multiple of 256) per tile
     int T;
     float* partial;  // [B][T][6+C][N]
+    const int* flag;
+    int want;
 };
 
 // Partial field order: 0 M0 = sum G e, 1 Mx = sum G e dx, 2 My, 3 Mxx, 4 Mxy, 5 Myy,
@@ -444,6 +459,7 @@ __device__ __forceinline__ PixQuad<CP> load_quad(const float* __restrict__ p) {
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     constexpr int CP = pix_stride_sep(C);
+    IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
     int n[G];
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
@@ -532,6 +548,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     constexpr int CP = pix_stride_gen(C);
+    IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
     int n[G];
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
@@ -605,7 +622,8 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
 // D = s^2 i0 + c^2 i1, i_k = 1/(s_k^2 + eps).
 template <bool kScaleRot>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
-    const float* __restrict__ partial, int T, const float* __restrict__ p0,
+    const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
+    const float* __restrict__ p0,
     const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ alphas,
     int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
@@ -613,6 +631,8 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n >= N) return;
+    // AUTO grid mode: T_in belongs to the separable plan, T_alt to the general one
+    const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + C;
     const size_t i = (size_t)b * N + n;
     const float* base = partial + (size_t)b * T * NF * N + n;
@@ -667,6 +687,28 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     }
 }
 
+// ----------------------------------------------------------------------------- grid class
+// flag = 1 iff x does not depend on the row and y does not depend on the column (bitwise).
+__global__ void k_flag_set(int* flag, int v) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *flag = v;
+}
+
+__global__ __launch_bounds__(kThreads) void k_grid_classify(const float* __restrict__ x,
+                                                            const float* __restrict__ y, long sxb,
+                                                            long sxh, long sxw, long syb, long syh,
+                                                            long syw, int H, int W,
+                                                            int* __restrict__ flag) {
+    const int p = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (p >= H * W) return;
+    const int h = p / W, w = p - h * W;
+    const float xv = x[b * sxb + h * sxh + w * sxw], x0 = x[b * sxb + w * sxw];
+    const float yv = y[b * syb + h * syh + w * syw], y0 = y[b * syb + h * syh];
+    // every writer stores the same value, so the race between them is benign
+    if (__float_as_uint(xv) != __float_as_uint(x0) || __float_as_uint(yv) != __float_as_uint(y0))
+        *flag = 0;
+}
+
 // ----------------------------------------------------------------------------- host side
 int g_cached_cus = 0;
 
@@ -719,7 +761,8 @@ FwdGeometry fwd_geometry(int B, int H, int W, bool sep) {
     return g;
 }
 
-int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
+// Plan of one kernel variant (grid_mode is GENERAL or SEPARABLE here).
+int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
     if (!p) return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, H, W)) return IGS_ERR_BAD_SHAPE;
     if (C < 1 || C > IGS_MAX_CHANNELS) return IGS_ERR_BAD_CHANNELS;
@@ -765,45 +808,27 @@ int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t*
     return IGS_OK;
 }
 
+// Public plan: AUTO reports the separable variant's geometry with the workspace sizes of
+// whichever variant needs more.
+int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
+    if (grid_mode != IGS_GRID_AUTO) return plan_one(B, N, H, W, C, grid_mode, p);
+    igs_gs2d_plan_t g;
+    int rc = plan_one(B, N, H, W, C, IGS_GRID_SEPARABLE, p);
+    if (rc) return rc;
+    rc = plan_one(B, N, H, W, C, IGS_GRID_GENERAL, &g);
+    if (rc) return rc;
+    if (g.fwd_ws_bytes > p->fwd_ws_bytes) p->fwd_ws_bytes = g.fwd_ws_bytes;
+    if (g.pix_bytes > p->pix_bytes) p->pix_bytes = g.pix_bytes;
+    if (g.partial_bytes > p->partial_bytes) p->partial_bytes = g.partial_bytes;
+    return IGS_OK;
+}
+
 inline int launch_status() {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? IGS_OK : (int)e;
 }
 
-template <int C>
-int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
-    const int blocks = ((a.total_tiles + 7) / 8) * 8;
-    const dim3 grid(blocks, a.S, 1);
-    if (sep)
-        hipLaunchKernelGGL((k_fwd_sep<C, kFwdSepP>), grid, dim3(kThreads), 0, st, a);
-    else
-        hipLaunchKernelGGL((k_fwd_gen<C, kFwdGenP>), grid, dim3(kThreads), 0, st, a);
-    return launch_status();
-}
-
-template <int C>
-int launch_backward(const BwdArgs& a, int B, bool sep, const float* out, const float* den,
-                    const float* gout, const float* x, const float* y, const int64_t* gs,
-                    float eps, float* pixrec, hipStream_t st) {
-    const int padded = sep ? a.H * a.Wp : a.HWp;
-    const dim3 pgrid(ceil_div(padded, kThreads), B, 1);
-    if (sep)
-        hipLaunchKernelGGL((k_bwd_pix<C, true>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
-                           gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
-                           pixrec);
-    else
-        hipLaunchKernelGGL((k_bwd_pix<C, false>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
-                           gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
-                           pixrec);
-    int rc = launch_status();
-    if (rc) return rc;
-    const dim3 grid(ceil_div(a.N, kThreads * kBwdG), a.T, B);
-    if (sep)
-        hipLaunchKernelGGL((k_bwd_sep<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
-    else
-        hipLaunchKernelGGL((k_bwd_gen<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
-    return launch_status();
-}
+bool channels_compiled(int C) { return C == 1 || C == 2 || C == 3 || C == 4 || C == 8 || C == 16; }
 
 // Channel counts with a compiled specialisation; other C <= 16 are rejected by the ABI
 // (the host wrapper zero-pads colours / grad_out up to the next one, which is exact).
@@ -818,7 +843,85 @@ int launch_backward(const BwdArgs& a, int B, bool sep, const float* out, const f
         default: return IGS_ERR_BAD_CHANNELS;            \
     }
 
-bool channels_compiled(int C) { return C == 1 || C == 2 || C == 3 || C == 4 || C == 8 || C == 16; }
+// The variants a grid mode runs: {variant mode, flag value it is gated on}; AUTO runs both.
+struct Variant {
+    int mode;
+    const int* flag;
+    int want;
+};
+
+int variants_of(int grid_mode, const int32_t* grid_flag, Variant (&v)[2]) {
+    if (grid_mode == IGS_GRID_AUTO) {
+        v[0] = {IGS_GRID_SEPARABLE, grid_flag, 1};
+        v[1] = {IGS_GRID_GENERAL, grid_flag, 0};
+        return 2;
+    }
+    v[0] = {grid_mode, nullptr, 0};
+    return 1;
+}
+
+template <int C>
+int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
+    const int blocks = ((a.total_tiles + 7) / 8) * 8;
+    const dim3 grid(blocks, a.S, 1);
+    if (sep)
+        hipLaunchKernelGGL((k_fwd_sep<C, kFwdSepP>), grid, dim3(kThreads), 0, st, a);
+    else
+        hipLaunchKernelGGL((k_fwd_gen<C, kFwdGenP>), grid, dim3(kThreads), 0, st, a);
+    return launch_status();
+}
+
+template <int C>
+int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, const float* den,
+                        const float* gout, const float* x, const float* y, const int64_t* gs,
+                        float eps, float* pixrec, hipStream_t st) {
+    const int padded = sep ? a.H * a.Wp : a.HWp;
+    const dim3 pgrid(ceil_div(padded, kThreads), B, 1);
+    if (sep)
+        hipLaunchKernelGGL((k_bwd_pix<C, true>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
+                           gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
+                           pixrec, a.flag, a.want);
+    else
+        hipLaunchKernelGGL((k_bwd_pix<C, false>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
+                           gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
+                           pixrec, a.flag, a.want);
+    return launch_status();
+}
+
+template <int C>
+int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
+    const dim3 grid(ceil_div(a.N, kThreads * kBwdG), a.T, B);
+    if (sep)
+        hipLaunchKernelGGL((k_bwd_sep<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
+    else
+        hipLaunchKernelGGL((k_bwd_gen<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
+    return launch_status();
+}
+
+int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* colors, const float* y,
+             const int64_t gs[6], int B, int N, int H, int W, int C, float* pix_ws, float* partial) {
+    igs_gs2d_plan_t plan;
+    const int rc = plan_one(B, N, H, W, C, v.mode, &plan);
+    if (rc) return rc;
+    const bool sep = v.mode == IGS_GRID_SEPARABLE;
+    a.packed = packed; a.colors = colors; a.pixrec = pix_ws;
+    a.xs = sep ? pix_ws + (size_t)B * H * plan.w_padded * plan.pix_stride : nullptr;
+    a.y = y;
+    a.syb = gs[3]; a.syh = gs[4];
+    a.N = N; a.Np = plan.n_padded; a.H = H; a.W = W; a.Wp = plan.w_padded; a.HWp = plan.hw_padded;
+    a.T = plan.bwd_tiles;
+    a.per_tile = plan.bwd_per_tile;
+    a.partial = partial;
+    a.flag = v.flag; a.want = v.want;
+    return IGS_OK;
+}
+
+int mode_ok(int grid_mode, const int32_t* grid_flag) {
+    if (grid_mode != IGS_GRID_GENERAL && grid_mode != IGS_GRID_SEPARABLE && grid_mode != IGS_GRID_AUTO)
+        return IGS_ERR_BAD_MODE;
+    if (grid_mode == IGS_GRID_AUTO && !grid_flag) return IGS_ERR_NULL_POINTER;
+    return IGS_OK;
+}
 
 }  // namespace
 
@@ -846,6 +949,18 @@ int igs_gs2d_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_pla
     const int rc = make_plan(B, N, H, W, C, grid_mode, plan);
     if (rc) return rc;
     return channels_compiled(C) ? IGS_OK : IGS_ERR_BAD_CHANNELS;
+}
+
+int igs_gs2d_grid_classify(const float* x, const float* y, const int64_t grid_strides[6], int B,
+                           int H, int W, int32_t* grid_flag, igs_stream_t stream) {
+    if (!x || !y || !grid_strides || !grid_flag) return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, 1, H, W)) return IGS_ERR_BAD_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_flag_set, dim3(1), dim3(64), 0, st, grid_flag, 1);
+    hipLaunchKernelGGL(k_grid_classify, dim3(ceil_div((long)H * W, kThreads), B), dim3(kThreads), 0, st,
+                       x, y, grid_strides[0], grid_strides[1], grid_strides[2], grid_strides[3],
+                       grid_strides[4], grid_strides[5], H, W, grid_flag);
+    return launch_status();
 }
 
 int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const float* cov_inv_01,
@@ -877,89 +992,163 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
 }
 
 int igs_gs2d_forward(const float* packed, const float* x, const float* y,
-                     const int64_t grid_strides[6], int grid_mode, int B, int N, int H, int W, int C,
-                     float eps, float* out, float* den, void* ws, size_t ws_bytes,
-                     igs_stream_t stream) {
+                     const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag, int B,
+                     int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
+                     size_t ws_bytes, igs_stream_t stream) {
     if (!packed || !x || !y || !grid_strides || !out || !den) return IGS_ERR_NULL_POINTER;
-    igs_gs2d_plan_t plan;
-    int rc = make_plan(B, N, H, W, C, grid_mode, &plan);
+    int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
-    if (plan.fwd_ws_bytes > 0 && (!ws || ws_bytes < plan.fwd_ws_bytes)) return IGS_ERR_WORKSPACE;
-    const bool sep = grid_mode == IGS_GRID_SEPARABLE;
-    const FwdGeometry fg = fwd_geometry(B, H, W, sep);
-    FwdArgs a;
-    a.packed = packed; a.x = x; a.y = y;
-    a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
-    a.syb = grid_strides[3]; a.syh = grid_strides[4]; a.syw = grid_strides[5];
-    a.B = B; a.Np = plan.n_padded; a.H = H; a.W = W;
-    a.S = plan.fwd_split;
-    a.n_per_split = plan.fwd_n_per_split;
-    a.tiles_x = fg.tiles_x; a.tiles_y = fg.tiles_y; a.total_tiles = fg.total_tiles; a.wx = fg.wx;
-    a.eps = eps; a.out = out; a.den = den; a.part = (float*)ws;
+    if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    igs_gs2d_plan_t total;
+    rc = make_plan(B, N, H, W, C, grid_mode, &total);
+    if (rc) return rc;
+    if (total.fwd_ws_bytes > 0 && (!ws || ws_bytes < total.fwd_ws_bytes)) return IGS_ERR_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
-    IGS_DISPATCH_C(C, rc = launch_forward<kC>(a, sep, st));
-    if (rc) return rc;
-    if (a.S > 1) {
-        hipLaunchKernelGGL(k_fwd_combine, dim3(ceil_div((long)H * W, kThreads), B), dim3(kThreads), 0,
-                           st, (const float*)ws, a.S, B, C, H * W, eps, out, den);
-        rc = launch_status();
+    Variant vs[2];
+    const int nv = variants_of(grid_mode, grid_flag, vs);
+    for (int i = 0; i < nv; ++i) {
+        igs_gs2d_plan_t plan;
+        rc = plan_one(B, N, H, W, C, vs[i].mode, &plan);
+        if (rc) return rc;
+        const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
+        const FwdGeometry fg = fwd_geometry(B, H, W, sep);
+        FwdArgs a;
+        a.packed = packed; a.x = x; a.y = y;
+        a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
+        a.syb = grid_strides[3]; a.syh = grid_strides[4]; a.syw = grid_strides[5];
+        a.B = B; a.Np = plan.n_padded; a.H = H; a.W = W;
+        a.S = plan.fwd_split;
+        a.n_per_split = plan.fwd_n_per_split;
+        a.tiles_x = fg.tiles_x; a.tiles_y = fg.tiles_y; a.total_tiles = fg.total_tiles; a.wx = fg.wx;
+        a.eps = eps; a.out = out; a.den = den; a.part = (float*)ws;
+        a.flag = vs[i].flag; a.want = vs[i].want;
+        IGS_DISPATCH_C(C, rc = launch_forward<kC>(a, sep, st));
+        if (rc) return rc;
+        if (a.S > 1) {
+            hipLaunchKernelGGL(k_fwd_combine, dim3(ceil_div((long)H * W, kThreads), B), dim3(kThreads),
+                               0, st, (const float*)ws, a.S, B, C, H * W, eps, out, den, a.flag, a.want);
+            rc = launch_status();
+            if (rc) return rc;
+        }
     }
-    return rc;
+    return IGS_OK;
+}
+
+int igs_gs2d_backward_prologue(const float* x, const float* y, const int64_t grid_strides[6],
+                               int grid_mode, const int32_t* grid_flag, const float* out,
+                               const float* den, const float* grad_out, int B, int N, int H, int W,
+                               int C, float eps, float* pix_ws, size_t pix_bytes,
+                               igs_stream_t stream) {
+    if (!x || !y || !grid_strides || !out || !den || !grad_out || !pix_ws) return IGS_ERR_NULL_POINTER;
+    int rc = mode_ok(grid_mode, grid_flag);
+    if (rc) return rc;
+    if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    igs_gs2d_plan_t total;
+    rc = make_plan(B, N, H, W, C, grid_mode, &total);
+    if (rc) return rc;
+    if (pix_bytes < total.pix_bytes) return IGS_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    Variant vs[2];
+    const int nv = variants_of(grid_mode, grid_flag, vs);
+    for (int i = 0; i < nv; ++i) {
+        BwdArgs a;
+        rc = bwd_args(a, vs[i], nullptr, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr);
+        if (rc) return rc;
+        const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
+        IGS_DISPATCH_C(C, rc = launch_bwd_prologue<kC>(a, B, sep, out, den, grad_out, x, y, grid_strides, eps, pix_ws, st));
+        if (rc) return rc;
+    }
+    return IGS_OK;
+}
+
+int igs_gs2d_backward_reduce(const float* packed, const float* colors, const float* y,
+                             const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                             int B, int N, int H, int W, int C, const float* pix_ws, size_t pix_bytes,
+                             float* partial, size_t partial_bytes, igs_stream_t stream) {
+    if (!packed || !colors || !y || !grid_strides || !pix_ws || !partial) return IGS_ERR_NULL_POINTER;
+    int rc = mode_ok(grid_mode, grid_flag);
+    if (rc) return rc;
+    if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    igs_gs2d_plan_t total;
+    rc = make_plan(B, N, H, W, C, grid_mode, &total);
+    if (rc) return rc;
+    if (pix_bytes < total.pix_bytes || partial_bytes < total.partial_bytes) return IGS_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    Variant vs[2];
+    const int nv = variants_of(grid_mode, grid_flag, vs);
+    for (int i = 0; i < nv; ++i) {
+        BwdArgs a;
+        rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C,
+                      const_cast<float*>(pix_ws), partial);
+        if (rc) return rc;
+        const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
+        IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, st));
+        if (rc) return rc;
+    }
+    return IGS_OK;
 }
 
 int igs_gs2d_backward(const float* packed, const float* colors, const float* x, const float* y,
-                      const int64_t grid_strides[6], int grid_mode, const float* out,
-                      const float* den, const float* grad_out, int B, int N, int H, int W, int C,
-                      float eps, float* pix_ws, size_t pix_bytes, float* partial,
+                      const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                      const float* out, const float* den, const float* grad_out, int B, int N, int H,
+                      int W, int C, float eps, float* pix_ws, size_t pix_bytes, float* partial,
                       size_t partial_bytes, igs_stream_t stream) {
-    if (!packed || !colors || !x || !y || !grid_strides || !out || !den || !grad_out || !pix_ws ||
-        !partial)
-        return IGS_ERR_NULL_POINTER;
-    igs_gs2d_plan_t plan;
-    int rc = make_plan(B, N, H, W, C, grid_mode, &plan);
+    int rc = igs_gs2d_backward_prologue(x, y, grid_strides, grid_mode, grid_flag, out, den, grad_out, B, N,
+                                        H, W, C, eps, pix_ws, pix_bytes, stream);
     if (rc) return rc;
-    if (pix_bytes < plan.pix_bytes || partial_bytes < plan.partial_bytes) return IGS_ERR_WORKSPACE;
-    const bool sep = grid_mode == IGS_GRID_SEPARABLE;
-    BwdArgs a;
-    a.packed = packed; a.colors = colors; a.pixrec = pix_ws;
-    a.xs = sep ? pix_ws + (size_t)B * H * plan.w_padded * plan.pix_stride : nullptr;
-    a.y = y;
-    a.syb = grid_strides[3]; a.syh = grid_strides[4];
-    a.N = N; a.Np = plan.n_padded; a.H = H; a.W = W; a.Wp = plan.w_padded; a.HWp = plan.hw_padded;
-    a.T = plan.bwd_tiles;
-    a.per_tile = plan.bwd_per_tile;
-    a.partial = partial;
-    hipStream_t st = (hipStream_t)stream;
-    IGS_DISPATCH_C(C, rc = launch_backward<kC>(a, B, sep, out, den, grad_out, x, y, grid_strides, eps, pix_ws, st));
-    return rc;
+    return igs_gs2d_backward_reduce(packed, colors, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C,
+                                    pix_ws, pix_bytes, partial, partial_bytes, stream);
 }
 
-int igs_gs2d_finalize_covinv(const float* partial, int T, const float* cov_inv_00,
-                             const float* cov_inv_01, const float* cov_inv_11, const float* alphas,
-                             int B, int N, int C, float* g_position, float* g_cov_inv_00,
-                             float* g_cov_inv_01, float* g_cov_inv_11, float* g_alphas,
-                             float* g_colors, igs_stream_t stream) {
+// T of the separable (or only) variant and of the general variant under AUTO.
+static int finalize_tiles(int grid_mode, int B, int N, int H, int W, int C, int* T, int* T_alt) {
+    igs_gs2d_plan_t plan;
+    int rc = plan_one(B, N, H, W, C, grid_mode == IGS_GRID_AUTO ? IGS_GRID_SEPARABLE : grid_mode, &plan);
+    if (rc) return rc;
+    *T = plan.bwd_tiles;
+    *T_alt = plan.bwd_tiles;
+    if (grid_mode == IGS_GRID_AUTO) {
+        rc = plan_one(B, N, H, W, C, IGS_GRID_GENERAL, &plan);
+        if (rc) return rc;
+        *T_alt = plan.bwd_tiles;
+    }
+    return IGS_OK;
+}
+
+int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t* grid_flag,
+                             const float* cov_inv_00, const float* cov_inv_01,
+                             const float* cov_inv_11, const float* alphas, int B, int N, int H, int W,
+                             int C, float* g_position, float* g_cov_inv_00, float* g_cov_inv_01,
+                             float* g_cov_inv_11, float* g_alphas, float* g_colors,
+                             igs_stream_t stream) {
     if (!partial || !cov_inv_00 || !cov_inv_01 || !cov_inv_11 || !alphas) return IGS_ERR_NULL_POINTER;
-    if (!shape_ok(B, N, 1, 1) || T < 1) return IGS_ERR_BAD_SHAPE;
-    if (C < 1 || C > IGS_MAX_CHANNELS) return IGS_ERR_BAD_CHANNELS;
+    int rc = mode_ok(grid_mode, grid_flag);
+    if (rc) return rc;
+    int T, T_alt;
+    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
+    if (rc) return rc;
     hipLaunchKernelGGL((k_bwd_finalize<false>), dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
-                       (hipStream_t)stream, partial, T, cov_inv_00, cov_inv_01, cov_inv_11, alphas, N,
-                       C, 0.0f, g_position, g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas,
-                       g_colors);
+                       (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
+                       T_alt, cov_inv_00, cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
+                       g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
     return launch_status();
 }
 
-int igs_gs2d_finalize_scale_rot(const float* partial, int T, const float* scales,
-                                const float* rotations, const float* alphas, int B, int N, int C,
-                                float eps, float* g_positions, float* g_scales, float* g_rotations,
-                                float* g_alphas, float* g_colors, igs_stream_t stream) {
+int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32_t* grid_flag,
+                                const float* scales, const float* rotations, const float* alphas,
+                                int B, int N, int H, int W, int C, float eps, float* g_positions,
+                                float* g_scales, float* g_rotations, float* g_alphas, float* g_colors,
+                                igs_stream_t stream) {
     if (!partial || !scales || !rotations || !alphas) return IGS_ERR_NULL_POINTER;
-    if (!shape_ok(B, N, 1, 1) || T < 1) return IGS_ERR_BAD_SHAPE;
-    if (C < 1 || C > IGS_MAX_CHANNELS) return IGS_ERR_BAD_CHANNELS;
+    int rc = mode_ok(grid_mode, grid_flag);
+    if (rc) return rc;
+    int T, T_alt;
+    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
+    if (rc) return rc;
     hipLaunchKernelGGL((k_bwd_finalize<true>), dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
-                       (hipStream_t)stream, partial, T, scales, rotations, (const float*)nullptr,
-                       alphas, N, C, eps, g_positions, g_scales, g_rotations, (float*)nullptr,
-                       g_alphas, g_colors);
+                       (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
+                       T_alt, scales, rotations, (const float*)nullptr, alphas, N, C, eps, g_positions,
+                       g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
     return launch_status();
 }
 

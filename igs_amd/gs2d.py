@@ -103,9 +103,19 @@ class _Grid:
         if min(self.sx + self.sy) < 0:
             self.x, self.y = x.contiguous(), y.contiguous()
             self.sx, self.sy = st(self.x), st(self.y)
-        # x independent of the row and y independent of the column -> factored kernels
-        self.mode = _lib.IGS_GRID_SEPARABLE if (self.sx[1] == 0 and self.sy[2] == 0) else _lib.IGS_GRID_GENERAL
         self.strides = _lib.strides6(self.sx, self.sy)
+        # x independent of the row and y independent of the column -> factored kernels.  Expanded
+        # (stride-0) grids prove it on the host; anything else is classified on the device into a
+        # flag that the kernels read, so there is no host synchronisation either way.
+        self.flag = None
+        if self.sx[1] == 0 and self.sy[2] == 0:
+            self.mode = _lib.IGS_GRID_SEPARABLE
+        else:
+            self.mode = _lib.IGS_GRID_AUTO
+            self.flag = torch.empty(1, dtype=torch.int32, device=x.device)
+            _lib.check(_lib.load().igs_gs2d_grid_classify(_ptr(self.x), _ptr(self.y), self.strides, B, self.H,
+                                                          self.W, _ptr(self.flag), _stream(x.device)),
+                       "igs_gs2d_grid_classify")
 
 
 class _Splat:
@@ -140,7 +150,8 @@ class _Splat:
         out = torch.empty(self.B, self.Cp, g.H, g.W, dtype=torch.float32, device=self.device)
         den = torch.empty(self.B, g.H, g.W, dtype=torch.float32, device=self.device)
         ws = self._empty(p.fwd_ws_bytes) if p.fwd_ws_bytes else None
-        _lib.check(self.lib.igs_gs2d_forward(_ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode, self.B, self.N,
+        _lib.check(self.lib.igs_gs2d_forward(_ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag),
+                                             self.B, self.N,
                                              g.H, g.W, self.Cp, self.eps, _ptr(out), _ptr(den), _ptr(ws),
                                              int(p.fwd_ws_bytes), _stream(self.device)), "igs_gs2d_forward")
         return out, den
@@ -150,7 +161,7 @@ class _Splat:
         pix = self._empty(p.pix_bytes)
         partial = self._empty(p.partial_bytes)
         _lib.check(self.lib.igs_gs2d_backward(_ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, g.mode,
-                                              _ptr(out), _ptr(den), _ptr(grad_out_p), self.B, self.N, g.H, g.W,
+                                              _ptr(g.flag), _ptr(out), _ptr(den), _ptr(grad_out_p), self.B, self.N, g.H, g.W,
                                               self.Cp, self.eps, _ptr(pix), int(p.pix_bytes), _ptr(partial),
                                               int(p.partial_bytes), _stream(self.device)), "igs_gs2d_backward")
         return partial
@@ -246,8 +257,9 @@ class GaussianSplatting2DKernel(torch.autograd.Function):
             g_d = new(B, N) if need[5] else None
             g_al = new(B, N) if need[6] else None
             g_col = new(B, N, Cp) if need[7] else None
-            _lib.check(op.lib.igs_gs2d_finalize_covinv(_ptr(partial), op.plan.bwd_tiles, _ptr(a), _ptr(b), _ptr(d),
-                                                       _ptr(al), B, N, Cp, _ptr(g_pos), _ptr(g_a), _ptr(g_b),
+            _lib.check(op.lib.igs_gs2d_finalize_covinv(_ptr(partial), op.grid.mode, _ptr(op.grid.flag), _ptr(a),
+                                                       _ptr(b), _ptr(d), _ptr(al), B, N, op.grid.H, op.grid.W,
+                                                       Cp, _ptr(g_pos), _ptr(g_a), _ptr(g_b),
                                                        _ptr(g_d), _ptr(g_al), _ptr(g_col), _stream(dev)),
                        "igs_gs2d_finalize_covinv")
         if g_col is not None and Cp != C:
@@ -317,8 +329,9 @@ class _RenderFused(torch.autograd.Function):
             g_sc = new(B, N, 2) if need[2] else None
             g_rot = new(B, N) if need[3] else None
             g_al = new(B, N) if need[4] else None
-            _lib.check(op.lib.igs_gs2d_finalize_scale_rot(_ptr(partial), op.plan.bwd_tiles, _ptr(sc), _ptr(rot),
-                                                          _ptr(al), B, N, Cp, op.eps, _ptr(g_pos), _ptr(g_sc),
+            _lib.check(op.lib.igs_gs2d_finalize_scale_rot(_ptr(partial), op.grid.mode, _ptr(op.grid.flag), _ptr(sc),
+                                                          _ptr(rot), _ptr(al), B, N, op.grid.H, op.grid.W, Cp,
+                                                          op.eps, _ptr(g_pos), _ptr(g_sc),
                                                           _ptr(g_rot), _ptr(g_al), _ptr(g_col), _stream(dev)),
                        "igs_gs2d_finalize_scale_rot")
         if g_col is not None and Cp != C:

@@ -48,10 +48,22 @@ typedef enum igs_status {
  *                        depend on w (every linspace/meshgrid grid, e.g. xy_grid,
  *                        src/igs/gs2d.py:503-522).  sxh and syw are then ignored and the
  *                        kernels factor the quadratic form by rows/columns.
+ *   IGS_GRID_AUTO      : decided on the device, without a host synchronisation: the caller
+ *                        runs igs_gs2d_grid_classify once into a 4-byte flag and passes that
+ *                        flag to every later call; both kernel variants are enqueued and the
+ *                        flag selects the one that does the work (the other exits at once).
+ *                        Workspace sizes are the larger of the two variants'.
+ * Entry points take `grid_flag` (device int32, 1 = separable); it is only read in AUTO mode
+ * and may be NULL otherwise.
  */
-typedef enum igs_grid_mode { IGS_GRID_GENERAL = 0, IGS_GRID_SEPARABLE = 1 } igs_grid_mode;
+typedef enum igs_grid_mode {
+    IGS_GRID_GENERAL = 0,
+    IGS_GRID_SEPARABLE = 1,
+    IGS_GRID_AUTO = 2
+} igs_grid_mode;
 
-/* Launch plan and workspace sizes for one problem shape (filled by igs_gs2d_plan). */
+/* Launch plan and workspace sizes for one problem shape (filled by igs_gs2d_plan).  In AUTO
+ * mode the geometry fields describe the separable variant. */
 typedef struct igs_gs2d_plan_t {
     int32_t B, N, H, W, C;
     int32_t rec_stride;      /* floats per packed Gaussian record                          */
@@ -76,6 +88,12 @@ const char *igs_status_string(int status);
  * query of the current device's compute-unit count.  grid_mode is an igs_grid_mode. */
 int igs_gs2d_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t *plan);
 
+/* Device-side test whether the grids are separable (bitwise: x(b,h,w) == x(b,0,w) and
+ * y(b,h,w) == y(b,h,0)); writes 1 or 0 to *grid_flag.  No counterpart in the reference,
+ * whose kernels always read per-pixel coordinates (src/igs/gs_triton.py:113-114). */
+int igs_gs2d_grid_classify(const float *x, const float *y, const int64_t grid_strides[6], int B,
+                           int H, int W, int32_t *grid_flag, igs_stream_t stream);
+
 /* Pack per-Gaussian parameters for the kernels (operator level: the caller already has
  * the inverse covariance).  position [B,N,2]; cov_inv_00/01/11 [B,N]; alphas [B,N];
  * colors [B,N,C]; packed: plan.packed_bytes.  Replaces nothing in the reference (its
@@ -95,38 +113,56 @@ int igs_gs2d_pack_scale_rot(const float *positions, const float *scales, const f
  * grid_strides = {sxb, sxh, sxw, syb, syh, syw}.  ws: plan.fwd_ws_bytes (may be NULL when
  * that is 0). */
 int igs_gs2d_forward(const float *packed, const float *x, const float *y,
-                     const int64_t grid_strides[6], int grid_mode, int B, int N, int H, int W,
-                     int C, float eps, float *out, float *den, void *ws, size_t ws_bytes,
-                     igs_stream_t stream);
+                     const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag, int B,
+                     int N, int H, int W, int C, float eps, float *out, float *den, void *ws,
+                     size_t ws_bytes, igs_stream_t stream);
 
-/* Backward, stage 1 and 2: per-pixel prologue (g^ = grad_out/(den+eps), s = <g^, out>)
- * and the recomputing per-Gaussian reduction over pixel tiles into `partial`.
- * Replaces the backward of src/igs/gs2d.py:146-262 / src/igs/gs_triton.py:159-405.
- * colors [B,N,C]; out, grad_out [B,C,H,W]; den [B,H,W]; pix_ws: plan.pix_bytes;
- * partial: plan.partial_bytes.  Neither grad_out nor out/den are modified. */
+/* Backward, stage 1: per-pixel prologue, g^ = grad_out/(den+eps), s = <g^, out>, written
+ * as one record per pixel into pix_ws (plan.pix_bytes).  Replaces the per-image pre-pass of
+ * the reference backward, src/igs/gs2d.py:175-177 (which also mutates its inputs; this does
+ * not).  out, grad_out [B,C,H,W]; den [B,H,W]. */
+int igs_gs2d_backward_prologue(const float *x, const float *y, const int64_t grid_strides[6],
+                               int grid_mode, const int32_t *grid_flag, const float *out,
+                               const float *den, const float *grad_out, int B, int N, int H, int W,
+                               int C, float eps, float *pix_ws, size_t pix_bytes,
+                               igs_stream_t stream);
+
+/* Backward, stage 2: the recomputing per-Gaussian reduction over pixel tiles into
+ * partial [B,T,6+C,N] (plan.partial_bytes).  Replaces the Gaussian loop of the reference
+ * backward, src/igs/gs2d.py:180-246 / src/igs/gs_triton.py:159-405.  colors [B,N,C]. */
+int igs_gs2d_backward_reduce(const float *packed, const float *colors, const float *y,
+                             const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag,
+                             int B, int N, int H, int W, int C, const float *pix_ws,
+                             size_t pix_bytes, float *partial, size_t partial_bytes,
+                             igs_stream_t stream);
+
+/* Stages 1 and 2 in one call. */
 int igs_gs2d_backward(const float *packed, const float *colors, const float *x, const float *y,
-                      const int64_t grid_strides[6], int grid_mode, const float *out,
-                      const float *den, const float *grad_out, int B, int N, int H, int W, int C,
-                      float eps, float *pix_ws, size_t pix_bytes, float *partial,
-                      size_t partial_bytes, igs_stream_t stream);
+                      const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag,
+                      const float *out, const float *den, const float *grad_out, int B, int N,
+                      int H, int W, int C, float eps, float *pix_ws, size_t pix_bytes,
+                      float *partial, size_t partial_bytes, igs_stream_t stream);
 
 /* Backward, stage 3 (operator level): fixed-order sum of the tile partials and the
- * gradients of the operator inputs.  Any output pointer may be NULL (not wanted).
+ * gradients of the operator inputs (the tail of src/igs/gs2d.py:207-246, :252-262).  The
+ * shape and grid mode must be those given to igs_gs2d_backward (they fix the tile count).
+ * Any output pointer may be NULL (not wanted).
  * g_position [B,N,2]; g_cov_inv_* [B,N]; g_alphas [B,N]; g_colors [B,N,C]. */
-int igs_gs2d_finalize_covinv(const float *partial, int T, const float *cov_inv_00,
-                             const float *cov_inv_01, const float *cov_inv_11,
-                             const float *alphas, int B, int N, int C, float *g_position,
-                             float *g_cov_inv_00, float *g_cov_inv_01, float *g_cov_inv_11,
-                             float *g_alphas, float *g_colors, igs_stream_t stream);
+int igs_gs2d_finalize_covinv(const float *partial, int grid_mode, const int32_t *grid_flag,
+                             const float *cov_inv_00, const float *cov_inv_01,
+                             const float *cov_inv_11, const float *alphas, int B, int N, int H,
+                             int W, int C, float *g_position, float *g_cov_inv_00,
+                             float *g_cov_inv_01, float *g_cov_inv_11, float *g_alphas,
+                             float *g_colors, igs_stream_t stream);
 
 /* Backward, stage 3 (function level): as above plus the chain rule through the closed-form
  * covariance inverse to scales [B,N,2] and rotations [B,N] (the autograd of
  * src/igs/gs2d.py:548-580). */
-int igs_gs2d_finalize_scale_rot(const float *partial, int T, const float *scales,
-                                const float *rotations, const float *alphas, int B, int N, int C,
-                                float eps, float *g_positions, float *g_scales,
-                                float *g_rotations, float *g_alphas, float *g_colors,
-                                igs_stream_t stream);
+int igs_gs2d_finalize_scale_rot(const float *partial, int grid_mode, const int32_t *grid_flag,
+                                const float *scales, const float *rotations, const float *alphas,
+                                int B, int N, int H, int W, int C, float eps, float *g_positions,
+                                float *g_scales, float *g_rotations, float *g_alphas,
+                                float *g_colors, igs_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,149 @@
+"""The C-ABI library loads and exports every symbol include/igs_hip.h declares; host-side
+plan arithmetic and argument checks (no kernel is launched, no GPU needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "igs_hip.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from igs_amd import _lib, build
+
+    if build.is_stale():
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(igs_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    from igs_amd import _lib
+
+    names = declared_symbols()
+    assert "igs_gs2d_forward" in names and "igs_gs2d_backward_reduce" in names and len(names) >= 12
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in igs_hip.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_header_cites_reference_for_each_entry_point():
+    text = open(HEADER).read()
+    assert text.count("src/igs/") >= 8
+
+
+def test_plan_struct_matches_header_layout(lib):
+    from igs_amd import _lib
+
+    text = open(HEADER).read()
+    body = text[text.index("typedef struct igs_gs2d_plan_t {"):text.index("} igs_gs2d_plan_t;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = []
+    for decl in body.split("{", 1)[1].split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        typ, rest = decl.split(None, 1)
+        fields += [(f.strip(), typ) for f in rest.split(",")]
+    assert [f for f, _ in fields] == [f for f, _ in _lib.Plan._fields_]
+    for (name, typ), (_, ct) in zip(fields, _lib.Plan._fields_):
+        assert ct is {"int32_t": ctypes.c_int32, "uint64_t": ctypes.c_uint64}[typ], name
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_plan_arithmetic(lib, mode):
+    from igs_amd import _lib
+
+    for (B, N, H, W, C) in [(1, 2048, 256, 256, 3), (16, 8192, 256, 256, 3), (4, 32768, 384, 640, 16), (2, 5, 3, 4, 1)]:
+        p = _lib.plan(B, N, H, W, C, mode)
+        assert p.n_padded % 4 == 0 and p.n_padded >= N
+        assert p.fwd_n_per_split % 4 == 0 and p.fwd_split * p.fwd_n_per_split >= p.n_padded
+        assert (p.fwd_split - 1) * p.fwd_n_per_split < p.n_padded          # no empty split
+        assert p.packed_bytes == B * p.n_padded * p.rec_stride * 4
+        assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
+        assert p.bwd_tiles >= 1 and p.partial_bytes >= B * p.bwd_tiles * (6 + C) * N * 4
+        if mode != 0:
+            assert p.w_padded % 8 == 0 and p.bwd_tiles * p.bwd_per_tile >= H
+        assert p.pix_bytes >= B * H * W * (C + 1) * 4
+    a, s_, g = (_lib.plan(8, 4096, 256, 256, 3, m) for m in (2, 1, 0))
+    assert a.pix_bytes == max(s_.pix_bytes, g.pix_bytes) and a.fwd_ws_bytes == max(s_.fwd_ws_bytes, g.fwd_ws_bytes)
+
+
+def test_argument_errors_are_status_codes_not_crashes(lib):
+    from igs_amd import _lib
+
+    p = _lib.Plan()
+    assert lib.igs_gs2d_plan(0, 8, 4, 4, 3, 1, ctypes.byref(p)) == -2
+    assert lib.igs_gs2d_plan(1, 8, 4, 4, 0, 1, ctypes.byref(p)) == -3
+    assert lib.igs_gs2d_plan(1, 8, 4, 4, 17, 1, ctypes.byref(p)) == -3
+    assert lib.igs_gs2d_plan(1, 8, 4, 4, 5, 1, ctypes.byref(p)) == -3     # not a compiled channel count
+    assert lib.igs_gs2d_plan(1, 8, 4, 4, 3, 7, ctypes.byref(p)) == -5
+    assert lib.igs_gs2d_plan(1, 8, 4, 4, 3, 1, None) == -1
+    # null pointers are rejected before anything is launched
+    st = _lib.strides6((0, 0, 1), (0, 4, 0))
+    assert lib.igs_gs2d_forward(None, None, None, st, 1, None, 1, 8, 4, 4, 3, 1e-6, None, None, None, 0, None) == -1
+    assert lib.igs_gs2d_pack_covinv(None, None, None, None, None, None, 1, 8, 3, None, None) == -1
+    assert lib.igs_gs2d_finalize_covinv(None, 1, None, None, None, None, None, 1, 8, 4, 4, 3,
+                                        None, None, None, None, None, None, None) == -1
+    assert b"workspace" in lib.igs_status_string(-4)
+    with pytest.raises(RuntimeError):
+        _lib.check(-2, "x")
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from igs_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libigs_hip.so")
+    with pytest.raises(_lib.IGSLibraryError):
+        _lib.load()
+
+
+def test_fused_path_refuses_cpu_tensors():
+    import torch
+
+    import igs_amd
+    from oracle import gs2d_oracle as O
+
+    d = O.make_config_inputs("c0", N=16, H=8, W=8)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        igs_amd.gaussian_splatting_2d(d["positions"], d["colors"], d["scales"], d["rotations"], d["alphas"],
+                                      d["x_grid"], d["y_grid"])
+    with pytest.raises(RuntimeError, match="GPU only"):
+        a = torch.ones(1, 16, 1, 1)
+        igs_amd.GaussianSplatting2DKernel.apply(d["x_grid"], d["y_grid"], d["positions"], a, a * 0, a, d["alphas"], d["colors"])
+
+
+def test_host_api_surface_and_module_init():
+    import torch
+
+    import igs_amd
+    from oracle import gs2d_oracle as O
+
+    for n in ("GaussianSplatting2D", "gaussian_splatting_2d", "naive_gaussian_2d", "GaussianSplatting2DKernel",
+              "TorchGaussianSplatting2DKernel", "TorchGaussianSplatting2DChunked", "GaussianSplatting2DChunkedKernel"):
+        assert hasattr(igs_amd, n)
+    torch.manual_seed(0)
+    m = igs_amd.GaussianSplatting2D(4, 32, output_dim=3)
+    assert sorted(m.state_dict()) == ["proj.bias", "proj.weight"]
+    assert m.proj.weight.shape == (4 * 9, 32)
+    b = m.proj.bias.view(4, 9)
+    assert torch.all(b[:, :2] == 0) and torch.all(b[:, 2:4] == -4)
+    xg, yg = igs_amd.GaussianSplatting2D.xy_grid((6, 10))
+    ox, oy = O.xy_grid((6, 10))
+    assert torch.equal(xg, ox) and torch.equal(yg, oy) and xg.stride(1) == 0 and yg.stride(2) == 0
+    # fused=False debug path on the CPU equals the oracle's naive expression
+    x = torch.randn(2, 3, 32)
+    img, feat = m(x, size=(6, 10), fused=False)
+    rimg, rfeat = O.module_forward(m.proj.weight.detach(), m.proj.bias.detach(), x, (6, 10), 4)
+    assert torch.allclose(img, rimg, rtol=1e-5, atol=1e-6) and torch.equal(feat, rfeat)

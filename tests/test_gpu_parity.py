@@ -141,8 +141,17 @@ def test_materialised_linspace_grid_equals_expanded(igs, dev):
     xe = d["x_grid"][:1, :, :1, :].expand(2, 1, 19, 45)
     ye = d["y_grid"][:1, :, :, :1].expand(2, 1, 19, 45)
     o_sep = igs.gaussian_splatting_2d(*args, xe, ye)
-    o_gen = igs.gaussian_splatting_2d(*args, xe.contiguous(), ye.contiguous())
-    assert torch.allclose(o_sep, o_gen, rtol=2e-5, atol=2e-6)
+    # materialised: separability is detected on the device, the same kernels run -> same bits
+    o_mat = igs.gaussian_splatting_2d(*args, xe.contiguous(), ye.contiguous())
+    assert torch.equal(o_sep, o_mat)
+    # one perturbed coordinate makes the grid non-separable -> general kernels, same values
+    xg = xe.contiguous()
+    xg[1, 0, 7, 3] += 1e-3
+    o_gen = igs.gaussian_splatting_2d(*args, xg, ye.contiguous())
+    mask = torch.ones_like(o_gen, dtype=torch.bool)
+    mask[1, :, 7, 3] = False
+    assert torch.allclose(o_gen[mask], o_sep[mask], rtol=2e-5, atol=2e-6)
+    assert not torch.equal(o_gen[1, :, 7, 3], o_sep[1, :, 7, 3])
 
 
 def test_run_to_run_bit_identical(igs, dev):
