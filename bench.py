@@ -40,6 +40,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
+                         "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over the batch with no "
@@ -78,6 +81,14 @@ def main() -> int:
         out.backward(d["grad_out"])
         for v in leaves.values():
             v.grad = None
+
+    if args.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- whole step: W warm-ups, then exactly K steps between two synchronisations
     for _ in range(args.warmup):
@@ -187,18 +198,19 @@ def main() -> int:
 
 
 def cpu_baseline(config: str, O):
-    """Chunked torch autograd path on the host cores, one image of the same workload."""
+    """Chunked torch autograd path on the host cores, on a bounded sample of the same workload
+    (a few images of it; cost is linear in the number of images)."""
     import torch
 
     from oracle.chunked_cpu import render_chunked_cpu
 
     threads = torch.get_num_threads()
-    d = O.make_config_inputs(config, B=1)
+    full = O.CONFIGS[config]
+    nb = {"c0": 1, "c1": 4, "c2": 1, "c4": 1}[config]
+    N = full["N"] // 8 if config == "c4" else full["N"]
+    d = O.make_config_inputs(config, B=nb, N=N)
     B, N, C = d["colors"].shape
     H, W = d["x_grid"].shape[-2:]
-    if config == "c4":
-        d = O.make_config_inputs(config, B=1, N=N // 8)
-        N = N // 8
     names = ("positions", "colors", "scales", "rotations", "alphas")
     leaves = {k: d[k].clone().requires_grad_(True) for k in names}
     xg, yg = d["x_grid"].contiguous(), d["y_grid"].contiguous()
@@ -219,7 +231,7 @@ def cpu_baseline(config: str, O):
     t = time.perf_counter() - t0
     pairs = B * N * H * W
     return {"value": pairs / t, "unit": "pairs/s", "cores": threads, "kind": "port",
-            "sample": f"one image of {config} (B=1, N={N}, {H}x{W}, C={C}), fwd+bwd once, {t:.1f} s, "
+            "sample": f"{B} image(s) of {config} (B={B}, N={N}, {H}x{W}, C={C}), fwd+bwd once, {t:.1f} s, "
                       f"eager torch fp32 with {threads} threads"}
 
 
