@@ -185,6 +185,28 @@ def test_zero_alpha_padding_is_exact_and_permutation_close(igs, dev):
     assert torch.allclose(outp, base, rtol=1e-5, atol=1e-6)
 
 
+def test_against_committed_golden_fixture(igs, dev):
+    import importlib.util
+    import os
+
+    import numpy as np
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(here, "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    blob = np.load(os.path.join(here, "gs2d_golden.npz"))
+    names = ("positions", "colors", "scales", "rotations", "alphas")
+    for case, kw in mg.CASES.items():
+        d = to_dev(O.make_inputs(dtype=F64, **kw), dev)
+        lv = {k: d[k].clone().requires_grad_(True) for k in names}
+        out = igs.gaussian_splatting_2d(*[lv[k] for k in names], d["x_grid"], d["y_grid"])
+        assert_fwd(out.detach(), torch.from_numpy(blob[f"{case}/out"]), case)
+        out.backward(d["grad_out"])
+        for k in names:
+            assert_grad(lv[k].grad, torch.from_numpy(blob[f"{case}/g_{k}"]), k, case)
+
+
 def _full_config(igs, dev, name, rows, **override):
     d64 = O.make_config_inputs(name, dtype=F64, **override)
     g64 = {k: v.to(dev) for k, v in d64.items()}   # oracle evaluated in fp64 on the device, in strips

@@ -246,3 +246,19 @@ def test_make_inputs_is_seeded_and_shaped():
     assert a["scales"].min() >= 0.25 and a["scales"].max() <= 0.75
     c4 = O.make_config_inputs("c4", B=1, N=8, H=12, W=20)
     assert math.isclose(float(c4["x_grid"].max()), 20 / 12, rel_tol=1e-6)
+
+
+# ---------------------------------------------------------------- committed fixtures
+def test_oracle_reproduces_golden_fixture():
+    import importlib.util
+    import os
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(here, "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    blob = np.load(os.path.join(here, "gs2d_golden.npz"))
+    for case in mg.CASES:
+        _, res = mg.compute(case)
+        for k, v in res.items():
+            assert np.allclose(v.numpy(), blob[f"{case}/{k}"], rtol=1e-11, atol=1e-14), (case, k)
