@@ -58,6 +58,8 @@ SIGNATURES = {
                                          _FP, c_size_t, _FP, c_size_t, c_void_p]),
     "igs_gs2d_backward": (c_int, [_FP, _FP, _FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int,
                                   c_int, c_int, c_int, c_float, _FP, c_size_t, _FP, c_size_t, c_void_p]),
+    "igs_gs2d_backward_grid": (c_int, [_FP, _FP, _FP, _STRIDES, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
+                                       c_float, _FP, _FP, c_void_p]),
     "igs_gs2d_finalize_covinv": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                          _FP, _FP, _FP, _FP, _FP, _FP, c_void_p]),
     "igs_gs2d_finalize_scale_rot": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,

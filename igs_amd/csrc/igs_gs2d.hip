@@ -687,6 +687,80 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     }
 }
 
+// ----------------------------------------------------------------------------- grid grads
+// Optional: d L / d x(pixel), d L / d y(pixel) = -sum_n G_n w_n (A dx + B dy), (B dx + D dy).
+// Pixel-major like the forward (lane = P pixels, Gaussian record wave-uniform); the per-pixel
+// g^, s are rebuilt from out/den/grad_out in the prologue of the same kernel.  With
+// t1 = A'dx + (B2'/2) dy and t2 = (B2'/2) dx + D'dy the exponent is q' = dx t1 + dy t2, and
+// the sums of G w t1, G w t2 are scaled by -1/k (k = -0.5 log2 e) at the end.
+struct GridGradArgs {
+    const float* packed;
+    const float* x;
+    const float* y;
+    long sxb, sxh, sxw, syb, syh, syw;
+    const float* out;
+    const float* den;
+    const float* gout;
+    int Np, H, W, tiles_per_img, total_tiles;
+    float eps;
+    float* gx;  // [B][H*W]
+    float* gy;
+};
+
+template <int C, int P>
+__global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
+    constexpr int RS = rec_stride_of(C);
+    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
+    if (tile >= a.total_tiles) return;
+    const int b = tile / a.tiles_per_img;
+    const int tl = tile - b * a.tiles_per_img;
+    const int HW = a.H * a.W;
+    float xv[P], yv[P], gh[P][C], negs[P], sx[P], sy[P];
+    int pix[P];
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+        pix[j] = tl * (kThreads * P) + j * kThreads + (int)threadIdx.x;
+        const int pc = min(pix[j], HW - 1);
+        const int h = pc / a.W, w = pc - h * a.W;
+        xv[j] = a.x[b * a.sxb + h * a.sxh + w * a.sxw];
+        yv[j] = a.y[b * a.syb + h * a.syh + w * a.syw];
+        const float inv = 1.0f / (a.den[(size_t)b * HW + pc] + a.eps);
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            gh[j][c] = a.gout[((size_t)b * C + c) * HW + pc] * inv;
+            s = fmaf(gh[j][c], a.out[((size_t)b * C + c) * HW + pc], s);
+        }
+        negs[j] = -s;
+        sx[j] = sy[j] = 0.0f;
+    }
+    stream_gaussians<C>(a.packed + (size_t)b * a.Np * RS, a.Np >> 2, [&](const GRec<C>& g) {
+        const float hb = 0.5f * g.B2;
+#pragma unroll
+        for (int j = 0; j < P; ++j) {
+            const float dx = xv[j] - g.px;
+            const float dy = yv[j] - g.py;
+            const float t1 = fmaf(g.A, dx, hb * dy);
+            const float t2 = fmaf(g.D, dy, hb * dx);
+            const float q = fmaf(dx, t1, dy * t2);
+            const float e = hw_exp2(q);
+            float Gv = negs[j] * g.al;  // alpha (<g^, c> - s)
+#pragma unroll
+            for (int c = 0; c < C; ++c) Gv = fmaf(gh[j][c], g.ac[c], Gv);
+            const float Gw = Gv * e;
+            sx[j] = fmaf(Gw, t1, sx[j]);
+            sy[j] = fmaf(Gw, t2, sy[j]);
+        }
+    });
+    constexpr float kScale = -1.0f / kNegHalfLog2e;  // A dx + B dy = t1 / k, and the leading minus
+#pragma unroll
+    for (int j = 0; j < P; ++j)
+        if (pix[j] < HW) {
+            a.gx[(size_t)b * HW + pix[j]] = kScale * sx[j];
+            a.gy[(size_t)b * HW + pix[j]] = kScale * sy[j];
+        }
+}
+
 // ----------------------------------------------------------------------------- grid class
 // flag = 1 iff x does not depend on the row and y does not depend on the column (bitwise).
 __global__ void k_flag_set(int* flag, int v) {
@@ -1098,6 +1172,33 @@ int igs_gs2d_backward(const float* packed, const float* colors, const float* x, 
     if (rc) return rc;
     return igs_gs2d_backward_reduce(packed, colors, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C,
                                     pix_ws, pix_bytes, partial, partial_bytes, stream);
+}
+
+int igs_gs2d_backward_grid(const float* packed, const float* x, const float* y,
+                           const int64_t grid_strides[6], const float* out, const float* den,
+                           const float* grad_out, int B, int N, int H, int W, int C, float eps,
+                           float* g_x, float* g_y, igs_stream_t stream) {
+    if (!packed || !x || !y || !grid_strides || !out || !den || !grad_out || !g_x || !g_y)
+        return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, N, H, W)) return IGS_ERR_BAD_SHAPE;
+    if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    GridGradArgs a;
+    a.packed = packed; a.x = x; a.y = y;
+    a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
+    a.syb = grid_strides[3]; a.syh = grid_strides[4]; a.syw = grid_strides[5];
+    a.out = out; a.den = den; a.gout = grad_out;
+    a.Np = (N + 3) & ~3; a.H = H; a.W = W;
+    a.eps = eps; a.gx = g_x; a.gy = g_y;
+    int rc = IGS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    IGS_DISPATCH_C(C, {
+        constexpr int P = kC > 4 ? 1 : 2;
+        a.tiles_per_img = ceil_div((long)H * W, kThreads * P);
+        a.total_tiles = B * a.tiles_per_img;
+        hipLaunchKernelGGL((k_bwd_grid<kC, P>), dim3(((a.total_tiles + 7) / 8) * 8), dim3(kThreads), 0, st, a);
+        rc = launch_status();
+    });
+    return rc;
 }
 
 // T of the separable (or only) variant and of the general variant under AUTO.

@@ -166,6 +166,24 @@ class _Splat:
                                               int(p.partial_bytes), _stream(self.device)), "igs_gs2d_backward")
         return partial
 
+    def grid_grads(self, packed, out, den, grad_out_p, x_like, y_like):
+        """d L / d x_grid, d L / d y_grid in the (shape, dtype) of the tensors the caller passed."""
+        g = self.grid
+        gx = torch.empty(self.B, g.H, g.W, dtype=torch.float32, device=self.device)
+        gy = torch.empty_like(gx)
+        _lib.check(self.lib.igs_gs2d_backward_grid(_ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, _ptr(out),
+                                                   _ptr(den), _ptr(grad_out_p), self.B, self.N, g.H, g.W, self.Cp,
+                                                   self.eps, _ptr(gx), _ptr(gy), _stream(self.device)),
+                   "igs_gs2d_backward_grid")
+
+        def fit(gr, like):
+            shape, dtype = like
+            if shape[0] == 1 and self.B > 1:      # batch-1 grid shared by all images
+                gr = gr.sum(0, keepdim=True)
+            return gr.reshape(shape).to(dtype)
+
+        return fit(gx, x_like), fit(gy, y_like)
+
     def pad_grad_out(self, grad_out: Tensor) -> Tensor:
         go = _f32c(grad_out)
         if self.Cp != self.C:
@@ -191,11 +209,6 @@ def _require_gpu(t: Tensor):
         raise RuntimeError("the fused Gaussian-splatting path runs on the GPU only (HIP kernels); got a tensor on "
                            f"{t.device}. Use fused=False for the plain-torch debug path.")
     _lib.load()
-
-
-def _grid_grad_unsupported(ctx):
-    if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-        raise NotImplementedError("gradients w.r.t. the pixel grids (x, y) are not implemented in the HIP path")
 
 
 # --------------------------------------------------------------------------------------
@@ -233,6 +246,7 @@ class GaussianSplatting2DKernel(torch.autograd.Function):
             packed = op.pack_covinv(pos, a, b, d, al, col)
             out, den = op.forward(packed)
         ctx.op = op
+        ctx.grid_like = ((x.shape, x.dtype), (y.shape, y.dtype))
         ctx.save_for_backward(packed, col, a, b, d, al, out, den)
         ctx.in_dtypes = tuple(t.dtype for t in (position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors))
         ctx.cov_shapes = (cov_inv_00.shape, cov_inv_01.shape, cov_inv_11.shape)
@@ -242,13 +256,16 @@ class GaussianSplatting2DKernel(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_result):
-        _grid_grad_unsupported(ctx)
         op: _Splat = ctx.op
         packed, col, a, b, d, al, out, den = ctx.saved_tensors
         B, N, C, Cp, dev = op.B, op.N, op.C, op.Cp, op.device
         need = ctx.needs_input_grad
+        g_x = g_y = None
         with torch.cuda.device(dev):
             go = op.pad_grad_out(grad_result)
+            if need[0] or need[1]:
+                g_x, g_y = op.grid_grads(packed, out, den, go, *ctx.grid_like)
+                g_x, g_y = (g_x if need[0] else None), (g_y if need[1] else None)
             partial = op.backward_partials(packed, col, out, den, go)
             new = lambda *s: torch.empty(*s, dtype=torch.float32, device=dev)
             g_pos = new(B, N, 2) if need[2] else None
@@ -267,7 +284,7 @@ class GaussianSplatting2DKernel(torch.autograd.Function):
         dt = ctx.in_dtypes
         cast = lambda g, k: None if g is None else g.to(dt[k])
         sh = ctx.cov_shapes
-        return (None, None, cast(g_pos, 0),
+        return (g_x, g_y, cast(g_pos, 0),
                 None if g_a is None else cast(g_a, 1).reshape(sh[0]),
                 None if g_b is None else cast(g_b, 2).reshape(sh[1]),
                 None if g_d is None else cast(g_d, 3).reshape(sh[2]),
@@ -306,6 +323,7 @@ class _RenderFused(torch.autograd.Function):
             packed = op.pack_scale_rot(pos, sc, rot, al, col)
             out, den = op.forward(packed)
         ctx.op = op
+        ctx.grid_like = ((x_grid.shape, x_grid.dtype), (y_grid.shape, y_grid.dtype))
         ctx.save_for_backward(packed, col, sc, rot, al, out, den)
         ctx.in_dtypes = tuple(t.dtype for t in (positions, colors, scales, rotations, alphas))
         res = out if op.Cp == C else out[:, :C]
@@ -314,14 +332,16 @@ class _RenderFused(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_result):
-        if ctx.needs_input_grad[5] or ctx.needs_input_grad[6]:
-            raise NotImplementedError("gradients w.r.t. the pixel grids are not implemented in the HIP path")
         op: _Splat = ctx.op
         packed, col, sc, rot, al, out, den = ctx.saved_tensors
         B, N, C, Cp, dev = op.B, op.N, op.C, op.Cp, op.device
         need = ctx.needs_input_grad
+        g_x = g_y = None
         with torch.cuda.device(dev):
             go = op.pad_grad_out(grad_result)
+            if need[5] or need[6]:
+                g_x, g_y = op.grid_grads(packed, out, den, go, *ctx.grid_like)
+                g_x, g_y = (g_x if need[5] else None), (g_y if need[6] else None)
             partial = op.backward_partials(packed, col, out, den, go)
             new = lambda *s: torch.empty(*s, dtype=torch.float32, device=dev)
             g_pos = new(B, N, 2) if need[0] else None
@@ -338,7 +358,7 @@ class _RenderFused(torch.autograd.Function):
             g_col = g_col[..., :C]
         dt = ctx.in_dtypes
         cast = lambda g, k: None if g is None else g.to(dt[k])
-        return cast(g_pos, 0), cast(g_col, 1), cast(g_sc, 2), cast(g_rot, 3), cast(g_al, 4), None, None, None
+        return cast(g_pos, 0), cast(g_col, 1), cast(g_sc, 2), cast(g_rot, 3), cast(g_al, 4), g_x, g_y, None
 
 
 def _cov_inverse_torch(scales, rotations, eps):

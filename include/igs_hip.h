@@ -143,6 +143,16 @@ int igs_gs2d_backward(const float *packed, const float *colors, const float *x, 
                       int H, int W, int C, float eps, float *pix_ws, size_t pix_bytes,
                       float *partial, size_t partial_bytes, igs_stream_t stream);
 
+/* Optional backward output: gradients w.r.t. the pixel coordinates, g_x, g_y [B,H,W]
+ * (grad_x / grad_y of the reference backward, src/igs/gs2d.py:222-231, :249-250; the Triton
+ * backward accumulates them with atomics, src/igs/gs_triton.py:365-366).  Independent of the
+ * other backward stages: reads packed, out, den, grad_out; needs no workspace.  Only run
+ * when the caller wants these gradients. */
+int igs_gs2d_backward_grid(const float *packed, const float *x, const float *y,
+                           const int64_t grid_strides[6], const float *out, const float *den,
+                           const float *grad_out, int B, int N, int H, int W, int C, float eps,
+                           float *g_x, float *g_y, igs_stream_t stream);
+
 /* Backward, stage 3 (operator level): fixed-order sum of the tile partials and the
  * gradients of the operator inputs (the tail of src/igs/gs2d.py:207-246, :252-262).  The
  * shape and grid mode must be those given to igs_gs2d_backward (they fix the tile count).

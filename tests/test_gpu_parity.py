@@ -125,6 +125,38 @@ def test_operator_level_apply(igs, dev, general):
         assert_grad(t.grad, ref_g[k], k, "operator bwd")
 
 
+@pytest.mark.parametrize("C", [3, 16])
+def test_grid_gradients(igs, dev, C):
+    B, N, H, W = 2, 90, 18, 26
+    d = small_case(B, N, H, W, C, seed=40 + C, general=True)
+    a, b, c_ = (t.float().double() for t in O.cov_inverse_closed(d["scales"], d["rotations"]))
+    _, ref_g = O.operator_autograd(d["x_grid"], d["y_grid"], d["positions"], a, b, c_, d["alphas"], d["colors"],
+                                   d["grad_out"])
+    f = lambda t: t.to(dev, torch.float32)
+    # operator level: x, y are leaves
+    xg, yg = f(d["x_grid"]).requires_grad_(True), f(d["y_grid"]).requires_grad_(True)
+    pos = f(d["positions"]).requires_grad_(True)
+    out = igs.GaussianSplatting2DKernel.apply(xg, yg, pos, f(a), f(b), f(c_), f(d["alphas"]), f(d["colors"]), 1e-6)
+    out.backward(f(d["grad_out"]))
+    assert xg.grad.shape == xg.shape and yg.grad.shape == yg.shape
+    assert_grad(xg.grad, ref_g["x"], "x", "grid grads")
+    assert_grad(yg.grad, ref_g["y"], "y", "grid grads")
+    assert_grad(pos.grad, ref_g["position"], "position", "grid grads")
+    # translation identity: sum_n dL/dpos_n = - sum_px (dL/dx, dL/dy)
+    assert torch.allclose(pos.grad[..., 0].sum(1), -xg.grad.sum((1, 2, 3)), rtol=1e-3, atol=1e-4 * float(pos.grad.abs().max()))
+    # function level with a shared batch-1 expanded grid: autograd reduces to the leaf's shape
+    xs = f(d["x_grid"])[:1, :, :1, :].clone().requires_grad_(True)     # [1,1,1,W]
+    ys = f(d["y_grid"])[:1, :, :, :1].clone().requires_grad_(True)     # [1,1,H,1]
+    out2 = igs.gaussian_splatting_2d(f(d["positions"]), f(d["colors"]), f(d["scales"]), f(d["rotations"]),
+                                     f(d["alphas"]), xs.expand(1, 1, H, W), ys.expand(1, 1, H, W))
+    out2.backward(f(d["grad_out"]))
+    x64 = d["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+    y64 = d["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+    _, rg = O.operator_autograd(x64, y64, d["positions"], a, b, c_, d["alphas"], d["colors"], d["grad_out"])
+    assert_grad(xs.grad, rg["x"].sum((0, 2), keepdim=True), "x shared", "grid grads")
+    assert_grad(ys.grad, rg["y"].sum((0, 3), keepdim=True), "y shared", "grid grads")
+
+
 def test_fused_false_debug_path_matches(igs, dev):
     d = to_dev(small_case(1, 40, 12, 14, 3, seed=9), dev)
     a = igs.gaussian_splatting_2d(d["positions"], d["colors"], d["scales"], d["rotations"], d["alphas"],
