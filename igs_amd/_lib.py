@@ -9,7 +9,9 @@ import ctypes
 import os
 from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libigs_hip.so")
+# IGS_HIP_LIBRARY overrides the in-tree location (e.g. to try a differently tuned build)
+LIB_PATH = os.environ.get("IGS_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                                                               "libigs_hip.so")
 
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1

@@ -39,9 +39,21 @@ namespace {
 
 constexpr float kNegHalfLog2e = -0.72134752044448170368f;  // -0.5 * log2(e)
 constexpr int kThreads = 256;
-constexpr int kFwdSepP = 8;  // rows per lane, separable forward
+#ifndef IGS_FWD_SEP_P
+#define IGS_FWD_SEP_P 8
+#endif
+#ifndef IGS_BWD_G
+#define IGS_BWD_G 2
+#endif
+#ifndef IGS_FWD_WAVES
+#define IGS_FWD_WAVES 4
+#endif
+#ifndef IGS_BWD_WAVES
+#define IGS_BWD_WAVES 8
+#endif
+constexpr int kFwdSepP = IGS_FWD_SEP_P;  // rows per lane, separable forward
 constexpr int kFwdGenP = 4;  // pixels per lane, general forward
-constexpr int kBwdG = 2;     // Gaussians per lane, backward
+constexpr int kBwdG = IGS_BWD_G;  // Gaussians per lane, backward
 
 __host__ __device__ constexpr int rec_stride_of(int C) { return (6 + C + 3) & ~3; }
 __host__ __device__ constexpr int pix_stride_sep(int C) { return (C + 1 + 3) & ~3; }
@@ -126,42 +138,100 @@ struct FwdArgs {
 #define IGS_GATE(a) \
     if ((a).flag != nullptr && *(a).flag != (a).want) return
 
+// On gfx950 a fp32 VALU op whose operands are all VGPRs (or literals) issues about every
+// 2.2-2.7 cycles per wave64, while any SGPR operand makes it a 4-cycle op (measured; the
+// constant bus broadcast is the slow part).  So wave-uniform operands are NOT fed from SGPRs:
+// the uniform record stream (Gaussians in the forward, pixels in the backward) goes
+// global -> LDS (cooperatively, double-buffered) -> VGPRs through broadcast ds_read_b128
+// (every lane reads the same address: conflict-free), and the hot loops contain VGPR-only
+// VALU instructions plus LDS reads that issue on their own port.
 template <int C>
 struct GRec {
     float px, py, A, B2, D, al;
     float ac[C];
 };
 
+// Reads one record from (wave-uniform) LDS address r.
 template <int C>
-__device__ __forceinline__ GRec<C> load_grec(const float* __restrict__ r) {
-    GRec<C> g;
-    g.px = r[0];
-    g.py = r[1];
-    g.A = r[2];
-    g.B2 = r[3];
-    g.D = r[4];
-    g.al = r[5];
+__device__ __forceinline__ GRec<C> lds_grec(const float4* r) {
+    constexpr int R4 = rec_stride_of(C) / 4;
+    float v[4 * R4];
 #pragma unroll
-    for (int c = 0; c < C; ++c) g.ac[c] = r[6 + c];
+    for (int i = 0; i < R4; ++i) {
+        const float4 t = r[i];
+        v[4 * i] = t.x;
+        v[4 * i + 1] = t.y;
+        v[4 * i + 2] = t.z;
+        v[4 * i + 3] = t.w;
+    }
+    GRec<C> g;
+    g.px = v[0];
+    g.py = v[1];
+    g.A = v[2];
+    g.B2 = v[3];
+    g.D = v[4];
+    g.al = v[5];
+#pragma unroll
+    for (int c = 0; c < C; ++c) g.ac[c] = v[6 + c];
     return g;
 }
 
-// Walks `groups` groups of 4 consecutive records starting at rec, two records in flight
-// ahead of the two being consumed.  f(const GRec<C>&) is the per-Gaussian body.
-template <int C, class F>
-__device__ __forceinline__ void stream_gaussians(const float* __restrict__ rec, int groups, F&& f) {
-    constexpr int RS = rec_stride_of(C);
-    GRec<C> a0 = load_grec<C>(rec), a1 = load_grec<C>(rec + RS);
-    for (int i = 0; i < groups; ++i) {
-        const GRec<C> b0 = load_grec<C>(rec + 2 * RS), b1 = load_grec<C>(rec + 3 * RS);
-        f(a0);
-        f(a1);
-        const float* nxt = (i + 1 < groups) ? rec + 4 * RS : rec;  // last: harmless re-read
-        a0 = load_grec<C>(nxt);
-        a1 = load_grec<C>(nxt + RS);
-        f(b0);
-        f(b1);
-        rec = nxt;
+// Keeps a wave-uniform value in a VGPR (an empty asm the compiler cannot see through), so that
+// instructions using it stay VGPR-only.
+__device__ __forceinline__ float in_vgpr(float v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+constexpr int kGaussChunk = 64;  // Gaussian records per LDS buffer
+
+// Streams `count` records of R4 float4 each from global memory to every wave of the
+// workgroup through the double-buffered LDS window sh[2][CH*R4]; body(const float4* rec) runs
+// once per record with a wave-uniform LDS pointer.  Records past `count` in the last chunk
+// read as all-zero (for a Gaussian record: alpha = 0, adds exactly 0).  Must be called by all
+// kThreads threads of the workgroup (it contains barriers).
+template <int R4, int CH, class Body>
+__device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
+                                                   float4* sh, Body&& body) {
+    constexpr int E = CH * R4;                          // float4 per chunk
+    constexpr int PRE = (E + kThreads - 1) / kThreads;  // float4 per thread per chunk
+    const int total = count * R4;
+    const int chunks = (count + CH - 1) / CH;
+    const int tid = threadIdx.x;
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float4 pre[PRE];
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int e = i * kThreads + tid;
+        pre[i] = (e < E && e < total) ? src[e] : zero;
+    }
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int e = i * kThreads + tid;
+        if (e < E) sh[e] = pre[i];
+    }
+    __syncthreads();
+    for (int k = 0; k < chunks; ++k) {
+        const int nbase = (k + 1) * E;
+        if (k + 1 < chunks) {
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                pre[i] = (e < E && nbase + e < total) ? src[nbase + e] : zero;
+            }
+        }
+        const float4* cur = sh + (k & 1) * E;
+#pragma unroll 2
+        for (int n = 0; n < CH; ++n) body(cur + n * R4);
+        if (k + 1 < chunks) {
+            float4* nxt = sh + ((k + 1) & 1) * E;
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                if (e < E) nxt[e] = pre[i];
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -183,29 +253,28 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 }
 
 // Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows;
-// workgroup = wx x (4/wx) waves.  Per Gaussian and lane: dx, A'dx^2, B2'dx once, then per
-// pixel dy, 2 fma, exp2, 1 + C fma.
+// workgroup = wx x (4/wx) waves, all four streaming the same Gaussians.  Per Gaussian and
+// lane: dx, A'dx^2, B2'dx once, then per pixel dy, 2 fma, exp2, 1 + C fma.
 template <int C, int P>
 __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
-    constexpr int RS = rec_stride_of(C);
+    constexpr int RS = rec_stride_of(C), R4 = RS / 4;
+    __shared__ float4 sh[2 * kGaussChunk * R4];
     IGS_GATE(a);
     const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
-    if (tile >= a.total_tiles) return;
+    if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int per_img = a.tiles_x * a.tiles_y;
     const int b = tile / per_img;
     const int tl = tile - b * per_img;
     const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int wxi = wave % a.wx, wyi = wave / a.wx;
-    const int col0 = (tx * a.wx + wxi) * 64;
+    const int col = (tx * a.wx + wxi) * 64 + lane;
     const int row0 = (ty * (4 / a.wx) + wyi) * P;
-    if (row0 >= a.H || col0 >= a.W) return;  // wave-uniform
-    const int col = col0 + lane;
     const float xv = a.x[b * a.sxb + (long)min(col, a.W - 1) * a.sxw];
     float yv[P];
 #pragma unroll
-    for (int p = 0; p < P; ++p) yv[p] = a.y[b * a.syb + (long)min(row0 + p, a.H - 1) * a.syh];
+    for (int p = 0; p < P; ++p) yv[p] = in_vgpr(a.y[b * a.syb + (long)min(row0 + p, a.H - 1) * a.syh]);
 
     float dsum[P], num[P][C];
 #pragma unroll
@@ -217,23 +286,24 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     const int s = blockIdx.y;
     const int n0 = s * a.n_per_split;
     const int n1 = min(a.Np, n0 + a.n_per_split);
-    stream_gaussians<C>(a.packed + ((size_t)b * a.Np + n0) * RS, (n1 - n0) >> 2,
-                        [&](const GRec<C>& g) {
-                            const float dx = xv - g.px;
-                            const float adx = g.A * dx;
-                            const float c0 = adx * dx;
-                            const float c1 = g.B2 * dx;
+    const float4* src = reinterpret_cast<const float4*>(a.packed + ((size_t)b * a.Np + n0) * RS);
+    stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r) {
+        const GRec<C> g = lds_grec<C>(r);
+        const float dx = xv - g.px;
+        const float adx = g.A * dx;
+        const float c0 = adx * dx;
+        const float c1 = g.B2 * dx;
 #pragma unroll
-                            for (int p = 0; p < P; ++p) {
-                                const float dy = yv[p] - g.py;
-                                const float t = fmaf(g.D, dy, c1);
-                                const float q = fmaf(t, dy, c0);
-                                const float e = hw_exp2(q);
-                                dsum[p] = fmaf(e, g.al, dsum[p]);
+        for (int p = 0; p < P; ++p) {
+            const float dy = yv[p] - g.py;
+            const float t = fmaf(g.D, dy, c1);
+            const float q = fmaf(t, dy, c0);
+            const float e = hw_exp2(q);
+            dsum[p] = fmaf(e, g.al, dsum[p]);
 #pragma unroll
-                                for (int c = 0; c < C; ++c) num[p][c] = fmaf(e, g.ac[c], num[p][c]);
-                            }
-                        });
+            for (int c = 0; c < C; ++c) num[p][c] = fmaf(e, g.ac[c], num[p][c]);
+        }
+    });
     if (col < a.W) {
 #pragma unroll
         for (int p = 0; p < P; ++p)
@@ -244,10 +314,11 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
 // General grid: lane = P pixels of a flat 256*P pixel tile.
 template <int C, int P>
 __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
-    constexpr int RS = rec_stride_of(C);
+    constexpr int RS = rec_stride_of(C), R4 = RS / 4;
+    __shared__ float4 sh[2 * kGaussChunk * R4];
     IGS_GATE(a);
     const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
-    if (tile >= a.total_tiles) return;
+    if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int per_img = a.tiles_x;
     const int b = tile / per_img;
     const int tl = tile - b * per_img;
@@ -256,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
     int pix[P];
 #pragma unroll
     for (int j = 0; j < P; ++j) {
-        pix[j] = tl * (kThreads * P) + j * kThreads + threadIdx.x;
+        pix[j] = tl * (kThreads * P) + j * kThreads + (int)threadIdx.x;
         const int pc = min(pix[j], HW - 1);
         const int h = pc / a.W, w = pc - h * a.W;
         xv[j] = a.x[b * a.sxb + h * a.sxh + w * a.sxw];
@@ -272,23 +343,24 @@ __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
     const int s = blockIdx.y;
     const int n0 = s * a.n_per_split;
     const int n1 = min(a.Np, n0 + a.n_per_split);
-    stream_gaussians<C>(a.packed + ((size_t)b * a.Np + n0) * RS, (n1 - n0) >> 2,
-                        [&](const GRec<C>& g) {
+    const float4* src = reinterpret_cast<const float4*>(a.packed + ((size_t)b * a.Np + n0) * RS);
+    stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r) {
+        const GRec<C> g = lds_grec<C>(r);
 #pragma unroll
-                            for (int j = 0; j < P; ++j) {
-                                const float dx = xv[j] - g.px;
-                                const float dy = yv[j] - g.py;
-                                float t = g.A * dx;
-                                t = fmaf(g.B2, dy, t);
-                                const float v = g.D * dy;
-                                float q = t * dx;
-                                q = fmaf(v, dy, q);
-                                const float e = hw_exp2(q);
-                                dsum[j] = fmaf(e, g.al, dsum[j]);
+        for (int j = 0; j < P; ++j) {
+            const float dx = xv[j] - g.px;
+            const float dy = yv[j] - g.py;
+            float t = g.A * dx;
+            t = fmaf(g.B2, dy, t);
+            const float v = g.D * dy;
+            float q = t * dx;
+            q = fmaf(v, dy, q);
+            const float e = hw_exp2(q);
+            dsum[j] = fmaf(e, g.al, dsum[j]);
 #pragma unroll
-                                for (int c = 0; c < C; ++c) num[j][c] = fmaf(e, g.ac[c], num[j][c]);
-                            }
-                        });
+            for (int c = 0; c < C; ++c) num[j][c] = fmaf(e, g.ac[c], num[j][c]);
+        }
+    });
 #pragma unroll
     for (int j = 0; j < P; ++j)
         if (pix[j] < HW) fwd_store<C>(a, b, s, pix[j], dsum[j], num[j]);
@@ -437,30 +509,25 @@ __device__ __forceinline__ void bwd_load_gaussians(const BwdArgs& a, int b, int 
     }
 }
 
-// Four consecutive pixel records (uniform -> SGPRs).
-template <int CP>
-struct PixQuad {
-    float v[4][CP];
-};
+constexpr int kPixChunk = 128;  // pixel records per LDS buffer
 
-template <int CP>
-__device__ __forceinline__ PixQuad<CP> load_quad(const float* __restrict__ p) {
-    PixQuad<CP> q;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int k = 0; k < CP; ++k) q.v[j][k] = p[j * CP + k];
-    return q;
-}
-
-// Separable grid: lane = G Gaussians; the tile is a range of full rows.  Per row the dy
-// part of q is hoisted, and row sums R0 = sum G e, R1 = sum G e dx, R2 = sum G e dx^2 (and
-// the colour sums) are folded into the totals once per row.
+// Separable grid: lane = G Gaussians; the tile is a range of full rows.  Pixel records and
+// column coordinates of 128-pixel row segments stream through LDS (double-buffered) and are
+// read with broadcast ds_read_b128.  Per row the dy part of q is hoisted, and row sums
+// R0 = sum G e, R1 = sum G e dx, R2 = sum G e dx^2 (and the colour sums) are folded into the
+// totals once per row.
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
-    constexpr int CP = pix_stride_sep(C);
+    constexpr int CP = pix_stride_sep(C), CP4 = CP / 4;
+    constexpr int PX = kPixChunk;
+    constexpr int ER = PX * CP4;   // float4 of pixel records per chunk
+    constexpr int EX = PX / 4;     // float4 of x coordinates per chunk
+    constexpr int E = ER + EX;
+    constexpr int PRE = (E + kThreads - 1) / kThreads;
+    __shared__ float4 sh[2 * E];
     IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
+    const int tid = threadIdx.x;
     int n[G];
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
     bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
@@ -473,144 +540,193 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
         for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
     }
     const int r0 = t * a.per_tile, r1 = min(a.H, r0 + a.per_tile);
-    const float* xrow = a.xs + (size_t)b * a.Wp;
-    const int octs = a.Wp >> 3;  // Wp % 8 == 0
-    for (int r = r0; r < r1; ++r) {
-        const float yv = a.y[b * a.syb + (long)r * a.syh];
-        float dy[G], cyy[G], bdy[G], R0[G], R1[G], R2[G], RC[G][C];
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            dy[g] = yv - py[g];
-            const float ddy = D[g] * dy[g];
-            cyy[g] = ddy * dy[g];
-            bdy[g] = B2[g] * dy[g];
-            R0[g] = R1[g] = R2[g] = 0.0f;
-#pragma unroll
-            for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
+    const int segs = (a.Wp + PX - 1) / PX;  // segments per row
+    const int chunks = (r1 - r0) * segs;
+    const float4* xsrc = reinterpret_cast<const float4*>(a.xs + (size_t)b * a.Wp);  // Wp % 8 == 0
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+
+    // element e of chunk k: e < ER -> pixel-record float4, else x-coordinate float4
+    auto fetch = [&](int k, int e) -> float4 {
+        const int r = r0 + k / segs, c0 = (k % segs) * PX;
+        if (e < ER) {
+            const int pxl = c0 + e / CP4;
+            if (pxl >= a.Wp) return zero;
+            const float4* row = reinterpret_cast<const float4*>(a.pixrec + ((size_t)b * a.H + r) * a.Wp * CP);
+            return row[(size_t)c0 * CP4 + e];
         }
-        auto body = [&](const PixQuad<CP>& pq, const float (&xq)[4]) {
+        const int xi = c0 / 4 + (e - ER);
+        return (e < E && xi * 4 < a.Wp) ? xsrc[xi] : zero;
+    };
+    float4 pre[PRE];
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int e = i * kThreads + tid;
+        if (e < E) sh[e] = fetch(0, e);
+    }
+    __syncthreads();
+
+    float dy[G], cyy[G], bdy[G], R0[G], R1[G], R2[G], RC[G][C];
+    for (int k = 0; k < chunks; ++k) {
+        const int seg = k % segs;
+        if (seg == 0) {  // a new row starts
+            const float yv = a.y[b * a.syb + (long)(r0 + k / segs) * a.syh];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                dy[g] = yv - py[g];
+                const float ddy = D[g] * dy[g];
+                cyy[g] = ddy * dy[g];
+                bdy[g] = B2[g] * dy[g];
+                R0[g] = R1[g] = R2[g] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
+            }
+        }
+        if (k + 1 < chunks) {
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                pre[i] = (e < E) ? fetch(k + 1, e) : zero;
+            }
+        }
+        const float4* cur = sh + (k & 1) * E;
+#pragma unroll 1
+        for (int i = 0; i < PX; i += 4) {
+            const float4 xq = cur[ER + (i >> 2)];
+            const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
+                float pv[CP];
+#pragma unroll
+                for (int q4 = 0; q4 < CP4; ++q4) {
+                    const float4 tq = cur[(i + j) * CP4 + q4];
+                    pv[4 * q4] = tq.x;
+                    pv[4 * q4 + 1] = tq.y;
+                    pv[4 * q4 + 2] = tq.z;
+                    pv[4 * q4 + 3] = tq.w;
+                }
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    const float dx = xq[j] - px[g];
+                    const float dx = xs4[j] - px[g];
                     const float tt = fmaf(A[g], dx, bdy[g]);
                     const float q = fmaf(tt, dx, cyy[g]);
                     const float e = hw_exp2(q);
-                    float Gv = pq.v[j][0] * col[g][0];
+                    float Gv = pv[C];  // -s
 #pragma unroll
-                    for (int c = 1; c < C; ++c) Gv = fmaf(pq.v[j][c], col[g][c], Gv);
-                    Gv += pq.v[j][C];
+                    for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[g][c], Gv);
                     const float ge = Gv * e;
                     R0[g] += ge;
                     const float t1 = ge * dx;
                     R1[g] += t1;
                     R2[g] = fmaf(t1, dx, R2[g]);
 #pragma unroll
-                    for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pq.v[j][c], RC[g][c]);
+                    for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[c], RC[g][c]);
                 }
             }
-        };
-        const float* prow = a.pixrec + ((size_t)b * a.H + r) * a.Wp * CP;
-        const float* xp = xrow;
-        PixQuad<CP> qa = load_quad<CP>(prow);
-        float xa[4] = {xp[0], xp[1], xp[2], xp[3]};
-        for (int o = 0; o < octs; ++o) {
-            const PixQuad<CP> qb = load_quad<CP>(prow + 4 * CP);
-            const float xb[4] = {xp[4], xp[5], xp[6], xp[7]};
-            body(qa, xa);
-            const bool more = o + 1 < octs;
-            const float* pn = more ? prow + 8 * CP : prow;  // last: harmless re-read
-            const float* xn = more ? xp + 8 : xp;
-            qa = load_quad<CP>(pn);
-            xa[0] = xn[0]; xa[1] = xn[1]; xa[2] = xn[2]; xa[3] = xn[3];
-            body(qb, xb);
-            prow = pn;
-            xp = xn;
         }
+        if (seg == segs - 1) {  // the row is complete
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-            M[g][0] += R0[g];
-            M[g][1] += R1[g];
-            M[g][3] += R2[g];
-            M[g][2] = fmaf(dy[g], R0[g], M[g][2]);
-            M[g][4] = fmaf(dy[g], R1[g], M[g][4]);
-            M[g][5] = fmaf(dy[g] * dy[g], R0[g], M[g][5]);
+            for (int g = 0; g < G; ++g) {
+                M[g][0] += R0[g];
+                M[g][1] += R1[g];
+                M[g][3] += R2[g];
+                M[g][2] = fmaf(dy[g], R0[g], M[g][2]);
+                M[g][4] = fmaf(dy[g], R1[g], M[g][4]);
+                M[g][5] = fmaf(dy[g] * dy[g], R0[g], M[g][5]);
 #pragma unroll
-            for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+                for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+            }
         }
+        if (k + 1 < chunks) {
+            float4* nxt = sh + ((k + 1) & 1) * E;
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                if (e < E) nxt[e] = pre[i];
+            }
+        }
+        __syncthreads();
     }
     bwd_store<C, G>(a, b, t, n, M, CG);
 }
 
 // General grid: the tile is a flat pixel range (multiple of 256); x and y come with the
-// pixel record.  Sums are flushed into the totals every 256 pixels (two-level summation).
+// pixel record.  Sums are flushed into the totals once per 128-pixel chunk.
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
-    constexpr int CP = pix_stride_gen(C);
+    constexpr int CP = pix_stride_gen(C), CP4 = CP / 4;
+    __shared__ float4 sh[2 * kPixChunk * CP4];
     IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
     int n[G];
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
     bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
-    float M[G][6], CG[G][C];
+    float M[G][6], CG[G][C], R[G][6], RC[G][C];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
 #pragma unroll
-        for (int f = 0; f < 6; ++f) M[g][f] = 0.0f;
+        for (int f = 0; f < 6; ++f) M[g][f] = R[g][f] = 0.0f;
 #pragma unroll
-        for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
+        for (int c = 0; c < C; ++c) CG[g][c] = RC[g][c] = 0.0f;
     }
-    const int p0 = t * a.per_tile, p1 = min(a.HWp, p0 + a.per_tile);  // HWp % 4 == 0
-    for (int pc = p0; pc < p1; pc += 256) {
-        const int pe = min(p1, pc + 256);
-        float R[G][6], RC[G][C];
+    const int p0 = t * a.per_tile, p1 = min(a.HWp, p0 + a.per_tile);
+    const float4* src = reinterpret_cast<const float4*>(a.pixrec + ((size_t)b * a.HWp + p0) * CP);
+    int seen = 0;
+    stream_records_lds<CP4, kPixChunk>(src, p1 - p0, sh, [&](const float4* r) {
+        float pv[CP];
+#pragma unroll
+        for (int q4 = 0; q4 < CP4; ++q4) {
+            const float4 tq = r[q4];
+            pv[4 * q4] = tq.x;
+            pv[4 * q4 + 1] = tq.y;
+            pv[4 * q4 + 2] = tq.z;
+            pv[4 * q4 + 3] = tq.w;
+        }
 #pragma unroll
         for (int g = 0; g < G; ++g) {
+            const float dx = pv[0] - px[g];
+            const float dy = pv[1] - py[g];
+            float tt = A[g] * dx;
+            tt = fmaf(B2[g], dy, tt);
+            const float v = D[g] * dy;
+            float q = tt * dx;
+            q = fmaf(v, dy, q);
+            const float e = hw_exp2(q);
+            float Gv = pv[2 + C];  // -s
 #pragma unroll
-            for (int f = 0; f < 6; ++f) R[g][f] = 0.0f;
+            for (int c = 0; c < C; ++c) Gv = fmaf(pv[2 + c], col[g][c], Gv);
+            const float ge = Gv * e;
+            R[g][0] += ge;
+            const float t1 = ge * dx, t2 = ge * dy;
+            R[g][1] += t1;
+            R[g][2] += t2;
+            R[g][3] = fmaf(t1, dx, R[g][3]);
+            R[g][4] = fmaf(t1, dy, R[g][4]);
+            R[g][5] = fmaf(t2, dy, R[g][5]);
 #pragma unroll
-            for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
+            for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[2 + c], RC[g][c]);
         }
-        const float* prec = a.pixrec + ((size_t)b * a.HWp + pc) * CP;
-        for (int p = pc; p < pe; p += 4, prec += 4 * CP) {
-            const PixQuad<CP> pq = load_quad<CP>(prec);
+        if ((++seen & (kPixChunk - 1)) == 0) {  // two-level summation
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int g = 0; g < G; ++g) {
 #pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    const float dx = pq.v[j][0] - px[g];
-                    const float dy = pq.v[j][1] - py[g];
-                    float tt = A[g] * dx;
-                    tt = fmaf(B2[g], dy, tt);
-                    const float v = D[g] * dy;
-                    float q = tt * dx;
-                    q = fmaf(v, dy, q);
-                    const float e = hw_exp2(q);
-                    float Gv = pq.v[j][2] * col[g][0];
+                for (int f = 0; f < 6; ++f) {
+                    M[g][f] += R[g][f];
+                    R[g][f] = 0.0f;
+                }
 #pragma unroll
-                    for (int c = 1; c < C; ++c) Gv = fmaf(pq.v[j][2 + c], col[g][c], Gv);
-                    Gv += pq.v[j][2 + C];
-                    const float ge = Gv * e;
-                    R[g][0] += ge;
-                    const float t1 = ge * dx, t2 = ge * dy;
-                    R[g][1] += t1;
-                    R[g][2] += t2;
-                    R[g][3] = fmaf(t1, dx, R[g][3]);
-                    R[g][4] = fmaf(t1, dy, R[g][4]);
-                    R[g][5] = fmaf(t2, dy, R[g][5]);
-#pragma unroll
-                    for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pq.v[j][2 + c], RC[g][c]);
+                for (int c = 0; c < C; ++c) {
+                    CG[g][c] += RC[g][c];
+                    RC[g][c] = 0.0f;
                 }
             }
         }
+    });
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
+    for (int g = 0; g < G; ++g) {
 #pragma unroll
-            for (int f = 0; f < 6; ++f) M[g][f] += R[g][f];
+        for (int f = 0; f < 6; ++f) M[g][f] += R[g][f];
 #pragma unroll
-            for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
-        }
+        for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
     }
     bwd_store<C, G>(a, b, t, n, M, CG);
 }
@@ -709,9 +825,10 @@ struct GridGradArgs {
 
 template <int C, int P>
 __global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
-    constexpr int RS = rec_stride_of(C);
+    constexpr int RS = rec_stride_of(C), R4 = RS / 4;
+    __shared__ float4 sh[2 * kGaussChunk * R4];
     const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
-    if (tile >= a.total_tiles) return;
+    if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int b = tile / a.tiles_per_img;
     const int tl = tile - b * a.tiles_per_img;
     const int HW = a.H * a.W;
@@ -734,7 +851,9 @@ __global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
         negs[j] = -s;
         sx[j] = sy[j] = 0.0f;
     }
-    stream_gaussians<C>(a.packed + (size_t)b * a.Np * RS, a.Np >> 2, [&](const GRec<C>& g) {
+    const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
+    stream_records_lds<R4, kGaussChunk>(src, a.Np, sh, [&](const float4* r) {
+        const GRec<C> g = lds_grec<C>(r);
         const float hb = 0.5f * g.B2;
 #pragma unroll
         for (int j = 0; j < P; ++j) {
@@ -844,7 +963,7 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     const bool sep = grid_mode == IGS_GRID_SEPARABLE;
     int cus = device_cus();
     if (cus <= 0) cus = 256;
-    const long target_waves = (long)cus * 4 * 4;  // 4 waves per SIMD
+    const long target_waves = (long)cus * 4 * IGS_FWD_WAVES;  // forward: waves per SIMD wanted
     p->B = B; p->N = N; p->H = H; p->W = W; p->C = C;
     p->rec_stride = rec_stride_of(C);
     p->n_padded = (N + 3) & ~3;
@@ -862,7 +981,7 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     p->fwd_split = (int)S;
     p->fwd_n_per_split = nps;
     const long groups = (long)B * ceil_div(N, kThreads * kBwdG) * 4;  // waves per tile
-    long T = (target_waves * 2 + groups - 1) / groups;                   // 8 waves per SIMD
+    long T = ((long)cus * 4 * IGS_BWD_WAVES + groups - 1) / groups;     // backward: waves per SIMD wanted
     const long maxT = sep ? H : ceil_div(p->hw_padded, 256);
     if (T > maxT) T = maxT;
     if (T < 1) T = 1;
