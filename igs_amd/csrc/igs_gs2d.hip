@@ -46,10 +46,10 @@ constexpr int kThreads = 256;
 #define IGS_BWD_G 2
 #endif
 #ifndef IGS_FWD_WAVES
-#define IGS_FWD_WAVES 4
+#define IGS_FWD_WAVES 8
 #endif
 #ifndef IGS_BWD_WAVES
-#define IGS_BWD_WAVES 8
+#define IGS_BWD_WAVES 16
 #endif
 constexpr int kFwdSepP = IGS_FWD_SEP_P;  // rows per lane, separable forward
 constexpr int kFwdGenP = 4;  // pixels per lane, general forward
@@ -151,7 +151,7 @@ struct GRec {
     float ac[C];
 };
 
-// Reads one record from (wave-uniform) LDS address r.
+// Unpacks one record held in R4 float4 registers (read from a wave-uniform LDS address).
 template <int C>
 __device__ __forceinline__ GRec<C> lds_grec(const float4* r) {
     constexpr int R4 = rec_stride_of(C) / 4;
@@ -221,8 +221,22 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
             }
         }
         const float4* cur = sh + (k & 1) * E;
-#pragma unroll 2
-        for (int n = 0; n < CH; ++n) body(cur + n * R4);
+        // register double-buffering of the LDS reads: record n+1 is read while n is consumed
+        float4 ra[R4], rb[R4];
+#pragma unroll
+        for (int i = 0; i < R4; ++i) ra[i] = cur[i];
+#pragma unroll 1
+        for (int n = 0; n < CH; n += 2) {
+#pragma unroll
+            for (int i = 0; i < R4; ++i) rb[i] = cur[(n + 1) * R4 + i];
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads above the work that hides them
+            body(ra);
+            const int nn = (n + 2 < CH) ? n + 2 : 0;  // last: harmless re-read
+#pragma unroll
+            for (int i = 0; i < R4; ++i) ra[i] = cur[nn * R4 + i];
+            __builtin_amdgcn_sched_barrier(0);
+            body(rb);
+        }
         if (k + 1 < chunks) {
             float4* nxt = sh + ((k + 1) & 1) * E;
 #pragma unroll
@@ -293,15 +307,22 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
         const float adx = g.A * dx;
         const float c0 = adx * dx;
         const float c1 = g.B2 * dx;
+        // three phases, so that the P independent chains overlap their latencies and the
+        // transcendental ops issue back to back
+        float e[P];
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             const float dy = yv[p] - g.py;
             const float t = fmaf(g.D, dy, c1);
-            const float q = fmaf(t, dy, c0);
-            const float e = hw_exp2(q);
-            dsum[p] = fmaf(e, g.al, dsum[p]);
+            e[p] = fmaf(t, dy, c0);
+        }
 #pragma unroll
-            for (int c = 0; c < C; ++c) num[p][c] = fmaf(e, g.ac[c], num[p][c]);
+        for (int p = 0; p < P; ++p) e[p] = hw_exp2(e[p]);
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            dsum[p] = fmaf(e[p], g.al, dsum[p]);
+#pragma unroll
+            for (int c = 0; c < C; ++c) num[p][c] = fmaf(e[p], g.ac[c], num[p][c]);
         }
     });
     if (col < a.W) {
@@ -593,6 +614,23 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
         for (int i = 0; i < PX; i += 4) {
             const float4 xq = cur[ER + (i >> 2)];
             const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
+            // phase 1: exponents of the 4 x G pairs (independent chains)
+            float dxs[4][G], ee[4][G];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const float dx = xs4[j] - px[g];
+                    const float tt = fmaf(A[g], dx, bdy[g]);
+                    ee[j][g] = fmaf(tt, dx, cyy[g]);
+                    dxs[j][g] = dx;
+                }
+            // phase 2: transcendentals back to back
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int g = 0; g < G; ++g) ee[j][g] = hw_exp2(ee[j][g]);
+            // phase 3: G = <g^, c> - s and the row sums
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float pv[CP];
@@ -606,10 +644,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
                 }
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    const float dx = xs4[j] - px[g];
-                    const float tt = fmaf(A[g], dx, bdy[g]);
-                    const float q = fmaf(tt, dx, cyy[g]);
-                    const float e = hw_exp2(q);
+                    const float e = ee[j][g], dx = dxs[j][g];
                     float Gv = pv[C];  // -s
 #pragma unroll
                     for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[g][c], Gv);
