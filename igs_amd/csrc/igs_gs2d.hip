@@ -40,7 +40,7 @@ namespace {
 constexpr float kNegHalfLog2e = -0.72134752044448170368f;  // -0.5 * log2(e)
 constexpr int kThreads = 256;
 #ifndef IGS_FWD_SEP_P
-#define IGS_FWD_SEP_P 8
+#define IGS_FWD_SEP_P 16
 #endif
 #ifndef IGS_BWD_G
 #define IGS_BWD_G 2
@@ -51,7 +51,8 @@ constexpr int kThreads = 256;
 #ifndef IGS_BWD_WAVES
 #define IGS_BWD_WAVES 16
 #endif
-constexpr int kFwdSepP = IGS_FWD_SEP_P;  // rows per lane, separable forward
+// rows per lane in the separable forward: as many as the accumulator VGPRs (P x (C+1)) allow
+__host__ __device__ constexpr int fwd_sep_p(int C) { return C <= 3 ? IGS_FWD_SEP_P : (C <= 8 ? 8 : 4); }
 constexpr int kFwdGenP = 4;  // pixels per lane, general forward
 constexpr int kBwdG = IGS_BWD_G;  // Gaussians per lane, backward
 
@@ -183,7 +184,13 @@ __device__ __forceinline__ float in_vgpr(float v) {
     return v;
 }
 
-constexpr int kGaussChunk = 64;  // Gaussian records per LDS buffer
+#ifndef IGS_GCHUNK
+#define IGS_GCHUNK 64
+#endif
+#ifndef IGS_PCHUNK
+#define IGS_PCHUNK 256
+#endif
+constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
 
 // Streams `count` records of R4 float4 each from global memory to every wave of the
 // workgroup through the double-buffered LDS window sh[2][CH*R4]; body(const float4* rec) runs
@@ -530,7 +537,8 @@ __device__ __forceinline__ void bwd_load_gaussians(const BwdArgs& a, int b, int 
     }
 }
 
-constexpr int kPixChunk = 128;  // pixel records per LDS buffer
+// pixel records per LDS buffer; wide records get a shorter chunk so the two buffers stay small
+__host__ __device__ constexpr int pix_chunk(int C) { return C <= 4 ? IGS_PCHUNK : 128; }
 
 // Separable grid: lane = G Gaussians; the tile is a range of full rows.  Pixel records and
 // column coordinates of 128-pixel row segments stream through LDS (double-buffered) and are
@@ -540,7 +548,7 @@ constexpr int kPixChunk = 128;  // pixel records per LDS buffer
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     constexpr int CP = pix_stride_sep(C), CP4 = CP / 4;
-    constexpr int PX = kPixChunk;
+    constexpr int PX = pix_chunk(C);
     constexpr int ER = PX * CP4;   // float4 of pixel records per chunk
     constexpr int EX = PX / 4;     // float4 of x coordinates per chunk
     constexpr int E = ER + EX;
@@ -689,6 +697,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     constexpr int CP = pix_stride_gen(C), CP4 = CP / 4;
+    constexpr int kPixChunk = pix_chunk(C);
     __shared__ float4 sh[2 * kPixChunk * CP4];
     IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
@@ -963,8 +972,9 @@ struct FwdGeometry {
     int wx, tiles_x, tiles_y, total_tiles;
 };
 
-FwdGeometry fwd_geometry(int B, int H, int W, bool sep) {
+FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
     FwdGeometry g;
+    const int kFwdSepP = fwd_sep_p(C);
     if (sep) {
         // choose the wave arrangement (wx waves along the columns) that wastes the fewest lanes
         long best = -1;
@@ -1004,7 +1014,7 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     p->n_padded = (N + 3) & ~3;
     p->w_padded = sep ? (W + 7) & ~7 : W;
     p->hw_padded = (H * W + 3) & ~3;
-    const FwdGeometry fg = fwd_geometry(B, H, W, sep);
+    const FwdGeometry fg = fwd_geometry(B, H, W, C, sep);
     long S = (target_waves + (long)fg.total_tiles * 4 - 1) / ((long)fg.total_tiles * 4);
     const long maxS = N / 64 > 0 ? N / 64 : 1;  // keep >= 64 Gaussians per split
     if (S > maxS) S = maxS;
@@ -1093,7 +1103,7 @@ int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
     const int blocks = ((a.total_tiles + 7) / 8) * 8;
     const dim3 grid(blocks, a.S, 1);
     if (sep)
-        hipLaunchKernelGGL((k_fwd_sep<C, kFwdSepP>), grid, dim3(kThreads), 0, st, a);
+        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C)>), grid, dim3(kThreads), 0, st, a);
     else
         hipLaunchKernelGGL((k_fwd_gen<C, kFwdGenP>), grid, dim3(kThreads), 0, st, a);
     return launch_status();
@@ -1239,7 +1249,7 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
         rc = plan_one(B, N, H, W, C, vs[i].mode, &plan);
         if (rc) return rc;
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
-        const FwdGeometry fg = fwd_geometry(B, H, W, sep);
+        const FwdGeometry fg = fwd_geometry(B, H, W, C, sep);
         FwdArgs a;
         a.packed = packed; a.x = x; a.y = y;
         a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
