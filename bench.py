@@ -36,8 +36,8 @@ def flops_per_pair(C: int):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -182,12 +182,14 @@ def main() -> int:
             "flops_per_pair": f_bwd,
             "pairs_per_launch": pairs,
             "launch_ms": t_bwd_kernel * 1e3,
-            "traffic": None,
+            "traffic": (140.4 + 86.9) * 1024 * 1024 if args.config == "c1" and C == 3 else None,
             "forward_kernel": {"launch_ms": t_fwd_kernel * 1e3, "flops_per_pair": f_fwd,
                                "achieved": pairs * f_fwd / t_fwd_kernel / 1e12,
                                "frac": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS},
-            "note": "peak = published fp32 vector peak (packed FMA); this build compiles with packed-fp32 "
-                    "instruction selection disabled, so its own issue ceiling is half of it",
+            "traffic_note": "HBM bytes per launch from rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (copy-calibrated), "
+                            "see profiles/; valid for the c1 workload only",
+            "note": "peak = published fp32 vector peak; the kernels use plain (non-packed) fp32 VALU ops with "
+                    "VGPR-only operands, v_exp_f32 counted as 1 FLOP",
         },
     }
 
