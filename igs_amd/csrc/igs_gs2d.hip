@@ -6,25 +6,25 @@
 //
 // Design in one paragraph.  The path is bound by fp32 VALU + transcendental issue, not by
 // HBM (a few tens of MB per call) and not by MFMA (colour contraction has C = 3), so the
-// kernels are organised to need no cross-lane reduction at all and the fewest VALU
-// instructions per (Gaussian, pixel) pair:
-//   * forward  : a lane owns pixels, the Gaussian record is wave-uniform and arrives
-//                through the scalar data path (s_load -> SGPR operands); den and the C
+// kernels are organised to need no cross-lane reduction at all and the fewest, cheapest
+// VALU instructions per (Gaussian, pixel) pair:
+//   * forward  : a lane owns pixels, the Gaussian record is wave-uniform; den and the C
 //                numerators stay in VGPRs for the whole Gaussian loop.
 //   * backward : a lane owns Gaussians, the pixel record (g^ = g/(den+eps), -s = -<g^,out>)
-//                is wave-uniform (SGPRs); the lane accumulates the six moments of G e and
-//                the C colour sums over its pixel tile in VGPRs.  Per-tile partials go to a
+//                is wave-uniform; the lane accumulates the six moments of G e and the C
+//                colour sums over its pixel tile in VGPRs.  Per-tile partials go to a
 //                [B,T,6+C,N] buffer which a finalize kernel sums in a fixed order (no
 //                float atomics anywhere, bit-reproducible).
+//   * the wave-uniform record stream goes global -> LDS (cooperative, double-buffered) ->
+//     VGPRs (broadcast ds_read_b128), because on gfx950 a VALU op with VGPR-only operands
+//     issues almost twice as fast as one with an SGPR operand.
 //   * separable grids (x independent of the row, y independent of the column: every
 //     linspace grid) let both kernels hoist the row/column part of the quadratic form and
 //     of the moment sums: 3 VALU ops per pair for q instead of 7, 5 instead of 9 for the
 //     moments.
 // exp() is one v_exp_f32: A, 2B, D are pre-multiplied by -0.5 log2(e) when packed.
-// Streams of uniform records are software-pipelined by hand: the next group of records is
-// requested right after the wait for the current one, so the scalar-load latency is
-// covered by the current group's VALU work.  Record arrays are zero-padded (alpha = 0 /
-// g^ = 0 records contribute exactly 0) so the hot loops have no tails.
+// Record arrays are zero-padded (alpha = 0 / g^ = 0 records contribute exactly 0) so the hot
+// loops have no tails.
 //
 // Build flags disable packed-fp32 instruction selection (-packed-fp32-ops), so every VALU
 // op below is a scalar-per-lane fp32 op.
