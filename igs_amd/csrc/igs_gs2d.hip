@@ -92,12 +92,14 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         return;
     }
     const size_t i = (size_t)b * N + n;
-    float A, Bc, D;
+    // The closed form runs in fp64 and is rounded once: an error of a few fp32 ulp in A', B2', D'
+    // would be multiplied by |q| (tens, for sharp Gaussians) in the exponent.  O(BN) work.
+    double A, Bc, D;
     if (kScaleRot) {
-        const float s0 = p0[2 * i], s1 = p0[2 * i + 1];
-        float sn, cs;
-        sincosf(p1[i], &sn, &cs);
-        const float i0 = 1.0f / (s0 * s0 + eps), i1 = 1.0f / (s1 * s1 + eps);
+        const double s0 = p0[2 * i], s1 = p0[2 * i + 1];
+        double sn, cs;
+        sincos((double)p1[i], &sn, &cs);
+        const double i0 = 1.0 / (s0 * s0 + (double)eps), i1 = 1.0 / (s1 * s1 + (double)eps);
         A = cs * cs * i0 + sn * sn * i1;
         Bc = cs * sn * (i0 - i1);
         D = sn * sn * i0 + cs * cs * i1;
@@ -106,12 +108,13 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         Bc = p1[i];
         D = p2[i];
     }
+    constexpr double k = -0.72134752044448170368;  // -0.5 * log2(e)
     const float al = alphas[i];
     r[0] = position[2 * i];
     r[1] = position[2 * i + 1];
-    r[2] = kNegHalfLog2e * A;
-    r[3] = 2.0f * kNegHalfLog2e * Bc;
-    r[4] = kNegHalfLog2e * D;
+    r[2] = (float)(k * A);
+    r[3] = (float)(2.0 * k * Bc);
+    r[4] = (float)(k * D);
     r[5] = al;
     for (int c = 0; c < C; ++c) r[6 + c] = al * colors[i * C + c];
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
@@ -803,14 +806,15 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
         for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + f) * N];
         M[f] = s;
     }
-    const float al = alphas[i];
-    float A, Bc, D, cs = 0.f, sn = 0.f, i0 = 0.f, i1 = 0.f, s0 = 0.f, s1 = 0.f;
+    const double al = alphas[i];
+    // O(BN) epilogue in fp64: the chain rule multiplies sums by 1/s^3-sized factors
+    double A, Bc, D, cs = 0., sn = 0., i0 = 0., i1 = 0., s0 = 0., s1 = 0.;
     if (kScaleRot) {
         s0 = p0[2 * i];
         s1 = p0[2 * i + 1];
-        sincosf(p1[i], &sn, &cs);
-        i0 = 1.0f / (s0 * s0 + eps);
-        i1 = 1.0f / (s1 * s1 + eps);
+        sincos((double)p1[i], &sn, &cs);
+        i0 = 1.0 / (s0 * s0 + (double)eps);
+        i1 = 1.0 / (s1 * s1 + (double)eps);
         A = cs * cs * i0 + sn * sn * i1;
         Bc = cs * sn * (i0 - i1);
         D = sn * sn * i0 + cs * cs * i1;
@@ -821,28 +825,28 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     }
     if (g_alpha) g_alpha[i] = M[0];
     if (g_pos) {
-        g_pos[2 * i] = al * (A * M[1] + Bc * M[2]);
-        g_pos[2 * i + 1] = al * (Bc * M[1] + D * M[2]);
+        g_pos[2 * i] = (float)(al * (A * M[1] + Bc * M[2]));
+        g_pos[2 * i + 1] = (float)(al * (Bc * M[1] + D * M[2]));
     }
-    const float gA = -0.5f * al * M[3], gB = -al * M[4], gD = -0.5f * al * M[5];
+    const double gA = -0.5 * al * M[3], gB = -al * M[4], gD = -0.5 * al * M[5];
     if (kScaleRot) {
         if (g0) {  // scales [B,N,2]
-            const float gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
-            const float gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
-            g0[2 * i] = gi0 * (-2.0f * s0 * i0 * i0);
-            g0[2 * i + 1] = gi1 * (-2.0f * s1 * i1 * i1);
+            const double gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
+            const double gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
+            g0[2 * i] = (float)(gi0 * (-2.0 * s0 * i0 * i0));
+            g0[2 * i + 1] = (float)(gi1 * (-2.0 * s1 * i1 * i1));
         }
-        if (g1) g1[i] = (gD - gA) * 2.0f * Bc + gB * (cs * cs - sn * sn) * (i0 - i1);
+        if (g1) g1[i] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
     } else {
-        if (g0) g0[i] = gA;
-        if (g1) g1[i] = gB;
-        if (g2) g2[i] = gD;
+        if (g0) g0[i] = (float)gA;
+        if (g1) g1[i] = (float)gB;
+        if (g2) g2[i] = (float)gD;
     }
     if (g_col) {
         for (int c = 0; c < C; ++c) {
             float s = 0.0f;
             for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + 6 + c) * N];
-            g_col[i * C + c] = al * s;
+            g_col[i * C + c] = (float)al * s;
         }
     }
 }

@@ -342,3 +342,19 @@ def make_config_inputs(name: str, dtype=torch.float32, **override):
     cfg.update(override)
     seed = 1000 + int(name[1:])
     return make_inputs(seed=seed, dtype=dtype, **cfg)
+
+
+def smooth_noise_target(H, W, seed, C=3, dtype=torch.float32):
+    """Seeded smooth target image for the single-image fit configuration: 64 random
+    sinusoids, `clip(0.5 + 1/8 sum_k a_kc sin(pi (fx_k x + fy_k y) + phi_k), 0, 1)` on the
+    x = linspace(-W/H, W/H, W), y = linspace(-1, 1, H) grid.  Returns [1, C, H, W]."""
+    g = torch.Generator().manual_seed(seed)
+    fx = torch.rand(64, generator=g, dtype=torch.float64) * 8 - 4
+    fy = torch.rand(64, generator=g, dtype=torch.float64) * 8 - 4
+    ph = torch.rand(64, generator=g, dtype=torch.float64) * (2 * math.pi)
+    amp = torch.rand(64, C, generator=g, dtype=torch.float64)
+    x = torch.linspace(-W / H, W / H, W, dtype=torch.float64).view(1, 1, W)
+    y = torch.linspace(-1, 1, H, dtype=torch.float64).view(1, H, 1)
+    s = torch.sin(math.pi * (fx.view(-1, 1, 1) * x + fy.view(-1, 1, 1) * y) + ph.view(-1, 1, 1))   # [64,H,W]
+    img = 0.5 + 0.125 * torch.einsum("khw,kc->chw", s, amp)
+    return img.clamp(0, 1)[None].to(dtype)
