@@ -66,6 +66,9 @@ SIGNATURES = {
                                          _FP, _FP, _FP, _FP, _FP, _FP, c_void_p]),
     "igs_gs2d_finalize_scale_rot": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                             c_float, _FP, _FP, _FP, _FP, _FP, c_void_p]),
+    "igs_gs2d_pack_feature": (c_int, [_FP, _FP, c_int, c_int, c_int, c_int, c_float, _FP, _FP, c_void_p]),
+    "igs_gs2d_finalize_feature": (c_int, [_FP, c_int, _FP, _FP, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                                          _FP, c_void_p]),
 }
 
 _lib = None

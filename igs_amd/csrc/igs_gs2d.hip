@@ -120,6 +120,53 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
 }
 
+// Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
+// opacity logit (unused), c_0..c_{C-1}] (reference src/igs/gs2d.py:635-644) and applies the
+// module's activations scales = exp(log_s) + eps, alpha = 1 (src/igs/gs2d.py:673-675), plus
+// an optional position offset (pos_map_offset, src/igs/gs2d.py:654-667).  Also writes the raw
+// colours [B][N][Cp] (zero-padded to the kernels' channel count) that the backward reads.
+__global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restrict__ feat,
+                                                           const float* __restrict__ pos_off, int N,
+                                                           int Np, int C, int Cp, int RS, float eps,
+                                                           float* __restrict__ packed,
+                                                           float* __restrict__ colors_out) {
+    const int n = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (n >= Np) return;
+    float* r = packed + ((size_t)b * Np + n) * RS;
+    if (n >= N) {
+        for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        return;
+    }
+    const size_t i = (size_t)b * N + n;
+    const float* f = feat + i * (6 + C);
+    const double s0 = (double)expf(f[2]) + (double)eps, s1 = (double)expf(f[3]) + (double)eps;
+    double sn, cs;
+    sincos((double)f[4], &sn, &cs);
+    const double i0 = 1.0 / (s0 * s0 + (double)eps), i1 = 1.0 / (s1 * s1 + (double)eps);
+    const double A = cs * cs * i0 + sn * sn * i1;
+    const double Bc = cs * sn * (i0 - i1);
+    const double D = sn * sn * i0 + cs * cs * i1;
+    constexpr double k = -0.72134752044448170368;
+    float px = f[0], py = f[1];
+    if (pos_off) {
+        px += pos_off[2 * i];
+        py += pos_off[2 * i + 1];
+    }
+    r[0] = px;
+    r[1] = py;
+    r[2] = (float)(k * A);
+    r[3] = (float)(2.0 * k * Bc);
+    r[4] = (float)(k * D);
+    r[5] = 1.0f;
+    for (int c = 0; c < Cp; ++c) {
+        const float col = c < C ? f[6 + c] : 0.0f;
+        r[6 + c] = col;
+        colors_out[i * Cp + c] = col;
+    }
+    for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
+}
+
 // ----------------------------------------------------------------------------- forward
 struct FwdArgs {
     const float* packed;  // [B][Np][RS]
@@ -851,6 +898,51 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     }
 }
 
+// Finalize for the fused module head: d gs_feature [B][N][6+C] from the tile partials, with
+// alpha = 1, d log_s_k = d s_k * exp(log_s_k) and a zero gradient for the unused opacity logit.
+__global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
+    const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
+    const float* __restrict__ feat, int N, int C, int Cp, float eps, float* __restrict__ g_feat) {
+    const int n = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (n >= N) return;
+    const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
+    const int NF = 6 + Cp;
+    const size_t i = (size_t)b * N + n;
+    const float* base = partial + (size_t)b * T * NF * N + n;
+    float M[6];
+#pragma unroll
+    for (int f = 0; f < 6; ++f) {
+        float s = 0.0f;
+        for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + f) * N];
+        M[f] = s;
+    }
+    const float* f = feat + i * (6 + C);
+    const double e0 = (double)expf(f[2]), e1 = (double)expf(f[3]);
+    const double s0 = e0 + (double)eps, s1 = e1 + (double)eps;
+    double sn, cs;
+    sincos((double)f[4], &sn, &cs);
+    const double i0 = 1.0 / (s0 * s0 + (double)eps), i1 = 1.0 / (s1 * s1 + (double)eps);
+    const double A = cs * cs * i0 + sn * sn * i1;
+    const double Bc = cs * sn * (i0 - i1);
+    const double D = sn * sn * i0 + cs * cs * i1;
+    const double gA = -0.5 * M[3], gB = -(double)M[4], gD = -0.5 * M[5];
+    const double gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
+    const double gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
+    float* g = g_feat + i * (6 + C);
+    g[0] = (float)(A * M[1] + Bc * M[2]);
+    g[1] = (float)(Bc * M[1] + D * M[2]);
+    g[2] = (float)(gi0 * (-2.0 * s0 * i0 * i0) * e0);
+    g[3] = (float)(gi1 * (-2.0 * s1 * i1 * i1) * e1);
+    g[4] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
+    g[5] = 0.0f;
+    for (int c = 0; c < C; ++c) {
+        float sum = 0.0f;
+        for (int t = 0; t < T; ++t) sum += base[((size_t)t * NF + 6 + c) * N];
+        g[6 + c] = sum;
+    }
+}
+
 // ----------------------------------------------------------------------------- grid grads
 // Optional: d L / d x(pixel), d L / d y(pixel) = -sum_n G_n w_n (A dx + B dy), (B dx + D dy).
 // Pixel-major like the forward (lane = P pixels, Gaussian record wave-uniform); the per-pixel
@@ -1418,6 +1510,35 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, scales, rotations, (const float*)nullptr, alphas, N, C, eps, g_positions,
                        g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
+    return launch_status();
+}
+
+int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int B, int N, int C,
+                          int C_kernel, float eps, float* packed, float* colors_out,
+                          igs_stream_t stream) {
+    if (!gs_feature || !packed || !colors_out) return IGS_ERR_NULL_POINTER;
+    if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
+    if (C < 1 || C > C_kernel || !channels_compiled(C_kernel)) return IGS_ERR_BAD_CHANNELS;
+    const int Np = (N + 3) & ~3;
+    hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
+                       (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
+                       rec_stride_of(C_kernel), eps, packed, colors_out);
+    return launch_status();
+}
+
+int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t* grid_flag,
+                              const float* gs_feature, int B, int N, int H, int W, int C,
+                              int C_kernel, float eps, float* g_feature, igs_stream_t stream) {
+    if (!partial || !gs_feature || !g_feature) return IGS_ERR_NULL_POINTER;
+    int rc = mode_ok(grid_mode, grid_flag);
+    if (rc) return rc;
+    if (C < 1 || C > C_kernel || !channels_compiled(C_kernel)) return IGS_ERR_BAD_CHANNELS;
+    int T, T_alt;
+    rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_bwd_finalize_feature, dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
+                       (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
+                       T_alt, gs_feature, N, C, C_kernel, eps, g_feature);
     return launch_status();
 }
 

@@ -60,8 +60,15 @@ def _padded_channels(C: int) -> int:
     for c in _lib.COMPILED_CHANNELS:
         if c >= C:
             return c
-    raise NotImplementedError(
-        f"output_dim / colour channels C={C} > {_lib.IGS_MAX_CHANNELS} is not supported by the HIP kernels")
+    raise ValueError(f"C={C} exceeds the {_lib.IGS_MAX_CHANNELS} channels of one kernel pass")
+
+
+def _channel_groups(C: int):
+    """More than IGS_MAX_CHANNELS channels are rendered in groups of that many: each group's output
+    depends on its own colours only, and autograd adds the groups' gradients w.r.t. the shared
+    geometry (the backward moments are additive over channel groups: s = sum_groups <g^, out>_group)."""
+    m = _lib.IGS_MAX_CHANNELS
+    return [(i, min(i + m, C)) for i in range(0, C, m)]
 
 
 def _pad_last(t: Tensor, Cp: int) -> Tensor:
@@ -230,6 +237,15 @@ class GaussianSplatting2DKernel(torch.autograd.Function):
     BLOCK_SIZE_H = BLOCK_SIZE_W = BWD_BLOCK_SIZE_H = BWD_BLOCK_SIZE_W = -1
     N_CHUNK_SIZE = 32
 
+    @classmethod
+    def apply(cls, x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
+        C = colors.shape[-1]
+        if C <= _lib.IGS_MAX_CHANNELS:
+            return super().apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps)
+        return torch.cat([super(GaussianSplatting2DKernel, cls).apply(
+            x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors[..., lo:hi], eps)
+            for lo, hi in _channel_groups(C)], dim=1)
+
     @staticmethod
     def forward(ctx, x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
         _require_gpu(position)
@@ -361,6 +377,65 @@ class _RenderFused(torch.autograd.Function):
         return cast(g_pos, 0), cast(g_col, 1), cast(g_sc, 2), cast(g_rot, 3), cast(g_al, 4), g_x, g_y, None
 
 
+class _RenderFromFeature(torch.autograd.Function):
+    """(gs_feature [B,N,6+C], pos_offset or None, x_grid, y_grid, eps) -> [B,C,H,W].
+
+    The module's split / exp(log_scale)+eps / alpha = 1 (src/igs/gs2d.py:638-675) run inside the
+    pack kernel and their autograd inside the finalize kernel, so the only torch ops left around
+    the splat are the two GEMMs of `proj`."""
+
+    @staticmethod
+    def forward(ctx, gs_feature, pos_offset, x_grid, y_grid, eps):
+        _require_gpu(gs_feature)
+        if gs_feature.dim() != 3 or gs_feature.shape[-1] < 7:
+            raise ValueError(f"gs_feature must be [B,N,6+C]; got {tuple(gs_feature.shape)}")
+        B, N, F6 = gs_feature.shape
+        C = F6 - 6
+        dev = gs_feature.device
+        with torch.cuda.device(dev):
+            grid = _Grid(x_grid, y_grid, B)
+            op = _Splat(B, N, C, grid, eps, dev)
+            feat = _f32c(gs_feature)
+            off = None if pos_offset is None else _f32c(pos_offset)
+            if off is not None and off.shape != (B, N, 2):
+                raise ValueError(f"pos_offset must be [B,N,2]; got {tuple(off.shape)}")
+            packed = op._empty(op.plan.packed_bytes)
+            col = torch.empty(B, N, op.Cp, dtype=torch.float32, device=dev)
+            _lib.check(op.lib.igs_gs2d_pack_feature(_ptr(feat), _ptr(off), B, N, C, op.Cp, op.eps, _ptr(packed),
+                                                    _ptr(col), _stream(dev)), "igs_gs2d_pack_feature")
+            out, den = op.forward(packed)
+        ctx.op = op
+        ctx.save_for_backward(packed, col, feat, out, den)
+        ctx.in_dtype = gs_feature.dtype
+        ctx.grid_like = ((x_grid.shape, x_grid.dtype), (y_grid.shape, y_grid.dtype))
+        res = out if op.Cp == C else out[:, :C]
+        return res.to(gs_feature.dtype) if gs_feature.dtype != torch.float32 else res
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_result):
+        op: _Splat = ctx.op
+        packed, col, feat, out, den = ctx.saved_tensors
+        B, N, C, Cp, dev = op.B, op.N, op.C, op.Cp, op.device
+        need = ctx.needs_input_grad
+        g_x = g_y = g_feat = g_off = None
+        with torch.cuda.device(dev):
+            go = op.pad_grad_out(grad_result)
+            if need[2] or need[3]:
+                g_x, g_y = op.grid_grads(packed, out, den, go, *ctx.grid_like)
+                g_x, g_y = (g_x if need[2] else None), (g_y if need[3] else None)
+            if need[0] or need[1]:
+                partial = op.backward_partials(packed, col, out, den, go)
+                g_feat = torch.empty(B, N, 6 + C, dtype=torch.float32, device=dev)
+                _lib.check(op.lib.igs_gs2d_finalize_feature(_ptr(partial), op.grid.mode, _ptr(op.grid.flag), _ptr(feat),
+                                                            B, N, op.grid.H, op.grid.W, C, Cp, op.eps, _ptr(g_feat),
+                                                            _stream(dev)), "igs_gs2d_finalize_feature")
+                if need[1]:
+                    g_off = g_feat[..., :2].contiguous()
+                g_feat = g_feat.to(ctx.in_dtype) if need[0] else None
+        return g_feat, g_off, g_x, g_y, None
+
+
 def _cov_inverse_torch(scales, rotations, eps):
     """Matrix route of the reference preamble (src/igs/gs2d.py:548-580) for the debug path,
     in the dtype of its inputs."""
@@ -416,7 +491,11 @@ class GaussianSplatting2D(nn.Module):
         x_grid, y_grid [B,1,H,W] (also accepted: [B,H,W], batch 1, expanded/stride-0).
         Returns [B,C,H,W] (src/igs/gs2d.py:524-609)."""
         if fused:
-            return _RenderFused.apply(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps)
+            C = colors.shape[-1]
+            if C <= _lib.IGS_MAX_CHANNELS:
+                return _RenderFused.apply(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps)
+            return torch.cat([_RenderFused.apply(positions, colors[..., lo:hi], scales, rotations, alphas, x_grid,
+                                                 y_grid, eps) for lo, hi in _channel_groups(C)], dim=1)
         # heavy debug path, plain torch (src/igs/gs2d.py:598-609)
         if x_grid.dim() == 3:
             x_grid, y_grid = x_grid[:, None], y_grid[:, None]
@@ -427,8 +506,6 @@ class GaussianSplatting2D(nn.Module):
         """feature [B,F,D] -> (image [B,C,H,W], gs_feature [B,F*n,6+C]) (src/igs/gs2d.py:611-689)."""
         gs_feature = self.proj(feature).unflatten(-1, (-1, 6 + self.output_dim)).flatten(1, 2)
         b = gs_feature.shape[0]
-        positions, log_scales, rotations, logit_opacity, colors = gs_feature.split(
-            [2, 2, 1, 1, self.output_dim], dim=-1)
 
         if grid is None:
             x_grid, y_grid = self.xy_grid(size, feature.device)
@@ -439,6 +516,7 @@ class GaussianSplatting2D(nn.Module):
         else:
             grid = grid.flip(1)  # pos_map order is (h, w): y first
             x_grid, y_grid = grid.split([1, 1], dim=1)
+        pos_map = None
         if self.pos_map_offset:
             pos_map = torch.concat([x_grid, y_grid], dim=1)
             if scale is not None:
@@ -446,8 +524,17 @@ class GaussianSplatting2D(nn.Module):
             pos_map = pos_map.flatten(2, 3).transpose(1, 2)
             assert pos_map.size(1) == feature.size(1)
             pos_map = pos_map[..., None, :].repeat(1, 1, self.num_gaussians_per_emb, 1).flatten(1, 2)
-            positions = positions + pos_map
 
+        if fused and self.output_dim <= _lib.IGS_MAX_CHANNELS:
+            # split, exp(log_scale) + eps, alpha = 1 and their autograd run inside the HIP pack /
+            # finalize kernels
+            output = _RenderFromFeature.apply(gs_feature, pos_map, x_grid, y_grid, eps)
+            return output, gs_feature
+
+        positions, log_scales, rotations, logit_opacity, colors = gs_feature.split(
+            [2, 2, 1, 1, self.output_dim], dim=-1)
+        if pos_map is not None:
+            positions = positions + pos_map
         alphas = torch.ones_like(logit_opacity[..., 0])  # opacity logit is unused, as in the reference
         scales = torch.exp(log_scales) + eps
         rotations = rotations[..., 0]

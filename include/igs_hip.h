@@ -174,6 +174,21 @@ int igs_gs2d_finalize_scale_rot(const float *partial, int grid_mode, const int32
                                 float *g_scales, float *g_rotations, float *g_alphas,
                                 float *g_colors, igs_stream_t stream);
 
+/* Module head fused into pack / finalize (replaces the split + activations of the module's
+ * forward, src/igs/gs2d.py:635-644 and :673-675, and their autograd).
+ * gs_feature [B,N,6+C] rows: px, py, log_s0, log_s1, theta, opacity logit (unused), c_0..;
+ * scales = exp(log_s) + eps, alpha = 1.  pos_offset [B,N,2] is added to the positions when not
+ * NULL (pos_map_offset, src/igs/gs2d.py:654-667).  C_kernel is the compiled channel count
+ * (>= C) the other calls are made with; colors_out [B,N,C_kernel] receives the zero-padded raw
+ * colours for igs_gs2d_backward.  g_feature [B,N,6+C] gets d L / d gs_feature (0 for the
+ * opacity logit); d L / d pos_offset equals its first two columns. */
+int igs_gs2d_pack_feature(const float *gs_feature, const float *pos_offset, int B, int N, int C,
+                          int C_kernel, float eps, float *packed, float *colors_out,
+                          igs_stream_t stream);
+int igs_gs2d_finalize_feature(const float *partial, int grid_mode, const int32_t *grid_flag,
+                              const float *gs_feature, int B, int N, int H, int W, int C,
+                              int C_kernel, float eps, float *g_feature, igs_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -165,3 +165,38 @@ def test_config4_full_size_properties(igs, dev):
     rhs = 1e-6 * ((d["grad_out"].double() * out.double()).sum(1) / (den.double() + 1e-6)).sum((1, 2))
     scale = float((d["alphas"].double() * g1["alphas"].double()).abs().sum(1).max())
     assert float((lhs - rhs).abs().max()) < 2e-5 * scale
+
+
+def test_module_fused_head_equals_unfused_render(igs, dev):
+    """The module's fused head (pack/finalize from gs_feature) against the same module driving
+    `render` through torch ops, incl. pos_map_offset and a user grid."""
+    for pos_off in (False, True):
+        torch.manual_seed(5)
+        m = igs.GaussianSplatting2D(4, 48, output_dim=3, pos_map_offset=pos_off).to(dev)
+        h, w = (8, 12)
+        x = torch.randn(2, h * w, 48, device=dev)
+        ys, xs = torch.meshgrid(torch.linspace(-1, 1, h, device=dev), torch.linspace(-1.5, 1.5, w, device=dev),
+                                indexing="ij")
+        grid = torch.stack([ys, xs])[None].repeat(2, 1, 1, 1)          # [B,2,H,W], (y, x) order
+        go = torch.randn(2, 3, h, w, device=dev)
+        res = []
+        for fused_head in (True, False):
+            xi = x.clone().requires_grad_(True)
+            m.zero_grad()
+            if fused_head:
+                img, feat = m(xi, grid=grid)
+            else:
+                feat = m.proj(xi).unflatten(-1, (-1, 9)).flatten(1, 2)
+                pos, ls, rot, op_, col = feat.split([2, 2, 1, 1, 3], dim=-1)
+                gx, gy = grid.flip(1).split([1, 1], dim=1)
+                if pos_off:
+                    pm = torch.concat([gx, gy], 1).flatten(2, 3).transpose(1, 2)
+                    pos = pos + pm[..., None, :].repeat(1, 1, 4, 1).flatten(1, 2)
+                img = igs.gaussian_splatting_2d(pos, col, torch.exp(ls) + 1e-6, rot[..., 0],
+                                                torch.ones_like(op_[..., 0]), gx, gy)
+            img.backward(go)
+            res.append((img.detach(), xi.grad.clone(), m.proj.weight.grad.clone(), m.proj.bias.grad.clone()))
+        (i1, x1, w1, b1), (i2, x2, w2, b2) = res
+        assert torch.allclose(i1, i2, rtol=1e-5, atol=1e-6)
+        for u, v in ((x1, x2), (w1, w2), (b1, b2)):
+            assert rel(u, v) < 1e-4

@@ -157,6 +157,26 @@ def test_grid_gradients(igs, dev, C):
     assert_grad(ys.grad, rg["y"].sum((0, 3), keepdim=True), "y shared", "grid grads")
 
 
+def test_more_than_16_channels_in_groups(igs, dev):
+    B, N, H, W, C = 1, 60, 10, 22, 21
+    d = small_case(B, N, H, W, C, seed=91)
+    ref_out, ref_g = O.render_autograd(d["positions"], d["colors"], d["scales"], d["rotations"], d["alphas"],
+                                       d["x_grid"], d["y_grid"], d["grad_out"])
+    g = to_dev(d, dev)
+    names = ("positions", "colors", "scales", "rotations", "alphas")
+    lv = {k: g[k].clone().requires_grad_(True) for k in names}
+    out = igs.gaussian_splatting_2d(*[lv[k] for k in names], g["x_grid"], g["y_grid"])
+    assert out.shape == (B, C, H, W)
+    assert_fwd(out.detach(), ref_out, "C=21 fwd")
+    out.backward(g["grad_out"])
+    for k in names:
+        assert_grad(lv[k].grad, ref_g[k], k, "C=21 bwd")
+    a, b, c_ = (t.float().to(dev) for t in O.cov_inverse_closed(d["scales"], d["rotations"]))
+    o2 = igs.GaussianSplatting2DKernel.apply(g["x_grid"], g["y_grid"], g["positions"], a, b, c_, g["alphas"],
+                                             g["colors"], 1e-6)
+    assert_fwd(o2, ref_out, "C=21 operator fwd")
+
+
 def test_fused_false_debug_path_matches(igs, dev):
     d = to_dev(small_case(1, 40, 12, 14, 3, seed=9), dev)
     a = igs.gaussian_splatting_2d(d["positions"], d["colors"], d["scales"], d["rotations"], d["alphas"],
