@@ -825,7 +825,38 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     bwd_store<C, G>(a, b, t, n, M, CG);
 }
 
-// Finalize: one thread per Gaussian; sums the T tile partials in order and applies
+// Fixed-order sum over the T tile partials of NV consecutive fields for one Gaussian, spread
+// over the 16 "t-lanes" of a workgroup laid out as 16 t-lanes x 16 Gaussians: t-lane k adds
+// tiles k, k+16, ... in order, the 16 lane sums are then added in order by every thread (so all
+// 16 t-lanes of a Gaussian hold the same, run-to-run identical value).  `red` is
+// [NV][16][17] floats of LDS.  Must be called by all 256 threads.
+constexpr int kFinT = 16, kFinN = 16;
+
+template <int NV>
+__device__ __forceinline__ void tile_sum(const float* __restrict__ base, int T, int NF, int N,
+                                         int f0, bool valid, float (&out)[NV], float* red) {
+    const int tl = threadIdx.x / kFinN, nl = threadIdx.x % kFinN;
+    float acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
+    if (valid)
+        for (int t = tl; t < T; t += kFinT)
+#pragma unroll
+            for (int v = 0; v < NV; ++v) acc[v] += base[((size_t)t * NF + f0 + v) * N];
+    __syncthreads();  // protects `red` against the previous call's readers
+#pragma unroll
+    for (int v = 0; v < NV; ++v) red[(v * kFinT + tl) * (kFinN + 1) + nl] = acc[v];
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kFinT; ++k) s += red[(v * kFinT + k) * (kFinN + 1) + nl];
+        out[v] = s;
+    }
+}
+
+// Finalize: 16 threads per Gaussian; sums the T tile partials in a fixed order and applies
 //   d alpha = M0, d color_c = alpha CG_c, d px = alpha (A Mx + B My), d py = alpha (B Mx + D My),
 //   dA = -1/2 alpha Mxx, dB = -alpha Mxy, dD = -1/2 alpha Myy,
 // and (function level) the chain rule through A = c^2 i0 + s^2 i1, B = c s (i0 - i1),
@@ -838,21 +869,18 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
     float* __restrict__ g_col) {
-    const int n = blockIdx.x * kThreads + threadIdx.x;
+    __shared__ float red[6 * kFinT * (kFinN + 1)];
+    const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
     const int b = blockIdx.y;
-    if (n >= N) return;
+    const bool valid = n < N;
+    const bool writer = valid && threadIdx.x < kFinN;  // t-lane 0 writes the results
     // AUTO grid mode: T_in belongs to the separable plan, T_alt to the general one
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + C;
-    const size_t i = (size_t)b * N + n;
-    const float* base = partial + (size_t)b * T * NF * N + n;
+    const size_t i = (size_t)b * N + min(n, N - 1);
+    const float* base = partial + (size_t)b * T * NF * N + min(n, N - 1);
     float M[6];
-#pragma unroll
-    for (int f = 0; f < 6; ++f) {
-        float s = 0.0f;
-        for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + f) * N];
-        M[f] = s;
-    }
+    tile_sum<6>(base, T, NF, N, 0, valid, M, red);
     const double al = alphas[i];
     // O(BN) epilogue in fp64: the chain rule multiplies sums by 1/s^3-sized factors
     double A, Bc, D, cs = 0., sn = 0., i0 = 0., i1 = 0., s0 = 0., s1 = 0.;
@@ -870,30 +898,30 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
         Bc = p1[i];
         D = p2[i];
     }
-    if (g_alpha) g_alpha[i] = M[0];
-    if (g_pos) {
+    if (g_alpha && writer) g_alpha[i] = M[0];
+    if (g_pos && writer) {
         g_pos[2 * i] = (float)(al * (A * M[1] + Bc * M[2]));
         g_pos[2 * i + 1] = (float)(al * (Bc * M[1] + D * M[2]));
     }
     const double gA = -0.5 * al * M[3], gB = -al * M[4], gD = -0.5 * al * M[5];
     if (kScaleRot) {
-        if (g0) {  // scales [B,N,2]
+        if (g0 && writer) {  // scales [B,N,2]
             const double gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
             const double gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
             g0[2 * i] = (float)(gi0 * (-2.0 * s0 * i0 * i0));
             g0[2 * i + 1] = (float)(gi1 * (-2.0 * s1 * i1 * i1));
         }
-        if (g1) g1[i] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
+        if (g1 && writer) g1[i] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
     } else {
-        if (g0) g0[i] = (float)gA;
-        if (g1) g1[i] = (float)gB;
-        if (g2) g2[i] = (float)gD;
+        if (g0 && writer) g0[i] = (float)gA;
+        if (g1 && writer) g1[i] = (float)gB;
+        if (g2 && writer) g2[i] = (float)gD;
     }
-    if (g_col) {
+    if (g_col) {  // kernel-argument uniform, so the barriers inside tile_sum are safe
         for (int c = 0; c < C; ++c) {
-            float s = 0.0f;
-            for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + 6 + c) * N];
-            g_col[i * C + c] = (float)al * s;
+            float s1[1];
+            tile_sum<1>(base, T, NF, N, 6 + c, valid, s1, red);
+            if (writer) g_col[i * C + c] = (float)al * s1[0];
         }
     }
 }
@@ -903,20 +931,17 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
     const float* __restrict__ feat, int N, int C, int Cp, float eps, float* __restrict__ g_feat) {
-    const int n = blockIdx.x * kThreads + threadIdx.x;
+    __shared__ float red[6 * kFinT * (kFinN + 1)];
+    const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
     const int b = blockIdx.y;
-    if (n >= N) return;
+    const bool valid = n < N;
+    const bool writer = valid && threadIdx.x < kFinN;
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + Cp;
-    const size_t i = (size_t)b * N + n;
-    const float* base = partial + (size_t)b * T * NF * N + n;
+    const size_t i = (size_t)b * N + min(n, N - 1);
+    const float* base = partial + (size_t)b * T * NF * N + min(n, N - 1);
     float M[6];
-#pragma unroll
-    for (int f = 0; f < 6; ++f) {
-        float s = 0.0f;
-        for (int t = 0; t < T; ++t) s += base[((size_t)t * NF + f) * N];
-        M[f] = s;
-    }
+    tile_sum<6>(base, T, NF, N, 0, valid, M, red);
     const float* f = feat + i * (6 + C);
     const double e0 = (double)expf(f[2]), e1 = (double)expf(f[3]);
     const double s0 = e0 + (double)eps, s1 = e1 + (double)eps;
@@ -930,16 +955,18 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const double gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
     const double gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
     float* g = g_feat + i * (6 + C);
-    g[0] = (float)(A * M[1] + Bc * M[2]);
-    g[1] = (float)(Bc * M[1] + D * M[2]);
-    g[2] = (float)(gi0 * (-2.0 * s0 * i0 * i0) * e0);
-    g[3] = (float)(gi1 * (-2.0 * s1 * i1 * i1) * e1);
-    g[4] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
-    g[5] = 0.0f;
+    if (writer) {
+        g[0] = (float)(A * M[1] + Bc * M[2]);
+        g[1] = (float)(Bc * M[1] + D * M[2]);
+        g[2] = (float)(gi0 * (-2.0 * s0 * i0 * i0) * e0);
+        g[3] = (float)(gi1 * (-2.0 * s1 * i1 * i1) * e1);
+        g[4] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
+        g[5] = 0.0f;
+    }
     for (int c = 0; c < C; ++c) {
-        float sum = 0.0f;
-        for (int t = 0; t < T; ++t) sum += base[((size_t)t * NF + 6 + c) * N];
-        g[6 + c] = sum;
+        float s1v[1];
+        tile_sum<1>(base, T, NF, N, 6 + c, valid, s1v, red);
+        if (writer) g[6 + c] = s1v[0];
     }
 }
 
@@ -1488,7 +1515,7 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     int T, T_alt;
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
     if (rc) return rc;
-    hipLaunchKernelGGL((k_bwd_finalize<false>), dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
+    hipLaunchKernelGGL((k_bwd_finalize<false>), dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, cov_inv_00, cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
                        g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
@@ -1506,7 +1533,7 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     int T, T_alt;
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
     if (rc) return rc;
-    hipLaunchKernelGGL((k_bwd_finalize<true>), dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
+    hipLaunchKernelGGL((k_bwd_finalize<true>), dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, scales, rotations, (const float*)nullptr, alphas, N, C, eps, g_positions,
                        g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
@@ -1536,7 +1563,7 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
     int T, T_alt;
     rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt);
     if (rc) return rc;
-    hipLaunchKernelGGL(k_bwd_finalize_feature, dim3(ceil_div(N, kThreads), B), dim3(kThreads), 0,
+    hipLaunchKernelGGL(k_bwd_finalize_feature, dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, gs_feature, N, C, C_kernel, eps, g_feature);
     return launch_status();
