@@ -240,6 +240,10 @@ __device__ __forceinline__ float in_vgpr(float v) {
 #ifndef IGS_PCHUNK
 #define IGS_PCHUNK 256
 #endif
+#ifndef IGS_STREAM_UNROLL
+#define IGS_STREAM_UNROLL 2
+#endif
+constexpr int kStreamUnroll = IGS_STREAM_UNROLL;  // records whose LDS reads are in flight together
 constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
 
 // Streams `count` records of R4 float4 each from global memory to every wave of the
@@ -278,21 +282,23 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
             }
         }
         const float4* cur = sh + (k & 1) * E;
-        // register double-buffering of the LDS reads: record n+1 is read while n is consumed
-        float4 ra[R4], rb[R4];
-#pragma unroll
-        for (int i = 0; i < R4; ++i) ra[i] = cur[i];
+        // The LDS reads of kStreamUnroll records are issued together and pinned above the work
+        // (the compiler would otherwise sink each read next to its first use and wait for it
+        // there); each record's body then only waits for its own reads, so one LDS latency is
+        // exposed per group instead of per record.
 #pragma unroll 1
-        for (int n = 0; n < CH; n += 2) {
+        for (int n = 0; n < CH; n += kStreamUnroll) {
+            float4 rr[kStreamUnroll][R4];
 #pragma unroll
-            for (int i = 0; i < R4; ++i) rb[i] = cur[(n + 1) * R4 + i];
-            __builtin_amdgcn_sched_barrier(0);  // keep the reads above the work that hides them
-            body(ra);
-            const int nn = (n + 2 < CH) ? n + 2 : 0;  // last: harmless re-read
+            for (int u = 0; u < kStreamUnroll; ++u)
 #pragma unroll
-            for (int i = 0; i < R4; ++i) ra[i] = cur[nn * R4 + i];
+                for (int i = 0; i < R4; ++i) rr[u][i] = cur[(n + u) * R4 + i];
             __builtin_amdgcn_sched_barrier(0);
-            body(rb);
+#pragma unroll
+            for (int u = 0; u < kStreamUnroll; ++u) {
+                body(rr[u]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         if (k + 1 < chunks) {
             float4* nxt = sh + ((k + 1) & 1) * E;
