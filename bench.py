@@ -40,6 +40,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the JSON line, print the operator-level table of the reference's "
+                         "scripts/profiling.py (B x N x H sweep, median of 32 timed calls after 4 warm-ups)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
@@ -48,6 +51,9 @@ def main() -> int:
         print("bench.py: this build measures one GPU only (the path shards over the batch with no "
               "exchange; no multi-GPU run is part of it). Use --gpus 1.", file=sys.stderr)
         return 2
+
+    if args.sweep:
+        return sweep()
 
     import torch
 
@@ -196,6 +202,54 @@ def main() -> int:
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args.config, O)
     print(json.dumps(result), flush=True)
+    return 0
+
+
+def sweep() -> int:
+    """Operator-level sweep in the protocol of the reference's scripts/profiling.py:30-49, :69-151, :199-211:
+    `.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors)` on randn/rand inputs (per-pixel
+    random coordinates, so the general-grid kernels run), 4 warm-ups, 32 timed calls with events, median;
+    forward+backward uses `output.mean().backward()`.  Columns as in the reference's table."""
+    import itertools
+
+    import torch
+
+    from igs_amd import GaussianSplatting2DKernel
+
+    dev = torch.device("cuda:0")
+    rows = []
+    for B, N, H in itertools.product([4, 8], [4096, 8192, 16384], [128, 256]):
+        W = H
+        for mode in ("fwd", "fwd_bwd"):
+            rg = mode == "fwd_bwd"
+            mk = lambda *sh, fn=torch.randn: fn(*sh, device=dev).requires_grad_(rg)
+            inputs = (mk(B, 1, H, W), mk(B, 1, H, W), mk(B, N, 2), mk(B, N, 1, 1), mk(B, N, 1, 1), mk(B, N, 1, 1),
+                      mk(B, N, fn=torch.rand), mk(B, N, 3, fn=torch.rand))
+
+            def call():
+                out = GaussianSplatting2DKernel.apply(*inputs)
+                if rg:
+                    out.mean().backward()
+                    for t in inputs:
+                        t.grad = None
+
+            for _ in range(4):
+                call()
+            torch.cuda.synchronize()
+            ts = []
+            for _ in range(32):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                call()
+                e1.record()
+                torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1))
+            ms = sorted(ts)[len(ts) // 2]
+            rows.append(("HipGaussianSplatting2D", B, N, H, "Forward" if mode == "fwd" else "Fwd+Bwd", ms,
+                         B * N * H * W / (ms * 1e-3) / 1e9, B * N / (ms * 1e-3) / 1e6))
+    print("%-24s %3s %6s %4s %-8s %10s %12s %14s" % ("Kernel", "B", "N", "H", "Pass", "ms", "G-pixels/s", "M-Gaussians/s"))
+    for r in rows:
+        print("%-24s %3d %6d %4d %-8s %10.4f %12.2f %14.2f" % r)
     return 0
 
 

@@ -53,7 +53,10 @@ constexpr int kThreads = 256;
 #endif
 // rows per lane in the separable forward: as many as the accumulator VGPRs (P x (C+1)) allow
 __host__ __device__ constexpr int fwd_sep_p(int C) { return C <= 3 ? IGS_FWD_SEP_P : (C <= 8 ? 8 : 4); }
-constexpr int kFwdGenP = 4;  // pixels per lane, general forward
+// pixels per lane, general forward
+__host__ __device__ constexpr int fwd_gen_p(int C) { return C <= 4 ? 8 : 4; }
+// Gaussians per lane, general backward (more independent chains per pixel record)
+__host__ __device__ constexpr int bwd_gen_g(int C) { return C <= 4 ? 4 : 2; }
 constexpr int kBwdG = IGS_BWD_G;  // Gaussians per lane, backward
 
 __host__ __device__ constexpr int rec_stride_of(int C) { return (6 + C + 3) & ~3; }
@@ -430,6 +433,7 @@ __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
     const float4* src = reinterpret_cast<const float4*>(a.packed + ((size_t)b * a.Np + n0) * RS);
     stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r) {
         const GRec<C> g = lds_grec<C>(r);
+        float e[P];
 #pragma unroll
         for (int j = 0; j < P; ++j) {
             const float dx = xv[j] - g.px;
@@ -438,11 +442,15 @@ __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
             t = fmaf(g.B2, dy, t);
             const float v = g.D * dy;
             float q = t * dx;
-            q = fmaf(v, dy, q);
-            const float e = hw_exp2(q);
-            dsum[j] = fmaf(e, g.al, dsum[j]);
+            e[j] = fmaf(v, dy, q);
+        }
 #pragma unroll
-            for (int c = 0; c < C; ++c) num[j][c] = fmaf(e, g.ac[c], num[j][c]);
+        for (int j = 0; j < P; ++j) e[j] = hw_exp2(e[j]);
+#pragma unroll
+        for (int j = 0; j < P; ++j) {
+            dsum[j] = fmaf(e[j], g.al, dsum[j]);
+#pragma unroll
+            for (int c = 0; c < C; ++c) num[j][c] = fmaf(e[j], g.ac[c], num[j][c]);
         }
     });
 #pragma unroll
@@ -781,6 +789,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
             pv[4 * q4 + 2] = tq.z;
             pv[4 * q4 + 3] = tq.w;
         }
+        float dxs[G], dys[G], ee[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             const float dx = pv[0] - px[g];
@@ -789,8 +798,15 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
             tt = fmaf(B2[g], dy, tt);
             const float v = D[g] * dy;
             float q = tt * dx;
-            q = fmaf(v, dy, q);
-            const float e = hw_exp2(q);
+            ee[g] = fmaf(v, dy, q);
+            dxs[g] = dx;
+            dys[g] = dy;
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) ee[g] = hw_exp2(ee[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float e = ee[g], dx = dxs[g], dy = dys[g];
             float Gv = pv[2 + C];  // -s
 #pragma unroll
             for (int c = 0; c < C; ++c) Gv = fmaf(pv[2 + c], col[g][c], Gv);
@@ -1028,20 +1044,26 @@ __global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
     stream_records_lds<R4, kGaussChunk>(src, a.Np, sh, [&](const float4* r) {
         const GRec<C> g = lds_grec<C>(r);
         const float hb = 0.5f * g.B2;
+        // phases: exponents, transcendentals back to back, accumulation
+        float t1[P], t2[P], e[P];
 #pragma unroll
         for (int j = 0; j < P; ++j) {
             const float dx = xv[j] - g.px;
             const float dy = yv[j] - g.py;
-            const float t1 = fmaf(g.A, dx, hb * dy);
-            const float t2 = fmaf(g.D, dy, hb * dx);
-            const float q = fmaf(dx, t1, dy * t2);
-            const float e = hw_exp2(q);
+            t1[j] = fmaf(g.A, dx, hb * dy);
+            t2[j] = fmaf(g.D, dy, hb * dx);
+            e[j] = fmaf(dx, t1[j], dy * t2[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < P; ++j) e[j] = hw_exp2(e[j]);
+#pragma unroll
+        for (int j = 0; j < P; ++j) {
             float Gv = negs[j] * g.al;  // alpha (<g^, c> - s)
 #pragma unroll
             for (int c = 0; c < C; ++c) Gv = fmaf(gh[j][c], g.ac[c], Gv);
-            const float Gw = Gv * e;
-            sx[j] = fmaf(Gw, t1, sx[j]);
-            sy[j] = fmaf(Gw, t2, sy[j]);
+            const float Gw = Gv * e[j];
+            sx[j] = fmaf(Gw, t1[j], sx[j]);
+            sy[j] = fmaf(Gw, t2[j], sy[j]);
         }
     });
     constexpr float kScale = -1.0f / kNegHalfLog2e;  // A dx + B dy = t1 / k, and the leading minus
@@ -1121,7 +1143,7 @@ FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
         g.tiles_y = ceil_div(H, kFwdSepP * (4 / g.wx));
     } else {
         g.wx = 4;
-        g.tiles_x = ceil_div((long)H * W, kThreads * kFwdGenP);
+        g.tiles_x = ceil_div((long)H * W, kThreads * fwd_gen_p(C));
         g.tiles_y = 1;
     }
     g.total_tiles = B * g.tiles_x * g.tiles_y;
@@ -1154,7 +1176,7 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     S = ceil_div(p->n_padded, nps);
     p->fwd_split = (int)S;
     p->fwd_n_per_split = nps;
-    const long groups = (long)B * ceil_div(N, kThreads * kBwdG) * 4;  // waves per tile
+    const long groups = (long)B * ceil_div(N, kThreads * (sep ? kBwdG : bwd_gen_g(C))) * 4;  // waves per tile
     long T = ((long)cus * 4 * IGS_BWD_WAVES + groups - 1) / groups;     // backward: waves per SIMD wanted
     const long maxT = sep ? H : ceil_div(p->hw_padded, 256);
     if (T > maxT) T = maxT;
@@ -1234,7 +1256,7 @@ int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
     if (sep)
         hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C)>), grid, dim3(kThreads), 0, st, a);
     else
-        hipLaunchKernelGGL((k_fwd_gen<C, kFwdGenP>), grid, dim3(kThreads), 0, st, a);
+        hipLaunchKernelGGL((k_fwd_gen<C, fwd_gen_p(C)>), grid, dim3(kThreads), 0, st, a);
     return launch_status();
 }
 
@@ -1257,11 +1279,13 @@ int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, con
 
 template <int C>
 int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
-    const dim3 grid(ceil_div(a.N, kThreads * kBwdG), a.T, B);
-    if (sep)
+    if (sep) {
+        const dim3 grid(ceil_div(a.N, kThreads * kBwdG), a.T, B);
         hipLaunchKernelGGL((k_bwd_sep<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
-    else
-        hipLaunchKernelGGL((k_bwd_gen<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
+    } else {
+        const dim3 grid(ceil_div(a.N, kThreads * bwd_gen_g(C)), a.T, B);
+        hipLaunchKernelGGL((k_bwd_gen<C, bwd_gen_g(C)>), grid, dim3(kThreads), 0, st, a);
+    }
     return launch_status();
 }
 
@@ -1485,7 +1509,7 @@ int igs_gs2d_backward_grid(const float* packed, const float* x, const float* y,
     int rc = IGS_OK;
     hipStream_t st = (hipStream_t)stream;
     IGS_DISPATCH_C(C, {
-        constexpr int P = kC > 4 ? 1 : 2;
+        constexpr int P = kC > 8 ? 2 : 4;
         a.tiles_per_img = ceil_div((long)H * W, kThreads * P);
         a.total_tiles = B * a.tiles_per_img;
         hipLaunchKernelGGL((k_bwd_grid<kC, P>), dim3(((a.total_tiles + 7) / 8) * 8), dim3(kThreads), 0, st, a);
