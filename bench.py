@@ -59,7 +59,7 @@ def main() -> int:
 
     import igs_amd
     from igs_amd import _lib
-    from igs_amd.gs2d import _Grid, _Splat, _ptr, _stream
+    from igs_amd._splat import Grid as _Grid, Splat as _Splat, _ptr, _stream
     from oracle import gs2d_oracle as O
 
     if not torch.cuda.is_available():
@@ -193,7 +193,7 @@ def main() -> int:
                                "achieved": pairs * f_fwd / t_fwd_kernel / 1e12,
                                "frac": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS},
             "traffic_note": "HBM bytes per launch from rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (copy-calibrated), "
-                            "see profiles/; valid for the c1 workload only",
+                            "from the committed rocprofv3 counter summary; valid for the c1 workload only",
             "note": "peak = published fp32 vector peak; the kernels use plain (non-packed) fp32 VALU ops with "
                     "VGPR-only operands, v_exp_f32 counted as 1 FLOP",
         },

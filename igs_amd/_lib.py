@@ -6,6 +6,7 @@ import of the product path raises.  Build it with ``python -m igs_amd.build``.
 from __future__ import annotations
 
 import ctypes
+import functools
 import os
 from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
@@ -107,7 +108,10 @@ def check(status: int, what: str) -> None:
         raise RuntimeError(f"{what} failed: {msg} (status {status})")
 
 
+@functools.lru_cache(maxsize=256)
 def plan(B: int, N: int, H: int, W: int, C: int, grid_mode: int) -> Plan:
+    """Launch plan / buffer sizes of a problem (pure host arithmetic in the library; cached, since
+    training loops ask for the same shape every step).  Treat the result as read-only."""
     p = Plan()
     check(load().igs_gs2d_plan(B, N, H, W, C, grid_mode, ctypes.byref(p)), "igs_gs2d_plan")
     return p

@@ -12,15 +12,13 @@ it raises.
 """
 from __future__ import annotations
 
-import ctypes
-from typing import Optional, Tuple
-
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 from torch.autograd.function import once_differentiable
 
-from . import _lib
+from . import _lib, _ops
+from ._splat import KIND_COVINV, KIND_FEATURE, KIND_SCALE_ROT, channel_groups, run_backward, run_forward
 
 Tensor = torch.Tensor
 
@@ -42,194 +40,58 @@ def naive_gaussian_2d(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas
 
 
 # --------------------------------------------------------------------------------------
-# helpers around the C ABI
-# --------------------------------------------------------------------------------------
-def _ptr(t: Optional[Tensor]):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
-
-
-def _stream(dev) -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-
-
-def _f32c(t: Tensor) -> Tensor:
-    return t.detach().to(torch.float32).contiguous()
-
-
-def _padded_channels(C: int) -> int:
-    for c in _lib.COMPILED_CHANNELS:
-        if c >= C:
-            return c
-    raise ValueError(f"C={C} exceeds the {_lib.IGS_MAX_CHANNELS} channels of one kernel pass")
-
-
-def _channel_groups(C: int):
-    """More than IGS_MAX_CHANNELS channels are rendered in groups of that many: each group's output
-    depends on its own colours only, and autograd adds the groups' gradients w.r.t. the shared
-    geometry (the backward moments are additive over channel groups: s = sum_groups <g^, out>_group)."""
-    m = _lib.IGS_MAX_CHANNELS
-    return [(i, min(i + m, C)) for i in range(0, C, m)]
-
-
-def _pad_last(t: Tensor, Cp: int) -> Tensor:
-    C = t.shape[-1]
-    return t if C == Cp else F.pad(t, (0, Cp - C))
-
-
-class _Grid:
-    """x/y coordinate tensors described by element strides (no copy for expanded grids)."""
-
-    def __init__(self, x: Tensor, y: Tensor, B: int):
-        if x.dim() == 3:
-            x = x[:, None]
-        if y.dim() == 3:
-            y = y[:, None]
-        if x.dim() != 4 or y.dim() != 4 or x.shape[1] != 1 or y.shape[1] != 1:
-            raise ValueError(f"x_grid/y_grid must be [B,1,H,W] (or [B,H,W]); got {tuple(x.shape)}, {tuple(y.shape)}")
-        if x.shape[-2:] != y.shape[-2:]:
-            raise ValueError("x_grid and y_grid must have the same H, W")
-        for g in (x, y):
-            if g.shape[0] not in (1, B):
-                raise ValueError(f"grid batch {g.shape[0]} does not match B={B}")
-        x = x.detach()
-        y = y.detach()
-        if x.dtype != torch.float32:
-            x = x.to(torch.float32)
-        if y.dtype != torch.float32:
-            y = y.to(torch.float32)
-        self.x, self.y = x, y
-        self.H, self.W = x.shape[-2:]
-
-        def st(g):
-            sb = 0 if (g.shape[0] == 1) else g.stride(0)
-            sh = 0 if self.H == 1 else g.stride(2)
-            sw = 0 if self.W == 1 else g.stride(3)
-            return (sb, sh, sw)
-
-        self.sx, self.sy = st(x), st(y)
-        if min(self.sx + self.sy) < 0:
-            self.x, self.y = x.contiguous(), y.contiguous()
-            self.sx, self.sy = st(self.x), st(self.y)
-        self.strides = _lib.strides6(self.sx, self.sy)
-        # x independent of the row and y independent of the column -> factored kernels.  Expanded
-        # (stride-0) grids prove it on the host; anything else is classified on the device into a
-        # flag that the kernels read, so there is no host synchronisation either way.
-        self.flag = None
-        if self.sx[1] == 0 and self.sy[2] == 0:
-            self.mode = _lib.IGS_GRID_SEPARABLE
-        else:
-            self.mode = _lib.IGS_GRID_AUTO
-            self.flag = torch.empty(1, dtype=torch.int32, device=x.device)
-            _lib.check(_lib.load().igs_gs2d_grid_classify(_ptr(self.x), _ptr(self.y), self.strides, B, self.H,
-                                                          self.W, _ptr(self.flag), _stream(x.device)),
-                       "igs_gs2d_grid_classify")
-
-
-class _Splat:
-    """One fused forward (+ backward) through the C ABI for a fixed problem."""
-
-    def __init__(self, B, N, C, grid: _Grid, eps: float, device):
-        self.lib = _lib.load()
-        self.B, self.N, self.C = B, N, C
-        self.Cp = _padded_channels(C)
-        self.grid, self.eps, self.device = grid, float(eps), device
-        self.plan = _lib.plan(B, N, grid.H, grid.W, self.Cp, grid.mode)
-
-    def _empty(self, nbytes: int) -> Tensor:
-        return torch.empty(max(int(nbytes) // 4, 1), dtype=torch.float32, device=self.device)
-
-    def pack_covinv(self, position, a, b, d, alphas, colors_p) -> Tensor:
-        packed = self._empty(self.plan.packed_bytes)
-        _lib.check(self.lib.igs_gs2d_pack_covinv(_ptr(position), _ptr(a), _ptr(b), _ptr(d), _ptr(alphas),
-                                                 _ptr(colors_p), self.B, self.N, self.Cp, _ptr(packed),
-                                                 _stream(self.device)), "igs_gs2d_pack_covinv")
-        return packed
-
-    def pack_scale_rot(self, positions, scales, rotations, alphas, colors_p) -> Tensor:
-        packed = self._empty(self.plan.packed_bytes)
-        _lib.check(self.lib.igs_gs2d_pack_scale_rot(_ptr(positions), _ptr(scales), _ptr(rotations), _ptr(alphas),
-                                                    _ptr(colors_p), self.B, self.N, self.Cp, self.eps,
-                                                    _ptr(packed), _stream(self.device)), "igs_gs2d_pack_scale_rot")
-        return packed
-
-    def forward(self, packed: Tensor) -> Tuple[Tensor, Tensor]:
-        g, p = self.grid, self.plan
-        out = torch.empty(self.B, self.Cp, g.H, g.W, dtype=torch.float32, device=self.device)
-        den = torch.empty(self.B, g.H, g.W, dtype=torch.float32, device=self.device)
-        ws = self._empty(p.fwd_ws_bytes) if p.fwd_ws_bytes else None
-        _lib.check(self.lib.igs_gs2d_forward(_ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag),
-                                             self.B, self.N,
-                                             g.H, g.W, self.Cp, self.eps, _ptr(out), _ptr(den), _ptr(ws),
-                                             int(p.fwd_ws_bytes), _stream(self.device)), "igs_gs2d_forward")
-        return out, den
-
-    def backward_partials(self, packed, colors_p, out, den, grad_out_p) -> Tensor:
-        g, p = self.grid, self.plan
-        pix = self._empty(p.pix_bytes)
-        partial = self._empty(p.partial_bytes)
-        _lib.check(self.lib.igs_gs2d_backward(_ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, g.mode,
-                                              _ptr(g.flag), _ptr(out), _ptr(den), _ptr(grad_out_p), self.B, self.N, g.H, g.W,
-                                              self.Cp, self.eps, _ptr(pix), int(p.pix_bytes), _ptr(partial),
-                                              int(p.partial_bytes), _stream(self.device)), "igs_gs2d_backward")
-        return partial
-
-    def grid_grads(self, packed, out, den, grad_out_p, x_like, y_like):
-        """d L / d x_grid, d L / d y_grid in the (shape, dtype) of the tensors the caller passed."""
-        g = self.grid
-        gx = torch.empty(self.B, g.H, g.W, dtype=torch.float32, device=self.device)
-        gy = torch.empty_like(gx)
-        _lib.check(self.lib.igs_gs2d_backward_grid(_ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, _ptr(out),
-                                                   _ptr(den), _ptr(grad_out_p), self.B, self.N, g.H, g.W, self.Cp,
-                                                   self.eps, _ptr(gx), _ptr(gy), _stream(self.device)),
-                   "igs_gs2d_backward_grid")
-
-        def fit(gr, like):
-            shape, dtype = like
-            if shape[0] == 1 and self.B > 1:      # batch-1 grid shared by all images
-                gr = gr.sum(0, keepdim=True)
-            return gr.reshape(shape).to(dtype)
-
-        return fit(gx, x_like), fit(gy, y_like)
-
-    def pad_grad_out(self, grad_out: Tensor) -> Tensor:
-        go = _f32c(grad_out)
-        if self.Cp != self.C:
-            go = F.pad(go, (0, 0, 0, 0, 0, self.Cp - self.C)).contiguous()
-        return go
-
-
-def _check_gaussian_shapes(position, alphas, colors):
-    if position.dim() != 3 or position.shape[-1] != 2:
-        raise ValueError(f"positions must be [B,N,2]; got {tuple(position.shape)}")
-    B, N, _ = position.shape
-    if alphas.shape != (B, N):
-        raise ValueError(f"alphas must be [B,N]={B, N}; got {tuple(alphas.shape)}")
-    if colors.dim() != 3 or colors.shape[:2] != (B, N):
-        raise ValueError(f"colors must be [B,N,C]; got {tuple(colors.shape)}")
-    if N == 0:
-        raise ValueError("need at least one Gaussian")
-    return B, N, colors.shape[-1]
-
-
-def _require_gpu(t: Tensor):
-    if t.device.type != "cuda":
-        raise RuntimeError("the fused Gaussian-splatting path runs on the GPU only (HIP kernels); got a tensor on "
-                           f"{t.device}. Use fused=False for the plain-torch debug path.")
-    _lib.load()
-
-
-# --------------------------------------------------------------------------------------
 # operator level: the `.apply` plugin boundary of the reference
 # --------------------------------------------------------------------------------------
-class GaussianSplatting2DKernel(torch.autograd.Function):
+def _as(t: Tensor, dtype) -> Tensor:
+    return t if t.dtype == dtype else t.to(dtype)
+
+
+def _visible(op, out: Tensor, dtype) -> Tensor:
+    """The caller's view of the kernel's [B,Cp,H,W] fp32 output."""
+    return _as(out if op.Cp == op.C else out[:, :op.C], dtype)
+
+
+class _Operator(torch.autograd.Function):
+    """(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps) -> [B,C,H,W]
+    for C <= IGS_MAX_CHANNELS; backward returns the reference's 9-tuple (src/igs/gs2d.py:252-262)."""
+
+    @staticmethod
+    def forward(ctx, x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
+        params = (position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors)
+        op, keep, packed, col, out, den = run_forward(KIND_COVINV, params, x, y, eps)
+        ctx.op = op
+        ctx.grid_like = ((x.shape, x.dtype), (y.shape, y.dtype))
+        ctx.n_keep = len(keep)
+        ctx.save_for_backward(*keep, packed, col, out, den)
+        ctx.like = tuple((t.shape, t.dtype) for t in params)
+        return _visible(op, out, x.dtype)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_result):
+        saved = ctx.saved_tensors
+        keep, (packed, col, out, den) = saved[:ctx.n_keep], saved[ctx.n_keep:]
+        need = ctx.needs_input_grad
+        grads, g_x, g_y = run_backward(KIND_COVINV, ctx.op, keep, packed, col, out, den, grad_result, need[2:8],
+                                       need[0], need[1], ctx.grid_like)
+        grads = [None if g is None else _as(g, dt).reshape(sh) for g, (sh, dt) in zip(grads, ctx.like)]
+        return (g_x, g_y, *grads, None)
+
+
+class GaussianSplatting2DKernel:
     """HIP-backed drop-in for the reference operator (src/igs/gs2d.py:47-262 and its Triton
     variants): `.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors,
-    eps=1e-6) -> [B,C,H,W]`; backward returns the same 9-tuple (last entry None).
+    eps=1e-6) -> [B,C,H,W]`, differentiable w.r.t. all eight tensors.
 
     x, y: [B,1,H,W] (batch-1 and stride-0/expanded grids are taken as they are);
     position [B,N,2]; cov_inv_* [B,N,1,1] (any shape with B*N elements); alphas [B,N];
     colors [B,N,C].  The backward computes the exact derivative of the forward expression
     (the d/d(den) term is -<g^, out>).
+
+    A plain class with the `torch.autograd.Function` calling convention rather than a Function
+    itself: `.apply` routes eager callers to the autograd.Function above and callers under
+    `torch.compile` to the registered operators (Dynamo would otherwise trace into the ctypes
+    calls of a Function's forward).
     """
 
     # advisory tunables kept for callers that set them (scripts/profiling.py:89-95); the
@@ -237,74 +99,19 @@ class GaussianSplatting2DKernel(torch.autograd.Function):
     BLOCK_SIZE_H = BLOCK_SIZE_W = BWD_BLOCK_SIZE_H = BWD_BLOCK_SIZE_W = -1
     N_CHUNK_SIZE = 32
 
-    @classmethod
-    def apply(cls, x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
+    @staticmethod
+    def apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
         C = colors.shape[-1]
-        if C <= _lib.IGS_MAX_CHANNELS:
-            return super().apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps)
-        return torch.cat([super(GaussianSplatting2DKernel, cls).apply(
-            x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors[..., lo:hi], eps)
-            for lo, hi in _channel_groups(C)], dim=1)
-
-    @staticmethod
-    def forward(ctx, x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
-        _require_gpu(position)
-        B, N, C = _check_gaussian_shapes(position, alphas, colors)
-        for t in (cov_inv_00, cov_inv_01, cov_inv_11):
-            if t.numel() != B * N:
-                raise ValueError(f"cov_inv_* must hold B*N={B * N} elements; got {tuple(t.shape)}")
-        dev = position.device
-        with torch.cuda.device(dev):
-            grid = _Grid(x, y, B)
-            op = _Splat(B, N, C, grid, eps, dev)
-            pos, a, b, d, al = (_f32c(t) for t in (position, cov_inv_00, cov_inv_01, cov_inv_11, alphas))
-            col = _pad_last(_f32c(colors), op.Cp).contiguous()
-            packed = op.pack_covinv(pos, a, b, d, al, col)
-            out, den = op.forward(packed)
-        ctx.op = op
-        ctx.grid_like = ((x.shape, x.dtype), (y.shape, y.dtype))
-        ctx.save_for_backward(packed, col, a, b, d, al, out, den)
-        ctx.in_dtypes = tuple(t.dtype for t in (position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors))
-        ctx.cov_shapes = (cov_inv_00.shape, cov_inv_01.shape, cov_inv_11.shape)
-        res = out if op.Cp == C else out[:, :C]
-        return res.to(x.dtype) if x.dtype != torch.float32 else res
-
-    @staticmethod
-    @once_differentiable
-    def backward(ctx, grad_result):
-        op: _Splat = ctx.op
-        packed, col, a, b, d, al, out, den = ctx.saved_tensors
-        B, N, C, Cp, dev = op.B, op.N, op.C, op.Cp, op.device
-        need = ctx.needs_input_grad
-        g_x = g_y = None
-        with torch.cuda.device(dev):
-            go = op.pad_grad_out(grad_result)
-            if need[0] or need[1]:
-                g_x, g_y = op.grid_grads(packed, out, den, go, *ctx.grid_like)
-                g_x, g_y = (g_x if need[0] else None), (g_y if need[1] else None)
-            partial = op.backward_partials(packed, col, out, den, go)
-            new = lambda *s: torch.empty(*s, dtype=torch.float32, device=dev)
-            g_pos = new(B, N, 2) if need[2] else None
-            g_a = new(B, N) if need[3] else None
-            g_b = new(B, N) if need[4] else None
-            g_d = new(B, N) if need[5] else None
-            g_al = new(B, N) if need[6] else None
-            g_col = new(B, N, Cp) if need[7] else None
-            _lib.check(op.lib.igs_gs2d_finalize_covinv(_ptr(partial), op.grid.mode, _ptr(op.grid.flag), _ptr(a),
-                                                       _ptr(b), _ptr(d), _ptr(al), B, N, op.grid.H, op.grid.W,
-                                                       Cp, _ptr(g_pos), _ptr(g_a), _ptr(g_b),
-                                                       _ptr(g_d), _ptr(g_al), _ptr(g_col), _stream(dev)),
-                       "igs_gs2d_finalize_covinv")
-        if g_col is not None and Cp != C:
-            g_col = g_col[..., :C]
-        dt = ctx.in_dtypes
-        cast = lambda g, k: None if g is None else g.to(dt[k])
-        sh = ctx.cov_shapes
-        return (g_x, g_y, cast(g_pos, 0),
-                None if g_a is None else cast(g_a, 1).reshape(sh[0]),
-                None if g_b is None else cast(g_b, 2).reshape(sh[1]),
-                None if g_d is None else cast(g_d, 3).reshape(sh[2]),
-                cast(g_al, 4), cast(g_col, 5), None)
+        if C > _lib.IGS_MAX_CHANNELS:
+            return torch.cat([GaussianSplatting2DKernel.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11,
+                                                              alphas, colors[..., lo:hi], eps)
+                              for lo, hi in channel_groups(C)], dim=1)
+        if torch.compiler.is_compiling():
+            B, N = position.shape[:2]
+            params = [position, cov_inv_00.reshape(B, N), cov_inv_01.reshape(B, N), cov_inv_11.reshape(B, N),
+                      alphas, colors]
+            return _ops.splat(KIND_COVINV, params, x, y, eps, C, x.dtype)
+        return _Operator.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps)
 
 
 # The reference exposes its torch variants under these names (src/igs/gs2d.py:468-469) and
@@ -326,55 +133,25 @@ class _RenderFused(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, positions, colors, scales, rotations, alphas, x_grid, y_grid, eps):
-        _require_gpu(positions)
-        B, N, C = _check_gaussian_shapes(positions, alphas, colors)
-        if scales.shape != (B, N, 2) or rotations.shape != (B, N):
-            raise ValueError(f"scales must be [B,N,2] and rotations [B,N]; got {tuple(scales.shape)}, {tuple(rotations.shape)}")
-        dev = positions.device
-        with torch.cuda.device(dev):
-            grid = _Grid(x_grid, y_grid, B)
-            op = _Splat(B, N, C, grid, eps, dev)
-            pos, sc, rot, al = (_f32c(t) for t in (positions, scales, rotations, alphas))
-            col = _pad_last(_f32c(colors), op.Cp).contiguous()
-            packed = op.pack_scale_rot(pos, sc, rot, al, col)
-            out, den = op.forward(packed)
+        params = (positions, colors, scales, rotations, alphas)
+        op, keep, packed, col, out, den = run_forward(KIND_SCALE_ROT, params, x_grid, y_grid, eps)
         ctx.op = op
         ctx.grid_like = ((x_grid.shape, x_grid.dtype), (y_grid.shape, y_grid.dtype))
-        ctx.save_for_backward(packed, col, sc, rot, al, out, den)
-        ctx.in_dtypes = tuple(t.dtype for t in (positions, colors, scales, rotations, alphas))
-        res = out if op.Cp == C else out[:, :C]
-        return res.to(positions.dtype) if positions.dtype != torch.float32 else res
+        ctx.n_keep = len(keep)
+        ctx.save_for_backward(*keep, packed, col, out, den)
+        ctx.in_dtypes = tuple(t.dtype for t in params)
+        return _visible(op, out, positions.dtype)
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_result):
-        op: _Splat = ctx.op
-        packed, col, sc, rot, al, out, den = ctx.saved_tensors
-        B, N, C, Cp, dev = op.B, op.N, op.C, op.Cp, op.device
+        saved = ctx.saved_tensors
+        keep, (packed, col, out, den) = saved[:ctx.n_keep], saved[ctx.n_keep:]
         need = ctx.needs_input_grad
-        g_x = g_y = None
-        with torch.cuda.device(dev):
-            go = op.pad_grad_out(grad_result)
-            if need[5] or need[6]:
-                g_x, g_y = op.grid_grads(packed, out, den, go, *ctx.grid_like)
-                g_x, g_y = (g_x if need[5] else None), (g_y if need[6] else None)
-            partial = op.backward_partials(packed, col, out, den, go)
-            new = lambda *s: torch.empty(*s, dtype=torch.float32, device=dev)
-            g_pos = new(B, N, 2) if need[0] else None
-            g_col = new(B, N, Cp) if need[1] else None
-            g_sc = new(B, N, 2) if need[2] else None
-            g_rot = new(B, N) if need[3] else None
-            g_al = new(B, N) if need[4] else None
-            _lib.check(op.lib.igs_gs2d_finalize_scale_rot(_ptr(partial), op.grid.mode, _ptr(op.grid.flag), _ptr(sc),
-                                                          _ptr(rot), _ptr(al), B, N, op.grid.H, op.grid.W, Cp,
-                                                          op.eps, _ptr(g_pos), _ptr(g_sc),
-                                                          _ptr(g_rot), _ptr(g_al), _ptr(g_col), _stream(dev)),
-                       "igs_gs2d_finalize_scale_rot")
-        if g_col is not None and Cp != C:
-            g_col = g_col[..., :C]
-        dt = ctx.in_dtypes
-        cast = lambda g, k: None if g is None else g.to(dt[k])
-        return cast(g_pos, 0), cast(g_col, 1), cast(g_sc, 2), cast(g_rot, 3), cast(g_al, 4), g_x, g_y, None
+        grads, g_x, g_y = run_backward(KIND_SCALE_ROT, ctx.op, keep, packed, col, out, den, grad_result, need[0:5],
+                                       need[5], need[6], ctx.grid_like)
+        grads = [None if g is None else _as(g, dt) for g, dt in zip(grads, ctx.in_dtypes)]
+        return (*grads, g_x, g_y, None)
 
 
 class _RenderFromFeature(torch.autograd.Function):
@@ -386,54 +163,42 @@ class _RenderFromFeature(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, gs_feature, pos_offset, x_grid, y_grid, eps):
-        _require_gpu(gs_feature)
-        if gs_feature.dim() != 3 or gs_feature.shape[-1] < 7:
-            raise ValueError(f"gs_feature must be [B,N,6+C]; got {tuple(gs_feature.shape)}")
-        B, N, F6 = gs_feature.shape
-        C = F6 - 6
-        dev = gs_feature.device
-        with torch.cuda.device(dev):
-            grid = _Grid(x_grid, y_grid, B)
-            op = _Splat(B, N, C, grid, eps, dev)
-            feat = _f32c(gs_feature)
-            off = None if pos_offset is None else _f32c(pos_offset)
-            if off is not None and off.shape != (B, N, 2):
-                raise ValueError(f"pos_offset must be [B,N,2]; got {tuple(off.shape)}")
-            packed = op._empty(op.plan.packed_bytes)
-            col = torch.empty(B, N, op.Cp, dtype=torch.float32, device=dev)
-            _lib.check(op.lib.igs_gs2d_pack_feature(_ptr(feat), _ptr(off), B, N, C, op.Cp, op.eps, _ptr(packed),
-                                                    _ptr(col), _stream(dev)), "igs_gs2d_pack_feature")
-            out, den = op.forward(packed)
+        params = (gs_feature,) if pos_offset is None else (gs_feature, pos_offset)
+        op, keep, packed, col, out, den = run_forward(KIND_FEATURE, params, x_grid, y_grid, eps)
         ctx.op = op
-        ctx.save_for_backward(packed, col, feat, out, den)
-        ctx.in_dtype = gs_feature.dtype
         ctx.grid_like = ((x_grid.shape, x_grid.dtype), (y_grid.shape, y_grid.dtype))
-        res = out if op.Cp == C else out[:, :C]
-        return res.to(gs_feature.dtype) if gs_feature.dtype != torch.float32 else res
+        ctx.n_keep = len(keep)
+        ctx.save_for_backward(*keep, packed, col, out, den)
+        ctx.in_dtypes = tuple(t.dtype for t in params)
+        return _visible(op, out, gs_feature.dtype)
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_result):
-        op: _Splat = ctx.op
-        packed, col, feat, out, den = ctx.saved_tensors
-        B, N, C, Cp, dev = op.B, op.N, op.C, op.Cp, op.device
+        saved = ctx.saved_tensors
+        keep, (packed, col, out, den) = saved[:ctx.n_keep], saved[ctx.n_keep:]
         need = ctx.needs_input_grad
-        g_x = g_y = g_feat = g_off = None
-        with torch.cuda.device(dev):
-            go = op.pad_grad_out(grad_result)
-            if need[2] or need[3]:
-                g_x, g_y = op.grid_grads(packed, out, den, go, *ctx.grid_like)
-                g_x, g_y = (g_x if need[2] else None), (g_y if need[3] else None)
-            if need[0] or need[1]:
-                partial = op.backward_partials(packed, col, out, den, go)
-                g_feat = torch.empty(B, N, 6 + C, dtype=torch.float32, device=dev)
-                _lib.check(op.lib.igs_gs2d_finalize_feature(_ptr(partial), op.grid.mode, _ptr(op.grid.flag), _ptr(feat),
-                                                            B, N, op.grid.H, op.grid.W, C, Cp, op.eps, _ptr(g_feat),
-                                                            _stream(dev)), "igs_gs2d_finalize_feature")
-                if need[1]:
-                    g_off = g_feat[..., :2].contiguous()
-                g_feat = g_feat.to(ctx.in_dtype) if need[0] else None
-        return g_feat, g_off, g_x, g_y, None
+        n = len(ctx.in_dtypes)
+        grads, g_x, g_y = run_backward(KIND_FEATURE, ctx.op, keep, packed, col, out, den, grad_result, need[0:n],
+                                       need[2], need[3], ctx.grid_like)
+        grads = [None if g is None else _as(g, dt) for g, dt in zip(grads, ctx.in_dtypes)]
+        if n == 1:
+            grads.append(None)
+        return (*grads, g_x, g_y, None)
+
+
+def _render_fused(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps):
+    if torch.compiler.is_compiling():
+        return _ops.splat(KIND_SCALE_ROT, [positions, colors, scales, rotations, alphas], x_grid, y_grid, eps,
+                          colors.shape[-1], positions.dtype)
+    return _RenderFused.apply(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps)
+
+
+def _render_from_feature(gs_feature, pos_offset, x_grid, y_grid, eps):
+    if torch.compiler.is_compiling():
+        params = [gs_feature] if pos_offset is None else [gs_feature, pos_offset]
+        return _ops.splat(KIND_FEATURE, params, x_grid, y_grid, eps, gs_feature.shape[-1] - 6, gs_feature.dtype)
+    return _RenderFromFeature.apply(gs_feature, pos_offset, x_grid, y_grid, eps)
 
 
 def _cov_inverse_torch(scales, rotations, eps):
@@ -493,9 +258,9 @@ class GaussianSplatting2D(nn.Module):
         if fused:
             C = colors.shape[-1]
             if C <= _lib.IGS_MAX_CHANNELS:
-                return _RenderFused.apply(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps)
-            return torch.cat([_RenderFused.apply(positions, colors[..., lo:hi], scales, rotations, alphas, x_grid,
-                                                 y_grid, eps) for lo, hi in _channel_groups(C)], dim=1)
+                return _render_fused(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps)
+            return torch.cat([_render_fused(positions, colors[..., lo:hi], scales, rotations, alphas, x_grid,
+                                            y_grid, eps) for lo, hi in channel_groups(C)], dim=1)
         # heavy debug path, plain torch (src/igs/gs2d.py:598-609)
         if x_grid.dim() == 3:
             x_grid, y_grid = x_grid[:, None], y_grid[:, None]
@@ -528,7 +293,7 @@ class GaussianSplatting2D(nn.Module):
         if fused and self.output_dim <= _lib.IGS_MAX_CHANNELS:
             # split, exp(log_scale) + eps, alpha = 1 and their autograd run inside the HIP pack /
             # finalize kernels
-            output = _RenderFromFeature.apply(gs_feature, pos_map, x_grid, y_grid, eps)
+            output = _render_from_feature(gs_feature, pos_map, x_grid, y_grid, eps)
             return output, gs_feature
 
         positions, log_scales, rotations, logit_opacity, colors = gs_feature.split(

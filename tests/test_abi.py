@@ -147,3 +147,30 @@ def test_host_api_surface_and_module_init():
     img, feat = m(x, size=(6, 10), fused=False)
     rimg, rfeat = O.module_forward(m.proj.weight.detach(), m.proj.bias.detach(), x, (6, 10), 4)
     assert torch.allclose(img, rimg, rtol=1e-5, atol=1e-6) and torch.equal(feat, rfeat)
+
+
+@pytest.mark.parametrize("B,N,H,W,C", [(2, 37, 8, 12, 3), (1, 1, 1, 1, 1), (3, 130, 5, 70, 5), (1, 64, 9, 9, 16)])
+def test_registered_operator_shape_functions(B, N, H, W, C):
+    """The shape functions that torch.compile uses for igs_amd::splat_fwd / splat_bwd agree with
+    the library's own plan (evaluated on meta tensors: no GPU, no kernel)."""
+    import torch
+
+    import igs_amd  # noqa: F401  (registers the operators)
+    from igs_amd import _lib, _splat
+
+    m = lambda *s: torch.empty(*s, device="meta")
+    Cp = _splat.padded_channels(C)
+    grids = (m(B, 1, H, W), m(1, 1, H, W))
+    for kind, params in ((_splat.KIND_SCALE_ROT, [m(B, N, 2), m(B, N, C), m(B, N, 2), m(B, N), m(B, N)]),
+                         (_splat.KIND_COVINV, [m(B, N, 2), m(B, N, 1, 1), m(B, N), m(B, N, 1), m(B, N), m(B, N, C)]),
+                         (_splat.KIND_FEATURE, [m(B, N, 6 + C), m(B, N, 2)])):
+        out, den, packed, col = torch.ops.igs_amd.splat_fwd(kind, params, *grids, 1e-6)
+        assert out.shape == (B, Cp, H, W) and den.shape == (B, H, W) and col.shape == (B, N, Cp)
+        assert packed.numel() * 4 == _lib.plan(B, N, H, W, Cp, _lib.IGS_GRID_AUTO).packed_bytes
+        assert out.dtype == torch.float32
+        g = torch.ops.igs_amd.splat_bwd(kind, params, *grids, packed, col, out, den, out, 1e-6, True)
+        assert [t.shape for t in g] == [p.shape for p in params] + [grids[0].shape, grids[1].shape]
+        assert len(torch.ops.igs_amd.splat_bwd(kind, params, *grids, packed, col, out, den, out, 1e-6, False)) == len(params)
+    with pytest.raises(ValueError):
+        torch.ops.igs_amd.splat_fwd(_splat.KIND_SCALE_ROT, [m(B, N, 2), m(B, N, C), m(B, N, 3), m(B, N), m(B, N)],
+                                    *grids, 1e-6)

@@ -153,7 +153,7 @@ def test_config4_full_size_properties(igs, dev):
         assert torch.allclose(g2[k], -2.0 * g1[k], rtol=1e-5, atol=1e-6 * float(g1[k].abs().max()))
     # Euler identity needs den: take it from a forward through the operator-level pieces
     a, b_, dd = O.cov_inverse_closed(d["scales"], d["rotations"])
-    from igs_amd.gs2d import _Grid, _Splat
+    from igs_amd._splat import Grid as _Grid, Splat as _Splat
 
     grid = _Grid(xg, yg, B)
     op = _Splat(B, N, C, grid, 1e-6, dev)
