@@ -15,7 +15,10 @@ from .gs2d import (  # noqa: F401
     naive_gaussian_2d,
 )
 
+from .fit import GaussianImageFit  # noqa: F401,E402
+
 __all__ = [
+    "GaussianImageFit",
     "GaussianSplatting2D",
     "gaussian_splatting_2d",
     "naive_gaussian_2d",

@@ -70,6 +70,11 @@ SIGNATURES = {
     "igs_gs2d_pack_feature": (c_int, [_FP, _FP, c_int, c_int, c_int, c_int, c_float, _FP, _FP, c_void_p]),
     "igs_gs2d_finalize_feature": (c_int, [_FP, c_int, _FP, _FP, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                           _FP, c_void_p]),
+    "igs_gs2d_mse_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "igs_gs2d_backward_prologue_mse": (c_int, [_FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int,
+                                               c_int, c_int, c_int, c_float, _FP, c_size_t, _FP, c_size_t, _FP,
+                                               c_void_p]),
+    "igs_adamw_step": (c_int, [_FP, _FP, _FP, _FP, c_int64, _FP, c_float, c_float, c_float, c_float, c_void_p]),
 }
 
 _lib = None

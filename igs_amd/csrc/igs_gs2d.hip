@@ -489,10 +489,17 @@ __global__ __launch_bounds__(kThreads) void k_fwd_combine(const float* __restric
 //              (padding columns repeat x of column W-1).
 //   general  : records [B][HWp][CP] = x, y, g^.., -s, 0..; padding pixels are zero records
 //              carrying the coordinates of the last pixel.
+// With `target` set (fit step), the upstream gradient is that of a mean-squared-error loss,
+// g_c = gscale (out_c - target_c), formed here instead of being read from `gout`, and each
+// workgroup writes its sum of (out - target)^2 (fixed-order LDS sum) to
+// loss_part[b * gridDim.x + blockIdx.x].
 template <int C, bool kSep>
 __global__ __launch_bounds__(kThreads) void k_bwd_pix(const float* __restrict__ out,
                                                       const float* __restrict__ den,
                                                       const float* __restrict__ gout,
+                                                      const float* __restrict__ target,
+                                                      float gscale,
+                                                      float* __restrict__ loss_part,
                                                       const float* __restrict__ x,
                                                       const float* __restrict__ y, long sxb,
                                                       long sxh, long sxw, long syb, long syh,
@@ -506,19 +513,19 @@ __global__ __launch_bounds__(kThreads) void k_bwd_pix(const float* __restrict__ 
     const int HW = H * W;
     const int i = blockIdx.x * kThreads + threadIdx.x;  // padded pixel index
     const int b = blockIdx.y;
-    int h, w;
-    bool valid;
+    int h = 0, w = 0;
+    bool valid, inside;  // inside: this thread owns a (padded) record; valid: a real pixel
     if (kSep) {
-        if (i >= H * Wp) return;
-        h = i / Wp;
-        w = i - h * Wp;
-        valid = w < W;
-        if (h == 0) {
+        inside = i < H * Wp;
+        h = inside ? i / Wp : 0;
+        w = inside ? i - h * Wp : 0;
+        valid = inside && w < W;
+        if (inside && h == 0) {
             float* xs = pixrec + (size_t)B * H * Wp * CP;
             xs[(size_t)b * Wp + w] = x[b * sxb + (long)min(w, W - 1) * sxw];
         }
     } else {
-        if (i >= HWp) return;
+        inside = i < HWp;
         valid = i < HW;
         const int pc = min(i, HW - 1);
         h = pc / W;
@@ -527,27 +534,102 @@ __global__ __launch_bounds__(kThreads) void k_bwd_pix(const float* __restrict__ 
     float r[CP];
 #pragma unroll
     for (int k = 0; k < CP; ++k) r[k] = 0.0f;
+    float sq = 0.0f;
     if (valid) {
         const int p = h * W + w;
         const float inv = 1.0f / (den[(size_t)b * HW + p] + eps);
         float s = 0.0f;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const float gh = gout[((size_t)b * C + c) * HW + p] * inv;
-            s = fmaf(gh, out[((size_t)b * C + c) * HW + p], s);
+            const size_t idx = ((size_t)b * C + c) * HW + p;
+            const float o = out[idx];
+            float g;
+            if (target != nullptr) {
+                const float d = o - target[idx];
+                sq = fmaf(d, d, sq);
+                g = gscale * d;
+            } else {
+                g = gout[idx];
+            }
+            const float gh = g * inv;
+            s = fmaf(gh, o, s);
             r[OFF + c] = gh;
         }
         r[OFF + C] = -s;
     }
-    if (!kSep) {
-        r[0] = x[b * sxb + h * sxh + w * sxw];
-        r[1] = y[b * syb + h * syh + w * syw];
-    }
-    const size_t rec = kSep ? ((size_t)b * H * Wp + i) : ((size_t)b * HWp + i);
-    float4* dst = reinterpret_cast<float4*>(pixrec + rec * CP);
+    if (inside) {
+        if (!kSep) {
+            r[0] = x[b * sxb + h * sxh + w * sxw];
+            r[1] = y[b * syb + h * syh + w * syw];
+        }
+        const size_t rec = kSep ? ((size_t)b * H * Wp + i) : ((size_t)b * HWp + i);
+        float4* dst = reinterpret_cast<float4*>(pixrec + rec * CP);
 #pragma unroll
-    for (int k = 0; k < CP / 4; ++k)
-        dst[k] = make_float4(r[4 * k], r[4 * k + 1], r[4 * k + 2], r[4 * k + 3]);
+        for (int k = 0; k < CP / 4; ++k)
+            dst[k] = make_float4(r[4 * k], r[4 * k + 1], r[4 * k + 2], r[4 * k + 3]);
+    }
+    if (loss_part != nullptr) {  // kernel-argument uniform: every thread reaches the barriers
+        __shared__ float red[kThreads];
+        red[threadIdx.x] = sq;
+        __syncthreads();
+        for (int k = kThreads / 2; k > 0; k >>= 1) {
+            if ((int)threadIdx.x < k) red[threadIdx.x] += red[threadIdx.x + k];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) loss_part[(size_t)b * gridDim.x + blockIdx.x] = red[0];
+    }
+}
+
+// loss = scale * sum(loss_part[0..count)), one workgroup, fixed order.
+__global__ __launch_bounds__(kThreads) void k_loss_sum(const float* __restrict__ loss_part, int count,
+                                                       float scale, float* __restrict__ loss,
+                                                       const int* __restrict__ flag, int want) {
+    if (flag != nullptr && *flag != want) return;
+    __shared__ float red[kThreads];
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < count; i += kThreads) s += loss_part[i];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int k = kThreads / 2; k > 0; k >>= 1) {
+        if ((int)threadIdx.x < k) red[threadIdx.x] += red[threadIdx.x + k];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *loss = red[0] * scale;
+}
+
+// ----------------------------------------------------------------------------- AdamW
+// Decoupled-weight-decay Adam over one flat parameter block, the update of torch.optim.AdamW
+// (amsgrad off) as the fit script configures it (scripts/2dgs_img_comp.py:186-193).  The
+// step counter and learning rate live in device memory so that a captured graph advances:
+//   state = {lr, t, 1 - beta1^t, sqrt(1 - beta2^t)}; lr is written by the host, the rest by
+// k_adamw_tick (one thread, powers in double).
+__global__ void k_adamw_tick(float* __restrict__ state, float beta1, float beta2) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const float t = state[1] + 1.0f;
+    state[1] = t;
+    state[2] = (float)(1.0 - pow((double)beta1, (double)t));
+    state[3] = (float)sqrt(1.0 - pow((double)beta2, (double)t));
+}
+
+__global__ __launch_bounds__(kThreads) void k_adamw(float* __restrict__ param,
+                                                    const float* __restrict__ grad,
+                                                    float* __restrict__ exp_avg,
+                                                    float* __restrict__ exp_avg_sq, long n,
+                                                    const float* __restrict__ state, float beta1,
+                                                    float beta2, float eps, float weight_decay) {
+    const long i = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= n) return;
+    const float lr = state[0], bc1 = state[2], bc2_sqrt = state[3];
+    const float g = grad[i];
+    float p = param[i] * (1.0f - lr * weight_decay);
+    float m = exp_avg[i];
+    m = fmaf(g - m, 1.0f - beta1, m);
+    const float v = fmaf(g * g, 1.0f - beta2, exp_avg_sq[i] * beta2);
+    const float denom = sqrtf(v) / bc2_sqrt + eps;
+    p -= (lr / bc1) * (m / denom);
+    param[i] = p;
+    exp_avg[i] = m;
+    exp_avg_sq[i] = v;
 }
 
 struct BwdArgs {
@@ -1252,6 +1334,15 @@ int variants_of(int grid_mode, const int32_t* grid_flag, Variant (&v)[2]) {
     return 1;
 }
 
+// Fused mean-squared-error upstream gradient of the fit step (all null/zero: plain backward).
+struct MseArgs {
+    const float* target = nullptr;  // [B,C,H,W]
+    float gscale = 0.0f;            // 2 / (number of real elements)
+    float* loss_part = nullptr;     // one float per prologue workgroup
+    float loss_scale = 0.0f;        // 1 / (number of real elements)
+    float* loss = nullptr;          // 1 float
+};
+
 template <int C>
 int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
     const int blocks = ((a.total_tiles + 7) / 8) * 8;
@@ -1265,18 +1356,24 @@ int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
 
 template <int C>
 int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, const float* den,
-                        const float* gout, const float* x, const float* y, const int64_t* gs,
-                        float eps, float* pixrec, hipStream_t st) {
+                        const float* gout, const MseArgs& mse, const float* x, const float* y,
+                        const int64_t* gs, float eps, float* pixrec, hipStream_t st) {
     const int padded = sep ? a.H * a.Wp : a.HWp;
     const dim3 pgrid(ceil_div(padded, kThreads), B, 1);
     if (sep)
-        hipLaunchKernelGGL((k_bwd_pix<C, true>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
+        hipLaunchKernelGGL((k_bwd_pix<C, true>), pgrid, dim3(kThreads), 0, st, out, den, gout,
+                           mse.target, mse.gscale, mse.loss_part, x, y,
                            gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
                            pixrec, a.flag, a.want);
     else
-        hipLaunchKernelGGL((k_bwd_pix<C, false>), pgrid, dim3(kThreads), 0, st, out, den, gout, x, y,
+        hipLaunchKernelGGL((k_bwd_pix<C, false>), pgrid, dim3(kThreads), 0, st, out, den, gout,
+                           mse.target, mse.gscale, mse.loss_part, x, y,
                            gs[0], gs[1], gs[2], gs[3], gs[4], gs[5], B, a.H, a.W, a.Wp, a.HWp, eps,
                            pixrec, a.flag, a.want);
+    int rc = launch_status();
+    if (rc || !mse.loss_part) return rc;
+    hipLaunchKernelGGL(k_loss_sum, dim3(1), dim3(kThreads), 0, st, mse.loss_part, (int)pgrid.x * B,
+                       mse.loss_scale, mse.loss, a.flag, a.want);
     return launch_status();
 }
 
@@ -1428,12 +1525,15 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
     return IGS_OK;
 }
 
-int igs_gs2d_backward_prologue(const float* x, const float* y, const int64_t grid_strides[6],
-                               int grid_mode, const int32_t* grid_flag, const float* out,
-                               const float* den, const float* grad_out, int B, int N, int H, int W,
-                               int C, float eps, float* pix_ws, size_t pix_bytes,
-                               igs_stream_t stream) {
-    if (!x || !y || !grid_strides || !out || !den || !grad_out || !pix_ws) return IGS_ERR_NULL_POINTER;
+}  // extern "C"
+
+namespace {
+int backward_prologue(const float* x, const float* y, const int64_t grid_strides[6], int grid_mode,
+                      const int32_t* grid_flag, const float* out, const float* den,
+                      const float* grad_out, const MseArgs& mse, int B, int N, int H, int W, int C,
+                      float eps, float* pix_ws, size_t pix_bytes, igs_stream_t stream) {
+    if (!x || !y || !grid_strides || !out || !den || !pix_ws) return IGS_ERR_NULL_POINTER;
+    if (!grad_out && !mse.target) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
     if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
@@ -1449,10 +1549,64 @@ int igs_gs2d_backward_prologue(const float* x, const float* y, const int64_t gri
         rc = bwd_args(a, vs[i], nullptr, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr);
         if (rc) return rc;
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
-        IGS_DISPATCH_C(C, rc = launch_bwd_prologue<kC>(a, B, sep, out, den, grad_out, x, y, grid_strides, eps, pix_ws, st));
+        IGS_DISPATCH_C(C, rc = launch_bwd_prologue<kC>(a, B, sep, out, den, grad_out, mse, x, y, grid_strides, eps, pix_ws, st));
         if (rc) return rc;
     }
     return IGS_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int igs_gs2d_backward_prologue(const float* x, const float* y, const int64_t grid_strides[6],
+                               int grid_mode, const int32_t* grid_flag, const float* out,
+                               const float* den, const float* grad_out, int B, int N, int H, int W,
+                               int C, float eps, float* pix_ws, size_t pix_bytes,
+                               igs_stream_t stream) {
+    if (!grad_out) return IGS_ERR_NULL_POINTER;
+    return backward_prologue(x, y, grid_strides, grid_mode, grid_flag, out, den, grad_out, MseArgs{}, B, N,
+                             H, W, C, eps, pix_ws, pix_bytes, stream);
+}
+
+size_t igs_gs2d_mse_workspace_bytes(int B, int H, int W) {
+    // one float per prologue workgroup of either grid variant (padded pixel counts differ)
+    if (B < 1 || H < 1 || W < 1) return 0;
+    const long sep = (long)H * ((W + 7) & ~7), gen = ((long)H * W + 3) & ~3L;
+    return (size_t)B * ceil_div(sep > gen ? sep : gen, kThreads) * sizeof(float);
+}
+
+int igs_gs2d_backward_prologue_mse(const float* x, const float* y, const int64_t grid_strides[6],
+                                   int grid_mode, const int32_t* grid_flag, const float* out,
+                                   const float* den, const float* target, int C_real, int B, int N,
+                                   int H, int W, int C, float eps, float* pix_ws, size_t pix_bytes,
+                                   float* loss_ws, size_t loss_ws_bytes, float* loss,
+                                   igs_stream_t stream) {
+    if (!target || !loss_ws || !loss) return IGS_ERR_NULL_POINTER;
+    if (C_real < 1 || C_real > C) return IGS_ERR_BAD_SHAPE;
+    if (loss_ws_bytes < igs_gs2d_mse_workspace_bytes(B, H, W)) return IGS_ERR_WORKSPACE;
+    MseArgs mse;
+    const double count = (double)B * C_real * H * W;
+    mse.target = target;
+    mse.gscale = (float)(2.0 / count);
+    mse.loss_part = loss_ws;
+    mse.loss_scale = (float)(1.0 / count);
+    mse.loss = loss;
+    return backward_prologue(x, y, grid_strides, grid_mode, grid_flag, out, den, nullptr, mse, B, N, H, W,
+                             C, eps, pix_ws, pix_bytes, stream);
+}
+
+int igs_adamw_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int64_t count,
+                   float* state, float beta1, float beta2, float eps, float weight_decay,
+                   igs_stream_t stream) {
+    if (!param || !grad || !exp_avg || !exp_avg_sq || !state) return IGS_ERR_NULL_POINTER;
+    if (count < 1 || count > (int64_t)kThreads * 0x7fffffff) return IGS_ERR_BAD_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_adamw_tick, dim3(1), dim3(64), 0, st, state, beta1, beta2);
+    int rc = launch_status();
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_adamw, dim3((unsigned)((count + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
+                       param, grad, exp_avg, exp_avg_sq, (long)count, state, beta1, beta2, eps, weight_decay);
+    return launch_status();
 }
 
 int igs_gs2d_backward_reduce(const float* packed, const float* colors, const float* y,

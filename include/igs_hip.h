@@ -189,6 +189,34 @@ int igs_gs2d_finalize_feature(const float *partial, int grid_mode, const int32_t
                               const float *gs_feature, int B, int N, int H, int W, int C,
                               int C_kernel, float eps, float *g_feature, igs_stream_t stream);
 
+/* Fit step (single-image fitting loop, scripts/2dgs_img_comp.py:186-193 and :219-232):
+ * render -> loss -> backward -> AdamW without leaving the library between the stages.
+ *
+ * igs_gs2d_backward_prologue_mse is igs_gs2d_backward_prologue with the upstream gradient of
+ * loss = mean((out - target)^2) (F.mse_loss, scripts/2dgs_img_comp.py:133) formed inside the
+ * per-pixel pass: g = 2 (out - target) / (B C_real H W).  out and target are [B,C,H,W] with the
+ * compiled channel count C; channels C_real..C-1 must be zero in both.  The loss value is
+ * written to loss[0] (device; fixed-order sum, bit-reproducible).  loss_ws needs
+ * igs_gs2d_mse_workspace_bytes(B,H,W) bytes.  Follow with igs_gs2d_backward_reduce. */
+size_t igs_gs2d_mse_workspace_bytes(int B, int H, int W);
+int igs_gs2d_backward_prologue_mse(const float *x, const float *y, const int64_t grid_strides[6],
+                                   int grid_mode, const int32_t *grid_flag, const float *out,
+                                   const float *den, const float *target, int C_real, int B, int N,
+                                   int H, int W, int C, float eps, float *pix_ws, size_t pix_bytes,
+                                   float *loss_ws, size_t loss_ws_bytes, float *loss,
+                                   igs_stream_t stream);
+
+/* One torch.optim.AdamW step (amsgrad off; the optimiser of scripts/2dgs_img_comp.py:186-193)
+ * over a flat block of `count` floats, in place:
+ *   p *= 1 - lr wd;  m += (g - m)(1 - beta1);  v = beta2 v + (1 - beta2) g^2;
+ *   p -= lr / (1 - beta1^t) * m / (sqrt(v) / sqrt(1 - beta2^t) + eps).
+ * state is 4 floats of device memory {lr, t, 1 - beta1^t, sqrt(1 - beta2^t)}: the caller
+ * writes lr (and t = 0 before the first step); every call increments t on the device, so a
+ * captured graph of the call advances on each replay. */
+int igs_adamw_step(float *param, const float *grad, float *exp_avg, float *exp_avg_sq,
+                   int64_t count, float *state, float beta1, float beta2, float eps,
+                   float weight_decay, igs_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,191 @@
+"""The fused fit step (render -> MSE -> backward -> AdamW, scripts/2dgs_img_comp.py:107-126,
+:186-193, :219-232) against the same iteration written with torch: this build's differentiable
+`gaussian_splatting_2d` (itself checked against the fp64 oracle elsewhere), `F.mse_loss` and
+`torch.optim.AdamW` with the fit script's hyper-parameters."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gs2d_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+HYPER = dict(eps=1e-6, betas=(0.9, 0.995), weight_decay=1e-4)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def igs():
+    import igs_amd
+
+    return igs_amd
+
+
+def make_block(B, N, C, seed, dev):
+    g = torch.Generator().manual_seed(seed)
+    pos = torch.rand(B, N, 2, generator=g) * 2 - 1
+    ls = torch.log(torch.rand(B, N, 2, generator=g) * 0.15 + 0.05)
+    rot = torch.rand(B, N, 1, generator=g) * 6.283
+    col = torch.rand(B, N, C, generator=g)
+    return torch.cat([pos, ls, rot, torch.zeros(B, N, 1), col], dim=-1).to(dev)
+
+
+def grids(igs, B, H, W, dev, general=False, seed=0):
+    if general:
+        g = torch.Generator().manual_seed(seed)
+        return ((torch.rand(B, 1, H, W, generator=g) * 2 - 1).to(dev), (torch.rand(B, 1, H, W, generator=g) * 2 - 1).to(dev))
+    x, y = igs.GaussianSplatting2D.xy_grid((H, W), dev)
+    return x[None].expand(B, 1, H, W), y[None].expand(B, 1, H, W)
+
+
+def torch_steps(igs, block0, target, xg, yg, steps, lr, n=None):
+    C = block0.shape[-1] - 6
+    p = block0.clone().requires_grad_(True)
+    opt = torch.optim.AdamW([p], lr=lr, **HYPER)
+    losses = []
+    for _ in range(steps):
+        q = p if n is None else p[:, :n]
+        pos, ls, rot, _, col = q.split([2, 2, 1, 1, C], dim=-1)
+        img = igs.gaussian_splatting_2d(pos, col, torch.exp(ls) + 1e-6, rot[..., 0], torch.ones_like(rot[..., 0]),
+                                        xg, yg)
+        loss = F.mse_loss(img, target)
+        loss.backward()
+        opt.step()
+        opt.zero_grad()
+        losses.append(loss.detach().clone())
+    return p.detach(), torch.stack(losses)
+
+
+def close(a, b, what, rtol=2e-5, atol=2e-6):
+    err = (a - b).abs()
+    ok = err <= atol + rtol * b.abs()
+    assert bool(ok.all()), f"{what}: max err {float(err.max()):.3e}, {int((~ok).sum())} of {ok.numel()} outside"
+
+
+@pytest.mark.parametrize("B,N,H,W,C,general", [(1, 200, 32, 48, 3, False), (2, 67, 17, 70, 3, True), (1, 96, 24, 40, 5, False)],
+                         ids=["B1-C3-linspace", "B2-C3-general", "B1-C5-padded-channels"])
+def test_fused_step_matches_torch_iteration(igs, dev, B, N, H, W, C, general):
+    from igs_amd.fit import GaussianImageFit
+
+    block = make_block(B, N, C, 1, dev)
+    xg, yg = grids(igs, B, H, W, dev, general, seed=3)
+    target = O.smooth_noise_target(H, W, seed=7, C=C).to(dev).expand(B, C, H, W).contiguous()
+    lr, steps = 0.02, 6
+    ref, ref_losses = torch_steps(igs, block, target, xg, yg, steps, lr)
+    fit = GaussianImageFit(block.clone(), target, xg, yg, lr=lr, adam_eps=HYPER["eps"], betas=HYPER["betas"],
+                           weight_decay=HYPER["weight_decay"])
+    losses = torch.stack([fit.step().clone() for _ in range(steps)])
+    assert fit.step_count == steps
+    close(losses, ref_losses, "loss", rtol=1e-5, atol=1e-9)
+    # the unused column has no gradient; torch leaves it at 0 * (1 - lr wd)^k = 0 as well
+    close(fit.params, ref, "parameters after 6 steps")
+    assert float((fit.params - block).abs().max()) > 1e-3          # it did move
+    named = fit.named_parameters()
+    assert named["position"].shape == (B, N, 2) and named["color"].shape == (B, N, C)
+
+
+def test_adamw_kernel_against_torch_optimizer(igs, dev):
+    """igs_adamw_step alone on random gradients of widely varying magnitude, 20 steps."""
+    from igs_amd import _lib
+    from igs_amd._splat import _ptr, _stream
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(5)
+    n = 10007
+    p0 = torch.randn(n, generator=g).to(dev)
+    p = p0.clone()
+    m, v = torch.zeros_like(p), torch.zeros_like(p)
+    state = torch.tensor([0.01, 0, 0, 0], dtype=torch.float32, device=dev)
+    q = p0.clone().requires_grad_(True)
+    opt = torch.optim.AdamW([q], lr=0.01, **HYPER)
+    for k in range(20):
+        grad = (torch.randn(n, generator=g) * 10.0 ** torch.randint(-9, 1, (n,), generator=g).float()).to(dev)
+        if k == 10:                                     # learning-rate change mid-run
+            state[0] = 0.003
+            opt.param_groups[0]["lr"] = 0.003
+        _lib.check(lib.igs_adamw_step(_ptr(p), _ptr(grad), _ptr(m), _ptr(v), n, _ptr(state), 0.9, 0.995, 1e-6, 1e-4,
+                                      _stream(dev)), "igs_adamw_step")
+        q.grad = grad.clone()
+        opt.step()
+    close(p, q.detach(), "AdamW parameters", rtol=1e-5, atol=1e-6)
+    st = opt.state[q]
+    # moments: sums of terms of either sign up to |g| ~ 30, so a few ulp of the largest term
+    close(m, st["exp_avg"], "exp_avg", rtol=1e-5, atol=1e-6)
+    close(v, st["exp_avg_sq"], "exp_avg_sq", rtol=1e-5, atol=1e-6)
+    assert float(state[1]) == 20.0
+
+
+def test_graph_replay_equals_eager_fused_steps(igs, dev):
+    from igs_amd.fit import GaussianImageFit
+
+    B, N, H, W, C = 1, 300, 40, 64, 3
+    block = make_block(B, N, C, 2, dev)
+    xg, yg = grids(igs, B, H, W, dev)
+    target = O.smooth_noise_target(H, W, seed=9, C=C).to(dev)
+    eager = GaussianImageFit(block.clone(), target, xg, yg, lr=0.02)
+    graphed = GaussianImageFit(block.clone(), target, xg, yg, lr=0.02)
+    graphed.capture()
+    assert torch.equal(graphed.params, block) and graphed.step_count == 0   # capture executes nothing
+    for k in range(8):
+        if k == 4:
+            eager.set_lr(0.005)
+            graphed.set_lr(0.005)
+        le = eager.step().clone()
+        lg = graphed.step().clone()
+        torch.cuda.synchronize()                       # the program's own work between replays
+        assert torch.equal(le, lg), k
+        assert torch.equal(eager.params, graphed.params), k
+    assert graphed.step_count == 8
+
+
+def test_prefix_of_gaussians_and_new_resolution(igs, dev):
+    """num_active (scripts/2dgs_img_comp.py:107-111) and a change of target size (:208-217)."""
+    from igs_amd.fit import GaussianImageFit
+
+    B, N, C = 1, 128, 3
+    block = make_block(B, N, C, 4, dev)
+    xg, yg = grids(igs, B, 24, 40, dev)
+    target = O.smooth_noise_target(24, 40, seed=11, C=C).to(dev)
+    fit = GaussianImageFit(block.clone(), target, xg, yg, lr=0.02)
+    ref, _ = torch_steps(igs, block, target, xg, yg, 3, 0.02, n=50)
+    for _ in range(3):
+        fit.step(num_active=50)
+    close(fit.params[:, :50], ref[:, :50], "active prefix")
+    assert torch.equal(fit.params[:, 50:], block[:, 50:])          # inactive Gaussians untouched
+    img = fit.render()
+    assert img.shape == (1, 3, 24, 40)
+    xg2, yg2 = grids(igs, B, 48, 80, dev)
+    fit.set_target(O.smooth_noise_target(48, 80, seed=11, C=C).to(dev), xg2, yg2)
+    l0 = float(fit.step())
+    for _ in range(30):
+        l = float(fit.step())
+    assert l < l0
+    with pytest.raises(ValueError):
+        GaussianImageFit(make_block(2, 16, 3, 0, dev), target.expand(2, -1, -1, -1), xg, yg).step(num_active=4)
+
+
+def test_fit_converges_config2_reduced(igs, dev):
+    """c2-shaped (one image, sigma 0.01-0.1) at reduced size: 100 fused steps lower the loss
+    steadily, as the same loop through torch does."""
+    from igs_amd.fit import GaussianImageFit
+
+    N, H, W = 2048, 128, 128
+    g = torch.Generator().manual_seed(1002)
+    pos = torch.rand(1, N, 2, generator=g) * 2 - 1
+    col = torch.rand(1, N, 3, generator=g)
+    sc = torch.rand(1, N, 2, generator=g) * 0.09 + 0.01
+    rot = torch.rand(1, N, generator=g) * 6.283
+    xg, yg = grids(igs, 1, H, W, dev)
+    target = O.smooth_noise_target(H, W, seed=1002).to(dev)
+    fit = GaussianImageFit.from_parameters(pos.to(dev), sc.log().to(dev), rot.to(dev), col.to(dev), target, xg, yg,
+                                           lr=min(0.05 * 4096 / N, 0.03))
+    fit.capture()
+    losses = [float(fit.step()) for _ in range(100)]
+    assert losses[10] < losses[0] and losses[99] < 0.5 * losses[10]
+    assert bool(torch.isfinite(fit.params).all())
