@@ -14,6 +14,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 LIB_PATH = os.environ.get("IGS_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "libigs_hip.so")
 
+ABI_VERSION = 2  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1
 IGS_GRID_AUTO = 2
@@ -39,6 +40,8 @@ class Plan(ctypes.Structure):
         ("fwd_ws_bytes", c_uint64),
         ("pix_bytes", c_uint64),
         ("partial_bytes", c_uint64),
+        ("fwd_tiles", c_int32),
+        ("bwd_tiles_x", c_int32),
     ]
 
 
@@ -101,8 +104,9 @@ def load() -> ctypes.CDLL:
             raise IGSLibraryError(f"{LIB_PATH} does not export {name}") from e
         fn.restype = res
         fn.argtypes = args
-    if lib.igs_abi_version() != 1:
-        raise IGSLibraryError(f"ABI version mismatch: library reports {lib.igs_abi_version()}, binding expects 1")
+    if lib.igs_abi_version() != ABI_VERSION:
+        raise IGSLibraryError(f"ABI version mismatch: library reports {lib.igs_abi_version()}, binding expects "
+                              f"{ABI_VERSION}")
     _lib = lib
     return lib
 

@@ -78,8 +78,37 @@ __device__ __forceinline__ int xcd_contiguous(int linear, int total) {
 }
 
 // ----------------------------------------------------------------------------- pack
+// Reach box of a Gaussian: the axis-aligned bounding box of the ellipse q <= kReachQ, outside
+// of which its weight is exactly zero in these kernels: there the exponent
+// q' = -0.5 log2(e) q is below -160, ten binades under the -149/-150 at which exp2 returns 0
+// in fp32 whatever the denormal mode (the margin covers the rounding of q' itself, which is
+// a few ulp of its largest term).  Pixels outside the box therefore receive exactly +0 from
+// this Gaussian and give exactly 0 to its gradient sums, so skipping them changes no bit.
+// Half extents: sqrt(kReachQ Sigma_xx), sqrt(kReachQ Sigma_yy) with Sigma the covariance that
+// (A, B, D) invert.  A record with a non-finite field or a non-positive-definite (A, B, D)
+// gets an unbounded box (its NaN/inf must propagate as without culling); padding records get
+// an empty one.  Stored as (xlo, xhi, ylo, yhi).
+constexpr double kReachQ = 160.0 / 0.72134752044448170368;
+
+__device__ __forceinline__ float4 reach_box(float px, float py, double sxx, double syy, bool bounded) {
+    const float inf = __builtin_inff();
+    if (!bounded || !(sxx >= 0.0) || !(syy >= 0.0) || !isfinite(px) || !isfinite(py))
+        return make_float4(-inf, inf, -inf, inf);
+    // rounded outwards: one part in 1e5 is far more than the fp32 rounding of the bounds
+    const double hx = sqrt(kReachQ * sxx) * 1.00001, hy = sqrt(kReachQ * syy) * 1.00001;
+    const double ax = fabs((double)px) * 1e-6 + 1e-30, ay = fabs((double)py) * 1e-6 + 1e-30;
+    return make_float4((float)((double)px - hx - ax), (float)((double)px + hx + ax),
+                       (float)((double)py - hy - ay), (float)((double)py + hy + ay));
+}
+
+__device__ __forceinline__ float4 empty_box() {
+    const float inf = __builtin_inff();
+    return make_float4(inf, -inf, inf, -inf);
+}
+
 // One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
 // with A' = k A, B2' = 2 k B, D' = k D, k = -0.5 log2 e.  Records N..Np-1 are zero.
+// The reach boxes [B][Np] follow the records in the packed buffer.
 template <bool kScaleRot>
 __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ position,
                                                    const float* __restrict__ p0,  // cov00 | scales
@@ -88,42 +117,60 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
                                                    const float* __restrict__ alphas,
                                                    const float* __restrict__ colors, int N,
                                                    int Np, int C, int RS, float eps,
-                                                   float* __restrict__ packed) {
+                                                   float* __restrict__ packed,
+                                                   float4* __restrict__ boxes) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n >= Np) return;
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {  // padding: alpha = 0 and e = exp2(0) = 1, so it contributes exactly 0
         for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        boxes[(size_t)b * Np + n] = empty_box();
         return;
     }
     const size_t i = (size_t)b * N + n;
     // The closed form runs in fp64 and is rounded once: an error of a few fp32 ulp in A', B2', D'
     // would be multiplied by |q| (tens, for sharp Gaussians) in the exponent.  O(BN) work.
-    double A, Bc, D;
+    double A, Bc, D, sxx, syy;
+    bool bounded;
     if (kScaleRot) {
         const double s0 = p0[2 * i], s1 = p0[2 * i + 1];
         double sn, cs;
         sincos((double)p1[i], &sn, &cs);
-        const double i0 = 1.0 / (s0 * s0 + (double)eps), i1 = 1.0 / (s1 * s1 + (double)eps);
+        const double v0 = s0 * s0 + (double)eps, v1 = s1 * s1 + (double)eps;
+        const double i0 = 1.0 / v0, i1 = 1.0 / v1;
         A = cs * cs * i0 + sn * sn * i1;
         Bc = cs * sn * (i0 - i1);
         D = sn * sn * i0 + cs * cs * i1;
+        sxx = cs * cs * v0 + sn * sn * v1;
+        syy = sn * sn * v0 + cs * cs * v1;
+        bounded = v0 > 0.0 && v1 > 0.0;
     } else {
         A = p0[i];
         Bc = p1[i];
         D = p2[i];
+        const double det = A * D - Bc * Bc;
+        bounded = A > 0.0 && det > 0.0;
+        sxx = D / det;
+        syy = A / det;
     }
     constexpr double k = -0.72134752044448170368;  // -0.5 * log2(e)
     const float al = alphas[i];
-    r[0] = position[2 * i];
-    r[1] = position[2 * i + 1];
+    const float px = position[2 * i], py = position[2 * i + 1];
+    r[0] = px;
+    r[1] = py;
     r[2] = (float)(k * A);
     r[3] = (float)(2.0 * k * Bc);
     r[4] = (float)(k * D);
     r[5] = al;
-    for (int c = 0; c < C; ++c) r[6 + c] = al * colors[i * C + c];
+    bool fin = isfinite(al) && isfinite(r[2]) && isfinite(r[3]) && isfinite(r[4]);
+    for (int c = 0; c < C; ++c) {
+        const float v = al * colors[i * C + c];
+        r[6 + c] = v;
+        fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
+    }
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
+    boxes[(size_t)b * Np + n] = reach_box(px, py, sxx, syy, bounded && fin);
 }
 
 // Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
@@ -135,6 +182,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
                                                            const float* __restrict__ pos_off, int N,
                                                            int Np, int C, int Cp, int RS, float eps,
                                                            float* __restrict__ packed,
+                                                           float4* __restrict__ boxes,
                                                            float* __restrict__ colors_out) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
@@ -142,6 +190,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {
         for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        boxes[(size_t)b * Np + n] = empty_box();
         return;
     }
     const size_t i = (size_t)b * N + n;
@@ -149,7 +198,8 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
     const double s0 = (double)expf(f[2]) + (double)eps, s1 = (double)expf(f[3]) + (double)eps;
     double sn, cs;
     sincos((double)f[4], &sn, &cs);
-    const double i0 = 1.0 / (s0 * s0 + (double)eps), i1 = 1.0 / (s1 * s1 + (double)eps);
+    const double v0 = s0 * s0 + (double)eps, v1 = s1 * s1 + (double)eps;
+    const double i0 = 1.0 / v0, i1 = 1.0 / v1;
     const double A = cs * cs * i0 + sn * sn * i1;
     const double Bc = cs * sn * (i0 - i1);
     const double D = sn * sn * i0 + cs * cs * i1;
@@ -165,12 +215,148 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
     r[3] = (float)(2.0 * k * Bc);
     r[4] = (float)(k * D);
     r[5] = 1.0f;
+    bool fin = isfinite(r[2]) && isfinite(r[3]) && isfinite(r[4]);
     for (int c = 0; c < Cp; ++c) {
         const float col = c < C ? f[6 + c] : 0.0f;
         r[6 + c] = col;
         colors_out[i * Cp + c] = col;
+        fin = fin && isfinite(col);
     }
     for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
+    boxes[(size_t)b * Np + n] = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
+                                          fin && v0 > 0.0 && v1 > 0.0);
+}
+
+// ----------------------------------------------------------------------------- binning
+// Per pixel tile, the Gaussians whose reach box meets the tile's coordinate range, as a list
+// of indices in increasing order (so that sums over a list keep the order of the unculled
+// sum), and the count.  One workgroup per (tile, image) scans all N boxes; positions come
+// from ballots and a fixed-order prefix over the four waves, so the lists are reproducible.
+// With `complement`, the Gaussians that do not meet the tile are written to the back of the
+// same list array (list[Np-1], list[Np-2], ...): every n < N then appears exactly once,
+// listed ones in [0, count), the others in [count + Np - N, Np).
+// Separable grids only: a tile is tile_w columns x tile_h rows and its coordinate range is
+// [min, max] of x over its columns and of y over its rows (no monotonicity assumed).
+struct BinArgs {
+    const float4* boxes;  // [B][Np]
+    const float* x;
+    const float* y;
+    long sxb, sxw, syb, syh;
+    int N, Np, H, W;
+    int tile_w, tile_h, tiles_x, tiles_y;
+    int* counts;  // [B][tiles]
+    int* lists;   // [B][tiles][Np]
+    int complement;
+    const int* flag;
+    int want;
+};
+
+constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads in flight per tile
+
+__global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
+    if (a.flag != nullptr && *a.flag != a.want) return;
+    __shared__ float red[4][kBinThreads];
+    __shared__ int wsum[2][kBinWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tiles = a.tiles_x * a.tiles_y;
+    const int t = blockIdx.x, b = blockIdx.y;
+    const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
+    const int c0 = tx * a.tile_w, c1 = min(a.W, c0 + a.tile_w);
+    const int r0 = ty * a.tile_h, r1 = min(a.H, r0 + a.tile_h);
+    const float inf = __builtin_inff();
+    float xlo = inf, xhi = -inf, ylo = inf, yhi = -inf;
+    bool bad = false;
+    for (int c = c0 + tid; c < c1; c += kBinThreads) {
+        const float v = a.x[b * a.sxb + (long)c * a.sxw];
+        bad = bad || !(v == v);
+        xlo = fminf(xlo, v);
+        xhi = fmaxf(xhi, v);
+    }
+    for (int r = r0 + tid; r < r1; r += kBinThreads) {
+        const float v = a.y[b * a.syb + (long)r * a.syh];
+        bad = bad || !(v == v);
+        ylo = fminf(ylo, v);
+        yhi = fmaxf(yhi, v);
+    }
+    if (bad) {  // a NaN coordinate: nothing may be culled for this tile
+        xlo = ylo = -inf;
+        xhi = yhi = inf;
+    }
+    red[0][tid] = xlo;
+    red[1][tid] = -xhi;
+    red[2][tid] = ylo;
+    red[3][tid] = -yhi;
+    __syncthreads();
+    for (int k = kBinThreads / 2; k > 0; k >>= 1) {
+        if (tid < k) {
+#pragma unroll
+            for (int f = 0; f < 4; ++f) red[f][tid] = fminf(red[f][tid], red[f][tid + k]);
+        }
+        __syncthreads();
+    }
+    const float txlo = red[0][0], txhi = -red[1][0], tylo = red[2][0], tyhi = -red[3][0];
+    int* list = a.lists + ((size_t)b * tiles + t) * a.Np;
+    const float4* boxes = a.boxes + (size_t)b * a.Np;
+    // Each wave scans one contiguous share of the Gaussians twice, without barriers: first to
+    // count, then (with the shares' counts prefixed in wave order) to write.
+    const int per_wave = ((a.N + kBinWaves - 1) / kBinWaves + 63) & ~63;
+    const int nb = wave * per_wave, ne = min(a.N, nb + per_wave);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    // kU boxes per lane are loaded together, so that kU loads are in flight instead of one
+    constexpr int kU = 8;
+    auto classify = [&](int n0, bool (&listed)[kU], bool (&unlisted)[kU]) {
+        float4 bb[kU];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int n = n0 + u * 64 + lane;
+            bb[u] = boxes[min(n, a.N - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const bool in = n0 + u * 64 + lane < ne;
+            // "definitely outside" negated, so that NaN bounds count as inside
+            listed[u] = in && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
+            unlisted[u] = in && !listed[u];
+        }
+    };
+    int cnt = 0, ucnt = 0;
+    for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
+        bool listed[kU], unlisted[kU];
+        classify(n0, listed, unlisted);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            cnt += __popcll(__ballot(listed[u]));
+            ucnt += __popcll(__ballot(unlisted[u]));
+        }
+    }
+    if (lane == 0) {
+        wsum[0][wave] = cnt;
+        wsum[1][wave] = ucnt;
+    }
+    __syncthreads();
+    int base = 0, ubase = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kBinWaves; ++w) {
+        if (w < wave) {
+            base += wsum[0][w];
+            ubase += wsum[1][w];
+        }
+        total += wsum[0][w];
+    }
+    for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
+        bool listed[kU], unlisted[kU];
+        classify(n0, listed, unlisted);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int n = n0 + u * 64 + lane;
+            const unsigned long long m = __ballot(listed[u]), um = __ballot(unlisted[u]);
+            if (listed[u]) list[base + __popcll(m & below)] = n;
+            if (a.complement && unlisted[u]) list[a.Np - 1 - (ubase + __popcll(um & below))] = n;
+            base += __popcll(m);
+            ubase += __popcll(um);
+        }
+    }
+    if (tid == 0) a.counts[(size_t)b * tiles + t] = total;
 }
 
 // ----------------------------------------------------------------------------- forward
@@ -186,6 +372,8 @@ struct FwdArgs {
     float* out;
     float* den;
     float* part;  // [S][B][C+1][HW] when S > 1
+    const int* counts;  // separable: Gaussians listed per tile [B][tiles]
+    const int* lists;   // separable: their indices [B][tiles][Np]
     const int* flag;  // AUTO grid mode: run only if *flag == want (nullptr: always run)
     int want;
 };
@@ -257,21 +445,42 @@ constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
 // once per record with a wave-uniform LDS pointer.  Records past `count` in the last chunk
 // read as all-zero (for a Gaussian record: alpha = 0, adds exactly 0).  Must be called by all
 // kThreads threads of the workgroup (it contains barriers).
-template <int R4, int CH, class Body>
+// With kGather, record i of the stream is src record index[i] (a tile's Gaussian list).
+template <int R4, int CH, bool kGather = false, class Body>
 __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
-                                                   float4* sh, Body&& body) {
+                                                   float4* sh, Body&& body,
+                                                   const int* __restrict__ index = nullptr) {
     constexpr int E = CH * R4;                          // float4 per chunk
     constexpr int PRE = (E + kThreads - 1) / kThreads;  // float4 per thread per chunk
     const int total = count * R4;
     const int chunks = (count + CH - 1) / CH;
     const int tid = threadIdx.x;
     const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    float4 pre[PRE];
+    // Gather: the record indices of a chunk are loaded one chunk before its records, so that
+    // no load in the loop waits for another load.
+    int idx[PRE];
+    auto load_idx = [&](int chunk) {
 #pragma unroll
-    for (int i = 0; i < PRE; ++i) {
-        const int e = i * kThreads + tid;
-        pre[i] = (e < E && e < total) ? src[e] : zero;
-    }
+        for (int i = 0; i < PRE; ++i) {
+            const int e = i * kThreads + tid, ge = chunk * E + e;
+            idx[i] = (kGather && e < E && ge < total) ? index[ge / R4] : 0;
+        }
+    };
+    float4 pre[PRE];
+    auto load_records = [&](int chunk) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int e = i * kThreads + tid, ge = chunk * E + e;
+            const bool valid = e < E && ge < total;
+            if (kGather)
+                pre[i] = valid ? src[(size_t)idx[i] * R4 + (ge % R4)] : zero;
+            else
+                pre[i] = valid ? src[ge] : zero;
+        }
+    };
+    load_idx(0);
+    load_records(0);
+    load_idx(1);
 #pragma unroll
     for (int i = 0; i < PRE; ++i) {
         const int e = i * kThreads + tid;
@@ -279,13 +488,9 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
     }
     __syncthreads();
     for (int k = 0; k < chunks; ++k) {
-        const int nbase = (k + 1) * E;
         if (k + 1 < chunks) {
-#pragma unroll
-            for (int i = 0; i < PRE; ++i) {
-                const int e = i * kThreads + tid;
-                pre[i] = (e < E && nbase + e < total) ? src[nbase + e] : zero;
-            }
+            load_records(k + 1);
+            load_idx(k + 2);
         }
         const float4* cur = sh + (k & 1) * E;
         // The LDS reads of kStreamUnroll records are issued together and pinned above the work
@@ -366,11 +571,15 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
 #pragma unroll
         for (int c = 0; c < C; ++c) num[p][c] = 0.0f;
     }
+    // this tile's Gaussians (those whose reach box meets it), split S ways by list position
     const int s = blockIdx.y;
-    const int n0 = s * a.n_per_split;
-    const int n1 = min(a.Np, n0 + a.n_per_split);
-    const float4* src = reinterpret_cast<const float4*>(a.packed + ((size_t)b * a.Np + n0) * RS);
-    stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r) {
+    const int count = a.counts[(size_t)b * per_img + tl];
+    const int per = ((count + a.S - 1) / a.S + 3) & ~3;
+    const int n0 = min(count, s * per);
+    const int n1 = min(count, n0 + per);
+    const int* list = a.lists + ((size_t)b * per_img + tl) * a.Np + n0;
+    const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
+    stream_records_lds<R4, kGaussChunk, true>(src, n1 - n0, sh, [&](const float4* r) {
         const GRec<C> g = lds_grec<C>(r);
         const float dx = xv - g.px;
         const float adx = g.A * dx;
@@ -393,7 +602,7 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
 #pragma unroll
             for (int c = 0; c < C; ++c) num[p][c] = fmaf(e[p], g.ac[c], num[p][c]);
         }
-    });
+    }, list);
     if (col < a.W) {
 #pragma unroll
         for (int p = 0; p < P; ++p)
@@ -641,7 +850,10 @@ struct BwdArgs {
     long syb, syh;
     int N, Np, H, W, Wp, HWp;
     int per_tile;  // rows (separable) or pixels (general, multiple of 256) per tile
-    int T;
+    int T;         // tiles per image (separable: tiles_x * row bands)
+    int tiles_x;   // separable: column bands of kBwdTileW columns
+    const int* counts;  // separable: Gaussians listed per tile [B][T]
+    const int* lists;   // separable: list + complement [B][T][Np]
     float* partial;  // [B][T][6+C][N]
     const int* flag;
     int want;
@@ -665,15 +877,15 @@ __device__ __forceinline__ void bwd_store(const BwdArgs& a, int b, int t, const 
     }
 }
 
+// Loads the G Gaussians of this lane; n[g] >= N marks an unused slot (nothing is stored for it).
 template <int C, int G>
-__device__ __forceinline__ void bwd_load_gaussians(const BwdArgs& a, int b, int (&n)[G],
+__device__ __forceinline__ void bwd_load_gaussians(const BwdArgs& a, int b, const int (&n)[G],
                                                    float (&px)[G], float (&py)[G], float (&A)[G],
                                                    float (&B2)[G], float (&D)[G],
                                                    float (&col)[G][C]) {
     constexpr int RS = rec_stride_of(C);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        n[g] = (blockIdx.x * G + g) * kThreads + threadIdx.x;
         const int nc = min(n[g], a.N - 1);
         const float* r = a.packed + ((size_t)b * a.Np + nc) * RS;
         px[g] = r[0];
@@ -689,26 +901,54 @@ __device__ __forceinline__ void bwd_load_gaussians(const BwdArgs& a, int b, int 
 // pixel records per LDS buffer; wide records get a shorter chunk so the two buffers stay small
 __host__ __device__ constexpr int pix_chunk(int C) { return C <= 4 ? IGS_PCHUNK : 128; }
 
-// Separable grid: lane = G Gaussians; the tile is a range of full rows.  Pixel records and
-// column coordinates of 128-pixel row segments stream through LDS (double-buffered) and are
-// read with broadcast ds_read_b128.  Per row the dy part of q is hoisted, and row sums
+// columns of a backward pixel tile on separable grids
+#ifndef IGS_BWD_MAX_ROWS
+#define IGS_BWD_MAX_ROWS 32
+#endif
+constexpr int kBwdMaxRows = IGS_BWD_MAX_ROWS;
+constexpr int kBwdMinRows = 4;
+#ifndef IGS_BWD_TILE_W
+#define IGS_BWD_TILE_W 64
+#endif
+constexpr int kBwdTileW = IGS_BWD_TILE_W;
+
+// Separable grid: lane = G Gaussians taken from the tile's list (those whose reach box meets
+// the tile; the others are known to get exactly zero from it); the tile is kBwdTileW columns x
+// per_tile rows.  Its pixel records stream through LDS in chunks of whole tile rows
+// (double-buffered) and are read with broadcast ds_read_b128; the tile's column coordinates sit
+// in LDS for the whole kernel.  Per row the dy part of q is hoisted, and row sums
 // R0 = sum G e, R1 = sum G e dx, R2 = sum G e dx^2 (and the colour sums) are folded into the
-// totals once per row.
+// totals once per row.  List positions past the count map to the unlisted Gaussians: a lane that
+// gets one computes (and stores) its exact zeros, and a workgroup made of such lanes only stores
+// zeros without computing, so every partial entry is written exactly once per launch.
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     constexpr int CP = pix_stride_sep(C), CP4 = CP / 4;
-    constexpr int PX = pix_chunk(C);
-    constexpr int ER = PX * CP4;   // float4 of pixel records per chunk
-    constexpr int EX = PX / 4;     // float4 of x coordinates per chunk
-    constexpr int E = ER + EX;
+    constexpr int PX = pix_chunk(C) > kBwdTileW ? pix_chunk(C) : kBwdTileW;
+    constexpr int RPC = PX / kBwdTileW;          // tile rows per chunk
+    constexpr int ROW4 = kBwdTileW * CP4;        // float4 per tile row
+    constexpr int E = RPC * ROW4;                // float4 per chunk
     constexpr int PRE = (E + kThreads - 1) / kThreads;
+    static_assert(PX % kBwdTileW == 0 && RPC >= 1, "chunk must hold whole tile rows");
     __shared__ float4 sh[2 * E];
+    __shared__ float4 xsh[kBwdTileW / 4];
+    __shared__ float ysh[2][RPC + 1];  // row coordinates of the chunk (+1: read-ahead slot)
     IGS_GATE(a);
-    const int b = blockIdx.z, t = blockIdx.y;
+    // tiles are the fastest grid dimension: consecutive workgroups (dealt round-robin to the
+    // XCDs) then belong to different tiles, and the list-position groups that have work (the
+    // low ones) are spread over all XCDs
+    const int b = blockIdx.z, t = blockIdx.x, grp = blockIdx.y;
     const int tid = threadIdx.x;
+    const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
+    const int count = a.counts[(size_t)b * a.T + t];
+    const int* list = a.lists + ((size_t)b * a.T + t) * a.Np;
     int n[G];
-    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
-    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int pos = (grp * G + g) * kThreads + tid;
+        const int idx = pos < count ? pos : pos + (a.Np - a.N);
+        n[g] = idx < a.Np ? list[idx] : a.N;
+    }
     float M[G][6], CG[G][C];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -717,37 +957,63 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
 #pragma unroll
         for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
     }
-    const int r0 = t * a.per_tile, r1 = min(a.H, r0 + a.per_tile);
-    const int segs = (a.Wp + PX - 1) / PX;  // segments per row
-    const int chunks = (r1 - r0) * segs;
-    const float4* xsrc = reinterpret_cast<const float4*>(a.xs + (size_t)b * a.Wp);  // Wp % 8 == 0
-    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (grp * G * kThreads >= count) {  // workgroup-uniform: unlisted Gaussians only
+        bwd_store<C, G>(a, b, t, n, M, CG);
+        return;
+    }
+    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
+    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
 
-    // element e of chunk k: e < ER -> pixel-record float4, else x-coordinate float4
+    const int c0 = tx * kBwdTileW;
+    const int cw = min(a.Wp, c0 + kBwdTileW) - c0;  // columns of this tile, a multiple of 8
+    const int r0 = ty * a.per_tile, r1 = min(a.H, r0 + a.per_tile);
+    const int chunks = (r1 - r0 + RPC - 1) / RPC;
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (tid < kBwdTileW / 4)
+        xsh[tid] = 4 * tid < cw ? reinterpret_cast<const float4*>(a.xs + (size_t)b * a.Wp + c0)[tid] : zero;
+
+    // element e of chunk k: float4 (e % ROW4) of tile row (e / ROW4)
     auto fetch = [&](int k, int e) -> float4 {
-        const int r = r0 + k / segs, c0 = (k % segs) * PX;
-        if (e < ER) {
-            const int pxl = c0 + e / CP4;
-            if (pxl >= a.Wp) return zero;
-            const float4* row = reinterpret_cast<const float4*>(a.pixrec + ((size_t)b * a.H + r) * a.Wp * CP);
-            return row[(size_t)c0 * CP4 + e];
-        }
-        const int xi = c0 / 4 + (e - ER);
-        return (e < E && xi * 4 < a.Wp) ? xsrc[xi] : zero;
+        const int rr = e / ROW4, rem = e - rr * ROW4;
+        const int r = r0 + k * RPC + rr;
+        if (r >= r1 || rem >= cw * CP4) return zero;
+        const float4* row = reinterpret_cast<const float4*>(a.pixrec + (((size_t)b * a.H + r) * a.Wp + c0) * CP);
+        return row[rem];
+    };
+    // y of tile row (k * RPC + rr), clamped to the tile (the clamped ones are never used)
+    auto fetch_y = [&](int k, int rr) -> float {
+        return a.y[b * a.syb + (long)min(r0 + k * RPC + rr, r1 - 1) * a.syh];
     };
     float4 pre[PRE];
+    float ypre = 0.0f;
 #pragma unroll
     for (int i = 0; i < PRE; ++i) {
         const int e = i * kThreads + tid;
         if (e < E) sh[e] = fetch(0, e);
     }
+    if (tid <= RPC) ysh[0][tid] = fetch_y(0, min(tid, RPC - 1));
     __syncthreads();
 
-    float dy[G], cyy[G], bdy[G], R0[G], R1[G], R2[G], RC[G][C];
     for (int k = 0; k < chunks; ++k) {
-        const int seg = k % segs;
-        if (seg == 0) {  // a new row starts
-            const float yv = a.y[b * a.syb + (long)(r0 + k / segs) * a.syh];
+        if (k + 1 < chunks) {
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                pre[i] = (e < E) ? fetch(k + 1, e) : zero;
+            }
+            if (tid <= RPC) ypre = fetch_y(k + 1, min(tid, RPC - 1));
+        }
+        const float4* cur = sh + (k & 1) * E;
+        const float* ycur = ysh[k & 1];
+        const int rows = min(RPC, r1 - r0 - k * RPC);
+        float ynext = ycur[0];
+#pragma unroll 1
+        for (int rr = 0; rr < rows; ++rr) {
+            // the row coordinate comes from LDS, read one row ahead: a scalar load here would
+            // drain the LDS/scalar counter once per tile row
+            const float yv = ynext;
+            ynext = ycur[rr + 1];
+            float dy[G], cyy[G], bdy[G], R0[G], R1[G], R2[G], RC[G][C];
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 dy[g] = yv - py[g];
@@ -758,64 +1024,56 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
 #pragma unroll
                 for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
             }
-        }
-        if (k + 1 < chunks) {
-#pragma unroll
-            for (int i = 0; i < PRE; ++i) {
-                const int e = i * kThreads + tid;
-                pre[i] = (e < E) ? fetch(k + 1, e) : zero;
-            }
-        }
-        const float4* cur = sh + (k & 1) * E;
+            const float4* rowrec = cur + rr * ROW4;
 #pragma unroll 1
-        for (int i = 0; i < PX; i += 4) {
-            const float4 xq = cur[ER + (i >> 2)];
-            const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
-            // phase 1: exponents of the 4 x G pairs (independent chains)
-            float dxs[4][G], ee[4][G];
+            for (int i = 0; i < cw; i += 4) {
+                const float4 xq = xsh[i >> 2];
+                const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
+                // phase 1: exponents of the 4 x G pairs (independent chains)
+                float dxs[4][G], ee[4][G];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    const float dx = xs4[j] - px[g];
-                    const float tt = fmaf(A[g], dx, bdy[g]);
-                    ee[j][g] = fmaf(tt, dx, cyy[g]);
-                    dxs[j][g] = dx;
-                }
-            // phase 2: transcendentals back to back
+                    for (int g = 0; g < G; ++g) {
+                        const float dx = xs4[j] - px[g];
+                        const float tt = fmaf(A[g], dx, bdy[g]);
+                        ee[j][g] = fmaf(tt, dx, cyy[g]);
+                        dxs[j][g] = dx;
+                    }
+                // phase 2: transcendentals back to back
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int g = 0; g < G; ++g) ee[j][g] = hw_exp2(ee[j][g]);
-            // phase 3: G = <g^, c> - s and the row sums
+                    for (int g = 0; g < G; ++g) ee[j][g] = hw_exp2(ee[j][g]);
+                // phase 3: G = <g^, c> - s and the row sums
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float pv[CP];
+                for (int j = 0; j < 4; ++j) {
+                    float pv[CP];
 #pragma unroll
-                for (int q4 = 0; q4 < CP4; ++q4) {
-                    const float4 tq = cur[(i + j) * CP4 + q4];
-                    pv[4 * q4] = tq.x;
-                    pv[4 * q4 + 1] = tq.y;
-                    pv[4 * q4 + 2] = tq.z;
-                    pv[4 * q4 + 3] = tq.w;
-                }
+                    for (int q4 = 0; q4 < CP4; ++q4) {
+                        const float4 tq = rowrec[(i + j) * CP4 + q4];
+                        pv[4 * q4] = tq.x;
+                        pv[4 * q4 + 1] = tq.y;
+                        pv[4 * q4 + 2] = tq.z;
+                        pv[4 * q4 + 3] = tq.w;
+                    }
 #pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    const float e = ee[j][g], dx = dxs[j][g];
-                    float Gv = pv[C];  // -s
+                    for (int g = 0; g < G; ++g) {
+                        const float e = ee[j][g], dx = dxs[j][g];
+                        float Gv = pv[C];  // -s
 #pragma unroll
-                    for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[g][c], Gv);
-                    const float ge = Gv * e;
-                    R0[g] += ge;
-                    const float t1 = ge * dx;
-                    R1[g] += t1;
-                    R2[g] = fmaf(t1, dx, R2[g]);
+                        for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[g][c], Gv);
+                        const float ge = Gv * e;
+                        R0[g] += ge;
+                        const float t1 = ge * dx;
+                        R1[g] += t1;
+                        R2[g] = fmaf(t1, dx, R2[g]);
 #pragma unroll
-                    for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[c], RC[g][c]);
+                        for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[c], RC[g][c]);
+                    }
                 }
             }
-        }
-        if (seg == segs - 1) {  // the row is complete
+            // the tile row is complete
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 M[g][0] += R0[g];
@@ -835,6 +1093,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
                 const int e = i * kThreads + tid;
                 if (e < E) nxt[e] = pre[i];
             }
+            if (tid <= RPC) ysh[(k + 1) & 1][tid] = ypre;
         }
         __syncthreads();
     }
@@ -851,6 +1110,8 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
     int n[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) n[g] = (blockIdx.x * G + g) * kThreads + threadIdx.x;
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
     bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
     float M[G][6], CG[G][C], R[G][6], RC[G][C];
@@ -1212,10 +1473,11 @@ FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
     FwdGeometry g;
     const int kFwdSepP = fwd_sep_p(C);
     if (sep) {
-        // choose the wave arrangement (wx waves along the columns) that wastes the fewest lanes
+        // choose the wave arrangement (wx waves along the columns) that wastes the fewest lanes;
+        // on a tie the squarest tile (fewest Gaussians reach it)
         long best = -1;
-        g.wx = 4;
-        for (int wx = 4; wx >= 1; wx >>= 1) {
+        g.wx = 1;
+        for (int wx = 1; wx <= 4; wx <<= 1) {
             const long cols = (long)ceil_div(W, 64 * wx) * 64 * wx;
             const long rows = (long)ceil_div(H, kFwdSepP * (4 / wx)) * kFwdSepP * (4 / wx);
             const long area = cols * rows;
@@ -1234,6 +1496,12 @@ FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
     g.total_tiles = B * g.tiles_x * g.tiles_y;
     return g;
 }
+
+// Tile lists of one launch: counts [B][tiles] (padded to 4 ints) then lists [B][tiles][Np].
+inline size_t bins_bytes(int B, int tiles, int Np) {
+    return ((((size_t)B * tiles + 3) & ~(size_t)3) + (size_t)B * tiles * Np) * sizeof(int);
+}
+inline size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
 
 // Plan of one kernel variant (grid_mode is GENERAL or SEPARABLE here).
 int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
@@ -1263,7 +1531,16 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     p->fwd_n_per_split = nps;
     const long groups = (long)B * ceil_div(N, kThreads * (sep ? kBwdG : bwd_gen_g(C))) * 4;  // waves per tile
     long T = ((long)cus * 4 * IGS_BWD_WAVES + groups - 1) / groups;     // backward: waves per SIMD wanted
-    const long maxT = sep ? H : ceil_div(p->hw_padded, 256);
+    p->bwd_tiles_x = sep ? ceil_div(p->w_padded, kBwdTileW) : 1;
+    if (sep) {
+        T = (T + p->bwd_tiles_x - 1) / p->bwd_tiles_x;                  // row bands
+        // small tiles keep the tile lists short when the Gaussians are small (a tile is skipped
+        // by every Gaussian whose reach box misses it): at most kBwdMaxRows rows per tile
+        const long bands = ceil_div(H, kBwdMaxRows);
+        if (T < bands) T = bands;
+    }
+    // (tiles of fewer than kBwdMinRows rows cost more in partial sums than they gain in fill)
+    const long maxT = sep ? ceil_div(H, kBwdMinRows) : ceil_div(p->hw_padded, 256);
     if (T > maxT) T = maxT;
     if (T < 1) T = 1;
     if (sep) {
@@ -1271,15 +1548,38 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     } else {
         p->bwd_per_tile = (ceil_div(p->hw_padded, T) + 255) & ~255;
     }
-    T = ceil_div(sep ? H : p->hw_padded, p->bwd_per_tile);
+    T = (long)ceil_div(sep ? H : p->hw_padded, p->bwd_per_tile) * p->bwd_tiles_x;
     p->bwd_tiles = (int)T;
+    p->fwd_tiles = sep ? fg.tiles_x * fg.tiles_y : 0;
     p->pix_stride = sep ? pix_stride_sep(C) : pix_stride_gen(C);
-    p->packed_bytes = (uint64_t)B * p->n_padded * p->rec_stride * sizeof(float);
+    // records, then one reach box (4 floats) per record
+    p->packed_bytes = (uint64_t)B * p->n_padded * (p->rec_stride + 4) * sizeof(float);
     p->fwd_ws_bytes = S > 1 ? (uint64_t)S * B * (C + 1) * H * W * sizeof(float) : 0;
     p->pix_bytes = sep ? ((uint64_t)B * H * p->w_padded * p->pix_stride + (uint64_t)B * p->w_padded) * sizeof(float)
                        : (uint64_t)B * p->hw_padded * p->pix_stride * sizeof(float);
+    if (sep) {  // the tile lists of each launch follow its other scratch
+        p->fwd_ws_bytes = align16(p->fwd_ws_bytes) + bins_bytes(B, p->fwd_tiles, p->n_padded);
+        p->pix_bytes = align16(p->pix_bytes) + bins_bytes(B, p->bwd_tiles, p->n_padded);
+    }
     p->partial_bytes = (uint64_t)B * T * (6 + C) * N * sizeof(float);
     return IGS_OK;
+}
+
+// Where the tile lists of a separable launch live inside its workspace.
+struct BinPlace {
+    int* counts;
+    int* lists;
+};
+inline BinPlace bins_at(void* ws, size_t scratch_bytes, int B, int tiles) {
+    char* base = static_cast<char*>(ws) + align16(scratch_bytes);
+    BinPlace bp;
+    bp.counts = reinterpret_cast<int*>(base);
+    bp.lists = bp.counts + (((size_t)B * tiles + 3) & ~(size_t)3);
+    return bp;
+}
+
+inline const float4* boxes_of(const float* packed, int B, int Np, int RS) {
+    return reinterpret_cast<const float4*>(packed + (size_t)B * Np * RS);
 }
 
 // Public plan: AUTO reports the separable variant's geometry with the workspace sizes of
@@ -1295,6 +1595,12 @@ int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t*
     if (g.pix_bytes > p->pix_bytes) p->pix_bytes = g.pix_bytes;
     if (g.partial_bytes > p->partial_bytes) p->partial_bytes = g.partial_bytes;
     return IGS_OK;
+}
+
+int launch_bin(const BinArgs& a, int B, hipStream_t st) {
+    hipLaunchKernelGGL(k_bin, dim3(a.tiles_x * a.tiles_y, B), dim3(kBinThreads), 0, st, a);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? IGS_OK : (int)e;
 }
 
 inline int launch_status() {
@@ -1380,7 +1686,8 @@ int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, con
 template <int C>
 int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     if (sep) {
-        const dim3 grid(ceil_div(a.N, kThreads * kBwdG), a.T, B);
+        // every list position up to Np is visited: listed Gaussians compute, the others store zeros
+        const dim3 grid(a.T, ceil_div(a.Np, kThreads * kBwdG), B);
         hipLaunchKernelGGL((k_bwd_sep<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
     } else {
         const dim3 grid(ceil_div(a.N, kThreads * bwd_gen_g(C)), a.T, B);
@@ -1401,7 +1708,14 @@ int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* col
     a.syb = gs[3]; a.syh = gs[4];
     a.N = N; a.Np = plan.n_padded; a.H = H; a.W = W; a.Wp = plan.w_padded; a.HWp = plan.hw_padded;
     a.T = plan.bwd_tiles;
+    a.tiles_x = plan.bwd_tiles_x;
     a.per_tile = plan.bwd_per_tile;
+    a.counts = nullptr; a.lists = nullptr;
+    if (sep && pix_ws) {
+        const size_t scratch = ((size_t)B * H * plan.w_padded * plan.pix_stride + (size_t)B * plan.w_padded) * sizeof(float);
+        const BinPlace bp = bins_at(pix_ws, scratch, B, plan.bwd_tiles);
+        a.counts = bp.counts; a.lists = bp.lists;
+    }
     a.partial = partial;
     a.flag = v.flag; a.want = v.want;
     return IGS_OK;
@@ -1464,7 +1778,8 @@ int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const f
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
-                       colors, N, Np, C, rec_stride_of(C), 0.0f, packed);
+                       colors, N, Np, C, rec_stride_of(C), 0.0f, packed,
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
@@ -1478,7 +1793,8 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
-                       alphas, colors, N, Np, C, rec_stride_of(C), eps, packed);
+                       alphas, colors, N, Np, C, rec_stride_of(C), eps, packed,
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
@@ -1494,6 +1810,7 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
     rc = make_plan(B, N, H, W, C, grid_mode, &total);
     if (rc) return rc;
     if (total.fwd_ws_bytes > 0 && (!ws || ws_bytes < total.fwd_ws_bytes)) return IGS_ERR_WORKSPACE;
+    if (((uintptr_t)packed | (uintptr_t)ws) & 15) return IGS_ERR_BAD_SHAPE;  // float4 / int lists inside
     hipStream_t st = (hipStream_t)stream;
     Variant vs[2];
     const int nv = variants_of(grid_mode, grid_flag, vs);
@@ -1512,7 +1829,24 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
         a.n_per_split = plan.fwd_n_per_split;
         a.tiles_x = fg.tiles_x; a.tiles_y = fg.tiles_y; a.total_tiles = fg.total_tiles; a.wx = fg.wx;
         a.eps = eps; a.out = out; a.den = den; a.part = (float*)ws;
+        a.counts = nullptr; a.lists = nullptr;
         a.flag = vs[i].flag; a.want = vs[i].want;
+        if (sep) {
+            const size_t split_bytes = a.S > 1 ? (size_t)a.S * B * (C + 1) * H * W * sizeof(float) : 0;
+            const BinPlace bp = bins_at(ws, split_bytes, B, plan.fwd_tiles);
+            BinArgs ba;
+            ba.boxes = boxes_of(packed, B, plan.n_padded, plan.rec_stride);
+            ba.x = x; ba.y = y;
+            ba.sxb = a.sxb; ba.sxw = a.sxw; ba.syb = a.syb; ba.syh = a.syh;
+            ba.N = N; ba.Np = plan.n_padded; ba.H = H; ba.W = W;
+            ba.tile_w = 64 * fg.wx; ba.tile_h = fwd_sep_p(C) * (4 / fg.wx);
+            ba.tiles_x = fg.tiles_x; ba.tiles_y = fg.tiles_y;
+            ba.counts = bp.counts; ba.lists = bp.lists; ba.complement = 0;
+            ba.flag = vs[i].flag; ba.want = vs[i].want;
+            rc = launch_bin(ba, B, st);
+            if (rc) return rc;
+            a.counts = bp.counts; a.lists = bp.lists;
+        }
         IGS_DISPATCH_C(C, rc = launch_forward<kC>(a, sep, st));
         if (rc) return rc;
         if (a.S > 1) {
@@ -1630,6 +1964,19 @@ int igs_gs2d_backward_reduce(const float* packed, const float* colors, const flo
                       const_cast<float*>(pix_ws), partial);
         if (rc) return rc;
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
+        if (sep) {
+            BinArgs ba;
+            ba.boxes = boxes_of(packed, B, a.Np, rec_stride_of(C));
+            ba.x = a.xs; ba.y = y;               // the prologue's compact column coordinates
+            ba.sxb = a.Wp; ba.sxw = 1; ba.syb = a.syb; ba.syh = a.syh;
+            ba.N = N; ba.Np = a.Np; ba.H = H; ba.W = W;
+            ba.tile_w = kBwdTileW; ba.tile_h = a.per_tile;
+            ba.tiles_x = a.tiles_x; ba.tiles_y = a.T / a.tiles_x;
+            ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists); ba.complement = 1;
+            ba.flag = a.flag; ba.want = a.want;
+            rc = launch_bin(ba, B, st);
+            if (rc) return rc;
+        }
         IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, st));
         if (rc) return rc;
     }
@@ -1736,7 +2083,8 @@ int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int 
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
-                       rec_stride_of(C_kernel), eps, packed, colors_out);
+                       rec_stride_of(C_kernel), eps, packed,
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
     return launch_status();
 }
 

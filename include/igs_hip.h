@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define IGS_ABI_VERSION 1
+#define IGS_ABI_VERSION 2
 #define IGS_MAX_CHANNELS 16
 
 typedef void *igs_stream_t; /* a hipStream_t */
@@ -72,13 +72,18 @@ typedef struct igs_gs2d_plan_t {
     int32_t hw_padded;       /* general: pixel records per image (H*W rounded up to 4)     */
     int32_t fwd_split;       /* number of Gaussian-range splits of the forward (>= 1)      */
     int32_t fwd_n_per_split; /* records per split (multiple of 4)                          */
-    int32_t bwd_tiles;       /* number of pixel tiles T of the backward partial buffer     */
+    int32_t bwd_tiles;       /* pixel tiles T per image of the backward partial buffer     */
     int32_t bwd_per_tile;    /* rows (separable) or pixels (general) per backward tile     */
     int32_t pix_stride;      /* floats per pixel record of the backward prologue           */
-    uint64_t packed_bytes;   /* packed Gaussian buffer: B*n_padded*rec_stride*4            */
-    uint64_t fwd_ws_bytes;   /* forward split workspace (0 when fwd_split == 1)            */
-    uint64_t pix_bytes;      /* backward per-pixel buffer                                  */
+    uint64_t packed_bytes;   /* packed Gaussian buffer: records, then one reach box (4
+                                floats) per record: B*n_padded*(rec_stride+4)*4            */
+    uint64_t fwd_ws_bytes;   /* forward scratch: split partials (fwd_split > 1) and, on
+                                separable grids, the per-tile Gaussian lists                */
+    uint64_t pix_bytes;      /* backward scratch: per-pixel records and, on separable
+                                grids, the per-tile Gaussian lists                          */
     uint64_t partial_bytes;  /* backward partial sums: B*T*(6+C)*N*4                       */
+    int32_t fwd_tiles;       /* separable: pixel tiles per image of the forward            */
+    int32_t bwd_tiles_x;     /* separable: column bands (64 columns) of the backward tiles */
 } igs_gs2d_plan_t;
 
 int igs_abi_version(void);

@@ -69,11 +69,15 @@ def test_plan_arithmetic(lib, mode):
         assert p.n_padded % 4 == 0 and p.n_padded >= N
         assert p.fwd_n_per_split % 4 == 0 and p.fwd_split * p.fwd_n_per_split >= p.n_padded
         assert (p.fwd_split - 1) * p.fwd_n_per_split < p.n_padded          # no empty split
-        assert p.packed_bytes == B * p.n_padded * p.rec_stride * 4
+        assert p.packed_bytes == B * p.n_padded * (p.rec_stride + 4) * 4    # records + reach boxes
         assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
         assert p.bwd_tiles >= 1 and p.partial_bytes >= B * p.bwd_tiles * (6 + C) * N * 4
         if mode != 0:
-            assert p.w_padded % 8 == 0 and p.bwd_tiles * p.bwd_per_tile >= H
+            assert p.w_padded % 8 == 0 and p.bwd_tiles % p.bwd_tiles_x == 0
+            assert (p.bwd_tiles // p.bwd_tiles_x) * p.bwd_per_tile >= H and p.bwd_tiles_x * 64 >= W
+            # room for the per-tile Gaussian lists behind the other scratch
+            assert p.fwd_tiles >= 1 and p.fwd_ws_bytes >= B * p.fwd_tiles * (p.n_padded + 1) * 4
+            assert p.pix_bytes >= B * H * W * (C + 1) * 4 + B * p.bwd_tiles * (p.n_padded + 1) * 4
         assert p.pix_bytes >= B * H * W * (C + 1) * 4
     a, s_, g = (_lib.plan(8, 4096, 256, 256, 3, m) for m in (2, 1, 0))
     assert a.pix_bytes == max(s_.pix_bytes, g.pix_bytes) and a.fwd_ws_bytes == max(s_.fwd_ws_bytes, g.fwd_ws_bytes)
