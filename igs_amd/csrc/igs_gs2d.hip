@@ -32,6 +32,7 @@
 #include <hip/hip_runtime.h>
 
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "igs_hip.h"
 
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
                                                    const float* __restrict__ colors, int N,
                                                    int Np, int C, int RS, float eps,
                                                    float* __restrict__ packed,
-                                                   float4* __restrict__ boxes) {
+                                                   float4* __restrict__ boxes, int cull) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n >= Np) return;
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
     }
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
-    boxes[(size_t)b * Np + n] = reach_box(px, py, sxx, syy, bounded && fin);
+    boxes[(size_t)b * Np + n] = reach_box(px, py, sxx, syy, cull && bounded && fin);
 }
 
 // Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
                                                            int Np, int C, int Cp, int RS, float eps,
                                                            float* __restrict__ packed,
                                                            float4* __restrict__ boxes,
-                                                           float* __restrict__ colors_out) {
+                                                           float* __restrict__ colors_out, int cull) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n >= Np) return;
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
     }
     for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
     boxes[(size_t)b * Np + n] = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
-                                          fin && v0 > 0.0 && v1 > 0.0);
+                                          cull && fin && v0 > 0.0 && v1 > 0.0);
 }
 
 // ----------------------------------------------------------------------------- binning
@@ -1582,6 +1583,13 @@ inline const float4* boxes_of(const float* packed, int B, int Np, int RS) {
     return reinterpret_cast<const float4*>(packed + (size_t)B * Np * RS);
 }
 
+// IGS_NO_CULL=1 in the environment makes every reach box unbounded (nothing is skipped): the
+// reference point for checking that culling changes no bit.  Read at every pack call.
+inline int culling_enabled() {
+    const char* e = getenv("IGS_NO_CULL");
+    return !(e && e[0] == '1');
+}
+
 // Public plan: AUTO reports the separable variant's geometry with the workspace sizes of
 // whichever variant needs more.
 int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
@@ -1779,7 +1787,7 @@ int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const f
     hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
                        colors, N, Np, C, rec_stride_of(C), 0.0f, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))), culling_enabled());
     return launch_status();
 }
 
@@ -1794,7 +1802,7 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
     hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
                        alphas, colors, N, Np, C, rec_stride_of(C), eps, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))), culling_enabled());
     return launch_status();
 }
 
@@ -2084,7 +2092,8 @@ int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int 
     hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
                        rec_stride_of(C_kernel), eps, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out,
+                       culling_enabled());
     return launch_status();
 }
 

@@ -1,0 +1,167 @@
+"""Culling on separable grids: a Gaussian is skipped for a pixel tile when its reach box (the
+bounding box of q <= 221.8, beyond which exp2 of the kernels' exponent is exactly 0) misses the
+tile.  The claim under test is that this changes no bit of any result: with IGS_NO_CULL=1 the
+library makes every box unbounded, and both runs must agree exactly; beside that, sparse scenes
+against the fp64 oracle, non-finite parameters, and grids whose coordinates are not monotone."""
+import os
+
+import pytest
+import torch
+
+from oracle import gs2d_oracle as O
+
+pytestmark = pytest.mark.gpu
+NAMES = ("positions", "colors", "scales", "rotations", "alphas")
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def igs():
+    import igs_amd
+
+    return igs_amd
+
+
+def sparse_case(dev, B, N, H, W, C, seed, smin=0.004, smax=0.04, dtype=torch.float32):
+    d = O.make_inputs(B, N, H, W, C, smin, smax, seed=seed, dtype=torch.float64, expand_grids=True)
+    g = {k: v.to(dev, dtype) for k, v in d.items()}
+    g["x_grid"] = g["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+    g["y_grid"] = g["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+    return d, g
+
+
+def run(igs, g, x=None, y=None):
+    leaves = {k: g[k].clone().requires_grad_(True) for k in NAMES}
+    out = igs.gaussian_splatting_2d(*(leaves[k] for k in NAMES), g["x_grid"] if x is None else x,
+                                    g["y_grid"] if y is None else y)
+    out.backward(g["grad_out"])
+    return out.detach(), {k: v.grad for k, v in leaves.items()}
+
+
+@pytest.fixture
+def no_cull():
+    """Context that disables culling in the library (read at every pack call)."""
+    class Ctx:
+        def __enter__(self):
+            os.environ["IGS_NO_CULL"] = "1"
+
+        def __exit__(self, *a):
+            os.environ.pop("IGS_NO_CULL", None)
+
+    return Ctx()
+
+
+@pytest.mark.parametrize("shape", [(2, 120, 70, 150, 3), (1, 100, 200, 64, 16), (3, 64, 33, 257, 1)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_culled_equals_unculled_bit_for_bit(igs, dev, no_cull, shape):
+    """N < 128 keeps the forward in one Gaussian split, so that both runs add the same terms in
+    the same order and the skipped ones are exact zeros."""
+    B, N, H, W, C = shape
+    _, g = sparse_case(dev, B, N, H, W, C, seed=sum(shape))
+    out, grads = run(igs, g)
+    with no_cull:
+        out0, grads0 = run(igs, g)
+    assert float(out.abs().max()) > 0
+    assert torch.equal(out, out0)
+    for k in NAMES:
+        assert torch.equal(grads[k], grads0[k]), k
+
+
+def test_sparse_scene_against_oracle(igs, dev):
+    """Small Gaussians (sigma of 1-10 pixels) on a 96x160 image, several tiles in both directions,
+    more than one forward split: forward and every gradient against the fp64 oracle."""
+    B, N, H, W, C = 2, 700, 96, 160, 3
+    d, g = sparse_case(dev, B, N, H, W, C, seed=31, smin=0.01, smax=0.1)
+    ref_out, ref_g = O.render_autograd(d["positions"], d["colors"], d["scales"], d["rotations"], d["alphas"],
+                                       d["x_grid"], d["y_grid"], d["grad_out"])
+    out, grads = run(igs, g)
+    err = (out.double() - ref_out.to(dev)).abs()
+    assert bool((err <= 1e-6 + 1e-5 * ref_out.to(dev).abs()).all()), float(err.max())
+    for k in NAMES:
+        r = ref_g[k].to(dev)
+        dlt = grads[k].double() - r
+        assert float(dlt.abs().max()) <= 1e-4 * float(r.abs().max()), k
+        assert float(dlt.norm()) <= 1e-4 * float(r.norm()), k
+
+
+def test_non_monotone_separable_grid(igs, dev, no_cull):
+    """A separable grid need not be sorted: tiles take [min, max] of their coordinates.  Permuting
+    the columns and rows of the grid permutes the image, and culling still changes no bit."""
+    B, N, H, W, C = 1, 90, 80, 140, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=8)
+    gen = torch.Generator().manual_seed(3)
+    pc, pr = torch.randperm(W, generator=gen).to(dev), torch.randperm(H, generator=gen).to(dev)
+    xs = g["x_grid"][0, 0, 0, :][pc].contiguous()
+    ys = g["y_grid"][0, 0, :, 0][pr].contiguous()
+    xg = xs.view(1, 1, 1, W).expand(B, 1, H, W)
+    yg = ys.view(1, 1, H, 1).expand(B, 1, H, W)
+    g2 = dict(g)
+    g2["grad_out"] = g["grad_out"][:, :, pr][:, :, :, pc].contiguous()
+    out, grads = run(igs, g2, xg, yg)
+    with no_cull:
+        out0, grads0 = run(igs, g2, xg, yg)
+    assert torch.equal(out, out0)
+    for k in NAMES:
+        assert torch.equal(grads[k], grads0[k]), k
+    base, base_g = run(igs, g)
+    torch.testing.assert_close(out, base[:, :, pr][:, :, :, pc], rtol=1e-5, atol=1e-6)
+    for k in NAMES:   # the same sums in another pixel order
+        torch.testing.assert_close(grads[k], base_g[k], rtol=2e-4, atol=1e-6 * float(base_g[k].abs().max()))
+
+
+def test_non_finite_parameters_propagate_as_without_culling(igs, dev, no_cull):
+    """A Gaussian with a NaN position or rotation or an infinite alpha poisons every pixel in the
+    plain torch expression (NaN - x, 0 * inf), an infinite colour every pixel of its channel that
+    the Gaussian's weight reaches or underflows at; the reach box of such a record is unbounded,
+    so the fused result has its NaN/inf exactly where the run without culling has them."""
+    B, N, H, W, C = 1, 40, 70, 130, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=12)
+    for field, index, value, all_nan in (("positions", (0, 3, 0), float("nan"), True),
+                                         ("alphas", (0, 5), float("inf"), True),
+                                         ("colors", (0, 7, 1), float("inf"), False),
+                                         ("rotations", (0, 9), float("nan"), True)):
+        h = {k: v.clone() for k, v in g.items()}
+        h[field][index] = value
+        with torch.no_grad():
+            got = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"])
+            with no_cull:
+                ref = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"])
+            want = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"], fused=False)
+        assert torch.equal(torch.isnan(got), torch.isnan(ref)), field
+        assert torch.equal(torch.nan_to_num(got, nan=7.0), torch.nan_to_num(ref, nan=7.0)), field
+        if all_nan:
+            assert bool(torch.isnan(want).all()) and bool(torch.isnan(got).all()), field
+        else:   # the other channels are untouched
+            torch.testing.assert_close(got[:, [0, 2]], want[:, [0, 2]], rtol=1e-4, atol=1e-5)
+            assert not bool(torch.isfinite(got[:, 1]).any())
+
+
+def test_operator_level_with_indefinite_cov_inverse(igs, dev, no_cull):
+    """cov_inv entries that are not positive definite (the operator accepts anything) grow instead
+    of decaying: such a Gaussian is never culled."""
+    B, N, H, W = 1, 30, 66, 130
+    _, g = sparse_case(dev, B, N, H, W, 3, seed=4)
+    with torch.no_grad():
+        a, b, d = O.cov_inverse_closed(g["scales"].double(), g["rotations"].double())
+    a, b, d = (t.float().reshape(B, N, 1, 1).contiguous() for t in (a, b, d))
+    a[0, 2] = -1e-3          # saddle: exp(+...) along x
+    d[0, 4] = 0.0            # degenerate: constant along y
+    K = igs.GaussianSplatting2DKernel
+    args = (g["x_grid"], g["y_grid"], g["positions"], a, b, d, g["alphas"], g["colors"])
+    with torch.no_grad():
+        out = K.apply(*args)
+        with no_cull:
+            out0 = K.apply(*args)
+        want = igs.naive_gaussian_2d(g["x_grid"], g["y_grid"], g["positions"], a, b, d, g["alphas"], g["colors"])
+    # the saddle overflows where it grows (inf / inf): same places, same values elsewhere
+    assert torch.equal(torch.isnan(out), torch.isnan(out0))
+    assert torch.equal(torch.nan_to_num(out, nan=7.0), torch.nan_to_num(out0, nan=7.0))
+    ok = torch.isfinite(want) & torch.isfinite(out)
+    assert float(ok.float().mean()) > 0.3
+    torch.testing.assert_close(out[ok], want[ok], rtol=1e-4, atol=1e-5)
