@@ -1752,6 +1752,7 @@ const char* igs_status_string(int status) {
         case IGS_ERR_WORKSPACE: return "workspace smaller than igs_gs2d_plan requires";
         case IGS_ERR_BAD_MODE: return "unknown grid mode";
         case IGS_ERR_NO_DEVICE: return "no usable HIP device";
+        case IGS_ERR_ALIGNMENT: return "buffer not 16-byte aligned";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -1818,7 +1819,7 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
     rc = make_plan(B, N, H, W, C, grid_mode, &total);
     if (rc) return rc;
     if (total.fwd_ws_bytes > 0 && (!ws || ws_bytes < total.fwd_ws_bytes)) return IGS_ERR_WORKSPACE;
-    if (((uintptr_t)packed | (uintptr_t)ws) & 15) return IGS_ERR_BAD_SHAPE;  // float4 / int lists inside
+    if (((uintptr_t)packed | (uintptr_t)ws) & 15) return IGS_ERR_ALIGNMENT;  // float4 / int lists inside
     hipStream_t st = (hipStream_t)stream;
     Variant vs[2];
     const int nv = variants_of(grid_mode, grid_flag, vs);
@@ -1953,7 +1954,7 @@ int igs_adamw_step(float* param, const float* grad, float* exp_avg, float* exp_a
 
 int igs_gs2d_backward_reduce(const float* packed, const float* colors, const float* y,
                              const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
-                             int B, int N, int H, int W, int C, const float* pix_ws, size_t pix_bytes,
+                             int B, int N, int H, int W, int C, float* pix_ws, size_t pix_bytes,
                              float* partial, size_t partial_bytes, igs_stream_t stream) {
     if (!packed || !colors || !y || !grid_strides || !pix_ws || !partial) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
@@ -1963,13 +1964,13 @@ int igs_gs2d_backward_reduce(const float* packed, const float* colors, const flo
     rc = make_plan(B, N, H, W, C, grid_mode, &total);
     if (rc) return rc;
     if (pix_bytes < total.pix_bytes || partial_bytes < total.partial_bytes) return IGS_ERR_WORKSPACE;
+    if (((uintptr_t)packed | (uintptr_t)pix_ws) & 15) return IGS_ERR_ALIGNMENT;  // float4 / int lists inside
     hipStream_t st = (hipStream_t)stream;
     Variant vs[2];
     const int nv = variants_of(grid_mode, grid_flag, vs);
     for (int i = 0; i < nv; ++i) {
         BwdArgs a;
-        rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C,
-                      const_cast<float*>(pix_ws), partial);
+        rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C, pix_ws, partial);
         if (rc) return rc;
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
         if (sep) {

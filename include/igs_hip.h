@@ -36,7 +36,8 @@ typedef enum igs_status {
     IGS_ERR_BAD_CHANNELS = -3,   /* C outside 1..IGS_MAX_CHANNELS */
     IGS_ERR_WORKSPACE = -4,      /* a workspace is smaller than igs_gs2d_plan says */
     IGS_ERR_BAD_MODE = -5,       /* unknown grid mode */
-    IGS_ERR_NO_DEVICE = -6       /* no usable HIP device */
+    IGS_ERR_NO_DEVICE = -6,      /* no usable HIP device */
+    IGS_ERR_ALIGNMENT = -7       /* a buffer that must be 16-byte aligned is not */
 } igs_status;
 
 /* How the pixel coordinates are described.
@@ -101,8 +102,15 @@ int igs_gs2d_grid_classify(const float *x, const float *y, const int64_t grid_st
 
 /* Pack per-Gaussian parameters for the kernels (operator level: the caller already has
  * the inverse covariance).  position [B,N,2]; cov_inv_00/01/11 [B,N]; alphas [B,N];
- * colors [B,N,C]; packed: plan.packed_bytes.  Replaces nothing in the reference (its
- * kernels read the tensors directly); it exists so the hot loops read one record. */
+ * colors [B,N,C]; packed: plan.packed_bytes, 16-byte aligned.  Replaces nothing in the
+ * reference (its kernels read the tensors directly); it exists so the hot loops read one
+ * record.  Behind the records the buffer holds one "reach box" per Gaussian: the bounding box
+ * of the ellipse outside of which the kernels' exp2 returns exactly 0 for it.  On separable
+ * grids the forward and the backward skip, per pixel tile, the Gaussians whose box misses the
+ * tile; since only exact zeros are skipped, results are bit-identical to not skipping (the
+ * reference evaluates every pair: src/igs/gs_triton_chunked.py:100-200).  Records with a
+ * non-finite field or a cov_inv that is not positive definite are never skipped.  Setting
+ * IGS_NO_CULL=1 in the environment (read at each pack call) makes every box unbounded. */
 int igs_gs2d_pack_covinv(const float *position, const float *cov_inv_00, const float *cov_inv_01,
                          const float *cov_inv_11, const float *alphas, const float *colors,
                          int B, int N, int C, float *packed, igs_stream_t stream);
@@ -115,8 +123,8 @@ int igs_gs2d_pack_scale_rot(const float *positions, const float *scales, const f
 
 /* Forward: out [B,C,H,W] = sum_n w_n c_n / (sum_n w_n + eps), den [B,H,W] = sum_n w_n.
  * Replaces the forward of src/igs/gs2d.py:68-144 / src/igs/gs_triton_chunked.py:551-680.
- * grid_strides = {sxb, sxh, sxw, syb, syh, syw}.  ws: plan.fwd_ws_bytes (may be NULL when
- * that is 0). */
+ * grid_strides = {sxb, sxh, sxw, syb, syh, syw}.  ws: scratch of plan.fwd_ws_bytes, 16-byte
+ * aligned (may be NULL when that is 0); its contents mean nothing after the call. */
 int igs_gs2d_forward(const float *packed, const float *x, const float *y,
                      const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag, int B,
                      int N, int H, int W, int C, float eps, float *out, float *den, void *ws,
@@ -134,10 +142,12 @@ int igs_gs2d_backward_prologue(const float *x, const float *y, const int64_t gri
 
 /* Backward, stage 2: the recomputing per-Gaussian reduction over pixel tiles into
  * partial [B,T,6+C,N] (plan.partial_bytes).  Replaces the Gaussian loop of the reference
- * backward, src/igs/gs2d.py:180-246 / src/igs/gs_triton.py:159-405.  colors [B,N,C]. */
+ * backward, src/igs/gs2d.py:180-246 / src/igs/gs_triton.py:159-405.  colors [B,N,C].
+ * pix_ws is the buffer stage 1 filled (16-byte aligned); on separable grids this stage also
+ * writes its per-tile Gaussian lists behind the pixel records in it. */
 int igs_gs2d_backward_reduce(const float *packed, const float *colors, const float *y,
                              const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag,
-                             int B, int N, int H, int W, int C, const float *pix_ws,
+                             int B, int N, int H, int W, int C, float *pix_ws,
                              size_t pix_bytes, float *partial, size_t partial_bytes,
                              igs_stream_t stream);
 
