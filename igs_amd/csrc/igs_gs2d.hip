@@ -233,9 +233,8 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
 // of indices in increasing order (so that sums over a list keep the order of the unculled
 // sum), and the count.  One workgroup per (tile, image) scans all N boxes; positions come
 // from ballots and a fixed-order prefix over the four waves, so the lists are reproducible.
-// With `complement`, the Gaussians that do not meet the tile are written to the back of the
-// same list array (list[Np-1], list[Np-2], ...): every n < N then appears exactly once,
-// listed ones in [0, count), the others in [count + Np - N, Np).
+// With `slots` set, the inverse map is written as well: slots[b][tile][n] = position of
+// Gaussian n in the tile's list, or -1 when it is not listed (every n < N is written).
 // Separable grids only: a tile is tile_w columns x tile_h rows and its coordinate range is
 // [min, max] of x over its columns and of y over its rows (no monotonicity assumed).
 struct BinArgs {
@@ -247,7 +246,7 @@ struct BinArgs {
     int tile_w, tile_h, tiles_x, tiles_y;
     int* counts;  // [B][tiles]
     int* lists;   // [B][tiles][Np]
-    int complement;
+    int* slots;   // [B][tiles][Np] or nullptr
     const int* flag;
     int want;
 };
@@ -257,7 +256,7 @@ constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads i
 __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     if (a.flag != nullptr && *a.flag != a.want) return;
     __shared__ float red[4][kBinThreads];
-    __shared__ int wsum[2][kBinWaves];
+    __shared__ int wsum[kBinWaves];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tiles = a.tiles_x * a.tiles_y;
     const int t = blockIdx.x, b = blockIdx.y;
@@ -297,6 +296,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     }
     const float txlo = red[0][0], txhi = -red[1][0], tylo = red[2][0], tyhi = -red[3][0];
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np;
+    int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     const float4* boxes = a.boxes + (size_t)b * a.Np;
     // Each wave scans one contiguous share of the Gaussians twice, without barriers: first to
     // count, then (with the shares' counts prefixed in wave order) to write.
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     const unsigned long long below = (1ull << lane) - 1ull;
     // kU boxes per lane are loaded together, so that kU loads are in flight instead of one
     constexpr int kU = 8;
-    auto classify = [&](int n0, bool (&listed)[kU], bool (&unlisted)[kU]) {
+    auto classify = [&](int n0, bool (&listed)[kU], bool (&in)[kU]) {
         float4 bb[kU];
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
@@ -314,47 +314,37 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
-            const bool in = n0 + u * 64 + lane < ne;
+            in[u] = n0 + u * 64 + lane < ne;
             // "definitely outside" negated, so that NaN bounds count as inside
-            listed[u] = in && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
-            unlisted[u] = in && !listed[u];
+            listed[u] = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
         }
     };
-    int cnt = 0, ucnt = 0;
+    int cnt = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
-        bool listed[kU], unlisted[kU];
-        classify(n0, listed, unlisted);
+        bool listed[kU], in[kU];
+        classify(n0, listed, in);
 #pragma unroll
-        for (int u = 0; u < kU; ++u) {
-            cnt += __popcll(__ballot(listed[u]));
-            ucnt += __popcll(__ballot(unlisted[u]));
-        }
+        for (int u = 0; u < kU; ++u) cnt += __popcll(__ballot(listed[u]));
     }
-    if (lane == 0) {
-        wsum[0][wave] = cnt;
-        wsum[1][wave] = ucnt;
-    }
+    if (lane == 0) wsum[wave] = cnt;
     __syncthreads();
-    int base = 0, ubase = 0, total = 0;
+    int base = 0, total = 0;
 #pragma unroll
     for (int w = 0; w < kBinWaves; ++w) {
-        if (w < wave) {
-            base += wsum[0][w];
-            ubase += wsum[1][w];
-        }
-        total += wsum[0][w];
+        if (w < wave) base += wsum[w];
+        total += wsum[w];
     }
     for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
-        bool listed[kU], unlisted[kU];
-        classify(n0, listed, unlisted);
+        bool listed[kU], in[kU];
+        classify(n0, listed, in);
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             const int n = n0 + u * 64 + lane;
-            const unsigned long long m = __ballot(listed[u]), um = __ballot(unlisted[u]);
-            if (listed[u]) list[base + __popcll(m & below)] = n;
-            if (a.complement && unlisted[u]) list[a.Np - 1 - (ubase + __popcll(um & below))] = n;
+            const unsigned long long m = __ballot(listed[u]);
+            const int pos = base + __popcll(m & below);
+            if (listed[u]) list[pos] = n;
+            if (slot != nullptr && in[u]) slot[n] = listed[u] ? pos : -1;
             base += __popcll(m);
-            ubase += __popcll(um);
         }
     }
     if (tid == 0) a.counts[(size_t)b * tiles + t] = total;
@@ -862,6 +852,8 @@ struct BwdArgs {
 
 // Partial field order: 0 M0 = sum G e, 1 Mx = sum G e dx, 2 My, 3 Mxx, 4 Mxy, 5 Myy,
 // 6+c = sum e g^_c.
+// n[g] is the column of the partial array the lane's sums go to (>= N: nothing is stored): the
+// Gaussian index on general grids, the position in the tile's list on separable ones.
 template <int C, int G>
 __device__ __forceinline__ void bwd_store(const BwdArgs& a, int b, int t, const int (&n)[G],
                                           const float (&M)[G][6], const float (&CG)[G][C]) {
@@ -919,9 +911,9 @@ constexpr int kBwdTileW = IGS_BWD_TILE_W;
 // (double-buffered) and are read with broadcast ds_read_b128; the tile's column coordinates sit
 // in LDS for the whole kernel.  Per row the dy part of q is hoisted, and row sums
 // R0 = sum G e, R1 = sum G e dx, R2 = sum G e dx^2 (and the colour sums) are folded into the
-// totals once per row.  List positions past the count map to the unlisted Gaussians: a lane that
-// gets one computes (and stores) its exact zeros, and a workgroup made of such lanes only stores
-// zeros without computing, so every partial entry is written exactly once per launch.
+// totals once per row.  A lane's sums are stored at its list position (coalesced); the finalize
+// kernel finds them through the tile's slot table and takes 0 for unlisted Gaussians, so tiles
+// that a Gaussian does not reach cost neither compute nor memory traffic.
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     constexpr int CP = pix_stride_sep(C), CP4 = CP / 4;
@@ -942,13 +934,14 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     const int tid = threadIdx.x;
     const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
     const int count = a.counts[(size_t)b * a.T + t];
+    if (grp * G * kThreads >= count) return;  // workgroup-uniform: no listed Gaussian left
     const int* list = a.lists + ((size_t)b * a.T + t) * a.Np;
-    int n[G];
+    int n[G], slot[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         const int pos = (grp * G + g) * kThreads + tid;
-        const int idx = pos < count ? pos : pos + (a.Np - a.N);
-        n[g] = idx < a.Np ? list[idx] : a.N;
+        n[g] = pos < count ? list[pos] : a.N;
+        slot[g] = pos < count ? pos : a.N;
     }
     float M[G][6], CG[G][C];
 #pragma unroll
@@ -957,10 +950,6 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
         for (int f = 0; f < 6; ++f) M[g][f] = 0.0f;
 #pragma unroll
         for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
-    }
-    if (grp * G * kThreads >= count) {  // workgroup-uniform: unlisted Gaussians only
-        bwd_store<C, G>(a, b, t, n, M, CG);
-        return;
     }
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
     bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
@@ -1098,7 +1087,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
         }
         __syncthreads();
     }
-    bwd_store<C, G>(a, b, t, n, M, CG);
+    bwd_store<C, G>(a, b, t, slot, M, CG);
 }
 
 // General grid: the tile is a flat pixel range (multiple of 256); x and y come with the
@@ -1195,23 +1184,38 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
 }
 
 // Fixed-order sum over the T tile partials of NV consecutive fields for one Gaussian, spread
-// over the 16 "t-lanes" of a workgroup laid out as 16 t-lanes x 16 Gaussians: t-lane k adds
-// tiles k, k+16, ... in order, the 16 lane sums are then added in order by every thread (so all
-// 16 t-lanes of a Gaussian hold the same, run-to-run identical value).  `red` is
-// [NV][16][17] floats of LDS.  Must be called by all 256 threads.
-constexpr int kFinT = 16, kFinN = 16;
+// over the kFinT "t-lanes" of a workgroup laid out as kFinT t-lanes x kFinN Gaussians: t-lane k
+// adds tiles k, k+kFinT, ... in order, the lane sums are then added in order by every thread (so
+// all t-lanes of a Gaussian hold the same, run-to-run identical value).  `red` is
+// [NV][kFinT][kFinN+1] floats of LDS.  Must be called by all 256 threads.  (8 x 32: with fewer
+// t-lanes the consecutive Gaussians of a wave read neighbouring columns of a tile's partials,
+// with more the sequential part of a sum over hundreds of tiles gets shorter.)
+#ifndef IGS_FIN_T
+#define IGS_FIN_T 8
+#endif
+constexpr int kFinT = IGS_FIN_T, kFinN = 256 / IGS_FIN_T;
+constexpr int kFinColours = 8;  // colour channels summed per pass (>= 6: the LDS array also serves the moments)
 
+// `part` is the image's partial array [T][NF][N]; the Gaussian's column in tile t is
+// slots[t * Np + n] when a slot table is given (negative: the tile holds nothing for it), else n.
+// Only the first `nv` (<= NV) of the fields are read.
 template <int NV>
-__device__ __forceinline__ void tile_sum(const float* __restrict__ base, int T, int NF, int N,
-                                         int f0, bool valid, float (&out)[NV], float* red) {
+__device__ __forceinline__ void tile_sum(const float* __restrict__ part, const int* __restrict__ slots,
+                                         int Np, int n, int T, int NF, int N, int f0, bool valid,
+                                         float (&out)[NV], float* red, int nv = NV) {
     const int tl = threadIdx.x / kFinN, nl = threadIdx.x % kFinN;
     float acc[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
     if (valid)
-        for (int t = tl; t < T; t += kFinT)
+        for (int t = tl; t < T; t += kFinT) {
+            const int col = slots ? slots[(size_t)t * Np + n] : n;
+            if (col >= 0) {
 #pragma unroll
-            for (int v = 0; v < NV; ++v) acc[v] += base[((size_t)t * NF + f0 + v) * N];
+                for (int v = 0; v < NV; ++v)
+                    if (v < nv) acc[v] += part[((size_t)t * NF + f0 + v) * N + col];
+            }
+        }
     __syncthreads();  // protects `red` against the previous call's readers
 #pragma unroll
     for (int v = 0; v < NV; ++v) red[(v * kFinT + tl) * (kFinN + 1) + nl] = acc[v];
@@ -1233,12 +1237,12 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ base, int T, 
 template <bool kScaleRot>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
-    const float* __restrict__ p0,
+    const int* __restrict__ slots_in, int Np, const float* __restrict__ p0,
     const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ alphas,
     int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
     float* __restrict__ g_col) {
-    __shared__ float red[6 * kFinT * (kFinN + 1)];
+    __shared__ float red[kFinColours * kFinT * (kFinN + 1)];
     const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
     const int b = blockIdx.y;
     const bool valid = n < N;
@@ -1247,9 +1251,13 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + C;
     const size_t i = (size_t)b * N + min(n, N - 1);
-    const float* base = partial + (size_t)b * T * NF * N + min(n, N - 1);
+    const float* part = partial + (size_t)b * T * NF * N;
+    // the slot table belongs to the separable variant
+    const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
+                           ? slots_in + (size_t)b * T * Np : nullptr;
+    const int nn = min(n, N - 1);
     float M[6];
-    tile_sum<6>(base, T, NF, N, 0, valid, M, red);
+    tile_sum<6>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
     const double al = alphas[i];
     // O(BN) epilogue in fp64: the chain rule multiplies sums by 1/s^3-sized factors
     double A, Bc, D, cs = 0., sn = 0., i0 = 0., i1 = 0., s0 = 0., s1 = 0.;
@@ -1287,10 +1295,14 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
         if (g2 && writer) g2[i] = (float)gD;
     }
     if (g_col) {  // kernel-argument uniform, so the barriers inside tile_sum are safe
-        for (int c = 0; c < C; ++c) {
-            float s1[1];
-            tile_sum<1>(base, T, NF, N, 6 + c, valid, s1, red);
-            if (writer) g_col[i * C + c] = (float)al * s1[0];
+        for (int c0 = 0; c0 < C; c0 += kFinColours) {  // colour sums, kFinColours channels per pass
+            float sc[kFinColours];
+            const int nc = min(kFinColours, C - c0);
+            tile_sum<kFinColours>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+            if (writer)
+#pragma unroll
+                for (int c = 0; c < kFinColours; ++c)
+                    if (c < nc) g_col[i * C + c0 + c] = (float)al * sc[c];
         }
     }
 }
@@ -1299,8 +1311,9 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
 // alpha = 1, d log_s_k = d s_k * exp(log_s_k) and a zero gradient for the unused opacity logit.
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
-    const float* __restrict__ feat, int N, int C, int Cp, float eps, float* __restrict__ g_feat) {
-    __shared__ float red[6 * kFinT * (kFinN + 1)];
+    const int* __restrict__ slots_in, int Np, const float* __restrict__ feat, int N, int C, int Cp,
+    float eps, float* __restrict__ g_feat) {
+    __shared__ float red[kFinColours * kFinT * (kFinN + 1)];
     const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
     const int b = blockIdx.y;
     const bool valid = n < N;
@@ -1308,9 +1321,12 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + Cp;
     const size_t i = (size_t)b * N + min(n, N - 1);
-    const float* base = partial + (size_t)b * T * NF * N + min(n, N - 1);
+    const float* part = partial + (size_t)b * T * NF * N;
+    const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
+                           ? slots_in + (size_t)b * T * Np : nullptr;
+    const int nn = min(n, N - 1);
     float M[6];
-    tile_sum<6>(base, T, NF, N, 0, valid, M, red);
+    tile_sum<6>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
     const float* f = feat + i * (6 + C);
     const double e0 = (double)expf(f[2]), e1 = (double)expf(f[3]);
     const double s0 = e0 + (double)eps, s1 = e1 + (double)eps;
@@ -1332,10 +1348,14 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
         g[4] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
         g[5] = 0.0f;
     }
-    for (int c = 0; c < C; ++c) {
-        float s1v[1];
-        tile_sum<1>(base, T, NF, N, 6 + c, valid, s1v, red);
-        if (writer) g[6 + c] = s1v[0];
+    for (int c0 = 0; c0 < C; c0 += kFinColours) {
+        float sc[kFinColours];
+        const int nc = min(kFinColours, C - c0);
+        tile_sum<kFinColours>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+        if (writer)
+#pragma unroll
+            for (int c = 0; c < kFinColours; ++c)
+                if (c < nc) g[6 + c0 + c] = sc[c];
     }
 }
 
@@ -1563,7 +1583,15 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
         p->pix_bytes = align16(p->pix_bytes) + bins_bytes(B, p->bwd_tiles, p->n_padded);
     }
     p->partial_bytes = (uint64_t)B * T * (6 + C) * N * sizeof(float);
+    if (sep)  // the slot tables [B][T][Np] (Gaussian -> position in the tile's list) follow
+        p->partial_bytes = align16(p->partial_bytes) + (uint64_t)B * T * p->n_padded * sizeof(int);
     return IGS_OK;
+}
+
+// The slot tables of the separable backward inside the partial buffer.
+inline int* slots_at(float* partial, int B, int T, int NF, int N) {
+    return reinterpret_cast<int*>(reinterpret_cast<char*>(partial) +
+                                  align16((size_t)B * T * NF * N * sizeof(float)));
 }
 
 // Where the tile lists of a separable launch live inside its workspace.
@@ -1850,7 +1878,7 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
             ba.N = N; ba.Np = plan.n_padded; ba.H = H; ba.W = W;
             ba.tile_w = 64 * fg.wx; ba.tile_h = fwd_sep_p(C) * (4 / fg.wx);
             ba.tiles_x = fg.tiles_x; ba.tiles_y = fg.tiles_y;
-            ba.counts = bp.counts; ba.lists = bp.lists; ba.complement = 0;
+            ba.counts = bp.counts; ba.lists = bp.lists; ba.slots = nullptr;
             ba.flag = vs[i].flag; ba.want = vs[i].want;
             rc = launch_bin(ba, B, st);
             if (rc) return rc;
@@ -1981,7 +2009,8 @@ int igs_gs2d_backward_reduce(const float* packed, const float* colors, const flo
             ba.N = N; ba.Np = a.Np; ba.H = H; ba.W = W;
             ba.tile_w = kBwdTileW; ba.tile_h = a.per_tile;
             ba.tiles_x = a.tiles_x; ba.tiles_y = a.T / a.tiles_x;
-            ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists); ba.complement = 1;
+            ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists);
+            ba.slots = slots_at(partial, B, a.T, 6 + C, N);
             ba.flag = a.flag; ba.want = a.want;
             rc = launch_bin(ba, B, st);
             if (rc) return rc;
@@ -2031,6 +2060,12 @@ int igs_gs2d_backward_grid(const float* packed, const float* x, const float* y,
     return rc;
 }
 
+// The slot tables that the separable backward left behind the partial sums (none on general grids).
+static const int* finalize_slots(const float* partial, int grid_mode, int B, int T, int NF, int N) {
+    if (grid_mode == IGS_GRID_GENERAL) return nullptr;
+    return slots_at(const_cast<float*>(partial), B, T, NF, N);
+}
+
 // T of the separable (or only) variant and of the general variant under AUTO.
 static int finalize_tiles(int grid_mode, int B, int N, int H, int W, int C, int* T, int* T_alt) {
     igs_gs2d_plan_t plan;
@@ -2060,7 +2095,8 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     if (rc) return rc;
     hipLaunchKernelGGL((k_bwd_finalize<false>), dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, cov_inv_00, cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
+                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), (N + 3) & ~3, cov_inv_00,
+                       cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
                        g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
     return launch_status();
 }
@@ -2078,7 +2114,8 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     if (rc) return rc;
     hipLaunchKernelGGL((k_bwd_finalize<true>), dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, scales, rotations, (const float*)nullptr, alphas, N, C, eps, g_positions,
+                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), (N + 3) & ~3, scales, rotations,
+                       (const float*)nullptr, alphas, N, C, eps, g_positions,
                        g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
     return launch_status();
 }
@@ -2110,7 +2147,8 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
     if (rc) return rc;
     hipLaunchKernelGGL(k_bwd_finalize_feature, dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, gs_feature, N, C, C_kernel, eps, g_feature);
+                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N), (N + 3) & ~3, gs_feature,
+                       N, C, C_kernel, eps, g_feature);
     return launch_status();
 }
 
