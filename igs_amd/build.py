@@ -39,7 +39,8 @@ def is_stale() -> bool:
     if not os.path.exists(LIB):
         return True
     t = os.path.getmtime(LIB)
-    deps = SOURCES + [os.path.join(ROOT, "include", "igs_hip.h")]
+    csrc = os.path.join(PKG, "csrc")
+    deps = [os.path.join(csrc, f) for f in os.listdir(csrc)] + [os.path.join(ROOT, "include", "igs_hip.h")]
     return any(os.path.getmtime(d) > t for d in deps)
 
 

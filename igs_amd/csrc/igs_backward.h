@@ -1,0 +1,469 @@
+// igs_backward.h -- backward kernels: per-pixel prologue (optionally with the MSE gradient), per-Gaussian reduction on separable and general grids.
+// Included by igs_gs2d.hip inside its anonymous namespace (one translation unit).
+#pragma once
+
+// ----------------------------------------------------------------------------- backward
+// Prologue, one thread per (padded) pixel: g^_c = g_c / (den + eps), s = <g^, out>.
+//   separable: records [B][H][Wp][CP] = g^_0..g^_{C-1}, -s, 0..; columns W..Wp-1 are zero
+//              records; followed by the compact column coordinates xs [B][Wp]
+//              (padding columns repeat x of column W-1).
+//   general  : records [B][HWp][CP] = x, y, g^.., -s, 0..; padding pixels are zero records
+//              carrying the coordinates of the last pixel.
+// With `target` set (fit step), the upstream gradient is that of a mean-squared-error loss,
+// g_c = gscale (out_c - target_c), formed here instead of being read from `gout`, and each
+// workgroup writes its sum of (out - target)^2 (fixed-order LDS sum) to
+// loss_part[b * gridDim.x + blockIdx.x].
+template <int C, bool kSep>
+__global__ __launch_bounds__(kThreads) void k_bwd_pix(const float* __restrict__ out,
+                                                      const float* __restrict__ den,
+                                                      const float* __restrict__ gout,
+                                                      const float* __restrict__ target,
+                                                      float gscale,
+                                                      float* __restrict__ loss_part,
+                                                      const float* __restrict__ x,
+                                                      const float* __restrict__ y, long sxb,
+                                                      long sxh, long sxw, long syb, long syh,
+                                                      long syw, int B, int H, int W, int Wp,
+                                                      int HWp, float eps,
+                                                      float* __restrict__ pixrec,
+                                                      const int* __restrict__ flag, int want) {
+    constexpr int CP = kSep ? pix_stride_sep(C) : pix_stride_gen(C);
+    constexpr int OFF = kSep ? 0 : 2;
+    if (flag != nullptr && *flag != want) return;
+    const int HW = H * W;
+    const int i = blockIdx.x * kThreads + threadIdx.x;  // padded pixel index
+    const int b = blockIdx.y;
+    int h = 0, w = 0;
+    bool valid, inside;  // inside: this thread owns a (padded) record; valid: a real pixel
+    if (kSep) {
+        inside = i < H * Wp;
+        h = inside ? i / Wp : 0;
+        w = inside ? i - h * Wp : 0;
+        valid = inside && w < W;
+        if (inside && h == 0) {
+            float* xs = pixrec + (size_t)B * H * Wp * CP;
+            xs[(size_t)b * Wp + w] = x[b * sxb + (long)min(w, W - 1) * sxw];
+        }
+    } else {
+        inside = i < HWp;
+        valid = i < HW;
+        const int pc = min(i, HW - 1);
+        h = pc / W;
+        w = pc - h * W;
+    }
+    float r[CP];
+#pragma unroll
+    for (int k = 0; k < CP; ++k) r[k] = 0.0f;
+    float sq = 0.0f;
+    if (valid) {
+        const int p = h * W + w;
+        const float inv = 1.0f / (den[(size_t)b * HW + p] + eps);
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const size_t idx = ((size_t)b * C + c) * HW + p;
+            const float o = out[idx];
+            float g;
+            if (target != nullptr) {
+                const float d = o - target[idx];
+                sq = fmaf(d, d, sq);
+                g = gscale * d;
+            } else {
+                g = gout[idx];
+            }
+            const float gh = g * inv;
+            s = fmaf(gh, o, s);
+            r[OFF + c] = gh;
+        }
+        r[OFF + C] = -s;
+    }
+    if (inside) {
+        if (!kSep) {
+            r[0] = x[b * sxb + h * sxh + w * sxw];
+            r[1] = y[b * syb + h * syh + w * syw];
+        }
+        const size_t rec = kSep ? ((size_t)b * H * Wp + i) : ((size_t)b * HWp + i);
+        float4* dst = reinterpret_cast<float4*>(pixrec + rec * CP);
+#pragma unroll
+        for (int k = 0; k < CP / 4; ++k)
+            dst[k] = make_float4(r[4 * k], r[4 * k + 1], r[4 * k + 2], r[4 * k + 3]);
+    }
+    if (loss_part != nullptr) {  // kernel-argument uniform: every thread reaches the barriers
+        __shared__ float red[kThreads];
+        red[threadIdx.x] = sq;
+        __syncthreads();
+        for (int k = kThreads / 2; k > 0; k >>= 1) {
+            if ((int)threadIdx.x < k) red[threadIdx.x] += red[threadIdx.x + k];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) loss_part[(size_t)b * gridDim.x + blockIdx.x] = red[0];
+    }
+}
+
+// loss = scale * sum(loss_part[0..count)), one workgroup, fixed order.
+__global__ __launch_bounds__(kThreads) void k_loss_sum(const float* __restrict__ loss_part, int count,
+                                                       float scale, float* __restrict__ loss,
+                                                       const int* __restrict__ flag, int want) {
+    if (flag != nullptr && *flag != want) return;
+    __shared__ float red[kThreads];
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < count; i += kThreads) s += loss_part[i];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int k = kThreads / 2; k > 0; k >>= 1) {
+        if ((int)threadIdx.x < k) red[threadIdx.x] += red[threadIdx.x + k];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *loss = red[0] * scale;
+}
+
+struct BwdArgs {
+    const float* packed;  // [B][Np][RS]
+    const float* colors;  // [B][N][C]
+    const float* pixrec;
+    const float* xs;      // separable: [B][Wp]
+    const float* y;
+    long syb, syh;
+    int N, Np, H, W, Wp, HWp;
+    int per_tile;  // rows (separable) or pixels (general, multiple of 256) per tile
+    int T;         // tiles per image (separable: tiles_x * row bands)
+    int tiles_x;   // separable: column bands of kBwdTileW columns
+    const int* counts;  // separable: Gaussians listed per tile [B][T]
+    const int* lists;   // separable: list + complement [B][T][Np]
+    float* partial;  // [B][T][6+C][N]
+    const int* flag;
+    int want;
+};
+
+// Partial field order: 0 M0 = sum G e, 1 Mx = sum G e dx, 2 My, 3 Mxx, 4 Mxy, 5 Myy,
+// 6+c = sum e g^_c.
+// n[g] is the column of the partial array the lane's sums go to (>= N: nothing is stored): the
+// Gaussian index on general grids, the position in the tile's list on separable ones.
+template <int C, int G>
+__device__ __forceinline__ void bwd_store(const BwdArgs& a, int b, int t, const int (&n)[G],
+                                          const float (&M)[G][6], const float (&CG)[G][C]) {
+    constexpr int NF = 6 + C;
+    float* base = a.partial + ((size_t)b * a.T + t) * NF * a.N;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        if (n[g] < a.N) {
+#pragma unroll
+            for (int f = 0; f < 6; ++f) base[(size_t)f * a.N + n[g]] = M[g][f];
+#pragma unroll
+            for (int c = 0; c < C; ++c) base[(size_t)(6 + c) * a.N + n[g]] = CG[g][c];
+        }
+    }
+}
+
+// Loads the G Gaussians of this lane; n[g] >= N marks an unused slot (nothing is stored for it).
+template <int C, int G>
+__device__ __forceinline__ void bwd_load_gaussians(const BwdArgs& a, int b, const int (&n)[G],
+                                                   float (&px)[G], float (&py)[G], float (&A)[G],
+                                                   float (&B2)[G], float (&D)[G],
+                                                   float (&col)[G][C]) {
+    constexpr int RS = rec_stride_of(C);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int nc = min(n[g], a.N - 1);
+        const float* r = a.packed + ((size_t)b * a.Np + nc) * RS;
+        px[g] = r[0];
+        py[g] = r[1];
+        A[g] = r[2];
+        B2[g] = r[3];
+        D[g] = r[4];
+#pragma unroll
+        for (int c = 0; c < C; ++c) col[g][c] = a.colors[((size_t)b * a.N + nc) * C + c];
+    }
+}
+
+// pixel records per LDS buffer; wide records get a shorter chunk so the two buffers stay small
+__host__ __device__ constexpr int pix_chunk(int C) { return C <= 4 ? IGS_PCHUNK : 128; }
+
+// columns of a backward pixel tile on separable grids
+#ifndef IGS_BWD_MAX_ROWS
+#define IGS_BWD_MAX_ROWS 32
+#endif
+constexpr int kBwdMaxRows = IGS_BWD_MAX_ROWS;
+constexpr int kBwdMinRows = 4;
+#ifndef IGS_BWD_TILE_W
+#define IGS_BWD_TILE_W 64
+#endif
+constexpr int kBwdTileW = IGS_BWD_TILE_W;
+
+// Separable grid: lane = G Gaussians taken from the tile's list (those whose reach box meets
+// the tile; the others are known to get exactly zero from it); the tile is kBwdTileW columns x
+// per_tile rows.  Its pixel records stream through LDS in chunks of whole tile rows
+// (double-buffered) and are read with broadcast ds_read_b128; the tile's column coordinates sit
+// in LDS for the whole kernel.  Per row the dy part of q is hoisted, and row sums
+// R0 = sum G e, R1 = sum G e dx, R2 = sum G e dx^2 (and the colour sums) are folded into the
+// totals once per row.  A lane's sums are stored at its list position (coalesced); the finalize
+// kernel finds them through the tile's slot table and takes 0 for unlisted Gaussians, so tiles
+// that a Gaussian does not reach cost neither compute nor memory traffic.
+template <int C, int G>
+__global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
+    constexpr int CP = pix_stride_sep(C), CP4 = CP / 4;
+    constexpr int PX = pix_chunk(C) > kBwdTileW ? pix_chunk(C) : kBwdTileW;
+    constexpr int RPC = PX / kBwdTileW;          // tile rows per chunk
+    constexpr int ROW4 = kBwdTileW * CP4;        // float4 per tile row
+    constexpr int E = RPC * ROW4;                // float4 per chunk
+    constexpr int PRE = (E + kThreads - 1) / kThreads;
+    static_assert(PX % kBwdTileW == 0 && RPC >= 1, "chunk must hold whole tile rows");
+    __shared__ float4 sh[2 * E];
+    __shared__ float4 xsh[kBwdTileW / 4];
+    __shared__ float ysh[2][RPC + 1];  // row coordinates of the chunk (+1: read-ahead slot)
+    IGS_GATE(a);
+    // tiles are the fastest grid dimension: consecutive workgroups (dealt round-robin to the
+    // XCDs) then belong to different tiles, and the list-position groups that have work (the
+    // low ones) are spread over all XCDs
+    const int b = blockIdx.z, t = blockIdx.x, grp = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
+    const int count = a.counts[(size_t)b * a.T + t];
+    if (grp * G * kThreads >= count) return;  // workgroup-uniform: no listed Gaussian left
+    const int* list = a.lists + ((size_t)b * a.T + t) * a.Np;
+    int n[G], slot[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int pos = (grp * G + g) * kThreads + tid;
+        n[g] = pos < count ? list[pos] : a.N;
+        slot[g] = pos < count ? pos : a.N;
+    }
+    float M[G][6], CG[G][C];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int f = 0; f < 6; ++f) M[g][f] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
+    }
+    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
+    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+
+    const int c0 = tx * kBwdTileW;
+    const int cw = min(a.Wp, c0 + kBwdTileW) - c0;  // columns of this tile, a multiple of 8
+    const int r0 = ty * a.per_tile, r1 = min(a.H, r0 + a.per_tile);
+    const int chunks = (r1 - r0 + RPC - 1) / RPC;
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (tid < kBwdTileW / 4)
+        xsh[tid] = 4 * tid < cw ? reinterpret_cast<const float4*>(a.xs + (size_t)b * a.Wp + c0)[tid] : zero;
+
+    // element e of chunk k: float4 (e % ROW4) of tile row (e / ROW4)
+    auto fetch = [&](int k, int e) -> float4 {
+        const int rr = e / ROW4, rem = e - rr * ROW4;
+        const int r = r0 + k * RPC + rr;
+        if (r >= r1 || rem >= cw * CP4) return zero;
+        const float4* row = reinterpret_cast<const float4*>(a.pixrec + (((size_t)b * a.H + r) * a.Wp + c0) * CP);
+        return row[rem];
+    };
+    // y of tile row (k * RPC + rr), clamped to the tile (the clamped ones are never used)
+    auto fetch_y = [&](int k, int rr) -> float {
+        return a.y[b * a.syb + (long)min(r0 + k * RPC + rr, r1 - 1) * a.syh];
+    };
+    float4 pre[PRE];
+    float ypre = 0.0f;
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int e = i * kThreads + tid;
+        if (e < E) sh[e] = fetch(0, e);
+    }
+    if (tid <= RPC) ysh[0][tid] = fetch_y(0, min(tid, RPC - 1));
+    __syncthreads();
+
+    for (int k = 0; k < chunks; ++k) {
+        if (k + 1 < chunks) {
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                pre[i] = (e < E) ? fetch(k + 1, e) : zero;
+            }
+            if (tid <= RPC) ypre = fetch_y(k + 1, min(tid, RPC - 1));
+        }
+        const float4* cur = sh + (k & 1) * E;
+        const float* ycur = ysh[k & 1];
+        const int rows = min(RPC, r1 - r0 - k * RPC);
+        float ynext = ycur[0];
+#pragma unroll 1
+        for (int rr = 0; rr < rows; ++rr) {
+            // the row coordinate comes from LDS, read one row ahead: a scalar load here would
+            // drain the LDS/scalar counter once per tile row
+            const float yv = ynext;
+            ynext = ycur[rr + 1];
+            float dy[G], cyy[G], bdy[G], R0[G], R1[G], R2[G], RC[G][C];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                dy[g] = yv - py[g];
+                const float ddy = D[g] * dy[g];
+                cyy[g] = ddy * dy[g];
+                bdy[g] = B2[g] * dy[g];
+                R0[g] = R1[g] = R2[g] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
+            }
+            const float4* rowrec = cur + rr * ROW4;
+#pragma unroll 1
+            for (int i = 0; i < cw; i += 4) {
+                const float4 xq = xsh[i >> 2];
+                const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
+                // phase 1: exponents of the 4 x G pairs (independent chains)
+                float dxs[4][G], ee[4][G];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        const float dx = xs4[j] - px[g];
+                        const float tt = fmaf(A[g], dx, bdy[g]);
+                        ee[j][g] = fmaf(tt, dx, cyy[g]);
+                        dxs[j][g] = dx;
+                    }
+                // phase 2: transcendentals back to back
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int g = 0; g < G; ++g) ee[j][g] = hw_exp2(ee[j][g]);
+                // phase 3: G = <g^, c> - s and the row sums
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float pv[CP];
+#pragma unroll
+                    for (int q4 = 0; q4 < CP4; ++q4) {
+                        const float4 tq = rowrec[(i + j) * CP4 + q4];
+                        pv[4 * q4] = tq.x;
+                        pv[4 * q4 + 1] = tq.y;
+                        pv[4 * q4 + 2] = tq.z;
+                        pv[4 * q4 + 3] = tq.w;
+                    }
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        const float e = ee[j][g], dx = dxs[j][g];
+                        float Gv = pv[C];  // -s
+#pragma unroll
+                        for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[g][c], Gv);
+                        const float ge = Gv * e;
+                        R0[g] += ge;
+                        const float t1 = ge * dx;
+                        R1[g] += t1;
+                        R2[g] = fmaf(t1, dx, R2[g]);
+#pragma unroll
+                        for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[c], RC[g][c]);
+                    }
+                }
+            }
+            // the tile row is complete
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                M[g][0] += R0[g];
+                M[g][1] += R1[g];
+                M[g][3] += R2[g];
+                M[g][2] = fmaf(dy[g], R0[g], M[g][2]);
+                M[g][4] = fmaf(dy[g], R1[g], M[g][4]);
+                M[g][5] = fmaf(dy[g] * dy[g], R0[g], M[g][5]);
+#pragma unroll
+                for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+            }
+        }
+        if (k + 1 < chunks) {
+            float4* nxt = sh + ((k + 1) & 1) * E;
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                if (e < E) nxt[e] = pre[i];
+            }
+            if (tid <= RPC) ysh[(k + 1) & 1][tid] = ypre;
+        }
+        __syncthreads();
+    }
+    bwd_store<C, G>(a, b, t, slot, M, CG);
+}
+
+// General grid: the tile is a flat pixel range (multiple of 256); x and y come with the
+// pixel record.  Sums are flushed into the totals once per 128-pixel chunk.
+template <int C, int G>
+__global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
+    constexpr int CP = pix_stride_gen(C), CP4 = CP / 4;
+    constexpr int kPixChunk = pix_chunk(C);
+    __shared__ float4 sh[2 * kPixChunk * CP4];
+    IGS_GATE(a);
+    const int b = blockIdx.z, t = blockIdx.y;
+    int n[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) n[g] = (blockIdx.x * G + g) * kThreads + threadIdx.x;
+    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
+    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+    float M[G][6], CG[G][C], R[G][6], RC[G][C];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int f = 0; f < 6; ++f) M[g][f] = R[g][f] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) CG[g][c] = RC[g][c] = 0.0f;
+    }
+    const int p0 = t * a.per_tile, p1 = min(a.HWp, p0 + a.per_tile);
+    const float4* src = reinterpret_cast<const float4*>(a.pixrec + ((size_t)b * a.HWp + p0) * CP);
+    int seen = 0;
+    stream_records_lds<CP4, kPixChunk>(src, p1 - p0, sh, [&](const float4* r) {
+        float pv[CP];
+#pragma unroll
+        for (int q4 = 0; q4 < CP4; ++q4) {
+            const float4 tq = r[q4];
+            pv[4 * q4] = tq.x;
+            pv[4 * q4 + 1] = tq.y;
+            pv[4 * q4 + 2] = tq.z;
+            pv[4 * q4 + 3] = tq.w;
+        }
+        float dxs[G], dys[G], ee[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float dx = pv[0] - px[g];
+            const float dy = pv[1] - py[g];
+            float tt = A[g] * dx;
+            tt = fmaf(B2[g], dy, tt);
+            const float v = D[g] * dy;
+            float q = tt * dx;
+            ee[g] = fmaf(v, dy, q);
+            dxs[g] = dx;
+            dys[g] = dy;
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) ee[g] = hw_exp2(ee[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float e = ee[g], dx = dxs[g], dy = dys[g];
+            float Gv = pv[2 + C];  // -s
+#pragma unroll
+            for (int c = 0; c < C; ++c) Gv = fmaf(pv[2 + c], col[g][c], Gv);
+            const float ge = Gv * e;
+            R[g][0] += ge;
+            const float t1 = ge * dx, t2 = ge * dy;
+            R[g][1] += t1;
+            R[g][2] += t2;
+            R[g][3] = fmaf(t1, dx, R[g][3]);
+            R[g][4] = fmaf(t1, dy, R[g][4]);
+            R[g][5] = fmaf(t2, dy, R[g][5]);
+#pragma unroll
+            for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[2 + c], RC[g][c]);
+        }
+        if ((++seen & (kPixChunk - 1)) == 0) {  // two-level summation
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+#pragma unroll
+                for (int f = 0; f < 6; ++f) {
+                    M[g][f] += R[g][f];
+                    R[g][f] = 0.0f;
+                }
+#pragma unroll
+                for (int c = 0; c < C; ++c) {
+                    CG[g][c] += RC[g][c];
+                    RC[g][c] = 0.0f;
+                }
+            }
+        }
+    });
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int f = 0; f < 6; ++f) M[g][f] += R[g][f];
+#pragma unroll
+        for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+    }
+    bwd_store<C, G>(a, b, t, n, M, CG);
+}

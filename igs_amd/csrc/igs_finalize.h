@@ -1,0 +1,179 @@
+// igs_finalize.h -- finalize kernels: fixed-order sum of the tile partials and the chain rule.
+// Included by igs_gs2d.hip inside its anonymous namespace (one translation unit).
+#pragma once
+
+// Fixed-order sum over the T tile partials of NV consecutive fields for one Gaussian, spread
+// over the kFinT "t-lanes" of a workgroup laid out as kFinT t-lanes x kFinN Gaussians: t-lane k
+// adds tiles k, k+kFinT, ... in order, the lane sums are then added in order by every thread (so
+// all t-lanes of a Gaussian hold the same, run-to-run identical value).  `red` is
+// [NV][kFinT][kFinN+1] floats of LDS.  Must be called by all 256 threads.  (8 x 32: with fewer
+// t-lanes the consecutive Gaussians of a wave read neighbouring columns of a tile's partials,
+// with more the sequential part of a sum over hundreds of tiles gets shorter.)
+#ifndef IGS_FIN_T
+#define IGS_FIN_T 8
+#endif
+constexpr int kFinT = IGS_FIN_T, kFinN = 256 / IGS_FIN_T;
+constexpr int kFinColours = 8;  // colour channels summed per pass (>= 6: the LDS array also serves the moments)
+
+// `part` is the image's partial array [T][NF][N]; the Gaussian's column in tile t is
+// slots[t * Np + n] when a slot table is given (negative: the tile holds nothing for it), else n.
+// Only the first `nv` (<= NV) of the fields are read.
+template <int NV>
+__device__ __forceinline__ void tile_sum(const float* __restrict__ part, const int* __restrict__ slots,
+                                         int Np, int n, int T, int NF, int N, int f0, bool valid,
+                                         float (&out)[NV], float* red, int nv = NV) {
+    const int tl = threadIdx.x / kFinN, nl = threadIdx.x % kFinN;
+    float acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
+    if (valid)
+        for (int t = tl; t < T; t += kFinT) {
+            const int col = slots ? slots[(size_t)t * Np + n] : n;
+            if (col >= 0) {
+#pragma unroll
+                for (int v = 0; v < NV; ++v)
+                    if (v < nv) acc[v] += part[((size_t)t * NF + f0 + v) * N + col];
+            }
+        }
+    __syncthreads();  // protects `red` against the previous call's readers
+#pragma unroll
+    for (int v = 0; v < NV; ++v) red[(v * kFinT + tl) * (kFinN + 1) + nl] = acc[v];
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kFinT; ++k) s += red[(v * kFinT + k) * (kFinN + 1) + nl];
+        out[v] = s;
+    }
+}
+
+// Finalize: 16 threads per Gaussian; sums the T tile partials in a fixed order and applies
+//   d alpha = M0, d color_c = alpha CG_c, d px = alpha (A Mx + B My), d py = alpha (B Mx + D My),
+//   dA = -1/2 alpha Mxx, dB = -alpha Mxy, dD = -1/2 alpha Myy,
+// and (function level) the chain rule through A = c^2 i0 + s^2 i1, B = c s (i0 - i1),
+// D = s^2 i0 + c^2 i1, i_k = 1/(s_k^2 + eps).
+template <bool kScaleRot>
+__global__ __launch_bounds__(kThreads) void k_bwd_finalize(
+    const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
+    const int* __restrict__ slots_in, int Np, const float* __restrict__ p0,
+    const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ alphas,
+    int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
+    float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
+    float* __restrict__ g_col) {
+    __shared__ float red[kFinColours * kFinT * (kFinN + 1)];
+    const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
+    const int b = blockIdx.y;
+    const bool valid = n < N;
+    const bool writer = valid && threadIdx.x < kFinN;  // t-lane 0 writes the results
+    // AUTO grid mode: T_in belongs to the separable plan, T_alt to the general one
+    const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
+    const int NF = 6 + C;
+    const size_t i = (size_t)b * N + min(n, N - 1);
+    const float* part = partial + (size_t)b * T * NF * N;
+    // the slot table belongs to the separable variant
+    const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
+                           ? slots_in + (size_t)b * T * Np : nullptr;
+    const int nn = min(n, N - 1);
+    float M[6];
+    tile_sum<6>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+    const double al = alphas[i];
+    // O(BN) epilogue in fp64: the chain rule multiplies sums by 1/s^3-sized factors
+    double A, Bc, D, cs = 0., sn = 0., i0 = 0., i1 = 0., s0 = 0., s1 = 0.;
+    if (kScaleRot) {
+        s0 = p0[2 * i];
+        s1 = p0[2 * i + 1];
+        sincos((double)p1[i], &sn, &cs);
+        i0 = 1.0 / (s0 * s0 + (double)eps);
+        i1 = 1.0 / (s1 * s1 + (double)eps);
+        A = cs * cs * i0 + sn * sn * i1;
+        Bc = cs * sn * (i0 - i1);
+        D = sn * sn * i0 + cs * cs * i1;
+    } else {
+        A = p0[i];
+        Bc = p1[i];
+        D = p2[i];
+    }
+    if (g_alpha && writer) g_alpha[i] = M[0];
+    if (g_pos && writer) {
+        g_pos[2 * i] = (float)(al * (A * M[1] + Bc * M[2]));
+        g_pos[2 * i + 1] = (float)(al * (Bc * M[1] + D * M[2]));
+    }
+    const double gA = -0.5 * al * M[3], gB = -al * M[4], gD = -0.5 * al * M[5];
+    if (kScaleRot) {
+        if (g0 && writer) {  // scales [B,N,2]
+            const double gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
+            const double gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
+            g0[2 * i] = (float)(gi0 * (-2.0 * s0 * i0 * i0));
+            g0[2 * i + 1] = (float)(gi1 * (-2.0 * s1 * i1 * i1));
+        }
+        if (g1 && writer) g1[i] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
+    } else {
+        if (g0 && writer) g0[i] = (float)gA;
+        if (g1 && writer) g1[i] = (float)gB;
+        if (g2 && writer) g2[i] = (float)gD;
+    }
+    if (g_col) {  // kernel-argument uniform, so the barriers inside tile_sum are safe
+        for (int c0 = 0; c0 < C; c0 += kFinColours) {  // colour sums, kFinColours channels per pass
+            float sc[kFinColours];
+            const int nc = min(kFinColours, C - c0);
+            tile_sum<kFinColours>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+            if (writer)
+#pragma unroll
+                for (int c = 0; c < kFinColours; ++c)
+                    if (c < nc) g_col[i * C + c0 + c] = (float)al * sc[c];
+        }
+    }
+}
+
+// Finalize for the fused module head: d gs_feature [B][N][6+C] from the tile partials, with
+// alpha = 1, d log_s_k = d s_k * exp(log_s_k) and a zero gradient for the unused opacity logit.
+__global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
+    const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
+    const int* __restrict__ slots_in, int Np, const float* __restrict__ feat, int N, int C, int Cp,
+    float eps, float* __restrict__ g_feat) {
+    __shared__ float red[kFinColours * kFinT * (kFinN + 1)];
+    const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
+    const int b = blockIdx.y;
+    const bool valid = n < N;
+    const bool writer = valid && threadIdx.x < kFinN;
+    const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
+    const int NF = 6 + Cp;
+    const size_t i = (size_t)b * N + min(n, N - 1);
+    const float* part = partial + (size_t)b * T * NF * N;
+    const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
+                           ? slots_in + (size_t)b * T * Np : nullptr;
+    const int nn = min(n, N - 1);
+    float M[6];
+    tile_sum<6>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+    const float* f = feat + i * (6 + C);
+    const double e0 = (double)expf(f[2]), e1 = (double)expf(f[3]);
+    const double s0 = e0 + (double)eps, s1 = e1 + (double)eps;
+    double sn, cs;
+    sincos((double)f[4], &sn, &cs);
+    const double i0 = 1.0 / (s0 * s0 + (double)eps), i1 = 1.0 / (s1 * s1 + (double)eps);
+    const double A = cs * cs * i0 + sn * sn * i1;
+    const double Bc = cs * sn * (i0 - i1);
+    const double D = sn * sn * i0 + cs * cs * i1;
+    const double gA = -0.5 * M[3], gB = -(double)M[4], gD = -0.5 * M[5];
+    const double gi0 = gA * cs * cs + gB * cs * sn + gD * sn * sn;
+    const double gi1 = gA * sn * sn - gB * cs * sn + gD * cs * cs;
+    float* g = g_feat + i * (6 + C);
+    if (writer) {
+        g[0] = (float)(A * M[1] + Bc * M[2]);
+        g[1] = (float)(Bc * M[1] + D * M[2]);
+        g[2] = (float)(gi0 * (-2.0 * s0 * i0 * i0) * e0);
+        g[3] = (float)(gi1 * (-2.0 * s1 * i1 * i1) * e1);
+        g[4] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
+        g[5] = 0.0f;
+    }
+    for (int c0 = 0; c0 < C; c0 += kFinColours) {
+        float sc[kFinColours];
+        const int nc = min(kFinColours, C - c0);
+        tile_sum<kFinColours>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+        if (writer)
+#pragma unroll
+            for (int c = 0; c < kFinColours; ++c)
+                if (c < nc) g[6 + c0 + c] = sc[c];
+    }
+}

@@ -1,0 +1,38 @@
+// igs_fit.h -- AdamW step of the fused fit iteration.
+// Included by igs_gs2d.hip inside its anonymous namespace (one translation unit).
+#pragma once
+
+// ----------------------------------------------------------------------------- AdamW
+// Decoupled-weight-decay Adam over one flat parameter block, the update of torch.optim.AdamW
+// (amsgrad off) as the fit script configures it (scripts/2dgs_img_comp.py:186-193).  The
+// step counter and learning rate live in device memory so that a captured graph advances:
+//   state = {lr, t, 1 - beta1^t, sqrt(1 - beta2^t)}; lr is written by the host, the rest by
+// k_adamw_tick (one thread, powers in double).
+__global__ void k_adamw_tick(float* __restrict__ state, float beta1, float beta2) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const float t = state[1] + 1.0f;
+    state[1] = t;
+    state[2] = (float)(1.0 - pow((double)beta1, (double)t));
+    state[3] = (float)sqrt(1.0 - pow((double)beta2, (double)t));
+}
+
+__global__ __launch_bounds__(kThreads) void k_adamw(float* __restrict__ param,
+                                                    const float* __restrict__ grad,
+                                                    float* __restrict__ exp_avg,
+                                                    float* __restrict__ exp_avg_sq, long n,
+                                                    const float* __restrict__ state, float beta1,
+                                                    float beta2, float eps, float weight_decay) {
+    const long i = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= n) return;
+    const float lr = state[0], bc1 = state[2], bc2_sqrt = state[3];
+    const float g = grad[i];
+    float p = param[i] * (1.0f - lr * weight_decay);
+    float m = exp_avg[i];
+    m = fmaf(g - m, 1.0f - beta1, m);
+    const float v = fmaf(g * g, 1.0f - beta2, exp_avg_sq[i] * beta2);
+    const float denom = sqrtf(v) / bc2_sqrt + eps;
+    p -= (lr / bc1) * (m / denom);
+    param[i] = p;
+    exp_avg[i] = m;
+    exp_avg_sq[i] = v;
+}

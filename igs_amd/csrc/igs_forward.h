@@ -1,0 +1,335 @@
+// igs_forward.h -- forward kernels: LDS record streaming, separable and general grids, split combine.
+// Included by igs_gs2d.hip inside its anonymous namespace (one translation unit).
+#pragma once
+
+// ----------------------------------------------------------------------------- forward
+struct FwdArgs {
+    const float* packed;  // [B][Np][RS]
+    const float* x;
+    const float* y;
+    long sxb, sxh, sxw, syb, syh, syw;
+    int B, Np, H, W;
+    int n_per_split, S;  // n_per_split % 4 == 0
+    int tiles_x, tiles_y, total_tiles, wx;
+    float eps;
+    float* out;
+    float* den;
+    float* part;  // [S][B][C+1][HW] when S > 1
+    const int* counts;  // separable: Gaussians listed per tile [B][tiles]
+    const int* lists;   // separable: their indices [B][tiles][Np]
+    const int* flag;  // AUTO grid mode: run only if *flag == want (nullptr: always run)
+    int want;
+};
+
+// AUTO grid mode launches both the separable and the general variant of a kernel; the
+// device-side classification flag (1 = separable) decides which one does the work.
+#define IGS_GATE(a) \
+    if ((a).flag != nullptr && *(a).flag != (a).want) return
+
+// On gfx950 a fp32 VALU op whose operands are all VGPRs (or literals) issues about every
+// 2.2-2.7 cycles per wave64, while any SGPR operand makes it a 4-cycle op (measured; the
+// constant bus broadcast is the slow part).  So wave-uniform operands are NOT fed from SGPRs:
+// the uniform record stream (Gaussians in the forward, pixels in the backward) goes
+// global -> LDS (cooperatively, double-buffered) -> VGPRs through broadcast ds_read_b128
+// (every lane reads the same address: conflict-free), and the hot loops contain VGPR-only
+// VALU instructions plus LDS reads that issue on their own port.
+template <int C>
+struct GRec {
+    float px, py, A, B2, D, al;
+    float ac[C];
+};
+
+// Unpacks one record held in R4 float4 registers (read from a wave-uniform LDS address).
+template <int C>
+__device__ __forceinline__ GRec<C> lds_grec(const float4* r) {
+    constexpr int R4 = rec_stride_of(C) / 4;
+    float v[4 * R4];
+#pragma unroll
+    for (int i = 0; i < R4; ++i) {
+        const float4 t = r[i];
+        v[4 * i] = t.x;
+        v[4 * i + 1] = t.y;
+        v[4 * i + 2] = t.z;
+        v[4 * i + 3] = t.w;
+    }
+    GRec<C> g;
+    g.px = v[0];
+    g.py = v[1];
+    g.A = v[2];
+    g.B2 = v[3];
+    g.D = v[4];
+    g.al = v[5];
+#pragma unroll
+    for (int c = 0; c < C; ++c) g.ac[c] = v[6 + c];
+    return g;
+}
+
+// Keeps a wave-uniform value in a VGPR (an empty asm the compiler cannot see through), so that
+// instructions using it stay VGPR-only.
+__device__ __forceinline__ float in_vgpr(float v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+#ifndef IGS_GCHUNK
+#define IGS_GCHUNK 64
+#endif
+#ifndef IGS_PCHUNK
+#define IGS_PCHUNK 256
+#endif
+#ifndef IGS_STREAM_UNROLL
+#define IGS_STREAM_UNROLL 2
+#endif
+constexpr int kStreamUnroll = IGS_STREAM_UNROLL;  // records whose LDS reads are in flight together
+constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
+
+// Streams `count` records of R4 float4 each from global memory to every wave of the
+// workgroup through the double-buffered LDS window sh[2][CH*R4]; body(const float4* rec) runs
+// once per record with a wave-uniform LDS pointer.  Records past `count` in the last chunk
+// read as all-zero (for a Gaussian record: alpha = 0, adds exactly 0).  Must be called by all
+// kThreads threads of the workgroup (it contains barriers).
+// With kGather, record i of the stream is src record index[i] (a tile's Gaussian list).
+template <int R4, int CH, bool kGather = false, class Body>
+__device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
+                                                   float4* sh, Body&& body,
+                                                   const int* __restrict__ index = nullptr) {
+    constexpr int E = CH * R4;                          // float4 per chunk
+    constexpr int PRE = (E + kThreads - 1) / kThreads;  // float4 per thread per chunk
+    const int total = count * R4;
+    const int chunks = (count + CH - 1) / CH;
+    const int tid = threadIdx.x;
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    // Gather: the record indices of a chunk are loaded one chunk before its records, so that
+    // no load in the loop waits for another load.
+    int idx[PRE];
+    auto load_idx = [&](int chunk) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int e = i * kThreads + tid, ge = chunk * E + e;
+            idx[i] = (kGather && e < E && ge < total) ? index[ge / R4] : 0;
+        }
+    };
+    float4 pre[PRE];
+    auto load_records = [&](int chunk) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int e = i * kThreads + tid, ge = chunk * E + e;
+            const bool valid = e < E && ge < total;
+            if (kGather)
+                pre[i] = valid ? src[(size_t)idx[i] * R4 + (ge % R4)] : zero;
+            else
+                pre[i] = valid ? src[ge] : zero;
+        }
+    };
+    load_idx(0);
+    load_records(0);
+    load_idx(1);
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int e = i * kThreads + tid;
+        if (e < E) sh[e] = pre[i];
+    }
+    __syncthreads();
+    for (int k = 0; k < chunks; ++k) {
+        if (k + 1 < chunks) {
+            load_records(k + 1);
+            load_idx(k + 2);
+        }
+        const float4* cur = sh + (k & 1) * E;
+        // The LDS reads of kStreamUnroll records are issued together and pinned above the work
+        // (the compiler would otherwise sink each read next to its first use and wait for it
+        // there); each record's body then only waits for its own reads, so one LDS latency is
+        // exposed per group instead of per record.
+#pragma unroll 1
+        for (int n = 0; n < CH; n += kStreamUnroll) {
+            float4 rr[kStreamUnroll][R4];
+#pragma unroll
+            for (int u = 0; u < kStreamUnroll; ++u)
+#pragma unroll
+                for (int i = 0; i < R4; ++i) rr[u][i] = cur[(n + u) * R4 + i];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < kStreamUnroll; ++u) {
+                body(rr[u]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if (k + 1 < chunks) {
+            float4* nxt = sh + ((k + 1) & 1) * E;
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                if (e < E) nxt[e] = pre[i];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int C>
+__device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p, float dsum,
+                                          const float (&num)[C]) {
+    const size_t HW = (size_t)a.H * a.W;
+    if (a.S == 1) {
+        const float inv = 1.0f / (dsum + a.eps);
+        a.den[(size_t)b * HW + p] = dsum;
+#pragma unroll
+        for (int c = 0; c < C; ++c) a.out[((size_t)b * C + c) * HW + p] = num[c] * inv;
+    } else {
+        float* dst = a.part + ((size_t)s * a.B + b) * (C + 1) * HW + p;
+#pragma unroll
+        for (int c = 0; c < C; ++c) dst[(size_t)c * HW] = num[c];
+        dst[(size_t)C * HW] = dsum;
+    }
+}
+
+// Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows;
+// workgroup = wx x (4/wx) waves, all four streaming the same Gaussians.  Per Gaussian and
+// lane: dx, A'dx^2, B2'dx once, then per pixel dy, 2 fma, exp2, 1 + C fma.
+template <int C, int P>
+__global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
+    constexpr int RS = rec_stride_of(C), R4 = RS / 4;
+    __shared__ float4 sh[2 * kGaussChunk * R4];
+    IGS_GATE(a);
+    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
+    if (tile >= a.total_tiles) return;  // workgroup-uniform
+    const int per_img = a.tiles_x * a.tiles_y;
+    const int b = tile / per_img;
+    const int tl = tile - b * per_img;
+    const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wxi = wave % a.wx, wyi = wave / a.wx;
+    const int col = (tx * a.wx + wxi) * 64 + lane;
+    const int row0 = (ty * (4 / a.wx) + wyi) * P;
+    const float xv = a.x[b * a.sxb + (long)min(col, a.W - 1) * a.sxw];
+    float yv[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) yv[p] = in_vgpr(a.y[b * a.syb + (long)min(row0 + p, a.H - 1) * a.syh]);
+
+    float dsum[P], num[P][C];
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        dsum[p] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) num[p][c] = 0.0f;
+    }
+    // this tile's Gaussians (those whose reach box meets it), split S ways by list position
+    const int s = blockIdx.y;
+    const int count = a.counts[(size_t)b * per_img + tl];
+    const int per = ((count + a.S - 1) / a.S + 3) & ~3;
+    const int n0 = min(count, s * per);
+    const int n1 = min(count, n0 + per);
+    const int* list = a.lists + ((size_t)b * per_img + tl) * a.Np + n0;
+    const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
+    stream_records_lds<R4, kGaussChunk, true>(src, n1 - n0, sh, [&](const float4* r) {
+        const GRec<C> g = lds_grec<C>(r);
+        const float dx = xv - g.px;
+        const float adx = g.A * dx;
+        const float c0 = adx * dx;
+        const float c1 = g.B2 * dx;
+        // three phases, so that the P independent chains overlap their latencies and the
+        // transcendental ops issue back to back
+        float e[P];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const float dy = yv[p] - g.py;
+            const float t = fmaf(g.D, dy, c1);
+            e[p] = fmaf(t, dy, c0);
+        }
+#pragma unroll
+        for (int p = 0; p < P; ++p) e[p] = hw_exp2(e[p]);
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            dsum[p] = fmaf(e[p], g.al, dsum[p]);
+#pragma unroll
+            for (int c = 0; c < C; ++c) num[p][c] = fmaf(e[p], g.ac[c], num[p][c]);
+        }
+    }, list);
+    if (col < a.W) {
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+            if (row0 + p < a.H) fwd_store<C>(a, b, s, (row0 + p) * a.W + col, dsum[p], num[p]);
+    }
+}
+
+// General grid: lane = P pixels of a flat 256*P pixel tile.
+template <int C, int P>
+__global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
+    constexpr int RS = rec_stride_of(C), R4 = RS / 4;
+    __shared__ float4 sh[2 * kGaussChunk * R4];
+    IGS_GATE(a);
+    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
+    if (tile >= a.total_tiles) return;  // workgroup-uniform
+    const int per_img = a.tiles_x;
+    const int b = tile / per_img;
+    const int tl = tile - b * per_img;
+    const int HW = a.H * a.W;
+    float xv[P], yv[P];
+    int pix[P];
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+        pix[j] = tl * (kThreads * P) + j * kThreads + (int)threadIdx.x;
+        const int pc = min(pix[j], HW - 1);
+        const int h = pc / a.W, w = pc - h * a.W;
+        xv[j] = a.x[b * a.sxb + h * a.sxh + w * a.sxw];
+        yv[j] = a.y[b * a.syb + h * a.syh + w * a.syw];
+    }
+    float dsum[P], num[P][C];
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+        dsum[j] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) num[j][c] = 0.0f;
+    }
+    const int s = blockIdx.y;
+    const int n0 = s * a.n_per_split;
+    const int n1 = min(a.Np, n0 + a.n_per_split);
+    const float4* src = reinterpret_cast<const float4*>(a.packed + ((size_t)b * a.Np + n0) * RS);
+    stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r) {
+        const GRec<C> g = lds_grec<C>(r);
+        float e[P];
+#pragma unroll
+        for (int j = 0; j < P; ++j) {
+            const float dx = xv[j] - g.px;
+            const float dy = yv[j] - g.py;
+            float t = g.A * dx;
+            t = fmaf(g.B2, dy, t);
+            const float v = g.D * dy;
+            float q = t * dx;
+            e[j] = fmaf(v, dy, q);
+        }
+#pragma unroll
+        for (int j = 0; j < P; ++j) e[j] = hw_exp2(e[j]);
+#pragma unroll
+        for (int j = 0; j < P; ++j) {
+            dsum[j] = fmaf(e[j], g.al, dsum[j]);
+#pragma unroll
+            for (int c = 0; c < C; ++c) num[j][c] = fmaf(e[j], g.ac[c], num[j][c]);
+        }
+    });
+#pragma unroll
+    for (int j = 0; j < P; ++j)
+        if (pix[j] < HW) fwd_store<C>(a, b, s, pix[j], dsum[j], num[j]);
+}
+
+// Split-N combine: fixed-order sum over the S partial images, then normalise.
+__global__ __launch_bounds__(kThreads) void k_fwd_combine(const float* __restrict__ part, int S,
+                                                          int B, int C, int HW, float eps,
+                                                          float* __restrict__ out,
+                                                          float* __restrict__ den,
+                                                          const int* __restrict__ flag, int want) {
+    if (flag != nullptr && *flag != want) return;
+    const int p = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (p >= HW) return;
+    float d = 0.0f;
+    for (int s = 0; s < S; ++s) d += part[(((size_t)s * B + b) * (C + 1) + C) * HW + p];
+    den[(size_t)b * HW + p] = d;
+    const float inv = 1.0f / (d + eps);
+    for (int c = 0; c < C; ++c) {
+        float v = 0.0f;
+        for (int s = 0; s < S; ++s) v += part[(((size_t)s * B + b) * (C + 1) + c) * HW + p];
+        out[((size_t)b * C + c) * HW + p] = v * inv;
+    }
+}

@@ -1,0 +1,275 @@
+// igs_pack_bin.h -- pack kernels (records + reach boxes) and the per-tile Gaussian lists (k_bin).
+// Included by igs_gs2d.hip inside its anonymous namespace (one translation unit).
+#pragma once
+
+// ----------------------------------------------------------------------------- pack
+// Reach box of a Gaussian: the axis-aligned bounding box of the ellipse q <= kReachQ, outside
+// of which its weight is exactly zero in these kernels: there the exponent
+// q' = -0.5 log2(e) q is below -160, ten binades under the -149/-150 at which exp2 returns 0
+// in fp32 whatever the denormal mode (the margin covers the rounding of q' itself, which is
+// a few ulp of its largest term).  Pixels outside the box therefore receive exactly +0 from
+// this Gaussian and give exactly 0 to its gradient sums, so skipping them changes no bit.
+// Half extents: sqrt(kReachQ Sigma_xx), sqrt(kReachQ Sigma_yy) with Sigma the covariance that
+// (A, B, D) invert.  A record with a non-finite field or a non-positive-definite (A, B, D)
+// gets an unbounded box (its NaN/inf must propagate as without culling); padding records get
+// an empty one.  Stored as (xlo, xhi, ylo, yhi).
+constexpr double kReachQ = 160.0 / 0.72134752044448170368;
+
+__device__ __forceinline__ float4 reach_box(float px, float py, double sxx, double syy, bool bounded) {
+    const float inf = __builtin_inff();
+    if (!bounded || !(sxx >= 0.0) || !(syy >= 0.0) || !isfinite(px) || !isfinite(py))
+        return make_float4(-inf, inf, -inf, inf);
+    // rounded outwards: one part in 1e5 is far more than the fp32 rounding of the bounds
+    const double hx = sqrt(kReachQ * sxx) * 1.00001, hy = sqrt(kReachQ * syy) * 1.00001;
+    const double ax = fabs((double)px) * 1e-6 + 1e-30, ay = fabs((double)py) * 1e-6 + 1e-30;
+    return make_float4((float)((double)px - hx - ax), (float)((double)px + hx + ax),
+                       (float)((double)py - hy - ay), (float)((double)py + hy + ay));
+}
+
+__device__ __forceinline__ float4 empty_box() {
+    const float inf = __builtin_inff();
+    return make_float4(inf, -inf, inf, -inf);
+}
+
+// One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
+// with A' = k A, B2' = 2 k B, D' = k D, k = -0.5 log2 e.  Records N..Np-1 are zero.
+// The reach boxes [B][Np] follow the records in the packed buffer.
+template <bool kScaleRot>
+__global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ position,
+                                                   const float* __restrict__ p0,  // cov00 | scales
+                                                   const float* __restrict__ p1,  // cov01 | rotations
+                                                   const float* __restrict__ p2,  // cov11 | unused
+                                                   const float* __restrict__ alphas,
+                                                   const float* __restrict__ colors, int N,
+                                                   int Np, int C, int RS, float eps,
+                                                   float* __restrict__ packed,
+                                                   float4* __restrict__ boxes, int cull) {
+    const int n = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (n >= Np) return;
+    float* r = packed + ((size_t)b * Np + n) * RS;
+    if (n >= N) {  // padding: alpha = 0 and e = exp2(0) = 1, so it contributes exactly 0
+        for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        boxes[(size_t)b * Np + n] = empty_box();
+        return;
+    }
+    const size_t i = (size_t)b * N + n;
+    // The closed form runs in fp64 and is rounded once: an error of a few fp32 ulp in A', B2', D'
+    // would be multiplied by |q| (tens, for sharp Gaussians) in the exponent.  O(BN) work.
+    double A, Bc, D, sxx, syy;
+    bool bounded;
+    if (kScaleRot) {
+        const double s0 = p0[2 * i], s1 = p0[2 * i + 1];
+        double sn, cs;
+        sincos((double)p1[i], &sn, &cs);
+        const double v0 = s0 * s0 + (double)eps, v1 = s1 * s1 + (double)eps;
+        const double i0 = 1.0 / v0, i1 = 1.0 / v1;
+        A = cs * cs * i0 + sn * sn * i1;
+        Bc = cs * sn * (i0 - i1);
+        D = sn * sn * i0 + cs * cs * i1;
+        sxx = cs * cs * v0 + sn * sn * v1;
+        syy = sn * sn * v0 + cs * cs * v1;
+        bounded = v0 > 0.0 && v1 > 0.0;
+    } else {
+        A = p0[i];
+        Bc = p1[i];
+        D = p2[i];
+        const double det = A * D - Bc * Bc;
+        bounded = A > 0.0 && det > 0.0;
+        sxx = D / det;
+        syy = A / det;
+    }
+    constexpr double k = -0.72134752044448170368;  // -0.5 * log2(e)
+    const float al = alphas[i];
+    const float px = position[2 * i], py = position[2 * i + 1];
+    r[0] = px;
+    r[1] = py;
+    r[2] = (float)(k * A);
+    r[3] = (float)(2.0 * k * Bc);
+    r[4] = (float)(k * D);
+    r[5] = al;
+    bool fin = isfinite(al) && isfinite(r[2]) && isfinite(r[3]) && isfinite(r[4]);
+    for (int c = 0; c < C; ++c) {
+        const float v = al * colors[i * C + c];
+        r[6 + c] = v;
+        fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
+    }
+    for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
+    boxes[(size_t)b * Np + n] = reach_box(px, py, sxx, syy, cull && bounded && fin);
+}
+
+// Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
+// opacity logit (unused), c_0..c_{C-1}] (reference src/igs/gs2d.py:635-644) and applies the
+// module's activations scales = exp(log_s) + eps, alpha = 1 (src/igs/gs2d.py:673-675), plus
+// an optional position offset (pos_map_offset, src/igs/gs2d.py:654-667).  Also writes the raw
+// colours [B][N][Cp] (zero-padded to the kernels' channel count) that the backward reads.
+__global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restrict__ feat,
+                                                           const float* __restrict__ pos_off, int N,
+                                                           int Np, int C, int Cp, int RS, float eps,
+                                                           float* __restrict__ packed,
+                                                           float4* __restrict__ boxes,
+                                                           float* __restrict__ colors_out, int cull) {
+    const int n = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (n >= Np) return;
+    float* r = packed + ((size_t)b * Np + n) * RS;
+    if (n >= N) {
+        for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        boxes[(size_t)b * Np + n] = empty_box();
+        return;
+    }
+    const size_t i = (size_t)b * N + n;
+    const float* f = feat + i * (6 + C);
+    const double s0 = (double)expf(f[2]) + (double)eps, s1 = (double)expf(f[3]) + (double)eps;
+    double sn, cs;
+    sincos((double)f[4], &sn, &cs);
+    const double v0 = s0 * s0 + (double)eps, v1 = s1 * s1 + (double)eps;
+    const double i0 = 1.0 / v0, i1 = 1.0 / v1;
+    const double A = cs * cs * i0 + sn * sn * i1;
+    const double Bc = cs * sn * (i0 - i1);
+    const double D = sn * sn * i0 + cs * cs * i1;
+    constexpr double k = -0.72134752044448170368;
+    float px = f[0], py = f[1];
+    if (pos_off) {
+        px += pos_off[2 * i];
+        py += pos_off[2 * i + 1];
+    }
+    r[0] = px;
+    r[1] = py;
+    r[2] = (float)(k * A);
+    r[3] = (float)(2.0 * k * Bc);
+    r[4] = (float)(k * D);
+    r[5] = 1.0f;
+    bool fin = isfinite(r[2]) && isfinite(r[3]) && isfinite(r[4]);
+    for (int c = 0; c < Cp; ++c) {
+        const float col = c < C ? f[6 + c] : 0.0f;
+        r[6 + c] = col;
+        colors_out[i * Cp + c] = col;
+        fin = fin && isfinite(col);
+    }
+    for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
+    boxes[(size_t)b * Np + n] = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
+                                          cull && fin && v0 > 0.0 && v1 > 0.0);
+}
+
+// ----------------------------------------------------------------------------- binning
+// Per pixel tile, the Gaussians whose reach box meets the tile's coordinate range, as a list
+// of indices in increasing order (so that sums over a list keep the order of the unculled
+// sum), and the count.  One workgroup per (tile, image) scans all N boxes; positions come
+// from ballots and a fixed-order prefix over the four waves, so the lists are reproducible.
+// With `slots` set, the inverse map is written as well: slots[b][tile][n] = position of
+// Gaussian n in the tile's list, or -1 when it is not listed (every n < N is written).
+// Separable grids only: a tile is tile_w columns x tile_h rows and its coordinate range is
+// [min, max] of x over its columns and of y over its rows (no monotonicity assumed).
+struct BinArgs {
+    const float4* boxes;  // [B][Np]
+    const float* x;
+    const float* y;
+    long sxb, sxw, syb, syh;
+    int N, Np, H, W;
+    int tile_w, tile_h, tiles_x, tiles_y;
+    int* counts;  // [B][tiles]
+    int* lists;   // [B][tiles][Np]
+    int* slots;   // [B][tiles][Np] or nullptr
+    const int* flag;
+    int want;
+};
+
+constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads in flight per tile
+
+__global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
+    if (a.flag != nullptr && *a.flag != a.want) return;
+    __shared__ float red[4][kBinThreads];
+    __shared__ int wsum[kBinWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tiles = a.tiles_x * a.tiles_y;
+    const int t = blockIdx.x, b = blockIdx.y;
+    const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
+    const int c0 = tx * a.tile_w, c1 = min(a.W, c0 + a.tile_w);
+    const int r0 = ty * a.tile_h, r1 = min(a.H, r0 + a.tile_h);
+    const float inf = __builtin_inff();
+    float xlo = inf, xhi = -inf, ylo = inf, yhi = -inf;
+    bool bad = false;
+    for (int c = c0 + tid; c < c1; c += kBinThreads) {
+        const float v = a.x[b * a.sxb + (long)c * a.sxw];
+        bad = bad || !(v == v);
+        xlo = fminf(xlo, v);
+        xhi = fmaxf(xhi, v);
+    }
+    for (int r = r0 + tid; r < r1; r += kBinThreads) {
+        const float v = a.y[b * a.syb + (long)r * a.syh];
+        bad = bad || !(v == v);
+        ylo = fminf(ylo, v);
+        yhi = fmaxf(yhi, v);
+    }
+    if (bad) {  // a NaN coordinate: nothing may be culled for this tile
+        xlo = ylo = -inf;
+        xhi = yhi = inf;
+    }
+    red[0][tid] = xlo;
+    red[1][tid] = -xhi;
+    red[2][tid] = ylo;
+    red[3][tid] = -yhi;
+    __syncthreads();
+    for (int k = kBinThreads / 2; k > 0; k >>= 1) {
+        if (tid < k) {
+#pragma unroll
+            for (int f = 0; f < 4; ++f) red[f][tid] = fminf(red[f][tid], red[f][tid + k]);
+        }
+        __syncthreads();
+    }
+    const float txlo = red[0][0], txhi = -red[1][0], tylo = red[2][0], tyhi = -red[3][0];
+    int* list = a.lists + ((size_t)b * tiles + t) * a.Np;
+    int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
+    const float4* boxes = a.boxes + (size_t)b * a.Np;
+    // Each wave scans one contiguous share of the Gaussians twice, without barriers: first to
+    // count, then (with the shares' counts prefixed in wave order) to write.
+    const int per_wave = ((a.N + kBinWaves - 1) / kBinWaves + 63) & ~63;
+    const int nb = wave * per_wave, ne = min(a.N, nb + per_wave);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    // kU boxes per lane are loaded together, so that kU loads are in flight instead of one
+    constexpr int kU = 8;
+    auto classify = [&](int n0, bool (&listed)[kU], bool (&in)[kU]) {
+        float4 bb[kU];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int n = n0 + u * 64 + lane;
+            bb[u] = boxes[min(n, a.N - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            in[u] = n0 + u * 64 + lane < ne;
+            // "definitely outside" negated, so that NaN bounds count as inside
+            listed[u] = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
+        }
+    };
+    int cnt = 0;
+    for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
+        bool listed[kU], in[kU];
+        classify(n0, listed, in);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) cnt += __popcll(__ballot(listed[u]));
+    }
+    if (lane == 0) wsum[wave] = cnt;
+    __syncthreads();
+    int base = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kBinWaves; ++w) {
+        if (w < wave) base += wsum[w];
+        total += wsum[w];
+    }
+    for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
+        bool listed[kU], in[kU];
+        classify(n0, listed, in);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int n = n0 + u * 64 + lane;
+            const unsigned long long m = __ballot(listed[u]);
+            const int pos = base + __popcll(m & below);
+            if (listed[u]) list[pos] = n;
+            if (slot != nullptr && in[u]) slot[n] = listed[u] ? pos : -1;
+            base += __popcll(m);
+        }
+    }
+    if (tid == 0) a.counts[(size_t)b * tiles + t] = total;
+}
