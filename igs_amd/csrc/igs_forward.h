@@ -37,7 +37,11 @@ template <int C>
 struct GRec {
     float px, py, A, B2, D, al;
     float ac[C];
+    float ylo, yhi;  // y range of the reach box (records with two spare floats only)
 };
+
+// whether a record of C channels has room for the y range of the reach box
+__host__ __device__ constexpr bool rec_has_yrange(int C) { return rec_stride_of(C) >= 8 + C; }
 
 // Unpacks one record held in R4 float4 registers (read from a wave-uniform LDS address).
 template <int C>
@@ -61,6 +65,12 @@ __device__ __forceinline__ GRec<C> lds_grec(const float4* r) {
     g.al = v[5];
 #pragma unroll
     for (int c = 0; c < C; ++c) g.ac[c] = v[6 + c];
+    if (rec_has_yrange(C)) {
+        g.ylo = v[6 + C];
+        g.yhi = v[7 + C];
+    } else {
+        g.ylo = g.yhi = 0.0f;
+    }
     return g;
 }
 
@@ -214,6 +224,18 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
 #pragma unroll
         for (int c = 0; c < C; ++c) num[p][c] = 0.0f;
     }
+    float wylo = yv[0], wyhi = yv[0];  // y range of this wave's rows (NaN-safe: see the test below)
+    bool ybad = !(yv[0] == yv[0]);
+#pragma unroll
+    for (int p = 1; p < P; ++p) {
+        wylo = fminf(wylo, yv[p]);
+        wyhi = fmaxf(wyhi, yv[p]);
+        ybad = ybad || !(yv[p] == yv[p]);
+    }
+    if (ybad) {
+        wylo = -__builtin_inff();
+        wyhi = __builtin_inff();
+    }
     // this tile's Gaussians (those whose reach box meets it), split S ways by list position
     const int s = blockIdx.y;
     const int count = a.counts[(size_t)b * per_img + tl];
@@ -222,8 +244,11 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     const int n1 = min(count, n0 + per);
     const int* list = a.lists + ((size_t)b * per_img + tl) * a.Np + n0;
     const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
-    stream_records_lds<R4, kGaussChunk, true>(src, n1 - n0, sh, [&](const float4* r) {
+    auto body = [&](auto wave_skip, const float4* r) {
         const GRec<C> g = lds_grec<C>(r);
+        // The tile list is per workgroup (4 waves of P rows each); a wave whose own rows the
+        // reach box misses skips the record (wave-uniform: the record is the same in all lanes).
+        if (decltype(wave_skip)::value && __ballot(!(g.yhi < wylo || g.ylo > wyhi)) == 0ull) return;
         const float dx = xv - g.px;
         const float adx = g.A * dx;
         const float c0 = adx * dx;
@@ -245,7 +270,16 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
 #pragma unroll
             for (int c = 0; c < C; ++c) num[p][c] = fmaf(e[p], g.ac[c], num[p][c]);
         }
-    }, list);
+    };
+    // The per-wave test costs a few percent when it never fires, so it is used only for tiles
+    // that fewer than 7/8 of the Gaussians reach (workgroup-uniform choice of the loop): there
+    // some boxes are small against the image, and those are often small against the tile too.
+    if (rec_has_yrange(C) && 8L * count < 7L * a.Np)
+        stream_records_lds<R4, kGaussChunk, true>(
+            src, n1 - n0, sh, [&](const float4* r) { body(std::true_type{}, r); }, list);
+    else
+        stream_records_lds<R4, kGaussChunk, true>(
+            src, n1 - n0, sh, [&](const float4* r) { body(std::false_type{}, r); }, list);
     if (col < a.W) {
 #pragma unroll
         for (int p = 0; p < P; ++p)

@@ -95,7 +95,12 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
     }
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
-    boxes[(size_t)b * Np + n] = reach_box(px, py, sxx, syy, cull && bounded && fin);
+    const float4 box = reach_box(px, py, sxx, syy, cull && bounded && fin);
+    boxes[(size_t)b * Np + n] = box;
+    if (RS >= 8 + C) {  // room in the record: the y range of the box travels with it
+        r[6 + C] = box.z;
+        r[7 + C] = box.w;
+    }
 }
 
 // Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
@@ -148,8 +153,13 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
         fin = fin && isfinite(col);
     }
     for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
-    boxes[(size_t)b * Np + n] = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
-                                          cull && fin && v0 > 0.0 && v1 > 0.0);
+    const float4 box = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
+                                 cull && fin && v0 > 0.0 && v1 > 0.0);
+    boxes[(size_t)b * Np + n] = box;
+    if (RS >= 8 + Cp) {
+        r[6 + Cp] = box.z;
+        r[7 + Cp] = box.w;
+    }
 }
 
 // ----------------------------------------------------------------------------- binning
