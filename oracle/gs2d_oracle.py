@@ -238,6 +238,25 @@ def operator_autograd(x, y, position, a, b_, d, alphas, colors, grad_out, eps=1e
 # --------------------------------------------------------------------------------------
 # scalar brute force (tiny inputs only) -- an independent pin for the vectorised code
 # --------------------------------------------------------------------------------------
+REACH_Q = 160.0 / (0.5 * math.log2(math.e))   # q beyond which the fp32 kernels' exp2 argument is < -160
+
+
+def reach_box(position, a, b_, d, q_max: float = REACH_Q):
+    """Axis-aligned bounding box of the ellipse q(dx, dy) = a dx^2 + 2 b dx dy + d dy^2 <= q_max
+    around each Gaussian, as (xlo, xhi, ylo, yhi) [...,4].  Textbook result: the extreme of dx on
+    the ellipse is sqrt(q_max * Sigma_xx) with Sigma = [[a, b], [b, d]]^-1, i.e.
+    Sigma_xx = d / (a d - b^2), Sigma_yy = a / (a d - b^2).  This is the test infrastructure's
+    restatement of the culling bound of the HIP pack kernels (no counterpart in the reference,
+    which evaluates every pair: src/igs/gs_triton_chunked.py:100-200); pixels outside the box
+    have q > q_max and therefore a weight of exactly zero in the fp32 kernels."""
+    a, b_, d = (t.reshape(position.shape[:-1]) for t in (a, b_, d))
+    det = a * d - b_ * b_
+    hx = torch.sqrt(q_max * d / det)
+    hy = torch.sqrt(q_max * a / det)
+    px, py = position[..., 0], position[..., 1]
+    return torch.stack([px - hx, px + hx, py - hy, py + hy], dim=-1)
+
+
 def brute_force_forward(x, y, position, a, b_, d, alphas, colors, eps=1e-6):
     """Plain Python triple loop over (image, pixel, gaussian) in Python floats (fp64)."""
     B, N, C = colors.shape

@@ -165,3 +165,62 @@ def test_operator_level_with_indefinite_cov_inverse(igs, dev, no_cull):
     ok = torch.isfinite(want) & torch.isfinite(out)
     assert float(ok.float().mean()) > 0.3
     torch.testing.assert_close(out[ok], want[ok], rtol=1e-4, atol=1e-5)
+
+
+def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev):
+    """The boxes behind the packed records (scale/rotation, cov-inverse and module-feature
+    packing) against the oracle's restatement: never inside it, and no more than the stated
+    outward rounding (1e-5 relative on the half extent) beyond it."""
+    from igs_amd._splat import Grid, Splat, _f32c
+
+    B, N, C = 2, 257, 3
+    d64, g = sparse_case(dev, B, N, 40, 72, C, seed=2, smin=0.003, smax=0.4)
+    grid = Grid(g["x_grid"], g["y_grid"], B)
+    op = Splat(B, N, C, grid, 1e-6, dev)
+    a, b, dd = O.cov_inverse_closed(d64["scales"].float().double(), d64["rotations"].float().double())
+    want = O.reach_box(d64["positions"].float().double(), a, b, dd).to(dev)
+
+    def boxes(packed):
+        p = op.plan
+        return packed[B * p.n_padded * p.rec_stride:].view(B, p.n_padded, 4)
+
+    col = _f32c(g["colors"])
+    cases = {"scale_rot": op.pack_scale_rot(_f32c(g["positions"]), _f32c(g["scales"]), _f32c(g["rotations"]),
+                                            _f32c(g["alphas"]), col)}
+    f = lambda t: t.to(dev, torch.float32).reshape(B, N).contiguous()
+    cases["covinv"] = op.pack_covinv(_f32c(g["positions"]), f(a), f(b), f(dd), _f32c(g["alphas"]), col)
+    feat = torch.cat([g["positions"], (g["scales"] - 1e-6).log(), g["rotations"][..., None],
+                      torch.zeros_like(g["rotations"])[..., None], g["colors"]], dim=-1).contiguous()
+    cases["feature"] = op.pack_feature(feat, None)[0]
+    half = torch.stack([want[..., 1] - want[..., 0], want[..., 3] - want[..., 2]], -1).repeat_interleave(2, -1) / 2
+    sign = torch.tensor([-1.0, 1.0, -1.0, 1.0], device=dev, dtype=torch.float64)
+    for name, packed in cases.items():
+        got = boxes(packed)[:, :N].double()
+        out = (got - want) * sign                      # how far outside the exact box each edge lies
+        # cov-inverse / feature inputs are fp32 roundings of the fp64 route: allow their error too
+        slack = 1e-4 if name != "scale_rot" else 3e-5
+        assert bool((out >= -slack * half).all()), (name, float((out / half).min()))
+        assert bool((out <= slack * half + 1e-6).all()), (name, float((out / half).max()))
+        pad = boxes(packed)[:, N:]
+        assert bool((pad[..., 0] > pad[..., 1]).all())  # padding records: empty boxes
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.bfloat16, torch.float16])
+def test_other_input_dtypes_round_trip(igs, dev, dtype):
+    """The kernels compute in fp32; other floating dtypes are converted on the way in and the
+    image and the gradients come back in the caller's dtype (the reference allocates its output
+    with the inputs' dtype, src/igs/gs_triton_chunked.py:606)."""
+    B, N, H, W, C = 1, 50, 20, 36, 3
+    _, g32 = sparse_case(dev, B, N, H, W, C, seed=9, smin=0.05, smax=0.3)
+    g = {k: v.to(dtype) for k, v in g32.items()}
+    g["x_grid"] = g["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+    g["y_grid"] = g["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+    out, grads = run(igs, g)
+    assert out.dtype == dtype and all(v.dtype == dtype for v in grads.values())
+    ref = {k: v.to(torch.float32) for k, v in g.items()}      # the same rounded values in fp32
+    ref["x_grid"] = ref["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+    ref["y_grid"] = ref["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+    out32, grads32 = run(igs, ref)
+    assert torch.equal(out, out32.to(dtype))
+    for k in NAMES:
+        assert torch.equal(grads[k], grads32[k].to(dtype)), k

@@ -262,3 +262,46 @@ def test_oracle_reproduces_golden_fixture():
         _, res = mg.compute(case)
         for k, v in res.items():
             assert np.allclose(v.numpy(), blob[f"{case}/{k}"], rtol=1e-11, atol=1e-14), (case, k)
+
+
+# ---------------------------------------------------------------- culling bound
+def test_reach_box_bounds_the_ellipse_tightly():
+    """Pins the bounding-box formula of the culling pass by brute force, not by retyping it:
+    the box must contain every point of the ellipse q <= Q (no point with q <= Q lies outside)
+    and touch it (the boundary point with the largest x sits on the box's right edge, same for
+    y), for rotated anisotropic Gaussians.  A swapped Sigma_xx/Sigma_yy, a wrong sign of the
+    rotation or a missing eps fails this."""
+    g = torch.Generator().manual_seed(7)
+    n = 64
+    sc = torch.rand(1, n, 2, generator=g, dtype=F64) * 0.3 + 0.005
+    rot = torch.rand(1, n, generator=g, dtype=F64) * 2 * math.pi
+    pos = torch.rand(1, n, 2, generator=g, dtype=F64) * 2 - 1
+    a, b, d = O.cov_inverse_closed(sc, rot)
+    a, b, d = (t.reshape(1, n) for t in (a, b, d))
+    Q = O.REACH_Q
+    assert math.isclose(-0.5 * math.log2(math.e) * Q, -160.0, rel_tol=1e-12)
+    box = O.reach_box(pos, a, b, d)
+    # points on the ellipse q = Q: p = pos + sqrt(Q) L^-T u(theta) with [[a,b],[b,d]] = L L^T
+    th = torch.linspace(0, 2 * math.pi, 20001, dtype=F64)
+    l11 = torch.sqrt(a)
+    l21 = b / l11
+    l22 = torch.sqrt(d - l21 * l21)
+    u, v = torch.cos(th), torch.sin(th)
+    dy = math.sqrt(Q) * v[None, None, :] / l22[..., None]
+    dx = (math.sqrt(Q) * u[None, None, :] - l21[..., None] * dy) / l11[..., None]
+    q = a[..., None] * dx * dx + 2 * b[..., None] * dx * dy + d[..., None] * dy * dy
+    assert torch.allclose(q, torch.full_like(q, Q), rtol=1e-9)
+    x, y = pos[..., 0, None] + dx, pos[..., 1, None] + dy
+    xlo, xhi, ylo, yhi = (box[..., k, None] for k in range(4))
+    tol = 1e-9
+    assert bool(((x >= xlo - tol) & (x <= xhi + tol) & (y >= ylo - tol) & (y <= yhi + tol)).all())   # contains
+    for ext, edge in ((x.max(-1).values, box[..., 1]), (x.min(-1).values, box[..., 0]),
+                      (y.max(-1).values, box[..., 3]), (y.min(-1).values, box[..., 2])):
+        assert torch.allclose(ext, edge, rtol=0, atol=1e-6 * float(edge.abs().max() + 1))           # tight
+    # and therefore: a point outside the box has q > Q
+    gx = torch.rand(1, n, 4000, generator=g, dtype=F64) * 8 - 4
+    gy = torch.rand(1, n, 4000, generator=g, dtype=F64) * 8 - 4
+    outside = (gx < xlo) | (gx > xhi) | (gy < ylo) | (gy > yhi)
+    ddx, ddy = gx - pos[..., 0, None], gy - pos[..., 1, None]
+    qq = a[..., None] * ddx * ddx + 2 * b[..., None] * ddx * ddy + d[..., None] * ddy * ddy
+    assert bool(outside.any()) and bool((qq[outside] > Q).all())
