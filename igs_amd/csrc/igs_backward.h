@@ -184,7 +184,10 @@ __host__ __device__ constexpr int pix_chunk(int C) { return C <= 4 ? IGS_PCHUNK 
 #define IGS_BWD_MAX_ROWS 32
 #endif
 constexpr int kBwdMaxRows = IGS_BWD_MAX_ROWS;
-constexpr int kBwdMinRows = 4;
+#ifndef IGS_BWD_MIN_ROWS
+#define IGS_BWD_MIN_ROWS 4
+#endif
+constexpr int kBwdMinRows = IGS_BWD_MIN_ROWS;
 #ifndef IGS_BWD_TILE_W
 #define IGS_BWD_TILE_W 64
 #endif

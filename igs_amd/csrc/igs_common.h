@@ -17,6 +17,9 @@ constexpr int kThreads = 256;
 #ifndef IGS_FWD_WAVES
 #define IGS_FWD_WAVES 8
 #endif
+#ifndef IGS_FWD_MAX_SPLIT
+#define IGS_FWD_MAX_SPLIT 64
+#endif
 #ifndef IGS_BWD_WAVES
 #define IGS_BWD_WAVES 16
 #endif

@@ -3,31 +3,33 @@
 #pragma once
 
 // Fixed-order sum over the T tile partials of NV consecutive fields for one Gaussian, spread
-// over the kFinT "t-lanes" of a workgroup laid out as kFinT t-lanes x kFinN Gaussians: t-lane k
-// adds tiles k, k+kFinT, ... in order, the lane sums are then added in order by every thread (so
+// over the FT "t-lanes" of a workgroup laid out as FT t-lanes x FN = 256/FT Gaussians: t-lane k
+// adds tiles k, k+FT, ... in order, the lane sums are then added in order by every thread (so
 // all t-lanes of a Gaussian hold the same, run-to-run identical value).  `red` is
-// [NV][kFinT][kFinN+1] floats of LDS.  Must be called by all 256 threads.  (8 x 32: with fewer
-// t-lanes the consecutive Gaussians of a wave read neighbouring columns of a tile's partials,
-// with more the sequential part of a sum over hundreds of tiles gets shorter.)
-#ifndef IGS_FIN_T
-#define IGS_FIN_T 8
+// [NV][FT][FN+1] floats of LDS.  Must be called by all 256 threads.  Two layouts are compiled:
+// 8 x 32 (the consecutive Gaussians of a wave read neighbouring columns of a tile's partials)
+// and, for problems too small to fill the device with that one, 32 x 8 (the sequential,
+// latency-bound part of a sum over hundreds of tiles gets 4 times shorter; timed against 16 and 64).
+#ifndef IGS_FIN_DEEP
+#define IGS_FIN_DEEP 32
 #endif
-constexpr int kFinT = IGS_FIN_T, kFinN = 256 / IGS_FIN_T;
+constexpr int kFinWide = 8, kFinDeep = IGS_FIN_DEEP;
 constexpr int kFinColours = 8;  // colour channels summed per pass (>= 6: the LDS array also serves the moments)
 
 // `part` is the image's partial array [T][NF][N]; the Gaussian's column in tile t is
 // slots[t * Np + n] when a slot table is given (negative: the tile holds nothing for it), else n.
 // Only the first `nv` (<= NV) of the fields are read.
-template <int NV>
+template <int NV, int FT>
 __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const int* __restrict__ slots,
                                          int Np, int n, int T, int NF, int N, int f0, bool valid,
                                          float (&out)[NV], float* red, int nv = NV) {
-    const int tl = threadIdx.x / kFinN, nl = threadIdx.x % kFinN;
+    constexpr int FN = 256 / FT;
+    const int tl = threadIdx.x / FN, nl = threadIdx.x % FN;
     float acc[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
     if (valid)
-        for (int t = tl; t < T; t += kFinT) {
+        for (int t = tl; t < T; t += FT) {
             const int col = slots ? slots[(size_t)t * Np + n] : n;
             if (col >= 0) {
 #pragma unroll
@@ -37,23 +39,23 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const i
         }
     __syncthreads();  // protects `red` against the previous call's readers
 #pragma unroll
-    for (int v = 0; v < NV; ++v) red[(v * kFinT + tl) * (kFinN + 1) + nl] = acc[v];
+    for (int v = 0; v < NV; ++v) red[(v * FT + tl) * (FN + 1) + nl] = acc[v];
     __syncthreads();
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         float s = 0.0f;
 #pragma unroll
-        for (int k = 0; k < kFinT; ++k) s += red[(v * kFinT + k) * (kFinN + 1) + nl];
+        for (int k = 0; k < FT; ++k) s += red[(v * FT + k) * (FN + 1) + nl];
         out[v] = s;
     }
 }
 
-// Finalize: 16 threads per Gaussian; sums the T tile partials in a fixed order and applies
+// Finalize: FT threads per Gaussian; sums the T tile partials in a fixed order and applies
 //   d alpha = M0, d color_c = alpha CG_c, d px = alpha (A Mx + B My), d py = alpha (B Mx + D My),
 //   dA = -1/2 alpha Mxx, dB = -alpha Mxy, dD = -1/2 alpha Myy,
 // and (function level) the chain rule through A = c^2 i0 + s^2 i1, B = c s (i0 - i1),
 // D = s^2 i0 + c^2 i1, i_k = 1/(s_k^2 + eps).
-template <bool kScaleRot>
+template <bool kScaleRot, int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
     const int* __restrict__ slots_in, int Np, const float* __restrict__ p0,
@@ -61,11 +63,12 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
     float* __restrict__ g_col) {
-    __shared__ float red[kFinColours * kFinT * (kFinN + 1)];
-    const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
+    constexpr int FN = 256 / FT;
+    __shared__ float red[kFinColours * FT * (FN + 1)];
+    const int n = blockIdx.x * FN + threadIdx.x % FN;
     const int b = blockIdx.y;
     const bool valid = n < N;
-    const bool writer = valid && threadIdx.x < kFinN;  // t-lane 0 writes the results
+    const bool writer = valid && threadIdx.x < FN;  // t-lane 0 writes the results
     // AUTO grid mode: T_in belongs to the separable plan, T_alt to the general one
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + C;
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
                            ? slots_in + (size_t)b * T * Np : nullptr;
     const int nn = min(n, N - 1);
     float M[6];
-    tile_sum<6>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+    tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
     const double al = alphas[i];
     // O(BN) epilogue in fp64: the chain rule multiplies sums by 1/s^3-sized factors
     double A, Bc, D, cs = 0., sn = 0., i0 = 0., i1 = 0., s0 = 0., s1 = 0.;
@@ -117,7 +120,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
         for (int c0 = 0; c0 < C; c0 += kFinColours) {  // colour sums, kFinColours channels per pass
             float sc[kFinColours];
             const int nc = min(kFinColours, C - c0);
-            tile_sum<kFinColours>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+            tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
             if (writer)
 #pragma unroll
                 for (int c = 0; c < kFinColours; ++c)
@@ -128,15 +131,17 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
 
 // Finalize for the fused module head: d gs_feature [B][N][6+C] from the tile partials, with
 // alpha = 1, d log_s_k = d s_k * exp(log_s_k) and a zero gradient for the unused opacity logit.
+template <int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
     const int* __restrict__ slots_in, int Np, const float* __restrict__ feat, int N, int C, int Cp,
     float eps, float* __restrict__ g_feat) {
-    __shared__ float red[kFinColours * kFinT * (kFinN + 1)];
-    const int n = blockIdx.x * kFinN + threadIdx.x % kFinN;
+    constexpr int FN = 256 / FT;
+    __shared__ float red[kFinColours * FT * (FN + 1)];
+    const int n = blockIdx.x * FN + threadIdx.x % FN;
     const int b = blockIdx.y;
     const bool valid = n < N;
-    const bool writer = valid && threadIdx.x < kFinN;
+    const bool writer = valid && threadIdx.x < FN;
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + Cp;
     const size_t i = (size_t)b * N + min(n, N - 1);
@@ -145,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
                            ? slots_in + (size_t)b * T * Np : nullptr;
     const int nn = min(n, N - 1);
     float M[6];
-    tile_sum<6>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+    tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
     const float* f = feat + i * (6 + C);
     const double e0 = (double)expf(f[2]), e1 = (double)expf(f[3]);
     const double s0 = e0 + (double)eps, s1 = e1 + (double)eps;
@@ -170,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     for (int c0 = 0; c0 < C; c0 += kFinColours) {
         float sc[kFinColours];
         const int nc = min(kFinColours, C - c0);
-        tile_sum<kFinColours>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+        tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
         if (writer)
 #pragma unroll
             for (int c = 0; c < kFinColours; ++c)

@@ -353,17 +353,51 @@ __global__ __launch_bounds__(kThreads) void k_fwd_combine(const float* __restric
                                                           float* __restrict__ out,
                                                           float* __restrict__ den,
                                                           const int* __restrict__ flag, int want) {
+    // 64 pixels x 4 channel lanes per workgroup: lane k sums channels k, k+4, ... (channel C is
+    // the denominator), the partials of 8 splits are loaded together; the pixel's denominator
+    // reaches the other lanes through LDS.
+    constexpr int kPix = 64, kLanes = kThreads / kPix, kBatch = 8;
+    __shared__ float dsh[kPix];
     if (flag != nullptr && *flag != want) return;
-    const int p = blockIdx.x * kThreads + threadIdx.x;
+    const int pl = threadIdx.x % kPix, k = threadIdx.x / kPix;
+    const int p = blockIdx.x * kPix + pl;
     const int b = blockIdx.y;
-    if (p >= HW) return;
-    float d = 0.0f;
-    for (int s = 0; s < S; ++s) d += part[(((size_t)s * B + b) * (C + 1) + C) * HW + p];
-    den[(size_t)b * HW + p] = d;
-    const float inv = 1.0f / (d + eps);
-    for (int c = 0; c < C; ++c) {
+    const bool valid = p < HW;
+    const int pc = min(p, HW - 1);
+    auto sum_channel = [&](int c) -> float {
+        const float* src = part + ((size_t)b * (C + 1) + c) * HW + pc;
+        const size_t stride = (size_t)B * (C + 1) * HW;
         float v = 0.0f;
-        for (int s = 0; s < S; ++s) v += part[(((size_t)s * B + b) * (C + 1) + c) * HW + p];
-        out[((size_t)b * C + c) * HW + p] = v * inv;
+        for (int s0 = 0; s0 < S; s0 += kBatch) {
+            float t[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) t[j] = s0 + j < S ? src[(size_t)(s0 + j) * stride] : 0.0f;
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) v += t[j];  // fixed order s = 0, 1, ...
+        }
+        return v;
+    };
+    constexpr int kMine = (IGS_MAX_CHANNELS + 1 + kLanes - 1) / kLanes;
+    float mine[kMine];
+#pragma unroll
+    for (int j = 0; j < kMine; ++j) {
+        const int c = k + j * kLanes;
+        mine[j] = 0.0f;
+        if (c <= C) {
+            mine[j] = sum_channel(c);
+            if (c == C) dsh[pl] = mine[j];
+        }
+    }
+    __syncthreads();
+    const float d = dsh[pl];
+    const float inv = 1.0f / (d + eps);
+#pragma unroll
+    for (int j = 0; j < kMine; ++j) {
+        const int c = k + j * kLanes;
+        if (!valid || c > C) continue;
+        if (c == C)
+            den[(size_t)b * HW + p] = d;
+        else
+            out[((size_t)b * C + c) * HW + p] = mine[j] * inv;
     }
 }

@@ -126,7 +126,7 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     long S = (target_waves + (long)fg.total_tiles * 4 - 1) / ((long)fg.total_tiles * 4);
     const long maxS = N / 64 > 0 ? N / 64 : 1;  // keep >= 64 Gaussians per split
     if (S > maxS) S = maxS;
-    if (S > 64) S = 64;
+    if (S > IGS_FWD_MAX_SPLIT) S = IGS_FWD_MAX_SPLIT;
     if (S < 1) S = 1;
     // Gaussians per split: a multiple of 4; drop splits that would be empty
     const int nps = (ceil_div(p->n_padded, S) + 3) & ~3;
@@ -470,7 +470,7 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
         IGS_DISPATCH_C(C, rc = launch_forward<kC>(a, sep, st));
         if (rc) return rc;
         if (a.S > 1) {
-            hipLaunchKernelGGL(k_fwd_combine, dim3(ceil_div((long)H * W, kThreads), B), dim3(kThreads),
+            hipLaunchKernelGGL(k_fwd_combine, dim3(ceil_div((long)H * W, 64), B), dim3(kThreads),
                                0, st, (const float*)ws, a.S, B, C, H * W, eps, out, den, a.flag, a.want);
             rc = launch_status();
             if (rc) return rc;
@@ -643,6 +643,21 @@ int igs_gs2d_backward_grid(const float* packed, const float* x, const float* y,
     return rc;
 }
 
+// Launches a finalize kernel in the layout that suits the problem size: 8 t-lanes x 32 Gaussians
+// per workgroup, or 32 x 8 when that would give fewer than two workgroups per compute unit.
+#define IGS_FINALIZE_LAUNCH(B, N, KERNEL, ...)                                                      \
+    do {                                                                                            \
+        if ((long)(B) * ceil_div((N), 256 / kFinWide) >= 512) {                                     \
+            constexpr int kFT = kFinWide;                                                           \
+            hipLaunchKernelGGL(KERNEL, dim3(ceil_div((N), 256 / kFT), (B)), dim3(kThreads), 0,      \
+                               __VA_ARGS__);                                                        \
+        } else {                                                                                    \
+            constexpr int kFT = kFinDeep;                                                           \
+            hipLaunchKernelGGL(KERNEL, dim3(ceil_div((N), 256 / kFT), (B)), dim3(kThreads), 0,      \
+                               __VA_ARGS__);                                                        \
+        }                                                                                           \
+    } while (0)
+
 // The slot tables that the separable backward left behind the partial sums (none on general grids).
 static const int* finalize_slots(const float* partial, int grid_mode, int B, int T, int NF, int N) {
     if (grid_mode == IGS_GRID_GENERAL) return nullptr;
@@ -676,7 +691,7 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     int T, T_alt;
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
     if (rc) return rc;
-    hipLaunchKernelGGL((k_bwd_finalize<false>), dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
+    IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<false, kFT>),
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), (N + 3) & ~3, cov_inv_00,
                        cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
@@ -695,7 +710,7 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     int T, T_alt;
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
     if (rc) return rc;
-    hipLaunchKernelGGL((k_bwd_finalize<true>), dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
+    IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<true, kFT>),
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), (N + 3) & ~3, scales, rotations,
                        (const float*)nullptr, alphas, N, C, eps, g_positions,
@@ -728,7 +743,7 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
     int T, T_alt;
     rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt);
     if (rc) return rc;
-    hipLaunchKernelGGL(k_bwd_finalize_feature, dim3(ceil_div(N, kFinN), B), dim3(kThreads), 0,
+    IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize_feature<kFT>),
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N), (N + 3) & ~3, gs_feature,
                        N, C, C_kernel, eps, g_feature);
