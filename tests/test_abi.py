@@ -178,3 +178,15 @@ def test_registered_operator_shape_functions(B, N, H, W, C):
     with pytest.raises(ValueError):
         torch.ops.igs_amd.splat_fwd(_splat.KIND_SCALE_ROT, [m(B, N, 2), m(B, N, C), m(B, N, 3), m(B, N), m(B, N)],
                                     *grids, 1e-6)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; with --gpus above 1 it exits with a message instead of running."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
