@@ -190,3 +190,42 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=120)
     assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_plan_invariants_over_random_shapes(lib):
+    """igs_gs2d_plan over a few hundred seeded random shapes (tiny to large, square to extreme
+    aspect ratios): every size positive and consistent, tiles cover the image, splits cover N."""
+    import random
+
+    from igs_amd import _lib
+
+    rng = random.Random(1234)
+    dims = [1, 2, 3, 7, 8, 9, 15, 16, 17, 31, 33, 63, 64, 65, 100, 127, 128, 129, 255, 256, 257, 384, 511, 640, 1000,
+            2048, 4099]
+    for _ in range(400):
+        B = rng.choice([1, 2, 3, 8, 16, 33])
+        N = rng.choice([1, 2, 3, 4, 5, 63, 64, 65, 100, 511, 512, 513, 2048, 8192, 32768, 100003])
+        H, W = rng.choice(dims), rng.choice(dims)
+        C = rng.choice(_lib.COMPILED_CHANNELS)
+        if B * N > 1 << 24:
+            continue
+        for mode in (0, 1, 2):
+            p = _lib.plan(B, N, H, W, C, mode)
+            Np = p.n_padded
+            assert Np % 4 == 0 and N <= Np < N + 4
+            assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
+            assert p.packed_bytes == B * Np * (p.rec_stride + 4) * 4
+            assert 1 <= p.fwd_split <= 64 and p.fwd_n_per_split % 4 == 0
+            assert p.fwd_split * p.fwd_n_per_split >= Np > (p.fwd_split - 1) * p.fwd_n_per_split
+            assert p.bwd_tiles >= 1 and p.bwd_per_tile >= 1
+            assert p.partial_bytes >= B * p.bwd_tiles * (6 + C) * N * 4
+            if mode != 0:
+                rows = p.bwd_tiles // p.bwd_tiles_x
+                assert p.bwd_tiles == rows * p.bwd_tiles_x and rows * p.bwd_per_tile >= H > (rows - 1) * p.bwd_per_tile
+                assert p.bwd_tiles_x * 64 >= p.w_padded >= W and p.w_padded % 8 == 0
+                assert p.fwd_tiles >= 1
+                assert p.fwd_ws_bytes >= B * p.fwd_tiles * (Np + 1) * 4
+                assert p.pix_bytes >= (B * H * p.w_padded * p.pix_stride + B * p.w_padded) * 4 + B * p.bwd_tiles * (Np + 1) * 4
+                assert p.partial_bytes >= B * p.bwd_tiles * ((6 + C) * N + Np) * 4      # + slot tables
+            else:
+                assert p.hw_padded % 4 == 0 and p.bwd_tiles * p.bwd_per_tile >= p.hw_padded >= H * W
