@@ -229,3 +229,26 @@ def test_plan_invariants_over_random_shapes(lib):
                 assert p.partial_bytes >= B * p.bwd_tiles * ((6 + C) * N + Np) * 4      # + slot tables
             else:
                 assert p.hw_padded % 4 == 0 and p.bwd_tiles * p.bwd_per_tile >= p.hw_padded >= H * W
+
+
+def test_header_is_valid_c_and_links_from_a_c_program(lib, tmp_path):
+    """include/igs_hip.h compiled as C (gcc -std=c99 -pedantic -Wall -Werror) by a program that
+    links the shared library and calls the plan entry point: the boundary is a C ABI, usable
+    without C++ or Python."""
+    import os
+    import subprocess
+
+    from igs_amd import _lib
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = str(tmp_path / "plan_from_c")
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-I", os.path.join(root, "include"),
+                    os.path.join(root, "tests", "c_abi", "plan_from_c.c"), "-o", exe, "-L", libdir, "-ligs_hip",
+                    "-Wl,-rpath," + libdir], check=True, capture_output=True, text=True, timeout=120)
+    r = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=60)
+    first, second = r.stdout.strip().splitlines()
+    p = _lib.plan(16, 8192, 256, 256, 3, _lib.IGS_GRID_SEPARABLE)
+    assert [int(v) for v in first.split()] == [_lib.ABI_VERSION, p.n_padded, p.rec_stride, p.bwd_tiles, p.packed_bytes,
+                                               p.fwd_ws_bytes, p.pix_bytes, p.partial_bytes]
+    assert second.startswith("-2 ")
