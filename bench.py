@@ -11,7 +11,7 @@ B=16, N=8192, 256x256, C=3, fp32.  Prints ONE JSON line:
   cpu_baseline : the chunked torch autograd path of the reference restated on the CPU
                  (oracle/chunked_cpu.py), timed on this box's host cores on a bounded sample.
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu]
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu] | --all | --sweep
 """
 from __future__ import annotations
 
@@ -43,6 +43,9 @@ def main() -> int:
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the JSON line, print the operator-level table of the reference's "
                          "scripts/profiling.py (B x N x H sweep, median of 32 timed calls after 4 warm-ups)")
+    ap.add_argument("--all", action="store_true",
+                    help="instead of the JSON line, print forward and forward+backward times of all five "
+                         "configurations (c0-c4; c3 is the module, c2 also as the fused fit step)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
@@ -54,6 +57,8 @@ def main() -> int:
 
     if args.sweep:
         return sweep()
+    if args.all:
+        return all_configs(args.steps, args.warmup)
 
     import torch
 
@@ -202,6 +207,81 @@ def main() -> int:
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args.config, O)
     print(json.dumps(result), flush=True)
+    return 0
+
+
+def all_configs(steps: int, warmup: int) -> int:
+    """Forward and forward+backward wall time of the five configurations through the public API
+    (allocation included), pairs/s counting all B N H W pairs as scripts/profiling.py:199-211 does,
+    and the fraction of the fp32 vector peak by the 42 + 6 C FLOP/pair model (above 1 is possible
+    where culling skips pairs)."""
+    import torch
+
+    import igs_amd
+    from igs_amd.fit import GaussianImageFit
+    from oracle import gs2d_oracle as O
+
+    dev = torch.device("cuda:0")
+    names = ("positions", "colors", "scales", "rotations", "alphas")
+
+    def timeit(fn, n):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    rows = []
+    for cfg in ("c0", "c1", "c2", "c3", "c4"):
+        if cfg == "c3":
+            torch.manual_seed(1003)
+            m = igs_amd.GaussianSplatting2D(32, 1024).to(dev)
+            x = torch.randn(8, 128, 1024, device=dev, requires_grad=True)
+            go = torch.randn(8, 3, 256, 256, device=dev)
+            B, N, H, W, C = 8, 4096, 256, 256, 3
+
+            def fwd():
+                with torch.no_grad():
+                    m(x, size=(256, 256))
+
+            def step():
+                m(x, size=(256, 256))[0].backward(go)
+                x.grad = None
+                m.zero_grad(set_to_none=True)
+        else:
+            d = {k: v.to(dev) for k, v in O.make_config_inputs(cfg).items()}
+            B, N, C = d["colors"].shape
+            H, W = d["x_grid"].shape[-2:]
+            d["x_grid"] = d["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+            d["y_grid"] = d["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+            lv = {k: d[k].clone().requires_grad_(True) for k in names}
+
+            def fwd(d=d, lv=lv):
+                with torch.no_grad():
+                    igs_amd.gaussian_splatting_2d(*(lv[k] for k in names), d["x_grid"], d["y_grid"])
+
+            def step(d=d, lv=lv):
+                igs_amd.gaussian_splatting_2d(*(lv[k] for k in names), d["x_grid"], d["y_grid"]).backward(d["grad_out"])
+                for v in lv.values():
+                    v.grad = None
+        n = max(3, steps // 3) if cfg == "c4" else steps
+        rows.append((cfg, B, N, H, W, C, timeit(fwd, n), timeit(step, n)))
+        if cfg == "c2":   # the fused fit iteration (render, MSE, backward, AdamW) on the same problem
+            block = torch.cat([d["positions"], d["scales"].log(), d["rotations"][..., None],
+                               torch.zeros_like(d["rotations"])[..., None], d["colors"]], -1)
+            fit = GaussianImageFit(block, O.smooth_noise_target(H, W, seed=1002).to(dev), d["x_grid"], d["y_grid"],
+                                   lr=min(0.05 * 4096 / N, 0.03))
+            fit.capture()
+            rows.append(("c2 fit step", B, N, H, W, C, float("nan"), timeit(fit.step, n)))
+    print("%-12s %3s %6s %4s %4s %3s %10s %12s %14s %10s" % ("config", "B", "N", "H", "W", "C", "fwd ms", "fwd+bwd ms",
+                                                           "pairs/s", "of peak"))
+    for cfg, B, N, H, W, C, tf, t in rows:
+        pairs = B * N * H * W
+        print("%-12s %3d %6d %4d %4d %3d %10.3f %12.3f %14.3e %10.2f" % (cfg, B, N, H, W, C, tf * 1e3, t * 1e3, pairs / t,
+                                                                       pairs * (42 + 6 * C) / t / 1e12 / FP32_VECTOR_PEAK_TFLOPS))
     return 0
 
 
