@@ -42,6 +42,20 @@ def naive_gaussian_2d(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas
 # --------------------------------------------------------------------------------------
 # operator level: the `.apply` plugin boundary of the reference
 # --------------------------------------------------------------------------------------
+def _degenerate(params, x_grid, B, N, C, dtype):
+    """No Gaussian, no image or no pixel: the plain expression (src/igs/gs2d.py:24-44) gives an
+    all-zero [B,C,H,W] image (den = 0, 0 / (0 + eps) = 0) and zero gradients; there is nothing
+    to launch.  Returns None for a real problem."""
+    H, W = x_grid.shape[-2:]
+    if B and N and H and W:
+        return None
+    out = torch.zeros(B, C, H, W, dtype=dtype, device=params[0].device)
+    for p in params:   # keeps the result attached to its inputs (their gradients are zeros)
+        if p.requires_grad:
+            out = out + p.sum() * 0
+    return out
+
+
 def _as(t: Tensor, dtype) -> Tensor:
     return t if t.dtype == dtype else t.to(dtype)
 
@@ -102,6 +116,10 @@ class GaussianSplatting2DKernel:
     @staticmethod
     def apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
         C = colors.shape[-1]
+        empty = _degenerate((position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors), x, position.shape[0],
+                            position.shape[1], C, x.dtype)
+        if empty is not None:
+            return empty
         if C > _lib.IGS_MAX_CHANNELS:
             return torch.cat([GaussianSplatting2DKernel.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11,
                                                               alphas, colors[..., lo:hi], eps)
@@ -188,6 +206,10 @@ class _RenderFromFeature(torch.autograd.Function):
 
 
 def _render_fused(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps):
+    empty = _degenerate((positions, colors, scales, rotations, alphas), x_grid, positions.shape[0],
+                        positions.shape[1], colors.shape[-1], positions.dtype)
+    if empty is not None:
+        return empty
     if torch.compiler.is_compiling():
         return _ops.splat(KIND_SCALE_ROT, [positions, colors, scales, rotations, alphas], x_grid, y_grid, eps,
                           colors.shape[-1], positions.dtype)
@@ -195,6 +217,10 @@ def _render_fused(positions, colors, scales, rotations, alphas, x_grid, y_grid, 
 
 
 def _render_from_feature(gs_feature, pos_offset, x_grid, y_grid, eps):
+    empty = _degenerate((gs_feature,) if pos_offset is None else (gs_feature, pos_offset), x_grid,
+                        gs_feature.shape[0], gs_feature.shape[1], gs_feature.shape[-1] - 6, gs_feature.dtype)
+    if empty is not None:
+        return empty
     if torch.compiler.is_compiling():
         params = [gs_feature] if pos_offset is None else [gs_feature, pos_offset]
         return _ops.splat(KIND_FEATURE, params, x_grid, y_grid, eps, gs_feature.shape[-1] - 6, gs_feature.dtype)

@@ -252,3 +252,28 @@ def test_header_is_valid_c_and_links_from_a_c_program(lib, tmp_path):
     assert [int(v) for v in first.split()] == [_lib.ABI_VERSION, p.n_padded, p.rec_stride, p.bwd_tiles, p.packed_bytes,
                                                p.fwd_ws_bytes, p.pix_bytes, p.partial_bytes]
     assert second.startswith("-2 ")
+
+
+def test_empty_inputs_give_the_plain_expression_s_result():
+    """No Gaussians, no images or no pixels: zeros / empty of the right shape, zero gradients --
+    what the plain expression (fused=False) gives; nothing is launched, so this runs anywhere."""
+    import torch
+
+    import igs_amd
+
+    z = lambda *s: torch.zeros(*s, requires_grad=True)
+    for (B, N, H, W, C) in [(2, 0, 4, 5, 3), (0, 7, 4, 5, 3), (1, 7, 0, 5, 2), (1, 7, 4, 0, 1)]:
+        p, c, s, r, a = z(B, N, 2), z(B, N, C), torch.ones(B, N, 2), torch.zeros(B, N), torch.ones(B, N)
+        x, y = torch.zeros(B, 1, H, W), torch.zeros(B, 1, H, W)
+        out = igs_amd.gaussian_splatting_2d(p, c, s, r, a, x, y)
+        assert out.shape == (B, C, H, W) and float(out.detach().abs().sum()) == 0.0
+        if B and H and W:
+            want = igs_amd.gaussian_splatting_2d(p, c, s, r, a, x, y, fused=False)
+            assert torch.equal(out, want)
+        out.sum().backward()
+        assert p.grad.shape == p.shape and c.grad.shape == c.shape and float(c.grad.abs().sum()) == 0.0
+        cov = torch.ones(B, N, 1, 1)
+        assert igs_amd.GaussianSplatting2DKernel.apply(x, y, p, cov, cov * 0, cov, a, c).shape == (B, C, H, W)
+    m = igs_amd.GaussianSplatting2D(4, 8)
+    img, feat = m(torch.zeros(2, 0, 8), size=(4, 6))       # no features -> no Gaussians
+    assert img.shape == (2, 3, 4, 6) and feat.shape == (2, 0, 9) and float(img.detach().abs().sum()) == 0.0
