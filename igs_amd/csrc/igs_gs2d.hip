@@ -66,6 +66,7 @@ bool shape_ok(int B, int N, int H, int W) {
     if (B <= 0 || N <= 0 || H <= 0 || W <= 0) return false;
     if (B > 65535) return false;
     if ((long)H * W > (1L << 28) || (long)B * N > (1L << 28)) return false;
+    if (N > (1 << 24)) return false;  // list-position groups of the backward are a 16-bit grid dimension
     return true;
 }
 

@@ -32,7 +32,8 @@ typedef void *igs_stream_t; /* a hipStream_t */
 typedef enum igs_status {
     IGS_OK = 0,
     IGS_ERR_NULL_POINTER = -1,
-    IGS_ERR_BAD_SHAPE = -2,      /* a dimension <= 0 or too large for 32-bit indexing */
+    IGS_ERR_BAD_SHAPE = -2,      /* a dimension <= 0 or too large: B <= 65535, N <= 2^24,
+                                    B*N <= 2^28, H*W <= 2^28 */
     IGS_ERR_BAD_CHANNELS = -3,   /* C outside 1..IGS_MAX_CHANNELS */
     IGS_ERR_WORKSPACE = -4,      /* a workspace is smaller than igs_gs2d_plan says */
     IGS_ERR_BAD_MODE = -5,       /* unknown grid mode */
