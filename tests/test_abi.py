@@ -93,6 +93,13 @@ def test_argument_errors_are_status_codes_not_crashes(lib):
     assert lib.igs_gs2d_plan(1, 8, 4, 4, 5, 1, ctypes.byref(p)) == -3     # not a compiled channel count
     assert lib.igs_gs2d_plan(1, 8, 4, 4, 3, 7, ctypes.byref(p)) == -5
     assert lib.igs_gs2d_plan(1, 8, 4, 4, 3, 1, None) == -1
+    # size limits: B <= 65535, N <= 2^24, B N <= 2^28, H W <= 2^28
+    assert lib.igs_gs2d_plan(65536, 8, 4, 4, 3, 1, ctypes.byref(p)) == -2
+    assert lib.igs_gs2d_plan(1, (1 << 24) + 1, 4, 4, 3, 1, ctypes.byref(p)) == -2
+    assert lib.igs_gs2d_plan(32, 1 << 24, 4, 4, 3, 1, ctypes.byref(p)) == -2
+    assert lib.igs_gs2d_plan(1, 8, 1 << 14, (1 << 14) + 1, 3, 1, ctypes.byref(p)) == -2
+    assert lib.igs_gs2d_plan(1, 1 << 24, 64, 64, 3, 1, ctypes.byref(p)) == 0
+    assert lib.igs_gs2d_plan(1, 8, 1 << 14, 1 << 14, 3, 1, ctypes.byref(p)) == 0
     # null pointers are rejected before anything is launched
     st = _lib.strides6((0, 0, 1), (0, 4, 0))
     assert lib.igs_gs2d_forward(None, None, None, st, 1, None, 1, 8, 4, 4, 3, 1e-6, None, None, None, 0, None) == -1
