@@ -16,9 +16,11 @@ from .gs2d import (  # noqa: F401
 )
 
 from .fit import GaussianImageFit  # noqa: F401,E402
+from .reg import koleo_diversity_loss  # noqa: F401,E402
 
 __all__ = [
     "GaussianImageFit",
+    "koleo_diversity_loss",
     "GaussianSplatting2D",
     "gaussian_splatting_2d",
     "naive_gaussian_2d",

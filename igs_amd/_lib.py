@@ -14,7 +14,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 LIB_PATH = os.environ.get("IGS_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "libigs_hip.so")
 
-ABI_VERSION = 2  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
+ABI_VERSION = 3  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1
 IGS_GRID_AUTO = 2
@@ -42,6 +42,19 @@ class Plan(ctypes.Structure):
         ("partial_bytes", c_uint64),
         ("fwd_tiles", c_int32),
         ("bwd_tiles_x", c_int32),
+    ]
+
+
+class KoleoPlan(ctypes.Structure):
+    """Mirror of igs_koleo_plan_t."""
+
+    _fields_ = [
+        ("B", c_int32), ("N", c_int32), ("D", c_int32),
+        ("d_padded", c_int32),
+        ("splits", c_int32),
+        ("tiles_per_split", c_int32),
+        ("saved_bytes", c_uint64),
+        ("scratch_bytes", c_uint64),
     ]
 
 
@@ -78,6 +91,9 @@ SIGNATURES = {
                                                c_int, c_int, c_int, c_float, _FP, c_size_t, _FP, c_size_t, _FP,
                                                c_void_p]),
     "igs_adamw_step": (c_int, [_FP, _FP, _FP, _FP, c_int64, _FP, c_float, c_float, c_float, c_float, c_void_p]),
+    "igs_koleo_plan": (c_int, [c_int, c_int, c_int, POINTER(KoleoPlan)]),
+    "igs_koleo_forward": (c_int, [_FP, c_int, c_int, c_int, _FP, _FP, c_size_t, _FP, c_size_t, c_void_p]),
+    "igs_koleo_backward": (c_int, [_FP, c_size_t, _FP, c_int, c_int, c_int, _FP, c_void_p]),
 }
 
 _lib = None
@@ -123,6 +139,14 @@ def plan(B: int, N: int, H: int, W: int, C: int, grid_mode: int) -> Plan:
     training loops ask for the same shape every step).  Treat the result as read-only."""
     p = Plan()
     check(load().igs_gs2d_plan(B, N, H, W, C, grid_mode, ctypes.byref(p)), "igs_gs2d_plan")
+    return p
+
+
+@functools.lru_cache(maxsize=64)
+def koleo_plan(B: int, N: int, D: int) -> KoleoPlan:
+    """Buffer sizes of the diversity loss for a [B, N, D] feature block (cached; read-only)."""
+    p = KoleoPlan()
+    check(load().igs_koleo_plan(B, N, D, ctypes.byref(p)), "igs_koleo_plan")
     return p
 
 

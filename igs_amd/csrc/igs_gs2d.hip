@@ -46,6 +46,7 @@ namespace {
 #include "igs_fit.h"
 #include "igs_finalize.h"
 #include "igs_grid.h"
+#include "igs_koleo.h"
 
 // ----------------------------------------------------------------------------- host side
 int g_cached_cus = 0;
@@ -748,6 +749,101 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N), (N + 3) & ~3, gs_feature,
                        N, C, C_kernel, eps, g_feature);
+    return launch_status();
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------ KoLeo diversity loss
+namespace {
+// saved buffer: fn [B N Dp] | norm [B N] | nn_val [B N] | nn_idx [B N], each part 16-byte aligned
+struct KoleoSaved {
+    float* fn;
+    float* norm;
+    float* nn_val;
+    int* nn_idx;
+};
+
+inline size_t koleo_rows_padded(long rows) { return (size_t)((rows + 3) & ~3L); }
+
+KoleoSaved koleo_saved(void* saved, const igs_koleo_plan_t& p) {
+    const long rows = (long)p.B * p.N;
+    KoleoSaved s;
+    s.fn = reinterpret_cast<float*>(saved);
+    s.norm = s.fn + (size_t)rows * p.d_padded;
+    s.nn_val = s.norm + koleo_rows_padded(rows);
+    s.nn_idx = reinterpret_cast<int*>(s.nn_val + koleo_rows_padded(rows));
+    return s;
+}
+
+int koleo_plan(int B, int N, int D, igs_koleo_plan_t* p) {
+    if (!p) return IGS_ERR_NULL_POINTER;
+    if (B <= 0 || B > 65535 || N < 2 || D <= 0 || D > (1 << 20)) return IGS_ERR_BAD_SHAPE;
+    const int Dp = (D + 3) & ~3;
+    if ((long)B * N > (1L << 28) || (long)B * N * Dp > (1L << 31)) return IGS_ERR_BAD_SHAPE;
+    const int cus = device_cus() > 0 ? device_cus() : 256;
+    const int tiles = ceil_div(N, kKoleoTile);
+    // enough workgroups for two per compute unit, by splitting the columns
+    int S = ceil_div(2L * cus, (long)tiles * B);
+    S = S < 1 ? 1 : (S > tiles ? tiles : S);
+    const int per = ceil_div(tiles, S);
+    S = ceil_div(tiles, per);
+    const long rows = (long)B * N;
+    p->B = B;
+    p->N = N;
+    p->D = D;
+    p->d_padded = Dp;
+    p->splits = S;
+    p->tiles_per_split = per;
+    p->saved_bytes = ((size_t)rows * Dp + 3 * koleo_rows_padded(rows)) * sizeof(float);
+    const size_t blocks = (size_t)ceil_div(rows, kThreads);
+    p->scratch_bytes = ((blocks + 1) & ~(size_t)1) * sizeof(double) + (size_t)B * S * N * 2 * sizeof(float);
+    return IGS_OK;
+}
+}  // namespace
+
+extern "C" {
+int igs_koleo_plan(int B, int N, int D, igs_koleo_plan_t* plan) { return koleo_plan(B, N, D, plan); }
+
+int igs_koleo_forward(const float* features, int B, int N, int D, float* loss, void* saved,
+                      size_t saved_bytes, void* scratch, size_t scratch_bytes, igs_stream_t stream) {
+    if (!features || !loss || !saved || !scratch) return IGS_ERR_NULL_POINTER;
+    igs_koleo_plan_t p;
+    int rc = koleo_plan(B, N, D, &p);
+    if (rc) return rc;
+    if (saved_bytes < p.saved_bytes || scratch_bytes < p.scratch_bytes) return IGS_ERR_WORKSPACE;
+    if (((uintptr_t)saved | (uintptr_t)scratch) & 15) return IGS_ERR_ALIGNMENT;
+    const KoleoSaved sv = koleo_saved(saved, p);
+    const long rows = (long)B * N;
+    const int blocks = ceil_div(rows, kThreads);
+    double* loss_part = reinterpret_cast<double*>(scratch);
+    float* part_val = reinterpret_cast<float*>(loss_part + ((blocks + 1) & ~1));
+    int* part_idx = reinterpret_cast<int*>(part_val + (size_t)B * p.splits * N);
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_koleo_normalize, dim3(ceil_div(rows, kThreads / 64)), dim3(kThreads), 0, st,
+                       features, rows, D, p.d_padded, sv.fn, sv.norm);
+    hipLaunchKernelGGL(k_koleo_nn, dim3(ceil_div(N, kKoleoTile), p.splits, B), dim3(kThreads), 0, st,
+                       (const float*)sv.fn, N, p.d_padded, p.tiles_per_split, part_val, part_idx);
+    hipLaunchKernelGGL(k_koleo_combine, dim3(blocks), dim3(kThreads), 0, st, (const float*)part_val,
+                       (const int*)part_idx, B, N, p.splits, sv.nn_val, sv.nn_idx, loss_part);
+    hipLaunchKernelGGL(k_koleo_sum, dim3(1), dim3(kThreads), 0, st, (const double*)loss_part, blocks,
+                       1.0 / (double)rows, loss);
+    return launch_status();
+}
+
+int igs_koleo_backward(const void* saved, size_t saved_bytes, const float* grad_loss, int B, int N,
+                       int D, float* grad_features, igs_stream_t stream) {
+    if (!saved || !grad_loss || !grad_features) return IGS_ERR_NULL_POINTER;
+    igs_koleo_plan_t p;
+    int rc = koleo_plan(B, N, D, &p);
+    if (rc) return rc;
+    if (saved_bytes < p.saved_bytes) return IGS_ERR_WORKSPACE;
+    if ((uintptr_t)saved & 15) return IGS_ERR_ALIGNMENT;
+    const KoleoSaved sv = koleo_saved(const_cast<void*>(saved), p);
+    const int rows_per_block = (kThreads / 64) * kKoleoBwdRows;
+    hipLaunchKernelGGL(k_koleo_bwd, dim3(ceil_div(N, rows_per_block), B), dim3(kThreads), 0,
+                       (hipStream_t)stream, (const float*)sv.fn, (const float*)sv.norm,
+                       (const int*)sv.nn_idx, grad_loss, B, N, D, p.d_padded, grad_features);
     return launch_status();
 }
 

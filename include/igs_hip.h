@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define IGS_ABI_VERSION 2
+#define IGS_ABI_VERSION 3
 #define IGS_MAX_CHANNELS 16
 
 typedef void *igs_stream_t; /* a hipStream_t */
@@ -235,6 +235,37 @@ int igs_gs2d_backward_prologue_mse(const float *x, const float *y, const int64_t
 int igs_adamw_step(float *param, const float *grad, float *exp_avg, float *exp_avg_sq,
                    int64_t count, float *state, float beta1, float beta2, float eps,
                    float weight_decay, igs_stream_t stream);
+
+/* ---- KoLeo diversity loss (src/igs/reg.py:5-40) ---------------------------------------------
+ * loss = mean over the B*N rows of relu(max_{j != i} cos(x_i, x_j) + 1), features [B,N,D] fp32
+ * contiguous.  The reference normalises the rows, forms the [B,N,N] similarity matrix with bmm,
+ * fills its diagonal with -inf and takes the row maxima; these entry points compute the same
+ * maxima tile by tile and never hold the matrix.  Equal similarities resolve to the lowest
+ * column index; every sum has a fixed order (results are bit-reproducible).  N >= 2 (the
+ * reference returns a constant 0 for N <= 1, src/igs/reg.py:19-20: callers handle that case). */
+typedef struct igs_koleo_plan_t {
+    int32_t B, N, D;
+    int32_t d_padded;        /* floats per normalised row (D rounded up to 4)                 */
+    int32_t splits;          /* column splits of the similarity tiles (>= 1)                  */
+    int32_t tiles_per_split; /* 64-column tiles per split                                      */
+    uint64_t saved_bytes;    /* kept from forward to backward: normalised rows, norms, nearest
+                                similarity and neighbour index per row                        */
+    uint64_t scratch_bytes;  /* forward only: per-split maxima, per-workgroup loss sums       */
+} igs_koleo_plan_t;
+
+int igs_koleo_plan(int B, int N, int D, igs_koleo_plan_t *plan);
+
+/* Forward: writes *loss (one float of device memory) and fills `saved` (plan.saved_bytes,
+ * 16-byte aligned) for the backward.  Replaces src/igs/reg.py:22-37. */
+int igs_koleo_forward(const float *features, int B, int N, int D, float *loss, void *saved,
+                      size_t saved_bytes, void *scratch, size_t scratch_bytes, igs_stream_t stream);
+
+/* Backward: grad_features [B,N,D] = grad_loss[0] * d loss / d features from the forward's
+ * `saved` buffer (what autograd derives from src/igs/reg.py:22-37: the gradient reaches a row
+ * through its own nearest neighbour and through the rows whose nearest neighbour it is, then
+ * through the normalisation).  grad_loss is one float of device memory. */
+int igs_koleo_backward(const void *saved, size_t saved_bytes, const float *grad_loss, int B, int N,
+                       int D, float *grad_features, igs_stream_t stream);
 
 #ifdef __cplusplus
 }
