@@ -46,6 +46,9 @@ def main() -> int:
     ap.add_argument("--all", action="store_true",
                     help="instead of the JSON line, print forward and forward+backward times of all five "
                          "configurations (c0-c4; c3 is the module, c2 also as the fused fit step)")
+    ap.add_argument("--koleo", action="store_true",
+                    help="instead of the JSON line, print forward and forward+backward times of the KoLeo "
+                         "diversity loss (src/igs/reg.py of the reference) beside the plain torch expression")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
@@ -59,6 +62,8 @@ def main() -> int:
         return sweep()
     if args.all:
         return all_configs(args.steps, args.warmup)
+    if args.koleo:
+        return koleo_table(args.no_cpu)
 
     import torch
 
@@ -282,6 +287,64 @@ def all_configs(steps: int, warmup: int) -> int:
         pairs = B * N * H * W
         print("%-12s %3d %6d %4d %4d %3d %10.3f %12.3f %14.3e %10.2f" % (cfg, B, N, H, W, C, tf * 1e3, t * 1e3, pairs / t,
                                                                        pairs * (42 + 6 * C) / t / 1e12 / FP32_VECTOR_PEAK_TFLOPS))
+    return 0
+
+
+def koleo_table(no_cpu: bool) -> int:
+    """KoLeo diversity loss: events around `koleo_diversity_loss(x)` and around loss + backward (4 warm-ups,
+    median of 32), for the two shapes scripts/gs2d_test.py:146,172 of the reference passes ([1, N, 9] Gaussian
+    features, [1, k <= 128, 512] latent features) and larger ones; beside it the same expression in eager fp32
+    torch on the GPU (the oracle's restatement of src/igs/reg.py:22-37, which holds the [B,N,N] matrix; skipped
+    above 4 GiB) and on the host cores.  FLOP model: 2 B N^2 D for the similarities (forward)."""
+    import torch
+
+    import igs_amd
+    from oracle import koleo_oracle as K
+
+    dev = torch.device("cuda:0")
+
+    def median_ms(fn):
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(32):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        return sorted(ts)[len(ts) // 2]
+
+    def both(loss_fn, x):
+        xg = x.clone().requires_grad_(True)
+
+        def step():
+            xg.grad = None
+            loss_fn(xg).backward()
+
+        with torch.no_grad():
+            f = median_ms(lambda: loss_fn(x))
+        return f, median_ms(step)
+
+    print("%-16s %10s %10s %12s %12s %12s %10s" % ("B x N x D", "fwd ms", "f+b ms", "torch fwd", "torch f+b",
+                                                   "TFLOP/s fwd", "cpu f+b ms"))
+    for shape in [(1, 128, 512), (1, 4096, 9), (8, 4096, 9), (1, 16384, 9), (4, 16384, 32), (1, 65536, 9)]:
+        B, N, D = shape
+        x = torch.randn(*shape, device=dev, generator=torch.Generator(dev).manual_seed(0))
+        f, fb = both(igs_amd.koleo_diversity_loss, x)
+        tf = tfb = float("nan")
+        if B * N * N * 4 <= 4 << 30:
+            tf, tfb = both(K.koleo_diversity_loss, x)
+        cpu = float("nan")
+        if not no_cpu and B * N * N <= 1 << 28:
+            xc = x.cpu()
+            t0 = time.perf_counter()
+            K.autograd_gradient(xc)
+            cpu = (time.perf_counter() - t0) * 1e3
+        print("%-16s %10.4f %10.4f %12.4f %12.4f %12.2f %10.1f" % ("%dx%dx%d" % shape, f, fb, tf, tfb,
+                                                                  2.0 * B * N * N * D / (f * 1e-3) / 1e12, cpu))
     return 0
 
 

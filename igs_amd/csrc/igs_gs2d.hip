@@ -782,8 +782,11 @@ int koleo_plan(int B, int N, int D, igs_koleo_plan_t* p) {
     const int Dp = (D + 3) & ~3;
     if ((long)B * N > (1L << 28) || (long)B * N * Dp > (1L << 31)) return IGS_ERR_BAD_SHAPE;
     const int cus = device_cus() > 0 ? device_cus() : 256;
-    const int tiles = ceil_div(N, kKoleoTile);
-    // enough workgroups for two per compute unit, by splitting the columns
+    // 64x64 similarity tiles, unless even one column tile per workgroup leaves most of the
+    // device idle; then enough workgroups for two per compute unit, by splitting the columns
+    const int t64 = ceil_div(N, 64);
+    const int tile = (long)t64 * t64 * B < 2L * cus ? 32 : 64;
+    const int tiles = ceil_div(N, tile);
     int S = ceil_div(2L * cus, (long)tiles * B);
     S = S < 1 ? 1 : (S > tiles ? tiles : S);
     const int per = ceil_div(tiles, S);
@@ -793,8 +796,19 @@ int koleo_plan(int B, int N, int D, igs_koleo_plan_t* p) {
     p->N = N;
     p->D = D;
     p->d_padded = Dp;
+    p->tile = tile;
     p->splits = S;
     p->tiles_per_split = per;
+    // backward: a wave owns bwd_rows rows.  More rows mean less scanning in total, but a wave
+    // handles its rows one after the other, each a chain of dependent loads, so it takes four
+    // waves per SIMD (4096 on the device) to hide that before rows are added.
+    p->bwd_chunk = Dp < kKoleoBwdChunk ? Dp : kKoleoBwdChunk;
+    int rw_max = kKoleoBwdLds / p->bwd_chunk;
+    rw_max = rw_max > kKoleoBwdMaxRows ? kKoleoBwdMaxRows : rw_max;
+    int rw = 1;
+    while (rw * 2 <= rw_max && (long)B * N / (rw * 2) >= 16L * cus) rw *= 2;
+    p->bwd_rows = rw;
+    p->reserved_ = 0;
     p->saved_bytes = ((size_t)rows * Dp + 3 * koleo_rows_padded(rows)) * sizeof(float);
     const size_t blocks = (size_t)ceil_div(rows, kThreads);
     p->scratch_bytes = ((blocks + 1) & ~(size_t)1) * sizeof(double) + (size_t)B * S * N * 2 * sizeof(float);
@@ -822,10 +836,26 @@ int igs_koleo_forward(const float* features, int B, int N, int D, float* loss, v
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(k_koleo_normalize, dim3(ceil_div(rows, kThreads / 64)), dim3(kThreads), 0, st,
                        features, rows, D, p.d_padded, sv.fn, sv.norm);
-    hipLaunchKernelGGL(k_koleo_nn, dim3(ceil_div(N, kKoleoTile), p.splits, B), dim3(kThreads), 0, st,
-                       (const float*)sv.fn, N, p.d_padded, p.tiles_per_split, part_val, part_idx);
+    const dim3 nn_grid(ceil_div(N, p.tile), p.splits, B);
+#define IGS_KOLEO_NN(M, KN)                                                                       \
+    hipLaunchKernelGGL((k_koleo_nn<M, KN>), nn_grid, dim3(kThreads), 0, st, (const float*)sv.fn, N,  \
+                       p.d_padded, p.tiles_per_split, part_val, part_idx)
+#define IGS_KOLEO_NN_K(KN)                                              \
+    do {                                                                \
+        if (p.tile == 64) IGS_KOLEO_NN(4, KN); else IGS_KOLEO_NN(2, KN); \
+    } while (0)
+    switch (p.d_padded <= kKoleoRegK ? p.d_padded : 0) {
+        case 4: IGS_KOLEO_NN_K(4); break;
+        case 8: IGS_KOLEO_NN_K(8); break;
+        case 12: IGS_KOLEO_NN_K(12); break;
+        case 16: IGS_KOLEO_NN_K(16); break;
+        default: IGS_KOLEO_NN_K(0); break;
+    }
+#undef IGS_KOLEO_NN_K
+#undef IGS_KOLEO_NN
     hipLaunchKernelGGL(k_koleo_combine, dim3(blocks), dim3(kThreads), 0, st, (const float*)part_val,
-                       (const int*)part_idx, B, N, p.splits, sv.nn_val, sv.nn_idx, loss_part);
+                       (const int*)part_idx, (const float*)sv.norm, B, N, p.splits, sv.nn_val, sv.nn_idx,
+                       loss_part);
     hipLaunchKernelGGL(k_koleo_sum, dim3(1), dim3(kThreads), 0, st, (const double*)loss_part, blocks,
                        1.0 / (double)rows, loss);
     return launch_status();
@@ -840,10 +870,10 @@ int igs_koleo_backward(const void* saved, size_t saved_bytes, const float* grad_
     if (saved_bytes < p.saved_bytes) return IGS_ERR_WORKSPACE;
     if ((uintptr_t)saved & 15) return IGS_ERR_ALIGNMENT;
     const KoleoSaved sv = koleo_saved(const_cast<void*>(saved), p);
-    const int rows_per_block = (kThreads / 64) * kKoleoBwdRows;
-    hipLaunchKernelGGL(k_koleo_bwd, dim3(ceil_div(N, rows_per_block), B), dim3(kThreads), 0,
-                       (hipStream_t)stream, (const float*)sv.fn, (const float*)sv.norm,
-                       (const int*)sv.nn_idx, grad_loss, B, N, D, p.d_padded, grad_features);
+    hipLaunchKernelGGL(k_koleo_bwd, dim3(ceil_div(N, p.bwd_rows), B), dim3(64),
+                       (size_t)p.bwd_rows * p.bwd_chunk * sizeof(float), (hipStream_t)stream,
+                       (const float*)sv.fn, (const float*)sv.norm, (const int*)sv.nn_idx, grad_loss, B, N, D,
+                       p.d_padded, p.bwd_rows, p.bwd_chunk, grad_features);
     return launch_status();
 }
 

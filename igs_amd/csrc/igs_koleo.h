@@ -3,7 +3,7 @@
 // that the reference materialises.  Included by igs_gs2d.hip inside its anonymous namespace.
 //
 //   k_koleo_normalize : fn = x / max(||x||, 1e-12), rows zero-padded to a multiple of 4 floats
-//   k_koleo_nn        : register-tiled fn fn^T (64x64 per workgroup, 4x4 per lane, K through LDS),
+//   k_koleo_nn        : register-tiled fn fn^T (64x64 or 32x32 per workgroup, K through LDS),
 //                       reduced on the fly to (max, argmax) per row and column split
 //   k_koleo_combine   : splits -> nearest neighbour per row, relu(. + 1), per-workgroup sums
 //   k_koleo_sum       : fixed-order sum of those -> loss
@@ -11,12 +11,12 @@
 // No atomics: equal similarities resolve to the lowest column index, every sum has a fixed order.
 #pragma once
 
-constexpr int kKoleoTile = 64;        // rows and columns of a similarity tile
-constexpr int kKoleoKC = 16;          // feature dimensions staged per LDS chunk
-constexpr int kKoleoLd = kKoleoTile + 4;  // LDS row stride (keeps float4 reads aligned)
+constexpr int kKoleoRegK = 16;        // up to this many (padded) dimensions the row tile stays in registers
 constexpr float kKoleoNormEps = 1e-12f;   // torch.nn.functional.normalize's default (src/igs/reg.py:22)
-constexpr int kKoleoBwdRows = 4;      // rows per wave in the backward
-constexpr int kKoleoBwdChunk = 256;   // feature dimensions per pass of a wave (one float4 per lane)
+constexpr int kKoleoBwdMaxRows = 64;  // rows per wave in the backward, at most
+constexpr int kKoleoBwdChunk = 2048;  // feature dimensions per pass of the backward, at most
+constexpr int kKoleoBwdLds = 8192;    // floats of LDS per backward wave
+constexpr int kKoleoScan = 8;         // loads of 64 neighbour indices in flight per backward wave (twice this)
 
 // Is candidate (v2, i2) to be preferred over (v1, i1)?  NaN wins and stays (torch.max propagates
 // it); equal values resolve to the lower index; index -1 (no candidate) loses every tie.
@@ -26,7 +26,8 @@ __device__ __forceinline__ bool koleo_better(float v2, int i2, float v1, int i1)
     return v2 > v1 || (v2 == v1 && (unsigned)i2 < (unsigned)i1);
 }
 
-// One wave per row: fn[row][0..Dp) and the unclamped norm.
+// One wave per row: fn[row][0..Dp) and the unclamped norm.  A row with a non-finite element
+// (which makes every similarity of its image NaN in the plain expression) gets norm = NaN.
 __global__ __launch_bounds__(kThreads) void k_koleo_normalize(const float* __restrict__ x, long rows,
                                                               int D, int Dp, float* __restrict__ fn,
                                                               float* __restrict__ norm) {
@@ -40,78 +41,183 @@ __global__ __launch_bounds__(kThreads) void k_koleo_normalize(const float* __res
     for (int k = 32; k > 0; k >>= 1) ss += __shfl_xor(ss, k);
     const float nrm = sqrtf(ss);
     const float den = fmaxf(nrm, kKoleoNormEps);
-    for (int d = lane; d < Dp; d += 64) fn[row * Dp + d] = d < D ? xr[d] / den : 0.0f;
-    if (lane == 0) norm[row] = nrm;
+    bool bad = false;
+    for (int d = lane; d < Dp; d += 64) {
+        const float v = d < D ? xr[d] / den : 0.0f;
+        bad = bad || !(fabsf(v) <= 1.0e30f);
+        fn[row * Dp + d] = v;
+    }
+    const bool any_bad = __ballot(bad) != 0ull;
+    if (lane == 0) norm[row] = any_bad ? __builtin_nanf("") : nrm;
 }
 
-// Workgroup (rt, s, b): rows [64 rt, 64 rt + 64) of image b against the column tiles
-// [s tiles_per_split, (s + 1) tiles_per_split).  Writes the best (value, column) per row of the
-// split; the diagonal and columns >= N are excluded.
+// Workgroup (rt, s, b): rows [TM rt, TM rt + TM) of image b against the column tiles
+// [s tiles_per_split, (s + 1) tiles_per_split), TM = 16 M: 256 lanes of M x M similarities each.
+// Writes the best (value, column) per row of the split; the diagonal and columns >= N are
+// excluded, NaN similarities are ignored (k_koleo_combine restores them from the norms).
+// Chunks of KC feature dimensions travel global -> registers -> LDS one step ahead of the
+// arithmetic (two LDS buffers, one barrier per step).  KN > 0 (= Dp <= 16): the row tile is read
+// once and kept in registers, a step stages only the column tile and the k loop is unrolled to
+// exactly KN; KN = 0: any Dp, 32 dimensions per step.
+template <int M, int KN>
 __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__ fn, int N, int Dp,
                                                        int tiles_per_split, float* __restrict__ part_val,
                                                        int* __restrict__ part_idx) {
-    __shared__ float As[kKoleoKC * kKoleoLd], Bs[kKoleoKC * kKoleoLd];
+    constexpr bool kRegA = KN > 0;
+    constexpr int KC = kRegA ? KN : 32;
+    constexpr int TM = 16 * M, LD = TM + 4;
+    constexpr int K4 = KC / 4;                    // float4 per tile row and chunk
+    constexpr int F4 = TM * K4;                   // float4 per tile chunk
+    constexpr int LPT = (2 * F4 + kThreads - 1) / kThreads;  // loader slots per thread and step (both tiles)
+    __shared__ float As[kRegA ? 1 : 2][KC * LD], Bs[2][KC * LD];
     const int b = blockIdx.z, s = blockIdx.y, S = gridDim.y;
-    const int row0 = blockIdx.x * kKoleoTile;
+    const int row0 = blockIdx.x * TM;
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const int lr = threadIdx.x >> 2, lk = (threadIdx.x & 3) * 4;  // loader: tile row, first k of a float4
     const float* img = fn + (size_t)b * N * Dp;
-    const int ntiles = (N + kKoleoTile - 1) / kKoleoTile;
+    const int ntiles = (N + TM - 1) / TM;
     const int ct0 = s * tiles_per_split, ct1 = min(ntiles, ct0 + tiles_per_split);
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
     const float ninf = -__builtin_inff();
-    float best[4] = {ninf, ninf, ninf, ninf};
-    int bidx[4] = {-1, -1, -1, -1};
-    auto stage = [&](float* dst, int first, int k0) {
-        const int r = first + lr;
-        const float4 v = (r < N && k0 + lk < Dp)
-                             ? *reinterpret_cast<const float4*>(img + (size_t)r * Dp + k0 + lk) : zero;
-        dst[(lk + 0) * kKoleoLd + lr] = v.x;
-        dst[(lk + 1) * kKoleoLd + lr] = v.y;
-        dst[(lk + 2) * kKoleoLd + lr] = v.z;
-        dst[(lk + 3) * kKoleoLd + lr] = v.w;
+    float best[M];
+    int bidx[M];
+#pragma unroll
+    for (int r = 0; r < M; ++r) {
+        best[r] = ninf;
+        bidx[r] = -1;
+    }
+    // loader slot j of this thread: which tile (0 = rows, 1 = columns, 2 = none), tile row, first k
+    auto slot = [&](int j, int& which, int& lr, int& lk) {
+        const int id = j * kThreads + (int)threadIdx.x;
+        which = id / F4;
+        lr = (id % F4) / K4;
+        lk = (id % K4) * 4;
     };
-    const bool one_chunk = Dp <= kKoleoKC;
-    if (one_chunk) stage(As, row0, 0);  // the row tile is staged once
-    for (int ct = ct0; ct < ct1; ++ct) {
-        const int col0 = ct * kKoleoTile;
-        float acc[4][4];
+    auto gload = [&](int j, int col0, int k0) {
+        int which, lr, lk;
+        slot(j, which, lr, lk);
+        if (which > 1 || (kRegA && which == 0)) return zero;
+        const int r = (which ? col0 : row0) + lr;
+        return (r < N && k0 + lk < Dp) ? *reinterpret_cast<const float4*>(img + (size_t)r * Dp + k0 + lk) : zero;
+    };
+    auto lstore = [&](int j, int buf, float4 v) {
+        int which, lr, lk;
+        slot(j, which, lr, lk);
+        if (which > 1 || (kRegA && which == 0)) return;
+        float* dst = which ? Bs[buf] : As[kRegA ? 0 : buf];
+        dst[(lk + 0) * LD + lr] = v.x;
+        dst[(lk + 1) * LD + lr] = v.y;
+        dst[(lk + 2) * LD + lr] = v.z;
+        dst[(lk + 3) * LD + lr] = v.w;
+    };
+    float areg[kRegA ? KN : 1][M];
+    if (kRegA) {  // stage the row tile through As once
+        for (int id = threadIdx.x; id < F4; id += kThreads) {
+            const int lr = id / K4, lk = (id % K4) * 4, r = row0 + lr;
+            const float4 v = r < N ? *reinterpret_cast<const float4*>(img + (size_t)r * Dp + lk) : zero;
+            As[0][(lk + 0) * LD + lr] = v.x;
+            As[0][(lk + 1) * LD + lr] = v.y;
+            As[0][(lk + 2) * LD + lr] = v.z;
+            As[0][(lk + 3) * LD + lr] = v.w;
+        }
+        __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int k = 0; k < KC; ++k)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
-        for (int k0 = 0; k0 < Dp; k0 += kKoleoKC) {
-            __syncthreads();  // the previous chunk's readers are done
-            if (!one_chunk) stage(As, row0, k0);
-            stage(Bs, col0, k0);
-            __syncthreads();
-            const int kn = min(kKoleoKC, Dp - k0);
+            for (int r = 0; r < M; ++r) areg[kRegA ? k : 0][r] = As[0][k * LD + ty * M + r];
+    }
+    const int kchunks = (Dp + KC - 1) / KC;
+    const int nsteps = (ct1 - ct0) * kchunks;
+    float4 pre[LPT];
+    if (nsteps > 0) {
+#pragma unroll
+        for (int j = 0; j < LPT; ++j) pre[j] = gload(j, ct0 * TM, 0);
+#pragma unroll
+        for (int j = 0; j < LPT; ++j) lstore(j, 0, pre[j]);
+    }
+    __syncthreads();
+    float acc[M][M];
+    int ct = ct0, kc = 0;
+    for (int step = 0; step < nsteps; ++step) {
+        const int buf = step & 1;
+        const int col0 = ct * TM, k0 = kc * KC;
+        int nct = ct, nkc = kc + 1;  // the step after this one
+        if (nkc == kchunks) {
+            nkc = 0;
+            ++nct;
+        }
+        const bool more = step + 1 < nsteps;
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < LPT; ++j) pre[j] = gload(j, nct * TM, nkc * KC);
+        }
+        if (kc == 0) {
+#pragma unroll
+            for (int r = 0; r < M; ++r)
+#pragma unroll
+                for (int q = 0; q < M; ++q) acc[r][q] = 0.0f;
+        }
+        if (kRegA) {  // fully unrolled: areg stays in registers
+#pragma unroll
+            for (int k = 0; k < KC; ++k) {
+                float cv[M];
+#pragma unroll
+                for (int r = 0; r < M; ++r) cv[r] = Bs[buf][k * LD + tx * M + r];
+#pragma unroll
+                for (int r = 0; r < M; ++r)
+#pragma unroll
+                    for (int q = 0; q < M; ++q) acc[r][q] = fmaf(areg[kRegA ? k : 0][r], cv[q], acc[r][q]);
+            }
+        } else {
+            const int kn = min(KC, Dp - k0);
+#pragma unroll 4
             for (int k = 0; k < kn; ++k) {
-                const float4 a = *reinterpret_cast<const float4*>(&As[k * kKoleoLd + ty * 4]);
-                const float4 c = *reinterpret_cast<const float4*>(&Bs[k * kKoleoLd + tx * 4]);
-                const float av[4] = {a.x, a.y, a.z, a.w}, cv[4] = {c.x, c.y, c.z, c.w};
+                float av[M], cv[M];
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
+                for (int r = 0; r < M; ++r) {
+                    av[r] = As[kRegA ? 0 : buf][k * LD + ty * M + r];
+                    cv[r] = Bs[buf][k * LD + tx * M + r];
+                }
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) acc[r][q] = fmaf(av[r], cv[q], acc[r][q]);
+                for (int r = 0; r < M; ++r)
+#pragma unroll
+                    for (int q = 0; q < M; ++q) acc[r][q] = fmaf(av[r], cv[q], acc[r][q]);
             }
         }
+        if (kc == kchunks - 1) {  // the tile's similarities are complete
+            if (col0 + TM > N || col0 == row0) {  // workgroup-uniform: the last column tile, the diagonal tile
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int grow = row0 + ty * 4 + r;
+                for (int r = 0; r < M; ++r)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int gcol = col0 + tx * 4 + q;
-                if (gcol < N && gcol != grow && koleo_better(acc[r][q], gcol, best[r], bidx[r])) {
-                    best[r] = acc[r][q];
-                    bidx[r] = gcol;
+                    for (int q = 0; q < M; ++q) {
+                        const int gcol = col0 + tx * M + q;
+                        if (gcol >= N || gcol == row0 + ty * M + r) acc[r][q] = ninf;
+                    }
+            }
+#pragma unroll
+            for (int r = 0; r < M; ++r) {
+                float m = acc[r][0];
+#pragma unroll
+                for (int q = 1; q < M; ++q) m = fmaxf(m, acc[r][q]);
+                int qi = M - 1;
+#pragma unroll
+                for (int q = M - 2; q >= 0; --q) qi = acc[r][q] == m ? q : qi;
+                if (m > best[r]) {  // columns come in increasing order: the first maximum stays
+                    best[r] = m;
+                    bidx[r] = col0 + tx * M + qi;
                 }
             }
         }
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < LPT; ++j) lstore(j, buf ^ 1, pre[j]);
+        }
+        __syncthreads();
+        ct = nct;
+        kc = nkc;
     }
     // the 16 lanes that share a row hold disjoint column sets
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < M; ++r) {
 #pragma unroll
         for (int k = 1; k < 16; k <<= 1) {
             const float ov = __shfl_xor(best[r], k);
@@ -121,7 +227,7 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
                 bidx[r] = oi;
             }
         }
-        const int grow = row0 + ty * 4 + r;
+        const int grow = row0 + ty * M + r;
         if (tx == 0 && grow < N) {
             part_val[((size_t)b * S + s) * N + grow] = best[r];
             part_idx[((size_t)b * S + s) * N + grow] = bidx[r];
@@ -132,7 +238,8 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
 // Thread per row: the best over the splits (in split order), the row's loss term, the gated
 // neighbour index (-1: relu passes no gradient) and the workgroup's sum of terms.
 __global__ __launch_bounds__(kThreads) void k_koleo_combine(const float* __restrict__ part_val,
-                                                            const int* __restrict__ part_idx, int B, int N,
+                                                            const int* __restrict__ part_idx,
+                                                            const float* __restrict__ norm, int B, int N,
                                                             int S, float* __restrict__ nn_val,
                                                             int* __restrict__ nn_idx,
                                                             double* __restrict__ loss_part) {
@@ -151,6 +258,7 @@ __global__ __launch_bounds__(kThreads) void k_koleo_combine(const float* __restr
                 idx = oi;
             }
         }
+        if (norm[row] != norm[row]) v = norm[row];  // non-finite row: NaN, which the sum below spreads
         const float t = v + 1.0f;
         nn_val[row] = v;
         nn_idx[row] = t > 0.0f ? idx : -1;
@@ -179,100 +287,111 @@ __global__ __launch_bounds__(kThreads) void k_koleo_sum(const double* __restrict
     if (threadIdx.x == 0) *loss = (float)(red[0] * scale);
 }
 
-// A wave owns kKoleoBwdRows consecutive rows r of image b.  With j(i) the gated neighbour of row i
-// and c = grad_loss / (B N):
+// One wave (a 64-thread workgroup) owns RW consecutive rows r of image b.  With j(i) the gated
+// neighbour of row i and c = grad_loss / (B N):
 //   d fn_r = c ( fn_j(r) + sum_{i: j(i) = r} fn_i )          (the sum in increasing i)
 //   d x_r  = (d fn_r - fn_r <fn_r, d fn_r>) / ||x_r||         if ||x_r|| > 1e-12, else d fn_r / 1e-12.
-// The wave scans the image's neighbour indices 64 at a time (ballot) and adds the few rows that
-// point at its own; d fn is parked in the output row until <fn, d fn> is known.
-__global__ __launch_bounds__(kThreads) void k_koleo_bwd(const float* __restrict__ fn,
-                                                        const float* __restrict__ norm,
-                                                        const int* __restrict__ nn_idx,
-                                                        const float* __restrict__ grad_loss, int B, int N,
-                                                        int D, int Dp, float* __restrict__ gx) {
-    constexpr int RW = kKoleoBwdRows;
+// The wave scans the image's neighbour indices 512 at a time (the next 512 in flight, ballots) and
+// adds the few rows that point at its own into LDS sums [RW][DC]; lane l owns the float4 groups
+// l, l + 64, ... of every row, so no LDS word is shared between lanes.  More than DC
+// dimensions are done DC at a time (another scan each).  d fn is parked in the output row until
+// <fn_r, d fn_r> is complete.
+__global__ __launch_bounds__(64) void k_koleo_bwd(const float* __restrict__ fn, const float* __restrict__ norm,
+                                                  const int* __restrict__ nn_idx,
+                                                  const float* __restrict__ grad_loss, int B, int N, int D,
+                                                  int Dp, int RW, int DC, float* __restrict__ gx) {
+    extern __shared__ __align__(16) float sums[];  // [RW][DC]
     const int b = blockIdx.y;
-    const int lane = threadIdx.x & 63;
-    const int r0 = (blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6)) * RW;
-    if (r0 >= N) return;  // wave-uniform
+    const int lane = threadIdx.x;
+    const int r0 = blockIdx.x * RW;
+    const int rows = min(RW, N - r0);
     const float c = grad_loss[0] / ((float)B * (float)N);
     const float* img = fn + (size_t)b * N * Dp;
     const int* idx = nn_idx + (size_t)b * N;
+    float* out0 = gx + ((size_t)b * N + r0) * D;
+    float mydot = 0.0f;  // lane q: <fn, d fn> of row r0 + q
+    float4* sums4 = reinterpret_cast<float4*>(sums);
+    const int DC4 = DC / 4;
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-    float dot[RW];
+    for (int dc = 0; dc < Dp; dc += DC) {
+        const int dn4 = min(DC, Dp - dc) / 4;  // float4 per row in this pass; lane l owns l, l + 64, ...
+        for (int q = 0; q < rows; ++q)
+            for (int d = lane; d < dn4; d += 64) sums4[q * DC4 + d] = zero;
+        // kKoleoScan x 64 neighbour indices per batch, the next batch's loads in flight meanwhile
+        int v[kKoleoScan], nxt[kKoleoScan];
 #pragma unroll
-    for (int q = 0; q < RW; ++q) dot[q] = 0.0f;
-    for (int dc = 0; dc < Dp; dc += kKoleoBwdChunk) {
-        const int d = dc + 4 * lane;
-        const bool live = d < Dp;
-        float4 acc[RW];
+        for (int u = 0; u < kKoleoScan; ++u) {
+            const int i = u * 64 + lane;
+            nxt[u] = i < N ? idx[i] : -1;
+        }
+        for (int i0 = 0; i0 < N; i0 += kKoleoScan * 64) {
 #pragma unroll
-        for (int q = 0; q < RW; ++q) acc[q] = zero;
-        for (int i0 = 0; i0 < N; i0 += 64) {
-            const int i = i0 + lane;
-            const int v = i < N ? idx[i] : -1;
-            unsigned long long mask = __ballot((unsigned)(v - r0) < (unsigned)RW);
-            while (mask) {  // wave-uniform
-                const int bit = __builtin_ctzll(mask);
-                mask &= mask - 1;
-                const int rr = __builtin_amdgcn_readlane(v, bit) - r0;
-                const float4 f = live ? *reinterpret_cast<const float4*>(img + (size_t)(i0 + bit) * Dp + d) : zero;
+            for (int u = 0; u < kKoleoScan; ++u) {
+                v[u] = nxt[u];
+                const int i = i0 + (kKoleoScan + u) * 64 + lane;
+                nxt[u] = i < N ? idx[i] : -1;
+            }
 #pragma unroll
-                for (int q = 0; q < RW; ++q)
-                    if (rr == q) {
-                        acc[q].x += f.x;
-                        acc[q].y += f.y;
-                        acc[q].z += f.z;
-                        acc[q].w += f.w;
+            for (int u = 0; u < kKoleoScan; ++u) {
+                unsigned long long mask = __ballot((unsigned)(v[u] - r0) < (unsigned)rows);
+                while (mask) {  // wave-uniform
+                    const int bit = __builtin_ctzll(mask);
+                    mask &= mask - 1;
+                    const int q = __builtin_amdgcn_readlane(v[u], bit) - r0;
+                    const float4* src = reinterpret_cast<const float4*>(img + (size_t)(i0 + u * 64 + bit) * Dp + dc);
+                    for (int d = lane; d < dn4; d += 64) {
+                        const float4 f = src[d];
+                        float4 a = sums4[q * DC4 + d];
+                        a.x += f.x;
+                        a.y += f.y;
+                        a.z += f.z;
+                        a.w += f.w;
+                        sums4[q * DC4 + d] = a;
                     }
+                }
             }
         }
-#pragma unroll
-        for (int q = 0; q < RW; ++q) {
+        for (int q = 0; q < rows; ++q) {
             const int r = r0 + q;
-            if (r >= N) break;  // wave-uniform
             const int j = idx[r];
-            if (j >= 0 && live) {
-                const float4 f = *reinterpret_cast<const float4*>(img + (size_t)j * Dp + d);
-                acc[q].x += f.x;
-                acc[q].y += f.y;
-                acc[q].z += f.z;
-                acc[q].w += f.w;
-            }
-            if (live) {
-                const float4 me = *reinterpret_cast<const float4*>(img + (size_t)r * Dp + d);
-                const float h[4] = {c * acc[q].x, c * acc[q].y, c * acc[q].z, c * acc[q].w};
-                const float m[4] = {me.x, me.y, me.z, me.w};
-                float* out = gx + ((size_t)b * N + r) * D;
+            const float4* nb = reinterpret_cast<const float4*>(img + (size_t)(j >= 0 ? j : r) * Dp + dc);
+            const float4* me = reinterpret_cast<const float4*>(img + (size_t)r * Dp + dc);
+            float part = 0.0f;
+            for (int d = lane; d < dn4; d += 64) {
+                const float4 a = sums4[q * DC4 + d];
+                const float4 f = j >= 0 ? nb[d] : zero;
+                const float4 m = me[d];
+                const float h[4] = {c * (a.x + f.x), c * (a.y + f.y), c * (a.z + f.z), c * (a.w + f.w)};
+                const float mv[4] = {m.x, m.y, m.z, m.w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    dot[q] = fmaf(m[e], h[e], dot[q]);  // padded dimensions hold 0
-                    if (d + e < D) out[d + e] = h[e];
+                    part = fmaf(mv[e], h[e], part);  // padded dimensions hold 0
+                    if (dc + 4 * d + e < D) out0[(size_t)q * D + dc + 4 * d + e] = h[e];
                 }
             }
+#pragma unroll
+            for (int k = 32; k > 0; k >>= 1) part += __shfl_xor(part, k);
+            if (lane == q) mydot += part;
         }
     }
+    for (int q = 0; q < rows; ++q) {
+        const int r = r0 + q;
+        const float dot = __shfl(mydot, q);
+        const float nrm = norm[(size_t)b * N + r];
+        const float4* me = reinterpret_cast<const float4*>(img + (size_t)r * Dp);
+        for (int dc = 0; dc < Dp; dc += DC) {
+            const int dn4 = min(DC, Dp - dc) / 4;
+            for (int d = lane; d < dn4; d += 64) {
+                const float4 m = me[dc / 4 + d];
+                const float mv[4] = {m.x, m.y, m.z, m.w};
 #pragma unroll
-    for (int q = 0; q < RW; ++q)
-#pragma unroll
-        for (int k = 32; k > 0; k >>= 1) dot[q] += __shfl_xor(dot[q], k);
-    for (int dc = 0; dc < Dp; dc += kKoleoBwdChunk) {
-        const int d = dc + 4 * lane;
-        if (d >= Dp) continue;
-#pragma unroll
-        for (int q = 0; q < RW; ++q) {
-            const int r = r0 + q;
-            if (r >= N) break;
-            const float nrm = norm[(size_t)b * N + r];
-            const float4 me = *reinterpret_cast<const float4*>(img + (size_t)r * Dp + d);
-            const float m[4] = {me.x, me.y, me.z, me.w};
-            float* out = gx + ((size_t)b * N + r) * D;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (d + e < D) {
-                    const float h = out[d + e];  // written by this lane above
-                    out[d + e] = nrm > kKoleoNormEps ? (h - m[e] * dot[q]) / nrm : h / kKoleoNormEps;
-                }
+                for (int e = 0; e < 4; ++e)
+                    if (dc + 4 * d + e < D) {
+                        float* o = out0 + (size_t)q * D + dc + 4 * d + e;
+                        const float h = *o;  // written by this lane above
+                        *o = nrm > kKoleoNormEps ? (h - mv[e] * dot) / nrm : h / kKoleoNormEps;
+                    }
+            }
         }
     }
 }

@@ -3,9 +3,10 @@
 loss = mean over the B*N rows of relu(max_{j != i} cos(x_i, x_j) + 1).  The reference forms the
 whole [B, N, N] similarity matrix (bmm, diagonal fill, row max) under `torch.compile`; here the
 row maxima come out of a tiled kernel that never stores the matrix, and the backward sends the
-gradient through each row's nearest neighbour only, as autograd does for `max`.  Registered as
-`igs_amd::koleo_fwd` / `igs_amd::koleo_bwd`, so that eager callers and callers under
-`torch.compile` take the same path.  There is no CPU path: tensors must live on the GPU.
+gradient through each row's nearest neighbour only, as autograd does for `max`.  Eager callers go
+through a `torch.autograd.Function`; under `torch.compile` the same two library calls are the
+registered operators `igs_amd::koleo_fwd` / `igs_amd::koleo_bwd`.  There is no CPU path: tensors
+must live on the GPU.
 """
 from __future__ import annotations
 
@@ -28,9 +29,7 @@ def saved_numel(B: int, N: int, D: int) -> int:
     return rows * ((D + 3) // 4 * 4) + 3 * ((rows + 3) // 4 * 4)
 
 
-@torch.library.custom_op("igs_amd::koleo_fwd", mutates_args=(), device_types="cuda")
-def koleo_fwd(features: Tensor) -> List[Tensor]:
-    """[loss (0-dim fp32), saved] for fp32 contiguous features [B, N >= 2, D]."""
+def _forward(features: Tensor) -> List[Tensor]:
     require_gpu(features)
     B, N, D = features.shape
     p = _lib.koleo_plan(B, N, D)
@@ -48,6 +47,40 @@ def koleo_fwd(features: Tensor) -> List[Tensor]:
     return [loss, saved]
 
 
+def _backward_call(saved: Tensor, grad_loss: Tensor, B: int, N: int, D: int) -> Tensor:
+    require_gpu(saved)
+    dev = saved.device
+    with torch.cuda.device(dev):
+        g = grad_loss.detach().to(torch.float32).reshape(1).contiguous()
+        out = torch.empty(B, N, D, device=dev, dtype=torch.float32)
+        _lib.check(_lib.load().igs_koleo_backward(_ptr(saved), saved.numel() * 4, _ptr(g), B, N, D, _ptr(out),
+                                                   _stream(dev)), "igs_koleo_backward")
+    return out
+
+
+class _Koleo(torch.autograd.Function):
+    """Eager path: the same two library calls without the operator dispatch (tens of microseconds
+    per call, which is most of the cost at the sizes the loss is used at)."""
+
+    @staticmethod
+    def forward(ctx, features):
+        loss, saved = _forward(features)
+        ctx.dims = tuple(features.shape)
+        ctx.save_for_backward(saved)
+        return loss
+
+    @staticmethod
+    def backward(ctx, g_loss):
+        (saved,) = ctx.saved_tensors
+        return _backward_call(saved, g_loss, *ctx.dims)
+
+
+@torch.library.custom_op("igs_amd::koleo_fwd", mutates_args=(), device_types="cuda")
+def koleo_fwd(features: Tensor) -> List[Tensor]:
+    """[loss (0-dim fp32), saved] for fp32 contiguous features [B, N >= 2, D]."""
+    return _forward(features)
+
+
 @koleo_fwd.register_fake
 def _(features):
     B, N, D = features.shape
@@ -57,14 +90,7 @@ def _(features):
 
 @torch.library.custom_op("igs_amd::koleo_bwd", mutates_args=(), device_types="cuda")
 def koleo_bwd(saved: Tensor, grad_loss: Tensor, B: int, N: int, D: int) -> Tensor:
-    require_gpu(saved)
-    dev = saved.device
-    with torch.cuda.device(dev):
-        g = grad_loss.detach().to(torch.float32).reshape(1).contiguous()
-        out = torch.empty(B, N, D, device=dev, dtype=torch.float32)
-        _lib.check(_lib.load().igs_koleo_backward(_ptr(saved), saved.numel() * 4, _ptr(g), B, N, D, _ptr(out),
-                                                   _stream(dev)), "igs_koleo_backward")
-    return out
+    return _backward_call(saved, grad_loss, B, N, D)
 
 
 @koleo_bwd.register_fake
@@ -120,5 +146,8 @@ def koleo_diversity_loss(features: Tensor) -> Tensor:
         # vectors normalise to zero, every similarity is 0, loss 1)
         return (features.sum() * 0 + (float("nan") if B == 0 else 1.0)).to(features.dtype)
     x = features.to(torch.float32).contiguous()
-    loss = torch.ops.igs_amd.koleo_fwd(x)[0]
+    if torch.compiler.is_compiling():
+        loss = torch.ops.igs_amd.koleo_fwd(x)[0]
+    else:
+        loss = _Koleo.apply(x)
     return loss if features.dtype == torch.float32 else loss.to(features.dtype)

@@ -284,3 +284,56 @@ def test_empty_inputs_give_the_plain_expression_s_result():
     m = igs_amd.GaussianSplatting2D(4, 8)
     img, feat = m(torch.zeros(2, 0, 8), size=(4, 6))       # no features -> no Gaussians
     assert img.shape == (2, 3, 4, 6) and feat.shape == (2, 0, 9) and float(img.detach().abs().sum()) == 0.0
+
+
+def test_koleo_plan_and_argument_errors(lib):
+    """Plan arithmetic of the diversity loss and its status codes (no GPU call is made)."""
+    from igs_amd import _lib
+    from igs_amd.reg import saved_numel
+
+    import random
+    rnd = random.Random(3)
+    for _ in range(200):
+        B, N, D = rnd.randint(1, 9), rnd.randint(2, 70000), rnd.randint(1, 600)
+        if B * N * ((D + 3) // 4 * 4) > 1 << 31:
+            continue
+        p = _lib.KoleoPlan()
+        assert lib.igs_koleo_plan(B, N, D, ctypes.byref(p)) == 0
+        assert (p.B, p.N, p.D) == (B, N, D) and p.d_padded == (D + 3) // 4 * 4
+        assert p.tile in (32, 64)
+        tiles = -(-N // p.tile)
+        assert 1 <= p.splits <= tiles and p.splits * p.tiles_per_split >= tiles
+        assert (p.splits - 1) * p.tiles_per_split < tiles            # no empty split
+        assert p.saved_bytes == 4 * saved_numel(B, N, D)
+        assert p.scratch_bytes >= 8 * -(-B * N // 256) + 8 * B * p.splits * N
+        assert 1 <= p.bwd_rows <= 64 and p.bwd_chunk % 4 == 0 and p.bwd_chunk <= 2048
+        assert p.bwd_rows * p.bwd_chunk <= 8192
+    p = _lib.KoleoPlan()
+    assert lib.igs_koleo_plan(1, 1, 3, ctypes.byref(p)) == -2          # N >= 2
+    assert lib.igs_koleo_plan(0, 5, 3, ctypes.byref(p)) == -2
+    assert lib.igs_koleo_plan(1, 5, 0, ctypes.byref(p)) == -2
+    assert lib.igs_koleo_plan(70000, 5, 3, ctypes.byref(p)) == -2
+    assert lib.igs_koleo_plan(1, 5, 3, None) == -1
+    assert lib.igs_koleo_forward(None, 1, 5, 3, None, None, 0, None, 0, None) == -1
+    assert lib.igs_koleo_backward(None, 0, None, 1, 5, 3, None, None) == -1
+    # workspace too small / misaligned are reported before anything is launched
+    fake = ctypes.c_void_p(4096)
+    assert lib.igs_koleo_forward(fake, 1, 5, 3, fake, fake, 8, fake, 8, None) == -4
+    assert lib.igs_koleo_forward(fake, 1, 5, 3, fake, ctypes.c_void_p(4100), 1 << 20, fake, 1 << 20, None) == -7
+    assert lib.igs_koleo_backward(fake, 8, fake, 1, 5, 3, fake, None) == -4
+
+
+def test_koleo_host_surface():
+    import torch
+
+    import igs_amd
+
+    assert float(igs_amd.koleo_diversity_loss(torch.randn(3, 1, 4))) == 0.0     # N <= 1: constant 0
+    assert float(igs_amd.koleo_diversity_loss(torch.randn(3, 0, 4))) == 0.0
+    with pytest.raises(RuntimeError):
+        igs_amd.koleo_diversity_loss(torch.randn(2, 5, 3))                      # no CPU path
+    with pytest.raises(ValueError):
+        igs_amd.koleo_diversity_loss(torch.randn(5, 3))
+    out = torch.ops.igs_amd.koleo_fwd(torch.empty(2, 50, 9, device="meta"))
+    assert out[0].shape == () and out[1].shape == (igs_amd.reg.saved_numel(2, 50, 9),)
+    assert torch.ops.igs_amd.koleo_bwd(out[1], out[0], 2, 50, 9).shape == (2, 50, 9)

@@ -3,7 +3,8 @@
 Tolerances: loss |d| <= 1e-6 + 1e-5 |ref|; gradient per tensor max|d| <= 1e-4 max|ref| and
 ||d|| <= 1e-4 ||ref||.  The gradient of a row maximum is discontinuous where two similarities
 are equal, so the neighbour the fp32 kernels chose is first checked to be a maximum to fp32
-rounding (2e-6) and the oracle's chain rule is then evaluated with that choice."""
+rounding (2e-6, times D/1024 for longer dot products) and the oracle's chain rule is then
+evaluated with that choice."""
 import math
 
 import pytest
@@ -47,7 +48,8 @@ def gpu_loss_and_grad(igs, x64, dev, scale=1.0):
 
 
 SHAPES = [(1, 2, 3), (2, 7, 4), (1, 65, 17), (3, 130, 9), (1, 128, 512), (2, 1000, 9), (1, 4096, 9),
-          (4, 300, 33), (5, 64, 16), (1, 257, 1), (2, 70, 300)]
+          (4, 300, 33), (5, 64, 16), (1, 257, 1), (2, 70, 300), (1, 40, 2500), (2, 33, 4100), (3, 2100, 16),
+          (1, 3000, 20)]
 
 
 @pytest.mark.parametrize("kind", ["normal", "offset", "scaled"])
@@ -63,17 +65,18 @@ def test_loss_and_gradient_against_oracle(igs, dev, shape, kind):
     # the neighbour the kernels chose is a maximum of the row to fp32 rounding
     val, idx = koleo_nearest_neighbours(x32.to(dev, torch.float32))
     rval, ridx, gap = K.nearest_neighbours(x32)
-    assert float((val.cpu().double() - rval).abs().max()) <= 2e-6
+    tol = 2e-6 * max(1.0, shape[2] / 1024)
+    assert float((val.cpu().double() - rval).abs().max()) <= tol
     idx = idx.cpu().long()
     open_gate = idx >= 0
-    assert bool((open_gate | (rval + 1 <= 2e-6)).all())
+    assert bool((open_gate | (rval + 1 <= tol)).all())
     fn, _ = K.normalize_rows(x32)
     chosen = torch.where(open_gate, idx, ridx)
     sim_chosen = (fn * torch.gather(fn, 1, chosen[..., None].expand_as(fn))).sum(-1)
-    assert float((rval - sim_chosen).max()) <= 2e-6
+    assert float((rval - sim_chosen).max()) <= tol
     assert bool((chosen != torch.arange(shape[1])[None]).all())
     differs = (chosen != ridx)
-    assert bool((gap[differs] <= 2e-6).all())           # only genuine near-ties may differ
+    assert bool((gap[differs] <= tol).all())            # only genuine near-ties may differ
     if kind == "normal" and shape[2] > 1:
         assert int(differs.sum()) <= max(1, shape[0] * shape[1] // 500)
     rgrad = K.koleo_backward(x32, grad_loss=1.3, neighbours=chosen)
