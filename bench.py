@@ -49,6 +49,8 @@ def main() -> int:
     ap.add_argument("--koleo", action="store_true",
                     help="instead of the JSON line, print forward and forward+backward times of the KoLeo "
                          "diversity loss (src/igs/reg.py of the reference) beside the plain torch expression")
+    ap.add_argument("--koleo-shape", default=None, metavar="BxNxD",
+                    help="with --koleo: time this one shape only, without the torch and CPU columns (for profiling)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
@@ -63,7 +65,7 @@ def main() -> int:
     if args.all:
         return all_configs(args.steps, args.warmup)
     if args.koleo:
-        return koleo_table(args.no_cpu)
+        return koleo_table(args.no_cpu, args.koleo_shape)
 
     import torch
 
@@ -290,7 +292,7 @@ def all_configs(steps: int, warmup: int) -> int:
     return 0
 
 
-def koleo_table(no_cpu: bool) -> int:
+def koleo_table(no_cpu: bool, only: str = None) -> int:
     """KoLeo diversity loss: events around `koleo_diversity_loss(x)` and around loss + backward (4 warm-ups,
     median of 32), for the two shapes scripts/gs2d_test.py:146,172 of the reference passes ([1, N, 9] Gaussian
     features, [1, k <= 128, 512] latent features) and larger ones; beside it the same expression in eager fp32
@@ -330,12 +332,15 @@ def koleo_table(no_cpu: bool) -> int:
 
     print("%-16s %10s %10s %12s %12s %12s %10s" % ("B x N x D", "fwd ms", "f+b ms", "torch fwd", "torch f+b",
                                                    "TFLOP/s fwd", "cpu f+b ms"))
-    for shape in [(1, 128, 512), (1, 4096, 9), (8, 4096, 9), (1, 16384, 9), (4, 16384, 32), (1, 65536, 9)]:
+    shapes = [(1, 128, 512), (1, 4096, 9), (8, 4096, 9), (1, 16384, 9), (4, 16384, 32), (1, 65536, 9)]
+    if only:
+        shapes, no_cpu = [tuple(int(v) for v in only.split("x"))], True
+    for shape in shapes:
         B, N, D = shape
         x = torch.randn(*shape, device=dev, generator=torch.Generator(dev).manual_seed(0))
         f, fb = both(igs_amd.koleo_diversity_loss, x)
         tf = tfb = float("nan")
-        if B * N * N * 4 <= 4 << 30:
+        if not only and B * N * N * 4 <= 4 << 30:
             tf, tfb = both(K.koleo_diversity_loss, x)
         cpu = float("nan")
         if not no_cpu and B * N * N <= 1 << 28:
