@@ -307,7 +307,7 @@ class GaussianSplatting2D(nn.Module):
         else:
             grid = grid.flip(1)  # pos_map order is (h, w): y first
             x_grid, y_grid = grid.split([1, 1], dim=1)
-        pos_map = None
+        pos_map = None  # the argument is not read by the reference either (:654-655 overwrites it)
         if self.pos_map_offset:
             pos_map = torch.concat([x_grid, y_grid], dim=1)
             if scale is not None:
