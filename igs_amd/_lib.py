@@ -51,12 +51,12 @@ class KoleoPlan(ctypes.Structure):
     _fields_ = [
         ("B", c_int32), ("N", c_int32), ("D", c_int32),
         ("d_padded", c_int32),
+        ("tile_rows", c_int32),
         ("tile", c_int32),
         ("splits", c_int32),
         ("tiles_per_split", c_int32),
         ("bwd_rows", c_int32),
         ("bwd_chunk", c_int32),
-        ("reserved_", c_int32),
         ("saved_bytes", c_uint64),
         ("scratch_bytes", c_uint64),
     ]

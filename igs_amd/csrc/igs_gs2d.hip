@@ -782,12 +782,17 @@ int koleo_plan(int B, int N, int D, igs_koleo_plan_t* p) {
     const int Dp = (D + 3) & ~3;
     if ((long)B * N > (1L << 28) || (long)B * N * Dp > (1L << 31)) return IGS_ERR_BAD_SHAPE;
     const int cus = device_cus() > 0 ? device_cus() : 256;
-    // 64x64 similarity tiles, unless even one column tile per workgroup leaves most of the
-    // device idle; then enough workgroups for two per compute unit, by splitting the columns
-    const int t64 = ceil_div(N, 64);
-    const int tile = (long)t64 * t64 * B < 2L * cus ? 32 : 64;
+    // similarity tiles of 128x64, unless one column tile per workgroup would leave most of the
+    // device idle (then 64x64, then 32x32); after that enough workgroups for two per compute
+    // unit, by splitting the columns
+    const long t128 = ceil_div(N, 128), t64 = ceil_div(N, 64);
+    // (128 rows pay only where the row tile is re-read from LDS at every step, Dp > kKoleoRegK)
+    const int tile_rows = (Dp > kKoleoRegK && t128 * t64 * B >= 2L * cus) ? 128
+                          : (t64 * t64 * B >= 2L * cus ? 64 : 32);
+    const int tile = tile_rows == 32 ? 32 : 64;
     const int tiles = ceil_div(N, tile);
-    int S = ceil_div(2L * cus, (long)tiles * B);
+    const int row_tiles = ceil_div(N, tile_rows);
+    int S = ceil_div(2L * cus, (long)row_tiles * B);
     S = S < 1 ? 1 : (S > tiles ? tiles : S);
     const int per = ceil_div(tiles, S);
     S = ceil_div(tiles, per);
@@ -796,6 +801,7 @@ int koleo_plan(int B, int N, int D, igs_koleo_plan_t* p) {
     p->N = N;
     p->D = D;
     p->d_padded = Dp;
+    p->tile_rows = tile_rows;
     p->tile = tile;
     p->splits = S;
     p->tiles_per_split = per;
@@ -808,7 +814,6 @@ int koleo_plan(int B, int N, int D, igs_koleo_plan_t* p) {
     int rw = 1;
     while (rw * 2 <= rw_max && (long)B * N / (rw * 2) >= 16L * cus) rw *= 2;
     p->bwd_rows = rw;
-    p->reserved_ = 0;
     p->saved_bytes = ((size_t)rows * Dp + 3 * koleo_rows_padded(rows)) * sizeof(float);
     const size_t blocks = (size_t)ceil_div(rows, kThreads);
     p->scratch_bytes = ((blocks + 1) & ~(size_t)1) * sizeof(double) + (size_t)B * S * N * 2 * sizeof(float);
@@ -836,13 +841,15 @@ int igs_koleo_forward(const float* features, int B, int N, int D, float* loss, v
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(k_koleo_normalize, dim3(ceil_div(rows, kThreads / 64)), dim3(kThreads), 0, st,
                        features, rows, D, p.d_padded, sv.fn, sv.norm);
-    const dim3 nn_grid(ceil_div(N, p.tile), p.splits, B);
-#define IGS_KOLEO_NN(M, KN)                                                                       \
-    hipLaunchKernelGGL((k_koleo_nn<M, KN>), nn_grid, dim3(kThreads), 0, st, (const float*)sv.fn, N,  \
+    const dim3 nn_grid(ceil_div(N, p.tile_rows), p.splits, B);
+#define IGS_KOLEO_NN(MR, MC, KN)                                                                       \
+    hipLaunchKernelGGL((k_koleo_nn<MR, MC, KN>), nn_grid, dim3(kThreads), 0, st, (const float*)sv.fn, N, \
                        p.d_padded, p.tiles_per_split, part_val, part_idx)
-#define IGS_KOLEO_NN_K(KN)                                              \
-    do {                                                                \
-        if (p.tile == 64) IGS_KOLEO_NN(4, KN); else IGS_KOLEO_NN(2, KN); \
+#define IGS_KOLEO_NN_K(KN)                                           \
+    do {                                                             \
+        if (p.tile_rows == 128 && KN == 0) IGS_KOLEO_NN(8, 4, 0);    \
+        else if (p.tile_rows == 64) IGS_KOLEO_NN(4, 4, KN);          \
+        else IGS_KOLEO_NN(2, 2, KN);                                 \
     } while (0)
     switch (p.d_padded <= kKoleoRegK ? p.d_padded : 0) {
         case 4: IGS_KOLEO_NN_K(4); break;

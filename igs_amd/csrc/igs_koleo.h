@@ -3,7 +3,7 @@
 // that the reference materialises.  Included by igs_gs2d.hip inside its anonymous namespace.
 //
 //   k_koleo_normalize : fn = x / max(||x||, 1e-12), rows zero-padded to a multiple of 4 floats
-//   k_koleo_nn        : register-tiled fn fn^T (64x64 or 32x32 per workgroup, K through LDS),
+//   k_koleo_nn        : register-tiled fn fn^T (128x64, 64x64 or 32x32 per workgroup, K through LDS),
 //                       reduced on the fly to (max, argmax) per row and column split
 //   k_koleo_combine   : splits -> nearest neighbour per row, relu(. + 1), per-workgroup sums
 //   k_koleo_sum       : fixed-order sum of those -> loss
@@ -51,95 +51,98 @@ __global__ __launch_bounds__(kThreads) void k_koleo_normalize(const float* __res
     if (lane == 0) norm[row] = any_bad ? __builtin_nanf("") : nrm;
 }
 
-// Workgroup (rt, s, b): rows [TM rt, TM rt + TM) of image b against the column tiles
-// [s tiles_per_split, (s + 1) tiles_per_split), TM = 16 M: 256 lanes of M x M similarities each.
-// Writes the best (value, column) per row of the split; the diagonal and columns >= N are
-// excluded, NaN similarities are ignored (k_koleo_combine restores them from the norms).
-// Chunks of KC feature dimensions travel global -> registers -> LDS one step ahead of the
-// arithmetic (two LDS buffers, one barrier per step).  KN > 0 (= Dp <= 16): the row tile is read
-// once and kept in registers, a step stages only the column tile and the k loop is unrolled to
-// exactly KN; KN = 0: any Dp, 32 dimensions per step.
-template <int M, int KN>
+// Workgroup (rt, s, b): rows [TR rt, TR rt + TR) of image b against the column tiles
+// [s tiles_per_split, (s + 1) tiles_per_split) of TC columns; TR = 16 MR, TC = 16 MC: 256 lanes of
+// MR x MC similarities each.  Writes the best (value, column) per row of the split; the diagonal
+// and columns >= N are excluded, NaN similarities are ignored (k_koleo_combine restores them from
+// the norms).  Chunks of KC feature dimensions travel global -> registers -> LDS one step ahead of
+// the arithmetic (two LDS buffers, one barrier per step).  KN > 0 (= Dp <= 16): the row tile is
+// read once and kept in registers, a step stages only the column tile and the k loop is unrolled
+// to exactly KN; KN = 0: any Dp, 32 dimensions per step.
+template <int MR, int MC, int KN>
 __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__ fn, int N, int Dp,
                                                        int tiles_per_split, float* __restrict__ part_val,
                                                        int* __restrict__ part_idx) {
     constexpr bool kRegA = KN > 0;
     constexpr int KC = kRegA ? KN : 32;
-    constexpr int TM = 16 * M, LD = TM + 4;
+    constexpr int TR = 16 * MR, TC = 16 * MC, LDA = TR + 4, LDB = TC + 4;
     constexpr int K4 = KC / 4;                    // float4 per tile row and chunk
-    constexpr int F4 = TM * K4;                   // float4 per tile chunk
-    constexpr int LPT = (2 * F4 + kThreads - 1) / kThreads;  // loader slots per thread and step (both tiles)
-    __shared__ float As[kRegA ? 1 : 2][KC * LD], Bs[2][KC * LD];
+    constexpr int F4A = kRegA ? 0 : TR * K4;      // float4 per step: row tile (none when it is in registers),
+    constexpr int F4B = TC * K4;                  // column tile
+    constexpr int LPT = (F4A + F4B + kThreads - 1) / kThreads;  // loader slots per thread and step
+    __shared__ float As[kRegA ? 1 : 2][KC * LDA], Bs[2][KC * LDB];
     const int b = blockIdx.z, s = blockIdx.y, S = gridDim.y;
-    const int row0 = blockIdx.x * TM;
+    const int row0 = blockIdx.x * TR;
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const float* img = fn + (size_t)b * N * Dp;
-    const int ntiles = (N + TM - 1) / TM;
+    const int ntiles = (N + TC - 1) / TC;
     const int ct0 = s * tiles_per_split, ct1 = min(ntiles, ct0 + tiles_per_split);
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
     const float ninf = -__builtin_inff();
-    float best[M];
-    int bidx[M];
+    float best[MR];
+    int bidx[MR];
 #pragma unroll
-    for (int r = 0; r < M; ++r) {
+    for (int r = 0; r < MR; ++r) {
         best[r] = ninf;
         bidx[r] = -1;
     }
     // loader slot j of this thread: which tile (0 = rows, 1 = columns, 2 = none), tile row, first k
     auto slot = [&](int j, int& which, int& lr, int& lk) {
         const int id = j * kThreads + (int)threadIdx.x;
-        which = id / F4;
-        lr = (id % F4) / K4;
-        lk = (id % K4) * 4;
+        which = id < F4A ? 0 : (id < F4A + F4B ? 1 : 2);
+        const int e = which ? id - F4A : id;
+        lr = e / K4;
+        lk = (e % K4) * 4;
     };
     auto gload = [&](int j, int col0, int k0) {
         int which, lr, lk;
         slot(j, which, lr, lk);
-        if (which > 1 || (kRegA && which == 0)) return zero;
+        if (which > 1) return zero;
         const int r = (which ? col0 : row0) + lr;
         return (r < N && k0 + lk < Dp) ? *reinterpret_cast<const float4*>(img + (size_t)r * Dp + k0 + lk) : zero;
     };
     auto lstore = [&](int j, int buf, float4 v) {
         int which, lr, lk;
         slot(j, which, lr, lk);
-        if (which > 1 || (kRegA && which == 0)) return;
+        if (which > 1) return;
         float* dst = which ? Bs[buf] : As[kRegA ? 0 : buf];
-        dst[(lk + 0) * LD + lr] = v.x;
-        dst[(lk + 1) * LD + lr] = v.y;
-        dst[(lk + 2) * LD + lr] = v.z;
-        dst[(lk + 3) * LD + lr] = v.w;
+        const int ld = which ? LDB : LDA;
+        dst[(lk + 0) * ld + lr] = v.x;
+        dst[(lk + 1) * ld + lr] = v.y;
+        dst[(lk + 2) * ld + lr] = v.z;
+        dst[(lk + 3) * ld + lr] = v.w;
     };
-    float areg[kRegA ? KN : 1][M];
+    float areg[kRegA ? KN : 1][MR];
     if (kRegA) {  // stage the row tile through As once
-        for (int id = threadIdx.x; id < F4; id += kThreads) {
+        for (int id = threadIdx.x; id < TR * K4; id += kThreads) {
             const int lr = id / K4, lk = (id % K4) * 4, r = row0 + lr;
             const float4 v = r < N ? *reinterpret_cast<const float4*>(img + (size_t)r * Dp + lk) : zero;
-            As[0][(lk + 0) * LD + lr] = v.x;
-            As[0][(lk + 1) * LD + lr] = v.y;
-            As[0][(lk + 2) * LD + lr] = v.z;
-            As[0][(lk + 3) * LD + lr] = v.w;
+            As[0][(lk + 0) * LDA + lr] = v.x;
+            As[0][(lk + 1) * LDA + lr] = v.y;
+            As[0][(lk + 2) * LDA + lr] = v.z;
+            As[0][(lk + 3) * LDA + lr] = v.w;
         }
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < KC; ++k)
 #pragma unroll
-            for (int r = 0; r < M; ++r) areg[kRegA ? k : 0][r] = As[0][k * LD + ty * M + r];
+            for (int r = 0; r < MR; ++r) areg[kRegA ? k : 0][r] = As[0][k * LDA + ty * MR + r];
     }
     const int kchunks = (Dp + KC - 1) / KC;
     const int nsteps = (ct1 - ct0) * kchunks;
     float4 pre[LPT];
     if (nsteps > 0) {
 #pragma unroll
-        for (int j = 0; j < LPT; ++j) pre[j] = gload(j, ct0 * TM, 0);
+        for (int j = 0; j < LPT; ++j) pre[j] = gload(j, ct0 * TC, 0);
 #pragma unroll
         for (int j = 0; j < LPT; ++j) lstore(j, 0, pre[j]);
     }
     __syncthreads();
-    float acc[M][M];
+    float acc[MR][MC];
     int ct = ct0, kc = 0;
     for (int step = 0; step < nsteps; ++step) {
         const int buf = step & 1;
-        const int col0 = ct * TM, k0 = kc * KC;
+        const int col0 = ct * TC, k0 = kc * KC;
         int nct = ct, nkc = kc + 1;  // the step after this one
         if (nkc == kchunks) {
             nkc = 0;
@@ -148,62 +151,62 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
         const bool more = step + 1 < nsteps;
         if (more) {
 #pragma unroll
-            for (int j = 0; j < LPT; ++j) pre[j] = gload(j, nct * TM, nkc * KC);
+            for (int j = 0; j < LPT; ++j) pre[j] = gload(j, nct * TC, nkc * KC);
         }
         if (kc == 0) {
 #pragma unroll
-            for (int r = 0; r < M; ++r)
+            for (int r = 0; r < MR; ++r)
 #pragma unroll
-                for (int q = 0; q < M; ++q) acc[r][q] = 0.0f;
+                for (int q = 0; q < MC; ++q) acc[r][q] = 0.0f;
         }
         if (kRegA) {  // fully unrolled: areg stays in registers
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
-                float cv[M];
+                float cv[MC];
 #pragma unroll
-                for (int r = 0; r < M; ++r) cv[r] = Bs[buf][k * LD + tx * M + r];
+                for (int q = 0; q < MC; ++q) cv[q] = Bs[buf][k * LDB + tx * MC + q];
 #pragma unroll
-                for (int r = 0; r < M; ++r)
+                for (int r = 0; r < MR; ++r)
 #pragma unroll
-                    for (int q = 0; q < M; ++q) acc[r][q] = fmaf(areg[kRegA ? k : 0][r], cv[q], acc[r][q]);
+                    for (int q = 0; q < MC; ++q) acc[r][q] = fmaf(areg[kRegA ? k : 0][r], cv[q], acc[r][q]);
             }
         } else {
             const int kn = min(KC, Dp - k0);
 #pragma unroll 4
             for (int k = 0; k < kn; ++k) {
-                float av[M], cv[M];
+                float av[MR], cv[MC];
 #pragma unroll
-                for (int r = 0; r < M; ++r) {
-                    av[r] = As[kRegA ? 0 : buf][k * LD + ty * M + r];
-                    cv[r] = Bs[buf][k * LD + tx * M + r];
-                }
+                for (int r = 0; r < MR; ++r) av[r] = As[kRegA ? 0 : buf][k * LDA + ty * MR + r];
 #pragma unroll
-                for (int r = 0; r < M; ++r)
+                for (int q = 0; q < MC; ++q) cv[q] = Bs[buf][k * LDB + tx * MC + q];
 #pragma unroll
-                    for (int q = 0; q < M; ++q) acc[r][q] = fmaf(av[r], cv[q], acc[r][q]);
+                for (int r = 0; r < MR; ++r)
+#pragma unroll
+                    for (int q = 0; q < MC; ++q) acc[r][q] = fmaf(av[r], cv[q], acc[r][q]);
             }
         }
         if (kc == kchunks - 1) {  // the tile's similarities are complete
-            if (col0 + TM > N || col0 == row0) {  // workgroup-uniform: the last column tile, the diagonal tile
+            // workgroup-uniform: the last column tile, the tiles that the diagonal crosses
+            if (col0 + TC > N || (col0 < row0 + TR && col0 + TC > row0)) {
 #pragma unroll
-                for (int r = 0; r < M; ++r)
+                for (int r = 0; r < MR; ++r)
 #pragma unroll
-                    for (int q = 0; q < M; ++q) {
-                        const int gcol = col0 + tx * M + q;
-                        if (gcol >= N || gcol == row0 + ty * M + r) acc[r][q] = ninf;
+                    for (int q = 0; q < MC; ++q) {
+                        const int gcol = col0 + tx * MC + q;
+                        if (gcol >= N || gcol == row0 + ty * MR + r) acc[r][q] = ninf;
                     }
             }
 #pragma unroll
-            for (int r = 0; r < M; ++r) {
+            for (int r = 0; r < MR; ++r) {
                 float m = acc[r][0];
 #pragma unroll
-                for (int q = 1; q < M; ++q) m = fmaxf(m, acc[r][q]);
-                int qi = M - 1;
+                for (int q = 1; q < MC; ++q) m = fmaxf(m, acc[r][q]);
+                int qi = MC - 1;
 #pragma unroll
-                for (int q = M - 2; q >= 0; --q) qi = acc[r][q] == m ? q : qi;
+                for (int q = MC - 2; q >= 0; --q) qi = acc[r][q] == m ? q : qi;
                 if (m > best[r]) {  // columns come in increasing order: the first maximum stays
                     best[r] = m;
-                    bidx[r] = col0 + tx * M + qi;
+                    bidx[r] = col0 + tx * MC + qi;
                 }
             }
         }
@@ -217,7 +220,7 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
     }
     // the 16 lanes that share a row hold disjoint column sets
 #pragma unroll
-    for (int r = 0; r < M; ++r) {
+    for (int r = 0; r < MR; ++r) {
 #pragma unroll
         for (int k = 1; k < 16; k <<= 1) {
             const float ov = __shfl_xor(best[r], k);
@@ -227,7 +230,7 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
                 bidx[r] = oi;
             }
         }
-        const int grow = row0 + ty * M + r;
+        const int grow = row0 + ty * MR + r;
         if (tx == 0 && grow < N) {
             part_val[((size_t)b * S + s) * N + grow] = best[r];
             part_idx[((size_t)b * S + s) * N + grow] = bidx[r];

@@ -246,12 +246,12 @@ int igs_adamw_step(float *param, const float *grad, float *exp_avg, float *exp_a
 typedef struct igs_koleo_plan_t {
     int32_t B, N, D;
     int32_t d_padded;        /* floats per normalised row (D rounded up to 4)                 */
-    int32_t tile;            /* rows = columns of a similarity tile: 64, or 32 for small N    */
+    int32_t tile_rows;       /* rows of a similarity tile: 128, 64 or 32 (by problem size)    */
+    int32_t tile;            /* columns of a similarity tile: 64 or 32                         */
     int32_t splits;          /* column splits of the similarity tiles (>= 1)                  */
     int32_t tiles_per_split; /* column tiles per split                                         */
     int32_t bwd_rows;        /* rows per wave of the backward                                  */
     int32_t bwd_chunk;       /* feature dimensions per pass of the backward                    */
-    int32_t reserved_;
     uint64_t saved_bytes;    /* kept from forward to backward: normalised rows, norms, nearest
                                 similarity and neighbour index per row                        */
     uint64_t scratch_bytes;  /* forward only: per-split maxima, per-workgroup loss sums       */
