@@ -200,13 +200,13 @@ def main() -> int:
             "flops_per_pair": f_bwd,
             "pairs_per_launch": pairs,
             "launch_ms": t_bwd_kernel * 1e3,
-            "traffic": (96.9 + 211.7) * 1024 * 1024 if args.config == "c1" and C == 3 else None,
+            "traffic": (94.2 + 138.6) * 1024 * 1024 if args.config == "c1" and C == 3 else None,
             "forward_kernel": {"launch_ms": t_fwd_kernel * 1e3, "flops_per_pair": f_fwd,
                                "achieved": pairs * f_fwd / t_fwd_kernel / 1e12,
                                "frac": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS},
             "traffic_note": "HBM bytes per launch from rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (copy-calibrated), "
                             "from the committed rocprofv3 counter summary; valid for the c1 workload only",
-            "note": "launch_ms brackets igs_gs2d_backward_reduce = k_bin (tile lists, ~11 us) + k_bwd_sep; peak = published fp32 vector peak; the kernels use plain (non-packed) fp32 VALU ops with "
+            "note": "launch_ms brackets igs_gs2d_backward_reduce = k_bin (tile lists, ~33 us) + k_bwd_sep; peak = published fp32 vector peak; the kernels use plain (non-packed) fp32 VALU ops with "
                     "VGPR-only operands, v_exp_f32 counted as 1 FLOP",
         },
     }

@@ -14,6 +14,7 @@
 #define IGS_FIN_DEEP 32
 #endif
 constexpr int kFinWide = 8, kFinDeep = IGS_FIN_DEEP;
+constexpr int kFinAhead = 4;    // tiles whose loads are issued together by a t-lane
 constexpr int kFinColours = 8;  // colour channels summed per pass (>= 6: the LDS array also serves the moments)
 
 // `part` is the image's partial array [T][NF][N]; the Gaussian's column in tile t is
@@ -28,15 +29,31 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const i
     float acc[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
-    if (valid)
-        for (int t = tl; t < T; t += FT) {
-            const int col = slots ? slots[(size_t)t * Np + n] : n;
-            if (col >= 0) {
+    if (valid) {
+        // kFinAhead tiles at a time: their slot entries first, then all their partials (loads of
+        // absent entries go to column 0 and are replaced by 0), then the sums in tile order, so that
+        // the loads of a group are in flight together instead of one dependent pair after the other
+        for (int t0 = tl; t0 < T; t0 += FT * kFinAhead) {
+            int col[kFinAhead];
 #pragma unroll
-                for (int v = 0; v < NV; ++v)
-                    if (v < nv) acc[v] += part[((size_t)t * NF + f0 + v) * N + col];
+            for (int u = 0; u < kFinAhead; ++u) {
+                const int t = t0 + u * FT;
+                col[u] = t < T ? (slots ? slots[(size_t)t * Np + n] : n) : -1;
             }
+            float val[kFinAhead][NV];
+#pragma unroll
+            for (int u = 0; u < kFinAhead; ++u) {
+                const int t = min(t0 + u * FT, T - 1);
+                const float* src = part + ((size_t)t * NF + f0) * N + max(col[u], 0);
+#pragma unroll
+                for (int v = 0; v < NV; ++v) val[u][v] = v < nv ? src[(size_t)v * N] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < kFinAhead; ++u)
+#pragma unroll
+                for (int v = 0; v < NV; ++v) acc[v] += col[u] >= 0 ? val[u][v] : 0.0f;
         }
+    }
     __syncthreads();  // protects `red` against the previous call's readers
 #pragma unroll
     for (int v = 0; v < NV; ++v) red[(v * FT + tl) * (FN + 1) + nl] = acc[v];

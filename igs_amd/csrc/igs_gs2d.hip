@@ -458,6 +458,7 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
             const BinPlace bp = bins_at(ws, split_bytes, B, plan.fwd_tiles);
             BinArgs ba;
             ba.boxes = boxes_of(packed, B, plan.n_padded, plan.rec_stride);
+            ba.packed = packed; ba.RS = plan.rec_stride;
             ba.x = x; ba.y = y;
             ba.sxb = a.sxb; ba.sxw = a.sxw; ba.syb = a.syb; ba.syh = a.syh;
             ba.N = N; ba.Np = plan.n_padded; ba.H = H; ba.W = W;
@@ -589,6 +590,7 @@ int igs_gs2d_backward_reduce(const float* packed, const float* colors, const flo
         if (sep) {
             BinArgs ba;
             ba.boxes = boxes_of(packed, B, a.Np, rec_stride_of(C));
+            ba.packed = packed; ba.RS = rec_stride_of(C);
             ba.x = a.xs; ba.y = y;               // the prologue's compact column coordinates
             ba.sxb = a.Wp; ba.sxw = 1; ba.syb = a.syb; ba.syh = a.syh;
             ba.N = N; ba.Np = a.Np; ba.H = H; ba.W = W;

@@ -163,8 +163,8 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
 }
 
 // ----------------------------------------------------------------------------- binning
-// Per pixel tile, the Gaussians whose reach box meets the tile's coordinate range, as a list
-// of indices in increasing order (so that sums over a list keep the order of the unculled
+// Per pixel tile, the Gaussians whose reach box meets the tile's coordinate range and whose
+// ellipse can reach it (ellipse_reaches), as a list of indices in increasing order (so that sums over a list keep the order of the unculled
 // sum), and the count.  One workgroup per (tile, image) scans all N boxes; positions come
 // from ballots and a fixed-order prefix over the four waves, so the lists are reproducible.
 // With `slots` set, the inverse map is written as well: slots[b][tile][n] = position of
@@ -173,6 +173,8 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
 // [min, max] of x over its columns and of y over its rows (no monotonicity assumed).
 struct BinArgs {
     const float4* boxes;  // [B][Np]
+    const float* packed;  // [B][Np][RS] records (the refined test reads px, py, A', B2', D')
+    int RS;
     const float* x;
     const float* y;
     long sxb, sxw, syb, syh;
@@ -186,6 +188,34 @@ struct BinArgs {
 };
 
 constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads in flight per tile
+
+// Second test for a Gaussian whose reach box meets the tile: can its ellipse reach the tile's
+// coordinate rectangle at all (the box of a long, rotated ellipse is mostly empty)?  With
+// P = -q' = a dx^2 + b2 dx dy + d dy^2 (a, b2, d = -A', -B2', -D' of the record), the minimum of
+// P over the rectangle is 0 when it holds the centre and else lies on an edge, where P is a
+// parabola in one variable (an error in the vertex only raises the value in second order).  The
+// kernels' weight is exactly 0 where their fp32 q' is below -150; both their q' and the P
+// evaluated here differ from the exact value by a few ulp of the largest term, bounded over the
+// rectangle by T below.  The tile is dropped only if min P - 4e-6 T > 155: the same margin
+// against rounding as the reach box has, so dropping it changes no bit either.  A
+// non-positive-definite or NaN record fails the comparison and stays listed.
+__device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, float txlo, float txhi,
+                                                float tylo, float tyhi) {
+    const float4 h = *reinterpret_cast<const float4*>(rec);  // px, py, A', B2'
+    const float a = -h.z, b2 = -h.w, d = -rec[4];
+    const float x0 = txlo - h.x, x1 = txhi - h.x, y0 = tylo - h.y, y1 = tyhi - h.y;
+    if (x0 <= 0.0f && x1 >= 0.0f && y0 <= 0.0f && y1 >= 0.0f) return true;
+    auto form = [&](float x, float y) { return fmaf(fmaf(b2, x, d * y), y, a * x * x); };
+    auto clamp = [](float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); };
+    const float ky = -0.5f * b2 / d, kx = -0.5f * b2 / a;  // vertex of the parabola on a vertical / horizontal edge
+    float pmin = form(x0, clamp(ky * x0, y0, y1));
+    pmin = fminf(pmin, form(x1, clamp(ky * x1, y0, y1)));
+    pmin = fminf(pmin, form(clamp(kx * y0, x0, x1), y0));
+    pmin = fminf(pmin, form(clamp(kx * y1, x0, x1), y1));
+    const float mx = fmaxf(fabsf(x0), fabsf(x1)), my = fmaxf(fabsf(y0), fabsf(y1));
+    const float T = a * mx * mx + fabsf(b2) * mx * my + d * my * my;
+    return !(pmin - 4e-6f * T > 155.0f);
+}
 
 __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     if (a.flag != nullptr && *a.flag != a.want) return;
@@ -232,6 +262,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     const float4* boxes = a.boxes + (size_t)b * a.Np;
+    const float* recs = a.packed + (size_t)b * a.Np * a.RS;
     // Each wave scans one contiguous share of the Gaussians twice, without barriers: first to
     // count, then (with the shares' counts prefixed in wave order) to write.
     const int per_wave = ((a.N + kBinWaves - 1) / kBinWaves + 63) & ~63;
@@ -251,14 +282,24 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             in[u] = n0 + u * 64 + lane < ne;
             // "definitely outside" negated, so that NaN bounds count as inside
             listed[u] = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
+            // bounded box (unbounded ones mark records that must never be skipped): refine
+            if (listed[u] && bb[u].x > -inf)
+                listed[u] = ellipse_reaches(recs + (size_t)(n0 + u * 64 + lane) * a.RS, txlo, txhi, tylo, tyhi);
         }
     };
-    int cnt = 0;
-    for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
+    // the first pass keeps its verdicts (one bit per box of this lane) for the second one when
+    // they fit in a register pair, i.e. up to 64 boxes per lane (N <= 65536)
+    const bool keep = per_wave <= 64 * 64;
+    unsigned long long verdicts = 0ull;
+    int cnt = 0, it = 0;
+    for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
         bool listed[kU], in[kU];
         classify(n0, listed, in);
 #pragma unroll
-        for (int u = 0; u < kU; ++u) cnt += __popcll(__ballot(listed[u]));
+        for (int u = 0; u < kU; ++u) {
+            cnt += __popcll(__ballot(listed[u]));
+            if (listed[u]) verdicts |= 1ull << ((it * kU + u) & 63);
+        }
     }
     if (lane == 0) wsum[wave] = cnt;
     __syncthreads();
@@ -268,9 +309,18 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         if (w < wave) base += wsum[w];
         total += wsum[w];
     }
-    for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
+    it = 0;
+    for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
         bool listed[kU], in[kU];
-        classify(n0, listed, in);
+        if (keep) {
+#pragma unroll
+            for (int u = 0; u < kU; ++u) {
+                in[u] = n0 + u * 64 + lane < ne;
+                listed[u] = (verdicts >> ((it * kU + u) & 63)) & 1ull;
+            }
+        } else {
+            classify(n0, listed, in);
+        }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             const int n = n0 + u * 64 + lane;

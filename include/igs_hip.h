@@ -108,7 +108,7 @@ int igs_gs2d_grid_classify(const float *x, const float *y, const int64_t grid_st
  * record.  Behind the records the buffer holds one "reach box" per Gaussian: the bounding box
  * of the ellipse outside of which the kernels' exp2 returns exactly 0 for it.  On separable
  * grids the forward and the backward skip, per pixel tile, the Gaussians whose box misses the
- * tile; only exact zeros are skipped and the order of the other terms is kept, so results
+ * tile or whose ellipse (same threshold) does not reach the tile's coordinate rectangle; only exact zeros are skipped and the order of the other terms is kept, so results
  * equal those of not skipping bit for bit while the forward runs one Gaussian split
  * (plan.fwd_split == 1) and to fp32 rounding otherwise, where a tile's list rather than the
  * index range is cut into the splits (the reference evaluates every pair:

@@ -257,6 +257,29 @@ def reach_box(position, a, b_, d, q_max: float = REACH_Q):
     return torch.stack([px - hx, px + hx, py - hy, py + hy], dim=-1)
 
 
+def min_q_over_rect(px, py, a, b_, d, xlo, xhi, ylo, yhi):
+    """Minimum of q(dx, dy) = a dx^2 + 2 b dx dy + d dy^2 (positive definite) over the rectangle
+    [xlo, xhi] x [ylo, yhi], dx = x - px, dy = y - py; tensors broadcast.  0 if the rectangle holds
+    the centre; else the minimum of a convex function lies on the boundary, and on an edge q is a
+    parabola in one variable whose vertex is clamped to the edge.  Restates the second culling test
+    of the HIP binning kernel (a tile is dropped for a Gaussian when this minimum is beyond the
+    zero-weight threshold); no counterpart in the reference."""
+    x0, x1, y0, y1 = xlo - px, xhi - px, ylo - py, yhi - py
+
+    def q(dx, dy):
+        return a * dx * dx + 2 * b_ * dx * dy + d * dy * dy
+
+    def clamp(v, lo, hi):
+        return torch.minimum(torch.maximum(v, lo), hi)
+
+    edges = torch.stack(torch.broadcast_tensors(
+        q(x0, clamp(-b_ * x0 / d, y0, y1)), q(x1, clamp(-b_ * x1 / d, y0, y1)),
+        q(clamp(-b_ * y0 / a, x0, x1), y0), q(clamp(-b_ * y1 / a, x0, x1), y1)))
+    inside = (x0 <= 0) & (x1 >= 0) & (y0 <= 0) & (y1 >= 0)
+    m = edges.min(dim=0).values
+    return torch.where(inside, torch.zeros_like(m), m)
+
+
 def brute_force_forward(x, y, position, a, b_, d, alphas, colors, eps=1e-6):
     """Plain Python triple loop over (image, pixel, gaussian) in Python floats (fp64)."""
     B, N, C = colors.shape

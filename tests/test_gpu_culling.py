@@ -74,6 +74,20 @@ def test_culled_equals_unculled_bit_for_bit(igs, dev, no_cull, shape):
         assert torch.equal(grads[k], grads0[k]), k
 
 
+def test_long_rotated_gaussians_bit_for_bit(igs, dev, no_cull):
+    """Aspect ratios up to 100 at random angles: the reach boxes are mostly empty and the second,
+    ellipse-against-tile test of the binning decides; it must drop exact zeros only."""
+    B, N, H, W, C = 2, 120, 192, 320, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=77, smin=0.002, smax=0.2)
+    out, grads = run(igs, g)
+    with no_cull:
+        out0, grads0 = run(igs, g)
+    assert float(out.abs().max()) > 0
+    assert torch.equal(out, out0)
+    for k in NAMES:
+        assert torch.equal(grads[k], grads0[k]), k
+
+
 def test_culled_equals_unculled_with_several_forward_splits(igs, dev, no_cull):
     """With S > 1 forward splits a tile's list (not the index range) is cut into S parts, so the
     same terms are grouped into other partial sums: equal to fp32 rounding, not bit for bit."""

@@ -219,3 +219,34 @@ def test_under_torch_compile_and_opcheck(igs, dev):
     out = torch.compile(f, fullgraph=True, dynamic=True)(xc)
     out.backward()
     assert torch.equal(out, f(x)) and torch.equal(xc.grad, xe.grad)
+
+
+def test_against_committed_golden_fixture(igs, dev):
+    """tests/golden/koleo_golden.npz (fp64 oracle results of seeded cases, made by
+    tests/golden/make_golden_koleo.py); every case has gaps between the two nearest similarities
+    far above fp32 rounding, so indices and gradients compare directly."""
+    import importlib.util
+    import os
+
+    import numpy as np
+    from igs_amd.reg import koleo_nearest_neighbours
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden_koleo", os.path.join(here, "make_golden_koleo.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    blob = np.load(os.path.join(here, "koleo_golden.npz"))
+    for case in mg.CASES:
+        x = mg.inputs(case).to(dev, torch.float32)
+        ref = {k: torch.from_numpy(blob[f"{case}/{k}"]) for k in ("loss", "nearest", "index", "gap", "grad")}
+        assert float(ref["gap"].min()) > 1e-5, case
+        xg = x.clone().requires_grad_(True)
+        loss = igs.koleo_diversity_loss(xg)
+        loss.backward()
+        assert abs(float(loss) - float(ref["loss"])) <= 1e-6 + 1e-5 * abs(float(ref["loss"])), case
+        val, idx = koleo_nearest_neighbours(x)
+        assert torch.equal(idx.cpu().long(), ref["index"]), case
+        assert float((val.cpu().double() - ref["nearest"]).abs().max()) <= 2e-6, case
+        d = xg.grad.cpu().double() - ref["grad"]
+        assert float(d.abs().max()) <= 1e-4 * float(ref["grad"].abs().max()), case
+        assert float(d.norm()) <= 1e-4 * float(ref["grad"].norm()), case

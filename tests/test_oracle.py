@@ -305,3 +305,40 @@ def test_reach_box_bounds_the_ellipse_tightly():
     ddx, ddy = gx - pos[..., 0, None], gy - pos[..., 1, None]
     qq = a[..., None] * ddx * ddx + 2 * b[..., None] * ddx * ddy + d[..., None] * ddy * ddy
     assert bool(outside.any()) and bool((qq[outside] > Q).all())
+
+
+def test_min_q_over_rect_against_dense_sampling():
+    """Pins the rectangle minimum used by the second culling test: never above the minimum over a
+    dense sample of the rectangle (it is a lower bound of every pixel's q), equal to it up to the
+    sampling step, 0 when the centre is inside, and the closed form a dist_x^2 + d dist_y^2 for
+    axis-aligned Gaussians.  A wrong vertex (sign, a/d swapped, factor 2) fails the first two."""
+    g = torch.Generator().manual_seed(11)
+    n = 300
+    sc = torch.rand(1, n, 2, generator=g, dtype=F64) * 0.3 + 0.01
+    rot = torch.rand(1, n, generator=g, dtype=F64) * 2 * math.pi
+    a, b, d = (t.reshape(n) for t in O.cov_inverse_closed(sc, rot))
+    px, py = (torch.rand(n, generator=g, dtype=F64) * 2 - 1 for _ in range(2))
+    cx, cy = (torch.rand(n, generator=g, dtype=F64) * 2 - 1 for _ in range(2))
+    hw, hh = (torch.rand(n, generator=g, dtype=F64) * 0.3 + 0.01 for _ in range(2))
+    xlo, xhi, ylo, yhi = cx - hw, cx + hw, cy - hh, cy + hh
+    m = O.min_q_over_rect(px, py, a, b, d, xlo, xhi, ylo, yhi)
+    k = 401
+    t = torch.linspace(0, 1, k, dtype=F64)
+    xs = xlo[:, None] + (xhi - xlo)[:, None] * t            # [n,k]
+    ys = ylo[:, None] + (yhi - ylo)[:, None] * t
+    dx = xs[:, :, None] - px[:, None, None]
+    dy = ys[:, None, :] - py[:, None, None]
+    q = a[:, None, None] * dx * dx + 2 * b[:, None, None] * dx * dy + d[:, None, None] * dy * dy
+    sampled = q.flatten(1).min(dim=1).values
+    assert bool((m <= sampled * (1 + 1e-12) + 1e-12).all())                       # a lower bound
+    # the sampled minimum is within one grid step of the true one: |grad q| * step
+    gmax = 2 * (a + b.abs() + d) * (hw + hh + (cx - px).abs() + (cy - py).abs())
+    assert bool((sampled - m <= gmax * (hw + hh) * 2 / (k - 1) + 1e-9).all())      # and attained
+    inside = (xlo <= px) & (px <= xhi) & (ylo <= py) & (py <= yhi)
+    assert bool(inside.any()) and bool((m[inside] == 0).all()) and bool((m[~inside] > 0).all())
+    # axis-aligned: distance to the rectangle per axis
+    z = torch.zeros(n, dtype=F64)
+    m0 = O.min_q_over_rect(px, py, a, z, d, xlo, xhi, ylo, yhi)
+    ddx = torch.clamp(torch.maximum(xlo - px, px - xhi), min=0)
+    ddy = torch.clamp(torch.maximum(ylo - py, py - yhi), min=0)
+    torch.testing.assert_close(m0, a * ddx * ddx + d * ddy * ddy, rtol=1e-12, atol=1e-15)

@@ -118,3 +118,27 @@ def test_backward_with_given_neighbours():
     sim = (fn * torch.gather(fn, 1, other[..., None].expand(2, 6, 3))).sum(-1)
     (g,) = torch.autograd.grad(torch.relu(sim + 1).mean() * 0.7, xr)
     torch.testing.assert_close(K.koleo_backward(x, 0.7, neighbours=other), g, rtol=1e-12, atol=1e-15)
+
+
+def _golden():
+    import importlib.util
+    import os
+
+    import numpy as np
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden_koleo", os.path.join(here, "make_golden_koleo.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    return mg, np.load(os.path.join(here, "koleo_golden.npz"))
+
+
+def test_oracle_reproduces_golden_fixture():
+    import numpy as np
+
+    mg, blob = _golden()
+    for case in mg.CASES:
+        x, res = mg.compute(case)
+        assert float(K.koleo_diversity_loss(x)) == pytest.approx(K.koleo_loops(x.tolist()), rel=1e-12)
+        for k, v in res.items():
+            assert np.allclose(v.numpy(), blob[f"{case}/{k}"], rtol=1e-11, atol=1e-14), (case, k)
