@@ -164,8 +164,8 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
 
 // ----------------------------------------------------------------------------- binning
 // Per pixel tile, the Gaussians whose reach box meets the tile's coordinate range and whose
-// ellipse can reach it (ellipse_reaches), as a list of indices in increasing order (so that sums over a list keep the order of the unculled
-// sum), and the count.  One workgroup per (tile, image) scans all N boxes; positions come
+// ellipse can reach it (ellipse_reaches), as a list of indices in increasing order (so that
+// sums over a list keep the order of the unculled sum), and the count.  One workgroup per (tile, image) scans all N boxes; positions come
 // from ballots and a fixed-order prefix over the four waves, so the lists are reproducible.
 // With `slots` set, the inverse map is written as well: slots[b][tile][n] = position of
 // Gaussian n in the tile's list, or -1 when it is not listed (every n < N is written).
@@ -193,8 +193,7 @@ constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads i
 // coordinate rectangle at all (the box of a long, rotated ellipse is mostly empty)?  With
 // P = -q' = a dx^2 + b2 dx dy + d dy^2 (a, b2, d = -A', -B2', -D' of the record), the minimum of
 // P over the rectangle is 0 when it holds the centre and else lies on an edge, where P is a
-// parabola in one variable (an error in the vertex only raises the value in second order).  The
-// kernels' weight is exactly 0 where their fp32 q' is below -150; both their q' and the P
+// parabola in one variable.  The kernels' weight is exactly 0 where their fp32 q' is below -150; both their q' and the P
 // evaluated here differ from the exact value by a few ulp of the largest term, bounded over the
 // rectangle by T below.  The tile is dropped only if min P - 4e-6 T > 155: the same margin
 // against rounding as the reach box has, so dropping it changes no bit either.  A
@@ -205,13 +204,21 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
     const float a = -h.z, b2 = -h.w, d = -rec[4];
     const float x0 = txlo - h.x, x1 = txhi - h.x, y0 = tylo - h.y, y1 = tyhi - h.y;
     if (x0 <= 0.0f && x1 >= 0.0f && y0 <= 0.0f && y1 >= 0.0f) return true;
+    // the argument below needs a form that is positive definite beyond the rounding of its
+    // (fp32) coefficients; ellipses thinner than about 1:600 simply stay listed
+    if (!(a > 0.0f && 4.0f * a * d - b2 * b2 > 4e-5f * a * d)) return true;
     auto form = [&](float x, float y) { return fmaf(fmaf(b2, x, d * y), y, a * x * x); };
     auto clamp = [](float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); };
-    const float ky = -0.5f * b2 / d, kx = -0.5f * b2 / a;  // vertex of the parabola on a vertical / horizontal edge
-    float pmin = form(x0, clamp(ky * x0, y0, y1));
-    pmin = fminf(pmin, form(x1, clamp(ky * x1, y0, y1)));
-    pmin = fminf(pmin, form(clamp(kx * y0, x0, x1), y0));
-    pmin = fminf(pmin, form(clamp(kx * y1, x0, x1), y1));
+    // Only the edges that face the centre can hold the minimum: P grows along every ray from the
+    // centre, and the ray to a point of the rectangle enters it through such an edge.  The vertex
+    // of an edge's parabola uses the hardware reciprocal (its error is of second order in P).
+    const float inf = __builtin_inff();
+    const bool vx = x0 > 0.0f || x1 < 0.0f, vy = y0 > 0.0f || y1 < 0.0f;
+    const float xe = x0 > 0.0f ? x0 : x1, ye = y0 > 0.0f ? y0 : y1;
+    const float ky = -0.5f * b2 * __builtin_amdgcn_rcpf(d), kx = -0.5f * b2 * __builtin_amdgcn_rcpf(a);
+    const float pv = vx ? form(xe, clamp(ky * xe, y0, y1)) : inf;
+    const float ph = vy ? form(clamp(kx * ye, x0, x1), ye) : inf;
+    const float pmin = fminf(pv, ph);
     const float mx = fmaxf(fabsf(x0), fabsf(x1)), my = fmaxf(fabsf(y0), fabsf(y1));
     const float T = a * mx * mx + fabsf(b2) * mx * my + d * my * my;
     return !(pmin - 4e-6f * T > 155.0f);
