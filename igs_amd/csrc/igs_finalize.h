@@ -67,6 +67,65 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const i
     }
 }
 
+// The same sum after a two-level binning: a tile's slot entry exists only where the super-tile
+// lists the Gaussian (cslots[st][n] >= 0), so the t-lanes walk the super-tiles (t-lane k takes
+// k, k + FT, ...) and, in a listed one, its tiles row by row (the four tiles of a row together).
+// A Gaussian reaches a few super-tiles, so this reads a fraction of the slot tables.
+struct SuperSlots {
+    const int* cslots;  // this image's [stiles][Np]; nullptr: one-level binning
+    int tiles_x, tiles_y, stiles_x, stiles;
+};
+
+template <int NV, int FT>
+__device__ __forceinline__ void tile_sum_super(const float* __restrict__ part, const int* __restrict__ slots,
+                                               const SuperSlots sup, int Np, int n, int NF, int N, int f0,
+                                               bool valid, float (&out)[NV], float* red, int nv = NV) {
+    constexpr int FN = 256 / FT;
+    const int tl = threadIdx.x / FN, nl = threadIdx.x % FN;
+    float acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
+    if (valid) {
+        for (int st = tl; st < sup.stiles; st += FT) {
+            if (sup.cslots[(size_t)st * Np + n] < 0) continue;
+            const int sy = st / sup.stiles_x, sx = st - sy * sup.stiles_x;
+            for (int j = 0; j < kSuperY; ++j) {
+                const int ty = sy * kSuperY + j;
+                if (ty >= sup.tiles_y) break;
+                int col[kSuperX];
+#pragma unroll
+                for (int u = 0; u < kSuperX; ++u) {
+                    const int tx = sx * kSuperX + u;
+                    col[u] = tx < sup.tiles_x ? slots[(size_t)(ty * sup.tiles_x + tx) * Np + n] : -1;
+                }
+                float val[kSuperX][NV];
+#pragma unroll
+                for (int u = 0; u < kSuperX; ++u) {
+                    const int t = ty * sup.tiles_x + min(sx * kSuperX + u, sup.tiles_x - 1);
+                    const float* src = part + ((size_t)t * NF + f0) * N + max(col[u], 0);
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) val[u][v] = v < nv ? src[(size_t)v * N] : 0.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < kSuperX; ++u)
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) acc[v] += col[u] >= 0 ? val[u][v] : 0.0f;
+            }
+        }
+    }
+    __syncthreads();  // protects `red` against the previous call's readers
+#pragma unroll
+    for (int v = 0; v < NV; ++v) red[(v * FT + tl) * (FN + 1) + nl] = acc[v];
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < FT; ++k) s += red[(v * FT + k) * (FN + 1) + nl];
+        out[v] = s;
+    }
+}
+
 // Finalize: FT threads per Gaussian; sums the T tile partials in a fixed order and applies
 //   d alpha = M0, d color_c = alpha CG_c, d px = alpha (A Mx + B My), d py = alpha (B Mx + D My),
 //   dA = -1/2 alpha Mxx, dB = -alpha Mxy, dD = -1/2 alpha Myy,
@@ -75,7 +134,7 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const i
 template <bool kScaleRot, int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
-    const int* __restrict__ slots_in, int Np, const float* __restrict__ p0,
+    const int* __restrict__ slots_in, const SuperSlots sup_in, int Np, const float* __restrict__ p0,
     const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ alphas,
     int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
@@ -94,9 +153,14 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     // the slot table belongs to the separable variant
     const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
                            ? slots_in + (size_t)b * T * Np : nullptr;
+    SuperSlots sup = sup_in;  // the super-tile tables belong to the separable variant as well
+    sup.cslots = (slots != nullptr && sup_in.cslots != nullptr) ? sup_in.cslots + (size_t)b * sup_in.stiles * Np : nullptr;
     const int nn = min(n, N - 1);
     float M[6];
-    tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+    if (sup.cslots != nullptr)  // kernel-argument and flag uniform: the barriers inside are safe
+        tile_sum_super<6, FT>(part, slots, sup, Np, nn, NF, N, 0, valid, M, red);
+    else
+        tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
     const double al = alphas[i];
     // O(BN) epilogue in fp64: the chain rule multiplies sums by 1/s^3-sized factors
     double A, Bc, D, cs = 0., sn = 0., i0 = 0., i1 = 0., s0 = 0., s1 = 0.;
@@ -137,7 +201,10 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
         for (int c0 = 0; c0 < C; c0 += kFinColours) {  // colour sums, kFinColours channels per pass
             float sc[kFinColours];
             const int nc = min(kFinColours, C - c0);
-            tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+            if (sup.cslots != nullptr)
+                tile_sum_super<kFinColours, FT>(part, slots, sup, Np, nn, NF, N, 6 + c0, valid, sc, red, nc);
+            else
+                tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
             if (writer)
 #pragma unroll
                 for (int c = 0; c < kFinColours; ++c)
@@ -151,7 +218,8 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
 template <int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
-    const int* __restrict__ slots_in, int Np, const float* __restrict__ feat, int N, int C, int Cp,
+    const int* __restrict__ slots_in, const SuperSlots sup_in, int Np, const float* __restrict__ feat, int N,
+    int C, int Cp,
     float eps, float* __restrict__ g_feat) {
     constexpr int FN = 256 / FT;
     __shared__ float red[kFinColours * FT * (FN + 1)];
@@ -165,9 +233,14 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const float* part = partial + (size_t)b * T * NF * N;
     const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
                            ? slots_in + (size_t)b * T * Np : nullptr;
+    SuperSlots sup = sup_in;  // the super-tile tables belong to the separable variant as well
+    sup.cslots = (slots != nullptr && sup_in.cslots != nullptr) ? sup_in.cslots + (size_t)b * sup_in.stiles * Np : nullptr;
     const int nn = min(n, N - 1);
     float M[6];
-    tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+    if (sup.cslots != nullptr)  // kernel-argument and flag uniform: the barriers inside are safe
+        tile_sum_super<6, FT>(part, slots, sup, Np, nn, NF, N, 0, valid, M, red);
+    else
+        tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
     const float* f = feat + i * (6 + C);
     const double e0 = (double)expf(f[2]), e1 = (double)expf(f[3]);
     const double s0 = e0 + (double)eps, s1 = e1 + (double)eps;
@@ -192,7 +265,10 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     for (int c0 = 0; c0 < C; c0 += kFinColours) {
         float sc[kFinColours];
         const int nc = min(kFinColours, C - c0);
-        tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+        if (sup.cslots != nullptr)
+            tile_sum_super<kFinColours, FT>(part, slots, sup, Np, nn, NF, N, 6 + c0, valid, sc, red, nc);
+        else
+            tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
         if (writer)
 #pragma unroll
             for (int c = 0; c < kFinColours; ++c)

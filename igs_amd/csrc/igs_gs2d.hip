@@ -109,6 +109,47 @@ inline size_t bins_bytes(int B, int tiles, int Np) {
 }
 inline size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
 
+// Two-level binning.  With many tiles and many Gaussians the cost of k_bin is every tile's
+// workgroup reading all N reach boxes.  In two levels, the Gaussians are first listed per
+// super-tile (kSuperX x kSuperY tiles; K workgroups per super-tile, each scanning one chunk of
+// the Gaussians into its own segment of the list), then every tile scans the segments of its
+// super-tile only; the finalize kernel looks at a tile's slot entry only where the super-tile
+// lists the Gaussian.  The tile lists, and with them the forward, are the same as with one level;
+// the finalize kernel adds the tiles in another order (super-tile by super-tile), so gradients
+// agree to rounding.  Space for the super-tile lists / tables is part of the plan whenever the
+// tile grid is large enough (a function of the shape only); whether a launch uses them depends
+// on the work, tiles x N, or on IGS_BIN_LEVELS=1|2 in the environment (read at every call).
+struct SuperGeometry {
+    int x, y, count;  // super-tiles along x, along y, per image
+    int chunk, K;     // Gaussians per first-level workgroup, workgroups per super-tile
+};
+inline SuperGeometry super_tiles(int tiles_x, int tiles_y, int B, int N) {
+    SuperGeometry g;
+    g.x = ceil_div(tiles_x, kSuperX);
+    g.y = ceil_div(tiles_y, kSuperY);
+    g.count = g.x * g.y;
+    // enough first-level workgroups for two per compute unit, of at least 4096 Gaussians each
+    int K = ceil_div(512, (long)g.count * B);
+    const int maxK = ceil_div(N, 4096);
+    K = K > maxK ? maxK : K;
+    K = K > kBinMaxChunks ? kBinMaxChunks : (K < 1 ? 1 : K);
+    g.chunk = (ceil_div(N, K) + 63) & ~63;
+    g.K = ceil_div(N, g.chunk);
+    return g;
+}
+inline bool super_reserved(int tiles_x, int tiles_y) { return tiles_x * tiles_y >= 32; }
+inline bool two_level(int N, int tiles_x, int tiles_y) {
+    if (!super_reserved(tiles_x, tiles_y)) return false;
+    const char* e = getenv("IGS_BIN_LEVELS");
+    if (e && e[0] == '1') return false;
+    if (e && e[0] == '2') return true;
+    return (long)N * tiles_x * tiles_y >= (1L << 25);  // measured break-even: N = 65536 on 256-512 tiles
+}
+// Super-tile lists of one launch: counts [B][stiles][kBinMaxChunks] then lists [B][stiles][Np].
+inline size_t super_bins_bytes(int B, int stiles, int Np) {
+    return ((size_t)B * stiles * kBinMaxChunks + (size_t)B * stiles * Np) * sizeof(int);
+}
+
 // Plan of one kernel variant (grid_mode is GENERAL or SEPARABLE here).
 int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
     if (!p) return IGS_ERR_NULL_POINTER;
@@ -163,13 +204,25 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     p->fwd_ws_bytes = S > 1 ? (uint64_t)S * B * (C + 1) * H * W * sizeof(float) : 0;
     p->pix_bytes = sep ? ((uint64_t)B * H * p->w_padded * p->pix_stride + (uint64_t)B * p->w_padded) * sizeof(float)
                        : (uint64_t)B * p->hw_padded * p->pix_stride * sizeof(float);
-    if (sep) {  // the tile lists of each launch follow its other scratch
+    const int bwd_tiles_y = sep ? (int)T / p->bwd_tiles_x : 1;
+    if (sep) {  // the tile lists of each launch follow its other scratch, then the super-tile lists
         p->fwd_ws_bytes = align16(p->fwd_ws_bytes) + bins_bytes(B, p->fwd_tiles, p->n_padded);
+        if (super_reserved(fg.tiles_x, fg.tiles_y))
+            p->fwd_ws_bytes = align16(p->fwd_ws_bytes) +
+                              super_bins_bytes(B, super_tiles(fg.tiles_x, fg.tiles_y, B, N).count, p->n_padded);
         p->pix_bytes = align16(p->pix_bytes) + bins_bytes(B, p->bwd_tiles, p->n_padded);
+        if (super_reserved(p->bwd_tiles_x, bwd_tiles_y))
+            p->pix_bytes = align16(p->pix_bytes) +
+                           super_bins_bytes(B, super_tiles(p->bwd_tiles_x, bwd_tiles_y, B, N).count, p->n_padded);
     }
     p->partial_bytes = (uint64_t)B * T * (6 + C) * N * sizeof(float);
-    if (sep)  // the slot tables [B][T][Np] (Gaussian -> position in the tile's list) follow
+    if (sep) {  // the slot tables [B][T][Np] (Gaussian -> position in the tile's list) follow,
+                // then those of the super-tiles
         p->partial_bytes = align16(p->partial_bytes) + (uint64_t)B * T * p->n_padded * sizeof(int);
+        if (super_reserved(p->bwd_tiles_x, bwd_tiles_y))
+            p->partial_bytes = align16(p->partial_bytes) +
+                               (uint64_t)B * super_tiles(p->bwd_tiles_x, bwd_tiles_y, B, N).count * p->n_padded * sizeof(int);
+    }
     return IGS_OK;
 }
 
@@ -190,6 +243,20 @@ inline BinPlace bins_at(void* ws, size_t scratch_bytes, int B, int tiles) {
     bp.counts = reinterpret_cast<int*>(base);
     bp.lists = bp.counts + (((size_t)B * tiles + 3) & ~(size_t)3);
     return bp;
+}
+
+// The super-tile lists that follow the tile lists of a launch.
+inline BinPlace super_bins_at(void* ws, size_t scratch_bytes, int B, int tiles, int Np, int stiles) {
+    char* base = static_cast<char*>(ws) + align16(align16(scratch_bytes) + bins_bytes(B, tiles, Np));
+    BinPlace bp;
+    bp.counts = reinterpret_cast<int*>(base);
+    bp.lists = bp.counts + (size_t)B * stiles * kBinMaxChunks;
+    return bp;
+}
+// The super-tile slot tables that follow the slot tables in the partial buffer.
+inline int* super_slots_at(float* partial, int B, int T, int NF, int N, int Np) {
+    char* slots = reinterpret_cast<char*>(slots_at(partial, B, T, NF, N));
+    return reinterpret_cast<int*>(slots + align16((size_t)B * T * Np * sizeof(int)));
 }
 
 inline const float4* boxes_of(const float* packed, int B, int Np, int RS) {
@@ -218,10 +285,30 @@ int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t*
     return IGS_OK;
 }
 
-int launch_bin(const BinArgs& a, int B, hipStream_t st) {
-    hipLaunchKernelGGL(k_bin, dim3(a.tiles_x * a.tiles_y, B), dim3(kBinThreads), 0, st, a);
+int launch_bin(const BinArgs& a, int K, int B, hipStream_t st) {
+    hipLaunchKernelGGL(k_bin, dim3(a.tiles_x * a.tiles_y, K, B), dim3(kBinThreads), 0, st, a);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? IGS_OK : (int)e;
+}
+
+// Tile lists in one or two levels.  `fine` describes the tiles (its slot table, if any, included);
+// `coarse` (and the super-tile slot table when `fine` has one) is used when `levels2`.
+int launch_bins(BinArgs fine, int B, bool levels2, const BinPlace& coarse, int* coarse_slots, hipStream_t st) {
+    fine.chunk = 0;
+    fine.cand_counts = nullptr; fine.cand_lists = nullptr;
+    fine.cand_K = 0; fine.cand_chunk = 0; fine.stiles_x = 0; fine.stiles = 0;
+    if (!levels2) return launch_bin(fine, 1, B, st);
+    const SuperGeometry sg = super_tiles(fine.tiles_x, fine.tiles_y, B, fine.N);
+    BinArgs c = fine;
+    c.tile_w = fine.tile_w * kSuperX; c.tile_h = fine.tile_h * kSuperY;
+    c.tiles_x = sg.x; c.tiles_y = sg.y;
+    c.counts = coarse.counts; c.lists = coarse.lists; c.slots = coarse_slots;
+    c.chunk = sg.chunk;
+    int rc = launch_bin(c, sg.K, B, st);
+    if (rc) return rc;
+    fine.cand_counts = coarse.counts; fine.cand_lists = coarse.lists;
+    fine.cand_K = sg.K; fine.cand_chunk = sg.chunk; fine.stiles_x = sg.x; fine.stiles = sg.count;
+    return launch_bin(fine, 1, B, st);
 }
 
 inline int launch_status() {
@@ -466,7 +553,11 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
             ba.tiles_x = fg.tiles_x; ba.tiles_y = fg.tiles_y;
             ba.counts = bp.counts; ba.lists = bp.lists; ba.slots = nullptr;
             ba.flag = vs[i].flag; ba.want = vs[i].want;
-            rc = launch_bin(ba, B, st);
+            const bool levels2 = two_level(N, fg.tiles_x, fg.tiles_y);
+            const BinPlace cp = levels2 ? super_bins_at(ws, split_bytes, B, plan.fwd_tiles, plan.n_padded,
+                                                        super_tiles(fg.tiles_x, fg.tiles_y, B, N).count)
+                                        : BinPlace{nullptr, nullptr};
+            rc = launch_bins(ba, B, levels2, cp, nullptr, st);
             if (rc) return rc;
             a.counts = bp.counts; a.lists = bp.lists;
         }
@@ -599,7 +690,15 @@ int igs_gs2d_backward_reduce(const float* packed, const float* colors, const flo
             ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists);
             ba.slots = slots_at(partial, B, a.T, 6 + C, N);
             ba.flag = a.flag; ba.want = a.want;
-            rc = launch_bin(ba, B, st);
+            const bool levels2 = two_level(N, ba.tiles_x, ba.tiles_y);
+            BinPlace cp{nullptr, nullptr};
+            int* cslots = nullptr;
+            if (levels2) {
+                const size_t scratch = ((size_t)B * H * a.Wp * pix_stride_sep(C) + (size_t)B * a.Wp) * sizeof(float);
+                cp = super_bins_at(pix_ws, scratch, B, a.T, a.Np, super_tiles(ba.tiles_x, ba.tiles_y, B, N).count);
+                cslots = super_slots_at(partial, B, a.T, 6 + C, N, a.Np);
+            }
+            rc = launch_bins(ba, B, levels2, cp, cslots, st);
             if (rc) return rc;
         }
         IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, st));
@@ -668,13 +767,27 @@ static const int* finalize_slots(const float* partial, int grid_mode, int B, int
     return slots_at(const_cast<float*>(partial), B, T, NF, N);
 }
 
-// T of the separable (or only) variant and of the general variant under AUTO.
-static int finalize_tiles(int grid_mode, int B, int N, int H, int W, int C, int* T, int* T_alt) {
+// T of the separable (or only) variant and of the general variant under AUTO; the super-tile slot
+// tables of the separable backward when it binned in two levels.
+static int finalize_tiles(int grid_mode, int B, int N, int H, int W, int C, int* T, int* T_alt,
+                          const float* partial, SuperSlots* sup) {
     igs_gs2d_plan_t plan;
     int rc = plan_one(B, N, H, W, C, grid_mode == IGS_GRID_AUTO ? IGS_GRID_SEPARABLE : grid_mode, &plan);
     if (rc) return rc;
     *T = plan.bwd_tiles;
     *T_alt = plan.bwd_tiles;
+    *sup = SuperSlots{nullptr, 1, 1, 1, 1};
+    if (grid_mode != IGS_GRID_GENERAL) {
+        const int tiles_y = plan.bwd_tiles / plan.bwd_tiles_x;
+        if (two_level(N, plan.bwd_tiles_x, tiles_y)) {
+            const SuperGeometry sg = super_tiles(plan.bwd_tiles_x, tiles_y, B, N);
+            sup->cslots = super_slots_at(const_cast<float*>(partial), B, plan.bwd_tiles, 6 + C, N, plan.n_padded);
+            sup->tiles_x = plan.bwd_tiles_x;
+            sup->tiles_y = tiles_y;
+            sup->stiles_x = sg.x;
+            sup->stiles = sg.count;
+        }
+    }
     if (grid_mode == IGS_GRID_AUTO) {
         rc = plan_one(B, N, H, W, C, IGS_GRID_GENERAL, &plan);
         if (rc) return rc;
@@ -693,11 +806,12 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
     int T, T_alt;
-    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
+    SuperSlots sup;
+    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
     if (rc) return rc;
     IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<false, kFT>),
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), (N + 3) & ~3, cov_inv_00,
+                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), sup, (N + 3) & ~3, cov_inv_00,
                        cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
                        g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
     return launch_status();
@@ -712,11 +826,12 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
     int T, T_alt;
-    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt);
+    SuperSlots sup;
+    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
     if (rc) return rc;
     IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<true, kFT>),
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), (N + 3) & ~3, scales, rotations,
+                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), sup, (N + 3) & ~3, scales, rotations,
                        (const float*)nullptr, alphas, N, C, eps, g_positions,
                        g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
     return launch_status();
@@ -745,11 +860,12 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
     if (rc) return rc;
     if (C < 1 || C > C_kernel || !channels_compiled(C_kernel)) return IGS_ERR_BAD_CHANNELS;
     int T, T_alt;
-    rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt);
+    SuperSlots sup;
+    rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt, partial, &sup);
     if (rc) return rc;
     IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize_feature<kFT>),
                        (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N), (N + 3) & ~3, gs_feature,
+                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N), sup, (N + 3) & ~3, gs_feature,
                        N, C, C_kernel, eps, g_feature);
     return launch_status();
 }

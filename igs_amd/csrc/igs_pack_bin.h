@@ -165,10 +165,15 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
 // ----------------------------------------------------------------------------- binning
 // Per pixel tile, the Gaussians whose reach box meets the tile's coordinate range and whose
 // ellipse can reach it (ellipse_reaches), as a list of indices in increasing order (so that
-// sums over a list keep the order of the unculled sum), and the count.  One workgroup per (tile, image) scans all N boxes; positions come
-// from ballots and a fixed-order prefix over the four waves, so the lists are reproducible.
+// sums over a list keep the order of the unculled sum), and the count.  One workgroup per
+// (tile, image) scans all N boxes — or, in a two-level binning, a chunk of them for a super-tile
+// (first level) or the segments of its super-tile's list (second level); positions come from
+// ballots and a fixed-order prefix over the waves, so the lists are reproducible.
 // With `slots` set, the inverse map is written as well: slots[b][tile][n] = position of
-// Gaussian n in the tile's list, or -1 when it is not listed (every n < N is written).
+// Gaussian n in the tile's list, or -1 when it is not listed; written for every candidate, i.e.
+// every n < N except at the second level of a two-level binning, where a tile's entries exist
+// only for the Gaussians listed for its super-tile (whose table, non-negative = listed, the
+// first level writes).
 // Separable grids only: a tile is tile_w columns x tile_h rows and its coordinate range is
 // [min, max] of x over its columns and of y over its rows (no monotonicity assumed).
 struct BinArgs {
@@ -180,12 +185,24 @@ struct BinArgs {
     long sxb, sxw, syb, syh;
     int N, Np, H, W;
     int tile_w, tile_h, tiles_x, tiles_y;
-    int* counts;  // [B][tiles]
+    int* counts;  // [B][tiles] ([B][tiles][K] with chunks)
     int* lists;   // [B][tiles][Np]
     int* slots;   // [B][tiles][Np] or nullptr
+    // Two-level binning.  First level (chunk > 0): the tiles are super-tiles of kSuperX x kSuperY
+    // tiles and gridDim.y = K workgroups share a super-tile, workgroup k scanning the Gaussians
+    // [k chunk, (k + 1) chunk) into segment k of the list (at offset k chunk, with its own count).
+    // Second level (cand_lists set): a tile scans the K segments of its super-tile's list, in order,
+    // instead of all N Gaussians.
+    int chunk;
+    const int* cand_counts;  // [B][stiles][cand_K]
+    const int* cand_lists;   // [B][stiles][Np], segment k at offset k cand_chunk
+    int cand_K, cand_chunk, stiles_x, stiles;
     const int* flag;
     int want;
 };
+
+// Tiles per super-tile of the two-level binning (each way) and the most segments per list.
+constexpr int kSuperX = 4, kSuperY = 4, kBinMaxChunks = 64;
 
 constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads in flight per tile
 
@@ -228,9 +245,10 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     if (a.flag != nullptr && *a.flag != a.want) return;
     __shared__ float red[4][kBinThreads];
     __shared__ int wsum[kBinWaves];
+    __shared__ int seg_first[kBinMaxChunks + 1];  // second level: first candidate index of each segment
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tiles = a.tiles_x * a.tiles_y;
-    const int t = blockIdx.x, b = blockIdx.y;
+    const int t = blockIdx.x, kc = blockIdx.y, K = gridDim.y, b = blockIdx.z;
     const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
     const int c0 = tx * a.tile_w, c1 = min(a.W, c0 + a.tile_w);
     const int r0 = ty * a.tile_h, r1 = min(a.H, r0 + a.tile_h);
@@ -266,24 +284,54 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         __syncthreads();
     }
     const float txlo = red[0][0], txhi = -red[1][0], tylo = red[2][0], tyhi = -red[3][0];
-    int* list = a.lists + ((size_t)b * tiles + t) * a.Np;
+    int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     const float4* boxes = a.boxes + (size_t)b * a.Np;
     const float* recs = a.packed + (size_t)b * a.Np * a.RS;
-    // Each wave scans one contiguous share of the Gaussians twice, without barriers: first to
+    // The candidates, numbered 0..M-1: all Gaussians; or this workgroup's chunk of them (first
+    // level); or the entries of the super-tile's list, segment after segment (second level).
+    int first = 0, M = a.N;
+    const int* cand = nullptr;
+    if (a.chunk > 0) {
+        first = kc * a.chunk;
+        M = max(0, min(a.N, first + a.chunk) - first);
+    }
+    if (a.cand_lists != nullptr) {
+        const size_t st = (size_t)b * a.stiles + (ty / kSuperY) * a.stiles_x + tx / kSuperX;
+        cand = a.cand_lists + st * a.Np;
+        if (tid == 0) {
+            int run = 0;
+            for (int j = 0; j < a.cand_K; ++j) {
+                seg_first[j] = run;
+                run += a.cand_counts[st * a.cand_K + j];
+            }
+            for (int j = a.cand_K; j <= kBinMaxChunks; ++j) seg_first[j] = run;
+        }
+        __syncthreads();
+        M = seg_first[kBinMaxChunks];
+    }
+    // candidate index -> Gaussian index
+    auto gaussian_of = [&](int i) {
+        if (cand == nullptr) return first + i;
+        int seg = 0;  // the last segment that starts at or before i (binary search over 64 entries)
+#pragma unroll
+        for (int step = kBinMaxChunks / 2; step > 0; step >>= 1)
+            if (seg_first[seg + step] <= i) seg += step;
+        return cand[(size_t)seg * a.cand_chunk + (i - seg_first[seg])];
+    };
+    // Each wave scans one contiguous share of the candidates twice, without barriers: first to
     // count, then (with the shares' counts prefixed in wave order) to write.
-    const int per_wave = ((a.N + kBinWaves - 1) / kBinWaves + 63) & ~63;
-    const int nb = wave * per_wave, ne = min(a.N, nb + per_wave);
+    const int per_wave = ((M + kBinWaves - 1) / kBinWaves + 63) & ~63;
+    const int nb = wave * per_wave, ne = min(M, nb + per_wave);
     const unsigned long long below = (1ull << lane) - 1ull;
     // kU boxes per lane are loaded together, so that kU loads are in flight instead of one
     constexpr int kU = 8;
-    auto classify = [&](int n0, bool (&listed)[kU], bool (&in)[kU]) {
+    auto classify = [&](int n0, bool (&listed)[kU], bool (&in)[kU], int (&n)[kU]) {
         float4 bb[kU];
 #pragma unroll
-        for (int u = 0; u < kU; ++u) {
-            const int n = n0 + u * 64 + lane;
-            bb[u] = boxes[min(n, a.N - 1)];
-        }
+        for (int u = 0; u < kU; ++u) n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));  // M > 0 inside the loops
+#pragma unroll
+        for (int u = 0; u < kU; ++u) bb[u] = boxes[n[u]];
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             in[u] = n0 + u * 64 + lane < ne;
@@ -291,17 +339,18 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             listed[u] = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
             // bounded box (unbounded ones mark records that must never be skipped): refine
             if (listed[u] && bb[u].x > -inf)
-                listed[u] = ellipse_reaches(recs + (size_t)(n0 + u * 64 + lane) * a.RS, txlo, txhi, tylo, tyhi);
+                listed[u] = ellipse_reaches(recs + (size_t)n[u] * a.RS, txlo, txhi, tylo, tyhi);
         }
     };
     // the first pass keeps its verdicts (one bit per box of this lane) for the second one when
-    // they fit in a register pair, i.e. up to 64 boxes per lane (N <= 65536)
+    // they fit in a register pair, i.e. up to 64 boxes per lane (65536 candidates)
     const bool keep = per_wave <= 64 * 64;
     unsigned long long verdicts = 0ull;
     int cnt = 0, it = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
         bool listed[kU], in[kU];
-        classify(n0, listed, in);
+        int n[kU];
+        classify(n0, listed, in, n);
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             cnt += __popcll(__ballot(listed[u]));
@@ -319,24 +368,27 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     it = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
         bool listed[kU], in[kU];
+        int n[kU];
         if (keep) {
 #pragma unroll
             for (int u = 0; u < kU; ++u) {
                 in[u] = n0 + u * 64 + lane < ne;
                 listed[u] = (verdicts >> ((it * kU + u) & 63)) & 1ull;
+                n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));
             }
         } else {
-            classify(n0, listed, in);
+            classify(n0, listed, in, n);
         }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
-            const int n = n0 + u * 64 + lane;
             const unsigned long long m = __ballot(listed[u]);
             const int pos = base + __popcll(m & below);
-            if (listed[u]) list[pos] = n;
-            if (slot != nullptr && in[u]) slot[n] = listed[u] ? pos : -1;
+            if (listed[u]) list[pos] = n[u];
+            // the slot of every candidate: its position (within the segment, at the first level,
+            // where only the sign is used) or -1
+            if (slot != nullptr && in[u]) slot[n[u]] = listed[u] ? pos : -1;
             base += __popcll(m);
         }
     }
-    if (tid == 0) a.counts[(size_t)b * tiles + t] = total;
+    if (tid == 0) a.counts[((size_t)b * tiles + t) * K + kc] = total;
 }

@@ -80,10 +80,12 @@ typedef struct igs_gs2d_plan_t {
     uint64_t packed_bytes;   /* packed Gaussian buffer: records, then one reach box (4
                                 floats) per record: B*n_padded*(rec_stride+4)*4            */
     uint64_t fwd_ws_bytes;   /* forward scratch: split partials (fwd_split > 1) and, on
-                                separable grids, the per-tile Gaussian lists                */
+                                separable grids, the per-tile Gaussian lists (plus those
+                                of the super-tiles when there are 32 tiles or more)         */
     uint64_t pix_bytes;      /* backward scratch: per-pixel records and, on separable
-                                grids, the per-tile Gaussian lists                          */
-    uint64_t partial_bytes;  /* backward partial sums: B*T*(6+C)*N*4                       */
+                                grids, the Gaussian lists as above                          */
+    uint64_t partial_bytes;  /* backward partial sums B*T*(6+C)*N*4 and, on separable
+                                grids, the slot tables of the tiles (and super-tiles)       */
     int32_t fwd_tiles;       /* separable: pixel tiles per image of the forward            */
     int32_t bwd_tiles_x;     /* separable: column bands (64 columns) of the backward tiles */
 } igs_gs2d_plan_t;
@@ -114,7 +116,12 @@ int igs_gs2d_grid_classify(const float *x, const float *y, const int64_t grid_st
  * index range is cut into the splits (the reference evaluates every pair:
  * src/igs/gs_triton_chunked.py:100-200).  Records with a
  * non-finite field or a cov_inv that is not positive definite are never skipped.  Setting
- * IGS_NO_CULL=1 in the environment (read at each pack call) makes every box unbounded. */
+ * IGS_NO_CULL=1 in the environment (read at each pack call) makes every box unbounded.
+ * Large problems (tiles x N >= 2^25) build the per-tile lists in two levels (super-tiles of
+ * 4 x 4 tiles first); IGS_BIN_LEVELS=1|2 in the environment (read at each forward / backward /
+ * finalize call; keep it fixed between a backward and its finalize) forces one or two.  The
+ * lists and the forward do not depend on it; the finalize kernels add the tiles in another
+ * order under two levels, so gradients agree to fp32 rounding. */
 int igs_gs2d_pack_covinv(const float *position, const float *cov_inv_00, const float *cov_inv_01,
                          const float *cov_inv_11, const float *alphas, const float *colors,
                          int B, int N, int C, float *packed, igs_stream_t stream);

@@ -88,6 +88,116 @@ def test_long_rotated_gaussians_bit_for_bit(igs, dev, no_cull):
         assert torch.equal(grads[k], grads0[k]), k
 
 
+class _Env:
+    def __init__(self, name, value):
+        self.name, self.value = name, value
+
+    def __enter__(self):
+        os.environ[self.name] = self.value
+
+    def __exit__(self, *a):
+        os.environ.pop(self.name, None)
+
+
+def _kernel_channels(C):
+    from igs_amd import _lib
+
+    return next(c for c in _lib.COMPILED_CHANNELS if c >= C)
+
+
+@pytest.mark.parametrize("shape,scales", [((2, 700, 256, 512, 3), (0.004, 0.04)), ((1, 1500, 384, 640, 16), (0.005, 0.05)),
+                                          ((3, 333, 200, 530, 1), (0.004, 0.1)), ((1, 70000, 256, 512, 3), (0.002, 0.01)),
+                                          ((1, 9000, 520, 1000, 3), (0.002, 0.02))],
+                         ids=lambda v: "x".join(map(str, v)))
+def test_two_level_binning(igs, dev, shape, scales):
+    """IGS_BIN_LEVELS=2 lists the Gaussians per super-tile (4 x 4 tiles, several workgroups per
+    super-tile, each filling its own segment) first and lets every tile scan those segments only.
+    The tile lists are the same as with one level, hence the forward bit for bit; the finalize kernel
+    then adds the tiles super-tile by super-tile, so the gradients agree to rounding."""
+    from igs_amd import _lib
+
+    B, N, H, W, C = shape
+    plan = _lib.plan(B, N, H, W, _kernel_channels(C), 1)
+    assert plan.fwd_tiles >= 32 and plan.bwd_tiles >= 32          # both launches have super-tiles
+    _, g = sparse_case(dev, B, N, H, W, C, seed=sum(shape), smin=scales[0], smax=scales[1])
+    with _Env("IGS_BIN_LEVELS", "1"):
+        out1, grads1 = run(igs, g)
+    with _Env("IGS_BIN_LEVELS", "2"):
+        out2, grads2 = run(igs, g)
+        out3, grads3 = run(igs, g)
+    assert float(out1.abs().max()) > 0
+    assert torch.equal(out1, out2)
+    for k in NAMES:
+        assert float(grads1[k].abs().max()) > 0
+        d = (grads1[k] - grads2[k]).double()
+        assert float(d.norm()) <= 1e-5 * float(grads1[k].double().norm()), k   # another order of the tile sums
+        assert torch.equal(grads2[k], grads3[k]), k                # reproducible run to run
+
+
+def test_two_level_binning_against_oracle(igs, dev):
+    """Long thin Gaussians (aspect ratios up to 40) under two levels against the fp64 oracle."""
+    B, N, H, W, C = 1, 300, 256, 512, 3
+    d, g = sparse_case(dev, B, N, H, W, C, seed=41, smin=0.005, smax=0.2)
+    ref_out, ref_g = O.render_autograd(d["positions"], d["colors"], d["scales"], d["rotations"], d["alphas"],
+                                       d["x_grid"], d["y_grid"], d["grad_out"])
+    with _Env("IGS_BIN_LEVELS", "2"):
+        out, grads = run(igs, g)
+    err = (out.double() - ref_out.to(dev)).abs()
+    assert bool((err <= 1e-6 + 1e-5 * ref_out.to(dev).abs()).all()), float(err.max())
+    for k in NAMES:
+        r = ref_g[k].to(dev)
+        dlt = grads[k].double() - r
+        assert float(dlt.abs().max()) <= 1e-4 * float(r.abs().max()), k
+        assert float(dlt.norm()) <= 1e-4 * float(r.norm()), k
+
+
+def test_two_level_binning_culled_equals_unculled(igs, dev, no_cull):
+    """Under two levels, too, culling drops exact zeros only (one forward split: N < 128)."""
+    B, N, H, W, C = 2, 120, 256, 512, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=21, smin=0.002, smax=0.2)
+    with _Env("IGS_BIN_LEVELS", "2"):
+        out, grads = run(igs, g)
+        with no_cull:
+            out0, grads0 = run(igs, g)
+    assert torch.equal(out, out0)
+    for k in NAMES:
+        assert torch.equal(grads[k], grads0[k]), k
+
+
+def test_two_level_binning_module_and_nan_tiles(igs, dev):
+    """The module path (feature parameterisation) and a grid with a NaN coordinate (its tiles list
+    everything at both levels) under both settings."""
+    torch.manual_seed(5)
+    m = igs.GaussianSplatting2D(8, 64).to(dev)
+    x = torch.randn(2, 100, 64, device=dev)
+    go = torch.randn(2, 3, 256, 512, device=dev)
+    res = []
+    for lv in ("1", "2"):
+        with _Env("IGS_BIN_LEVELS", lv):
+            xx = x.clone().requires_grad_(True)
+            img, _ = m(xx, size=(256, 512))
+            img.backward(go)
+            res.append((img.detach(), xx.grad.clone(), m.proj.weight.grad.clone()))
+            m.zero_grad()
+    assert torch.equal(res[0][0], res[1][0])
+    for a, b in zip(res[0][1:], res[1][1:]):
+        assert float((a - b).norm()) <= 1e-5 * float(a.norm())
+    _, g = sparse_case(dev, 1, 300, 256, 512, 3, seed=3)
+    xs = g["x_grid"][0, 0, 0, :].clone()
+    xs[100] = float("nan")
+    xg = xs.view(1, 1, 1, -1).expand(1, 1, 256, 512)
+    outs = []
+    for lv in ("1", "2"):
+        with _Env("IGS_BIN_LEVELS", lv):
+            outs.append(run(igs, g, xg, None))
+    assert torch.equal(torch.nan_to_num(outs[0][0], nan=7.0), torch.nan_to_num(outs[1][0], nan=7.0))
+    for k in NAMES:   # NaN in the same places, the rest to rounding
+        a, b = outs[0][1][k], outs[1][1][k]
+        assert torch.equal(torch.isnan(a), torch.isnan(b)), k
+        a, b = torch.nan_to_num(a, nan=0.0), torch.nan_to_num(b, nan=0.0)
+        assert float((a - b).norm()) <= 1e-5 * float(a.norm()) + 1e-30, k
+
+
 def test_culled_equals_unculled_with_several_forward_splits(igs, dev, no_cull):
     """With S > 1 forward splits a tile's list (not the index range) is cut into S parts, so the
     same terms are grouped into other partial sums: equal to fp32 rounding, not bit for bit."""
