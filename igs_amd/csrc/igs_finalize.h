@@ -15,7 +15,8 @@
 #endif
 constexpr int kFinWide = 8, kFinDeep = IGS_FIN_DEEP;
 constexpr int kFinAhead = 4;    // tiles whose loads are issued together by a t-lane
-constexpr int kFinColours = 8;  // colour channels summed per pass (>= 6: the LDS array also serves the moments)
+constexpr int kFinColours = 8;  // colour channels summed per further pass
+constexpr int kFinFirst = 9;    // fields of the first pass: the six moments and up to three colours (C <= 3: one pass)
 
 // `part` is the image's partial array [T][NF][N]; the Gaussian's column in tile t is
 // slots[t * Np + n] when a slot table is given (negative: the tile holds nothing for it), else n.
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
     float* __restrict__ g_col) {
     constexpr int FN = 256 / FT;
-    __shared__ float red[kFinColours * FT * (FN + 1)];
+    __shared__ float red[kFinFirst * FT * (FN + 1)];
     const int n = blockIdx.x * FN + threadIdx.x % FN;
     const int b = blockIdx.y;
     const bool valid = n < N;
@@ -156,11 +157,14 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     SuperSlots sup = sup_in;  // the super-tile tables belong to the separable variant as well
     sup.cslots = (slots != nullptr && sup_in.cslots != nullptr) ? sup_in.cslots + (size_t)b * sup_in.stiles * Np : nullptr;
     const int nn = min(n, N - 1);
-    float M[6];
+    // first pass: the moments and, when wanted, the first colours (they follow the moments)
+    constexpr int kC0 = kFinFirst - 6;
+    float M[kFinFirst];
+    const int nfirst = g_col ? min(kFinFirst, NF) : 6;
     if (sup.cslots != nullptr)  // kernel-argument and flag uniform: the barriers inside are safe
-        tile_sum_super<6, FT>(part, slots, sup, Np, nn, NF, N, 0, valid, M, red);
+        tile_sum_super<kFinFirst, FT>(part, slots, sup, Np, nn, NF, N, 0, valid, M, red, nfirst);
     else
-        tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+        tile_sum<kFinFirst, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red, nfirst);
     const double al = alphas[i];
     // O(BN) epilogue in fp64: the chain rule multiplies sums by 1/s^3-sized factors
     double A, Bc, D, cs = 0., sn = 0., i0 = 0., i1 = 0., s0 = 0., s1 = 0.;
@@ -198,7 +202,11 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
         if (g2 && writer) g2[i] = (float)gD;
     }
     if (g_col) {  // kernel-argument uniform, so the barriers inside tile_sum are safe
-        for (int c0 = 0; c0 < C; c0 += kFinColours) {  // colour sums, kFinColours channels per pass
+        if (writer)
+#pragma unroll
+            for (int c = 0; c < kC0; ++c)
+                if (c < C) g_col[i * C + c] = (float)al * M[6 + c];
+        for (int c0 = kC0; c0 < C; c0 += kFinColours) {  // further colour sums, kFinColours channels per pass
             float sc[kFinColours];
             const int nc = min(kFinColours, C - c0);
             if (sup.cslots != nullptr)
@@ -222,7 +230,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     int C, int Cp,
     float eps, float* __restrict__ g_feat) {
     constexpr int FN = 256 / FT;
-    __shared__ float red[kFinColours * FT * (FN + 1)];
+    __shared__ float red[kFinFirst * FT * (FN + 1)];
     const int n = blockIdx.x * FN + threadIdx.x % FN;
     const int b = blockIdx.y;
     const bool valid = n < N;
@@ -236,11 +244,12 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     SuperSlots sup = sup_in;  // the super-tile tables belong to the separable variant as well
     sup.cslots = (slots != nullptr && sup_in.cslots != nullptr) ? sup_in.cslots + (size_t)b * sup_in.stiles * Np : nullptr;
     const int nn = min(n, N - 1);
-    float M[6];
+    constexpr int kC0 = kFinFirst - 6;
+    float M[kFinFirst];
     if (sup.cslots != nullptr)  // kernel-argument and flag uniform: the barriers inside are safe
-        tile_sum_super<6, FT>(part, slots, sup, Np, nn, NF, N, 0, valid, M, red);
+        tile_sum_super<kFinFirst, FT>(part, slots, sup, Np, nn, NF, N, 0, valid, M, red, min(kFinFirst, NF));
     else
-        tile_sum<6, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red);
+        tile_sum<kFinFirst, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red, min(kFinFirst, NF));
     const float* f = feat + i * (6 + C);
     const double e0 = (double)expf(f[2]), e1 = (double)expf(f[3]);
     const double s0 = e0 + (double)eps, s1 = e1 + (double)eps;
@@ -261,8 +270,11 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
         g[3] = (float)(gi1 * (-2.0 * s1 * i1 * i1) * e1);
         g[4] = (float)((gD - gA) * 2.0 * Bc + gB * (cs * cs - sn * sn) * (i0 - i1));
         g[5] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < kC0; ++c)
+            if (c < C) g[6 + c] = M[6 + c];
     }
-    for (int c0 = 0; c0 < C; c0 += kFinColours) {
+    for (int c0 = kC0; c0 < C; c0 += kFinColours) {
         float sc[kFinColours];
         const int nc = min(kFinColours, C - c0);
         if (sup.cslots != nullptr)
