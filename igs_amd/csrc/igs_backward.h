@@ -130,7 +130,7 @@ struct BwdArgs {
     int tiles_x;   // separable: column bands of kBwdTileW columns
     const int* counts;  // separable: Gaussians listed per tile [B][T]
     const int* lists;   // separable: list + complement [B][T][Np]
-    float* partial;  // [B][T][6+C][N]
+    float* partial;  // [B][T][N][6+C]
     const int* flag;
     int want;
 };
@@ -147,10 +147,11 @@ __device__ __forceinline__ void bwd_store(const BwdArgs& a, int b, int t, const 
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         if (n[g] < a.N) {
+            float* rec = base + (size_t)n[g] * NF;  // one record of NF floats per column
 #pragma unroll
-            for (int f = 0; f < 6; ++f) base[(size_t)f * a.N + n[g]] = M[g][f];
+            for (int f = 0; f < 6; ++f) rec[f] = M[g][f];
 #pragma unroll
-            for (int c = 0; c < C; ++c) base[(size_t)(6 + c) * a.N + n[g]] = CG[g][c];
+            for (int c = 0; c < C; ++c) rec[6 + c] = CG[g][c];
         }
     }
 }

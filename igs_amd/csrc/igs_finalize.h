@@ -18,7 +18,7 @@ constexpr int kFinAhead = 4;    // tiles whose loads are issued together by a t-
 constexpr int kFinColours = 8;  // colour channels summed per further pass
 constexpr int kFinFirst = 9;    // fields of the first pass: the six moments and up to three colours (C <= 3: one pass)
 
-// `part` is the image's partial array [T][NF][N]; the Gaussian's column in tile t is
+// `part` is the image's partial array [T][N][NF]; the Gaussian's column in tile t is
 // slots[t * Np + n] when a slot table is given (negative: the tile holds nothing for it), else n.
 // Only the first `nv` (<= NV) of the fields are read.
 template <int NV, int FT>
@@ -45,9 +45,9 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const i
 #pragma unroll
             for (int u = 0; u < kFinAhead; ++u) {
                 const int t = min(t0 + u * FT, T - 1);
-                const float* src = part + ((size_t)t * NF + f0) * N + max(col[u], 0);
+                const float* src = part + ((size_t)t * N + max(col[u], 0)) * NF + f0;
 #pragma unroll
-                for (int v = 0; v < NV; ++v) val[u][v] = v < nv ? src[(size_t)v * N] : 0.0f;
+                for (int v = 0; v < NV; ++v) val[u][v] = v < nv ? src[v] : 0.0f;
             }
 #pragma unroll
             for (int u = 0; u < kFinAhead; ++u)
@@ -103,9 +103,9 @@ __device__ __forceinline__ void tile_sum_super(const float* __restrict__ part, c
 #pragma unroll
                 for (int u = 0; u < kSuperX; ++u) {
                     const int t = ty * sup.tiles_x + min(sx * kSuperX + u, sup.tiles_x - 1);
-                    const float* src = part + ((size_t)t * NF + f0) * N + max(col[u], 0);
+                    const float* src = part + ((size_t)t * N + max(col[u], 0)) * NF + f0;
 #pragma unroll
-                    for (int v = 0; v < NV; ++v) val[u][v] = v < nv ? src[(size_t)v * N] : 0.0f;
+                    for (int v = 0; v < NV; ++v) val[u][v] = v < nv ? src[v] : 0.0f;
                 }
 #pragma unroll
                 for (int u = 0; u < kSuperX; ++u)

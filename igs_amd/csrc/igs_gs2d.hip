@@ -13,7 +13,7 @@
 //   * backward : a lane owns Gaussians, the pixel record (g^ = g/(den+eps), -s = -<g^,out>)
 //                is wave-uniform; the lane accumulates the six moments of G e and the C
 //                colour sums over its pixel tile in VGPRs.  Per-tile partials go to a
-//                [B,T,6+C,N] buffer which a finalize kernel sums in a fixed order (no
+//                [B,T,N,6+C] buffer which a finalize kernel sums in a fixed order (no
 //                float atomics anywhere, bit-reproducible).
 //   * the wave-uniform record stream goes global -> LDS (cooperative, double-buffered) ->
 //     VGPRs (broadcast ds_read_b128), because on gfx950 a VALU op with VGPR-only operands
