@@ -152,7 +152,7 @@ int igs_gs2d_backward_prologue(const float *x, const float *y, const int64_t gri
                                igs_stream_t stream);
 
 /* Backward, stage 2: the recomputing per-Gaussian reduction over pixel tiles into
- * partial [B,T,6+C,N] (plan.partial_bytes).  Replaces the Gaussian loop of the reference
+ * partial [B,T,N,6+C] (plan.partial_bytes).  Replaces the Gaussian loop of the reference
  * backward, src/igs/gs2d.py:180-246 / src/igs/gs_triton.py:159-405.  colors [B,N,C].
  * pix_ws is the buffer stage 1 filled (16-byte aligned); on separable grids this stage also
  * writes its per-tile Gaussian lists behind the pixel records in it. */
