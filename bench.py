@@ -16,7 +16,6 @@ usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-c
 from __future__ import annotations
 
 import argparse
-import ctypes
 import json
 import os
 import sys

@@ -10,7 +10,6 @@ must live on the GPU.
 """
 from __future__ import annotations
 
-import ctypes
 from typing import List
 
 import torch
