@@ -107,7 +107,7 @@ def _kernel_channels(C):
 
 @pytest.mark.parametrize("shape,scales", [((2, 700, 256, 512, 3), (0.004, 0.04)), ((1, 1500, 384, 640, 16), (0.005, 0.05)),
                                           ((3, 333, 200, 530, 1), (0.004, 0.1)), ((1, 70000, 256, 512, 3), (0.002, 0.01)),
-                                          ((1, 9000, 520, 1000, 3), (0.002, 0.02))],
+                                          ((1, 9000, 520, 1000, 3), (0.002, 0.02)), ((2, 20000, 256, 512, 3), (0.002, 0.01))],
                          ids=lambda v: "x".join(map(str, v)))
 def test_two_level_binning(igs, dev, shape, scales):
     """IGS_BIN_LEVELS=2 lists the Gaussians per super-tile (4 x 4 tiles, several workgroups per
@@ -132,6 +132,20 @@ def test_two_level_binning(igs, dev, shape, scales):
         d = (grads1[k] - grads2[k]).double()
         assert float(d.norm()) <= 1e-5 * float(grads1[k].double().norm()), k   # another order of the tile sums
         assert torch.equal(grads2[k], grads3[k]), k                # reproducible run to run
+
+
+def test_two_level_binning_on_materialised_grids(igs, dev):
+    """Grids stored in full are classified on the device and both kernel variants are enqueued
+    behind the flag; the two binning passes are gated like the kernels they serve."""
+    B, N, H, W, C = 2, 9000, 256, 512, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=12, smin=0.003, smax=0.03)
+    xg, yg = g["x_grid"].contiguous(), g["y_grid"].contiguous()
+    with _Env("IGS_BIN_LEVELS", "2"):
+        out_e, grads_e = run(igs, g)
+        out_m, grads_m = run(igs, g, xg, yg)
+    assert torch.equal(out_e, out_m)
+    for k in NAMES:
+        assert torch.equal(grads_e[k], grads_m[k]), k
 
 
 def test_two_level_binning_against_oracle(igs, dev):
