@@ -189,3 +189,30 @@ def test_fit_converges_config2_reduced(igs, dev):
     losses = [float(fit.step()) for _ in range(100)]
     assert losses[10] < losses[0] and losses[99] < 0.5 * losses[10]
     assert bool(torch.isfinite(fit.params).all())
+
+
+def test_fused_step_under_two_level_binning(igs, dev):
+    """IGS_BIN_LEVELS=2 (the tile lists built through super-tiles) changes the order in which the
+    finalize kernel adds the tiles and nothing else: the first loss is bit-identical, the
+    parameters after a few steps agree to rounding."""
+    import os
+
+    B, N, H, W, C = 1, 3000, 256, 512, 3
+    block0 = make_block(B, N, C, 5, dev)
+    block0[..., 2:4] -= 2.0                                   # small Gaussians: sigma of 1-4 pixels
+    xg, yg = grids(igs, B, H, W, dev)
+    target = torch.rand(B, C, H, W, generator=torch.Generator().manual_seed(6)).to(dev)
+    res = {}
+    for levels in ("1", "2"):
+        os.environ["IGS_BIN_LEVELS"] = levels
+        try:
+            fit = igs.GaussianImageFit(block0.clone(), target, xg, yg, lr=0.01)
+            losses = [float(fit.step()) for _ in range(4)]
+            res[levels] = (losses, fit.params.clone())
+        finally:
+            os.environ.pop("IGS_BIN_LEVELS", None)
+    assert res["1"][0][0] == res["2"][0][0]
+    assert res["1"][0][-1] < res["1"][0][0]
+    torch.testing.assert_close(res["1"][1], res["2"][1], rtol=1e-4, atol=1e-5)
+    for a, b in zip(res["1"][0], res["2"][0]):
+        assert a == pytest.approx(b, rel=1e-5)
