@@ -210,9 +210,9 @@ constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads i
 // coordinate rectangle at all (the box of a long, rotated ellipse is mostly empty)?  With
 // P = -q' = a dx^2 + b2 dx dy + d dy^2 (a, b2, d = -A', -B2', -D' of the record), the minimum of
 // P over the rectangle is 0 when it holds the centre and else lies on an edge, where P is a
-// parabola in one variable.  The kernels' weight is exactly 0 where their fp32 q' is below -150; both their q' and the P
-// evaluated here differ from the exact value by a few ulp of the largest term, bounded over the
-// rectangle by T below.  The tile is dropped only if min P - 4e-6 T > 155: the same margin
+// parabola in one variable.  The kernels' weight is exactly 0 where their fp32 q' is below -150;
+// both their q' and the P evaluated here differ from the exact value by a few ulp of the largest
+// term, bounded over the rectangle by T below.  The tile is dropped only if min P - 4e-6 T > 155: the same margin
 // against rounding as the reach box has, so dropping it changes no bit either.  A
 // non-positive-definite or NaN record fails the comparison and stays listed.
 __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, float txlo, float txhi,
