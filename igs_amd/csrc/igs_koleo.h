@@ -130,10 +130,26 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
     }
     const int kchunks = (Dp + KC - 1) / KC;
     const int nsteps = (ct1 - ct0) * kchunks;
+    // kRegA: a step is a column tile, so a loader slot walks down the rows with a fixed stride
+    const float* nptr[LPT];
+    int nrow[LPT];
+#pragma unroll
+    for (int j = 0; j < LPT; ++j) {
+        int which, lr, lk;
+        slot(j, which, lr, lk);
+        nrow[j] = which == 1 ? ct0 * TC + lr : N;  // N: never loads
+        nptr[j] = img + (size_t)min(nrow[j], N - 1) * Dp + lk;
+    }
+    auto next_tile = [&](int j) {  // kRegA only: this slot's float4 of the next column tile
+        const float4 v = nrow[j] < N ? *reinterpret_cast<const float4*>(nptr[j]) : zero;
+        nrow[j] += TC;
+        nptr[j] += (size_t)TC * Dp;
+        return v;
+    };
     float4 pre[LPT];
     if (nsteps > 0) {
 #pragma unroll
-        for (int j = 0; j < LPT; ++j) pre[j] = gload(j, ct0 * TC, 0);
+        for (int j = 0; j < LPT; ++j) pre[j] = kRegA ? next_tile(j) : gload(j, ct0 * TC, 0);
 #pragma unroll
         for (int j = 0; j < LPT; ++j) lstore(j, 0, pre[j]);
     }
@@ -151,15 +167,15 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
         const bool more = step + 1 < nsteps;
         if (more) {
 #pragma unroll
-            for (int j = 0; j < LPT; ++j) pre[j] = gload(j, nct * TC, nkc * KC);
+            for (int j = 0; j < LPT; ++j) pre[j] = kRegA ? next_tile(j) : gload(j, nct * TC, nkc * KC);
         }
-        if (kc == 0) {
+        if (!kRegA && kc == 0) {
 #pragma unroll
             for (int r = 0; r < MR; ++r)
 #pragma unroll
                 for (int q = 0; q < MC; ++q) acc[r][q] = 0.0f;
         }
-        if (kRegA) {  // fully unrolled: areg stays in registers
+        if (kRegA) {  // fully unrolled: areg stays in registers; the first product starts the sums
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
                 float cv[MC];
@@ -168,7 +184,8 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
 #pragma unroll
                 for (int r = 0; r < MR; ++r)
 #pragma unroll
-                    for (int q = 0; q < MC; ++q) acc[r][q] = fmaf(areg[kRegA ? k : 0][r], cv[q], acc[r][q]);
+                    for (int q = 0; q < MC; ++q)
+                        acc[r][q] = k == 0 ? areg[0][r] * cv[q] : fmaf(areg[kRegA ? k : 0][r], cv[q], acc[r][q]);
             }
         } else {
             const int kn = min(KC, Dp - k0);
