@@ -192,6 +192,28 @@ class Splat:
                                               int(p.partial_bytes), self.stream), "igs_gs2d_backward")
         return partial
 
+    def backward_partials_with_grid(self, packed, colors_p, out, den, grad_out_p, x_like, y_like):
+        """The per-Gaussian partial sums and d L / d x_grid, d L / d y_grid from one call (on general
+        grids the grid sums are formed inside the per-Gaussian reduction)."""
+        g, p = self.grid, self.plan
+        pix = self._empty(p.pix_bytes)
+        partial = self._empty(p.partial_bytes)
+        gws_bytes = int(self.lib.igs_gs2d_grid_workspace_bytes(self.B, self.N, g.H, g.W, self.Cp))
+        gws = self._empty(gws_bytes)
+        gx = self._new(self.B, g.H, g.W)
+        gy = torch.empty_like(gx)
+        _lib.check(self.lib.igs_gs2d_backward_with_grid(
+            _ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), _ptr(out), _ptr(den),
+            _ptr(grad_out_p), self.B, self.N, g.H, g.W, self.Cp, self.eps, _ptr(pix), int(p.pix_bytes), _ptr(partial),
+            int(p.partial_bytes), _ptr(gws), gws_bytes, _ptr(gx), _ptr(gy), self.stream), "igs_gs2d_backward_with_grid")
+        return partial, self._fit_grid(gx, x_like), self._fit_grid(gy, y_like)
+
+    def _fit_grid(self, gr, like):
+        shape, dtype = like
+        if shape[0] == 1 and self.B > 1:      # batch-1 grid shared by all images
+            gr = gr.sum(0, keepdim=True)
+        return gr.reshape(shape).to(dtype)
+
     def grid_grads(self, packed, out, den, grad_out_p, x_like, y_like):
         """d L / d x_grid, d L / d y_grid in the (shape, dtype) of the tensors the caller passed."""
         g = self.grid
@@ -202,13 +224,7 @@ class Splat:
                                                    self.eps, _ptr(gx), _ptr(gy), self.stream),
                    "igs_gs2d_backward_grid")
 
-        def fit(gr, like):
-            shape, dtype = like
-            if shape[0] == 1 and self.B > 1:      # batch-1 grid shared by all images
-                gr = gr.sum(0, keepdim=True)
-            return gr.reshape(shape).to(dtype)
-
-        return fit(gx, x_like), fit(gy, y_like)
+        return self._fit_grid(gx, x_like), self._fit_grid(gy, y_like)
 
     def pad_grad_out(self, grad_out: Tensor) -> Tensor:
         """fp32 contiguous [B,Cp,H,W] upstream gradient (zero in the padding channels)."""
@@ -314,12 +330,16 @@ def run_backward(kind: int, op: Splat, keep, packed, col, out, den, grad_result:
     with torch.cuda.device(dev):
         op.use_current_stream()
         go = op.pad_grad_out(grad_result)
-        if need_x or need_y:
-            g_x, g_y = op.grid_grads(packed, out, den, go, *grid_like)
+        if (need_x or need_y) and any(need):
+            partial, g_x, g_y = op.backward_partials_with_grid(packed, col, out, den, go, *grid_like)
             g_x, g_y = (g_x if need_x else None), (g_y if need_y else None)
-        if not any(need):
-            return grads, g_x, g_y
-        partial = op.backward_partials(packed, col, out, den, go)
+        else:
+            if need_x or need_y:
+                g_x, g_y = op.grid_grads(packed, out, den, go, *grid_like)
+                g_x, g_y = (g_x if need_x else None), (g_y if need_y else None)
+            if not any(need):
+                return grads, g_x, g_y
+            partial = op.backward_partials(packed, col, out, den, go)
         mode, flag, H, W = op.grid.mode, _ptr(op.grid.flag), op.grid.H, op.grid.W
         if kind == KIND_COVINV:
             a, b, d, al = keep

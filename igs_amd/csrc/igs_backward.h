@@ -131,6 +131,7 @@ struct BwdArgs {
     const int* counts;  // separable: Gaussians listed per tile [B][T]
     const int* lists;   // separable: list + complement [B][T][Np]
     float* partial;  // [B][T][N][6+C]
+    float2* grid_part;  // general grids with grid gradients: [B][groups][HWp] sums of G w (t1, t2)
     const int* flag;
     int want;
 };
@@ -381,11 +382,12 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
 
 // General grid: the tile is a flat pixel range (multiple of 256); x and y come with the
 // pixel record.  Sums are flushed into the totals once per 128-pixel chunk.
-template <int C, int G>
+template <int C, int G, bool kGrid>
 __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     constexpr int CP = pix_stride_gen(C), CP4 = CP / 4;
     constexpr int kPixChunk = pix_chunk(C);
     __shared__ float4 sh[2 * kPixChunk * CP4];
+    __shared__ float2 gacc[kGrid ? kThreads / 64 : 1][kGrid ? kPixChunk : 1];  // per wave and record of the chunk
     IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
     int n[G];
@@ -393,6 +395,21 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     for (int g = 0; g < G; ++g) n[g] = (blockIdx.x * G + g) * kThreads + threadIdx.x;
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
     bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+    // Grid gradients (kGrid): d L / d x(pixel) = -sum_n G_n w_n (A dx + B dy), same with (B dx + D dy)
+    // for y.  With t1 = A'dx + (B2'/2) dy, t2 = (B2'/2) dx + D'dy the exponent is dx t1 + dy t2, and
+    // a lane adds alpha G e (t1, t2) of its G Gaussians per pixel record; the 64 lanes are summed
+    // by a butterfly, the four waves and the workgroups of the other Gaussians in a fixed order
+    // (LDS, then k_grid_reduce), which also applies the factor -1/k of t1 = k (A dx + B dy).
+    float hb[G], al[G];
+    if (kGrid) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            hb[g] = 0.5f * B2[g];
+            // unused lane slots (n >= N) must add nothing
+            al[g] = n[g] < a.N ? a.packed[((size_t)b * a.Np + n[g]) * rec_stride_of(C) + 5] : 0.0f;
+        }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     float M[G][6], CG[G][C], R[G][6], RC[G][C];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -414,21 +431,28 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
             pv[4 * q4 + 2] = tq.z;
             pv[4 * q4 + 3] = tq.w;
         }
-        float dxs[G], dys[G], ee[G];
+        float dxs[G], dys[G], ee[G], t1[G], t2[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             const float dx = pv[0] - px[g];
             const float dy = pv[1] - py[g];
-            float tt = A[g] * dx;
-            tt = fmaf(B2[g], dy, tt);
-            const float v = D[g] * dy;
-            float q = tt * dx;
-            ee[g] = fmaf(v, dy, q);
+            if (kGrid) {
+                t1[g] = fmaf(A[g], dx, hb[g] * dy);
+                t2[g] = fmaf(D[g], dy, hb[g] * dx);
+                ee[g] = fmaf(dx, t1[g], dy * t2[g]);
+            } else {
+                float tt = A[g] * dx;
+                tt = fmaf(B2[g], dy, tt);
+                const float v = D[g] * dy;
+                float q = tt * dx;
+                ee[g] = fmaf(v, dy, q);
+            }
             dxs[g] = dx;
             dys[g] = dy;
         }
 #pragma unroll
         for (int g = 0; g < G; ++g) ee[g] = hw_exp2(ee[g]);
+        float gxl = 0.0f, gyl = 0.0f;
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             const float e = ee[g], dx = dxs[g], dy = dys[g];
@@ -437,14 +461,27 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
             for (int c = 0; c < C; ++c) Gv = fmaf(pv[2 + c], col[g][c], Gv);
             const float ge = Gv * e;
             R[g][0] += ge;
-            const float t1 = ge * dx, t2 = ge * dy;
-            R[g][1] += t1;
-            R[g][2] += t2;
-            R[g][3] = fmaf(t1, dx, R[g][3]);
-            R[g][4] = fmaf(t1, dy, R[g][4]);
-            R[g][5] = fmaf(t2, dy, R[g][5]);
+            const float m1 = ge * dx, m2 = ge * dy;
+            R[g][1] += m1;
+            R[g][2] += m2;
+            R[g][3] = fmaf(m1, dx, R[g][3]);
+            R[g][4] = fmaf(m1, dy, R[g][4]);
+            R[g][5] = fmaf(m2, dy, R[g][5]);
 #pragma unroll
             for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[2 + c], RC[g][c]);
+            if (kGrid) {
+                const float gw = ge * al[g];
+                gxl = fmaf(gw, t1[g], gxl);
+                gyl = fmaf(gw, t2[g], gyl);
+            }
+        }
+        if (kGrid) {
+#pragma unroll
+            for (int k = 32; k > 0; k >>= 1) {
+                gxl += __shfl_xor(gxl, k);
+                gyl += __shfl_xor(gyl, k);
+            }
+            if (lane == 0) gacc[kGrid ? wave : 0][kGrid ? (seen & (kPixChunk - 1)) : 0] = make_float2(gxl, gyl);
         }
         if ((++seen & (kPixChunk - 1)) == 0) {  // two-level summation
 #pragma unroll
@@ -459,6 +496,20 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
                     CG[g][c] += RC[g][c];
                     RC[g][c] = 0.0f;
                 }
+            }
+            if (kGrid) {  // the chunk's records are complete in all four waves: add them in wave order
+                __syncthreads();
+                const int p = p0 + seen - kPixChunk + (int)threadIdx.x;
+                if ((int)threadIdx.x < kPixChunk && p < p1) {
+                    float2 sum = gacc[0][kGrid ? threadIdx.x : 0];
+#pragma unroll
+                    for (int w = 1; w < kThreads / 64; ++w) {
+                        sum.x += gacc[kGrid ? w : 0][kGrid ? threadIdx.x : 0].x;
+                        sum.y += gacc[kGrid ? w : 0][kGrid ? threadIdx.x : 0].y;
+                    }
+                    a.grid_part[((size_t)b * gridDim.x + blockIdx.x) * a.HWp + p] = sum;
+                }
+                __syncthreads();
             }
         }
     });

@@ -20,12 +20,15 @@ struct GridGradArgs {
     float eps;
     float* gx;  // [B][H*W]
     float* gy;
+    const int* flag;  // AUTO grid mode: run only if *flag == want
+    int want;
 };
 
 template <int C, int P>
 __global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
     constexpr int RS = rec_stride_of(C), R4 = RS / 4;
     __shared__ float4 sh[2 * kGaussChunk * R4];
+    IGS_GATE(a);
     const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
     if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int b = tile / a.tiles_per_img;
@@ -83,6 +86,26 @@ __global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
             a.gx[(size_t)b * HW + pix[j]] = kScale * sx[j];
             a.gy[(size_t)b * HW + pix[j]] = kScale * sy[j];
         }
+}
+
+// Grid gradients of the general backward with the grid sums fused in (k_bwd_gen<.., true>): adds
+// the `groups` workgroup partials of every pixel in order and applies the factor -1/k.
+__global__ __launch_bounds__(kThreads) void k_grid_reduce(const float2* __restrict__ part, int groups, int HW,
+                                                          int HWp, float* __restrict__ gx, float* __restrict__ gy,
+                                                          const int* __restrict__ flag, int want) {
+    if (flag != nullptr && *flag != want) return;
+    const int p = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (p >= HW) return;
+    float sx = 0.0f, sy = 0.0f;
+    for (int g = 0; g < groups; ++g) {
+        const float2 v = part[((size_t)b * groups + g) * HWp + p];
+        sx += v.x;
+        sy += v.y;
+    }
+    constexpr float kScale = -1.0f / kNegHalfLog2e;
+    gx[(size_t)b * HW + p] = kScale * sx;
+    gy[(size_t)b * HW + p] = kScale * sy;
 }
 
 // ----------------------------------------------------------------------------- grid class

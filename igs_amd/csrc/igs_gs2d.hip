@@ -391,6 +391,10 @@ int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, con
     return launch_status();
 }
 
+// Workgroups of the general backward along the Gaussians (= partial sums per pixel of its fused
+// grid gradients).
+inline int bwd_gen_groups(int N, int C) { return ceil_div(N, kThreads * bwd_gen_g(C)); }
+
 template <int C>
 int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     if (sep) {
@@ -398,8 +402,11 @@ int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
         const dim3 grid(a.T, ceil_div(a.Np, kThreads * kBwdG), B);
         hipLaunchKernelGGL((k_bwd_sep<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
     } else {
-        const dim3 grid(ceil_div(a.N, kThreads * bwd_gen_g(C)), a.T, B);
-        hipLaunchKernelGGL((k_bwd_gen<C, bwd_gen_g(C)>), grid, dim3(kThreads), 0, st, a);
+        const dim3 grid(bwd_gen_groups(a.N, C), a.T, B);
+        if (a.grid_part != nullptr)
+            hipLaunchKernelGGL((k_bwd_gen<C, bwd_gen_g(C), true>), grid, dim3(kThreads), 0, st, a);
+        else
+            hipLaunchKernelGGL((k_bwd_gen<C, bwd_gen_g(C), false>), grid, dim3(kThreads), 0, st, a);
     }
     return launch_status();
 }
@@ -425,6 +432,7 @@ int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* col
         a.counts = bp.counts; a.lists = bp.lists;
     }
     a.partial = partial;
+    a.grid_part = nullptr;
     a.flag = v.flag; a.want = v.want;
     return IGS_OK;
 }
@@ -657,10 +665,47 @@ int igs_adamw_step(float* param, const float* grad, float* exp_avg, float* exp_a
     return launch_status();
 }
 
-int igs_gs2d_backward_reduce(const float* packed, const float* colors, const float* y,
-                             const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
-                             int B, int N, int H, int W, int C, float* pix_ws, size_t pix_bytes,
-                             float* partial, size_t partial_bytes, igs_stream_t stream) {
+}  // extern "C"
+
+namespace {
+// What the grid gradients need beside the reduction's own arguments (all null: none wanted).
+struct GridGradOut {
+    const float* x = nullptr;
+    const float* out = nullptr;
+    const float* den = nullptr;
+    const float* grad_out = nullptr;
+    float eps = 0.0f;
+    void* ws = nullptr;  // general variant: [B][groups][HWp] float2 partial sums
+    float* g_x = nullptr;
+    float* g_y = nullptr;
+};
+
+int launch_grid_standalone(const float* packed, const float* x, const float* y, const int64_t gs[6],
+                           const float* out, const float* den, const float* grad_out, int B, int N, int H, int W,
+                           int C, float eps, float* g_x, float* g_y, const int* flag, int want, hipStream_t st) {
+    GridGradArgs a;
+    a.packed = packed; a.x = x; a.y = y;
+    a.sxb = gs[0]; a.sxh = gs[1]; a.sxw = gs[2];
+    a.syb = gs[3]; a.syh = gs[4]; a.syw = gs[5];
+    a.out = out; a.den = den; a.gout = grad_out;
+    a.Np = (N + 3) & ~3; a.H = H; a.W = W;
+    a.eps = eps; a.gx = g_x; a.gy = g_y;
+    a.flag = flag; a.want = want;
+    int rc = IGS_OK;
+    IGS_DISPATCH_C(C, {
+        constexpr int P = kC > 8 ? 2 : 4;
+        a.tiles_per_img = ceil_div((long)H * W, kThreads * P);
+        a.total_tiles = B * a.tiles_per_img;
+        hipLaunchKernelGGL((k_bwd_grid<kC, P>), dim3(((a.total_tiles + 7) / 8) * 8), dim3(kThreads), 0, st, a);
+        rc = launch_status();
+    });
+    return rc;
+}
+
+int backward_reduce(const float* packed, const float* colors, const float* y,
+                    const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                    int B, int N, int H, int W, int C, float* pix_ws, size_t pix_bytes,
+                    float* partial, size_t partial_bytes, const GridGradOut& gg, igs_stream_t stream) {
     if (!packed || !colors || !y || !grid_strides || !pix_ws || !partial) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
@@ -701,10 +746,58 @@ int igs_gs2d_backward_reduce(const float* packed, const float* colors, const flo
             rc = launch_bins(ba, B, levels2, cp, cslots, st);
             if (rc) return rc;
         }
+        if (gg.g_x != nullptr && !sep) a.grid_part = reinterpret_cast<float2*>(gg.ws);
         IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, st));
+        if (rc) return rc;
+        if (gg.g_x == nullptr) continue;
+        if (sep) {  // the pixel-major kernel of its own
+            rc = launch_grid_standalone(packed, gg.x, y, grid_strides, gg.out, gg.den, gg.grad_out, B, N, H, W, C,
+                                        gg.eps, gg.g_x, gg.g_y, a.flag, a.want, st);
+        } else {
+            hipLaunchKernelGGL(k_grid_reduce, dim3(ceil_div((long)H * W, kThreads), B), dim3(kThreads), 0, st,
+                               (const float2*)gg.ws, bwd_gen_groups(N, C), H * W, a.HWp, gg.g_x, gg.g_y, a.flag,
+                               a.want);
+            rc = launch_status();
+        }
         if (rc) return rc;
     }
     return IGS_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int igs_gs2d_backward_reduce(const float* packed, const float* colors, const float* y,
+                             const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                             int B, int N, int H, int W, int C, float* pix_ws, size_t pix_bytes,
+                             float* partial, size_t partial_bytes, igs_stream_t stream) {
+    return backward_reduce(packed, colors, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, pix_ws,
+                           pix_bytes, partial, partial_bytes, GridGradOut{}, stream);
+}
+
+size_t igs_gs2d_grid_workspace_bytes(int B, int N, int H, int W, int C) {
+    if (!shape_ok(B, N, H, W) || !channels_compiled(C)) return 0;
+    const size_t hwp = ((size_t)H * W + 3) & ~(size_t)3;
+    return (size_t)B * bwd_gen_groups(N, C) * hwp * sizeof(float2);
+}
+
+int igs_gs2d_backward_with_grid(const float* packed, const float* colors, const float* x, const float* y,
+                                const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                                const float* out, const float* den, const float* grad_out, int B, int N,
+                                int H, int W, int C, float eps, float* pix_ws, size_t pix_bytes, float* partial,
+                                size_t partial_bytes, void* grid_ws, size_t grid_ws_bytes, float* g_x,
+                                float* g_y, igs_stream_t stream) {
+    if (!x || !out || !den || !grad_out || !grid_ws || !g_x || !g_y) return IGS_ERR_NULL_POINTER;
+    if (grid_ws_bytes < igs_gs2d_grid_workspace_bytes(B, N, H, W, C)) return IGS_ERR_WORKSPACE;
+    if ((uintptr_t)grid_ws & 7) return IGS_ERR_ALIGNMENT;
+    int rc = igs_gs2d_backward_prologue(x, y, grid_strides, grid_mode, grid_flag, out, den, grad_out, B, N,
+                                        H, W, C, eps, pix_ws, pix_bytes, stream);
+    if (rc) return rc;
+    GridGradOut gg;
+    gg.x = x; gg.out = out; gg.den = den; gg.grad_out = grad_out; gg.eps = eps;
+    gg.ws = grid_ws; gg.g_x = g_x; gg.g_y = g_y;
+    return backward_reduce(packed, colors, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, pix_ws,
+                           pix_bytes, partial, partial_bytes, gg, stream);
 }
 
 int igs_gs2d_backward(const float* packed, const float* colors, const float* x, const float* y,
@@ -727,23 +820,8 @@ int igs_gs2d_backward_grid(const float* packed, const float* x, const float* y,
         return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, H, W)) return IGS_ERR_BAD_SHAPE;
     if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
-    GridGradArgs a;
-    a.packed = packed; a.x = x; a.y = y;
-    a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
-    a.syb = grid_strides[3]; a.syh = grid_strides[4]; a.syw = grid_strides[5];
-    a.out = out; a.den = den; a.gout = grad_out;
-    a.Np = (N + 3) & ~3; a.H = H; a.W = W;
-    a.eps = eps; a.gx = g_x; a.gy = g_y;
-    int rc = IGS_OK;
-    hipStream_t st = (hipStream_t)stream;
-    IGS_DISPATCH_C(C, {
-        constexpr int P = kC > 8 ? 2 : 4;
-        a.tiles_per_img = ceil_div((long)H * W, kThreads * P);
-        a.total_tiles = B * a.tiles_per_img;
-        hipLaunchKernelGGL((k_bwd_grid<kC, P>), dim3(((a.total_tiles + 7) / 8) * 8), dim3(kThreads), 0, st, a);
-        rc = launch_status();
-    });
-    return rc;
+    return launch_grid_standalone(packed, x, y, grid_strides, out, den, grad_out, B, N, H, W, C, eps, g_x, g_y,
+                                  nullptr, 0, (hipStream_t)stream);
 }
 
 // Launches a finalize kernel in the layout that suits the problem size: 8 t-lanes x 32 Gaussians

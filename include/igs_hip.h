@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define IGS_ABI_VERSION 3
+#define IGS_ABI_VERSION 4
 #define IGS_MAX_CHANNELS 16
 
 typedef void *igs_stream_t; /* a hipStream_t */
@@ -168,6 +168,21 @@ int igs_gs2d_backward(const float *packed, const float *colors, const float *x, 
                       const float *out, const float *den, const float *grad_out, int B, int N,
                       int H, int W, int C, float eps, float *pix_ws, size_t pix_bytes,
                       float *partial, size_t partial_bytes, igs_stream_t stream);
+
+/* Stages 1 and 2 plus the gradients w.r.t. the pixel coordinates g_x, g_y [B,H,W] (grad_x /
+ * grad_y of the reference backward, src/igs/gs2d.py:222-231, :249-250, which always computes
+ * them) in one call.  On general grids the per-pixel sums are formed inside the per-Gaussian
+ * reduction (one exponential per pair instead of two) into grid_ws
+ * (igs_gs2d_grid_workspace_bytes, 8-byte aligned) and added in a fixed order; on separable
+ * grids this equals igs_gs2d_backward followed by igs_gs2d_backward_grid. */
+size_t igs_gs2d_grid_workspace_bytes(int B, int N, int H, int W, int C);
+int igs_gs2d_backward_with_grid(const float *packed, const float *colors, const float *x,
+                                const float *y, const int64_t grid_strides[6], int grid_mode,
+                                const int32_t *grid_flag, const float *out, const float *den,
+                                const float *grad_out, int B, int N, int H, int W, int C, float eps,
+                                float *pix_ws, size_t pix_bytes, float *partial,
+                                size_t partial_bytes, void *grid_ws, size_t grid_ws_bytes,
+                                float *g_x, float *g_y, igs_stream_t stream);
 
 /* Optional backward output: gradients w.r.t. the pixel coordinates, g_x, g_y [B,H,W]
  * (grad_x / grad_y of the reference backward, src/igs/gs2d.py:222-231, :249-250; the Triton

@@ -353,3 +353,46 @@ def test_random_small_shapes_against_oracle(igs, dev):
             # lone or far-apart Gaussians: gradients are differences of nearly equal numbers of
             # size eps-ish (see test_function_level_forward_backward); absolute bound there
             assert_grad(v.grad, ref_g[k], k, tag, atol=1e-6 if N <= 5 else 0.0)
+
+
+@pytest.mark.parametrize("C", [3, 16])
+def test_grid_gradients_fused_into_the_general_backward(igs, dev, C):
+    """When parameter and grid gradients are both wanted on a general grid, the per-pixel sums are
+    formed inside the per-Gaussian reduction (several workgroups along the Gaussians, several pixel
+    chunks, a ragged last chunk) and must agree with the pixel-major kernel that runs when only the
+    grid gradients are wanted, and with the fp64 oracle."""
+    B, N, H, W = 2, 2500, 37, 53
+    d = small_case(B, N, H, W, C, seed=70 + C, general=True)
+    f = lambda t: t.to(dev, torch.float32)
+    names = ("positions", "colors", "scales", "rotations", "alphas")
+
+    def run(params_need_grad):
+        lv = {k: f(d[k]).requires_grad_(params_need_grad) for k in names}
+        xg, yg = f(d["x_grid"]).requires_grad_(True), f(d["y_grid"]).requires_grad_(True)
+        out = igs.gaussian_splatting_2d(*(lv[k] for k in names), xg, yg)
+        out.backward(f(d["grad_out"]))
+        return xg.grad, yg.grad, lv
+
+    gx_f, gy_f, lv = run(True)          # fused
+    gx_s, gy_s, _ = run(False)          # the kernel of its own
+    for a, b in ((gx_f, gx_s), (gy_f, gy_s)):
+        assert float((a - b).norm()) <= 1e-5 * float(b.norm())
+        assert float((a - b).abs().max()) <= 1e-4 * float(b.abs().max())
+    a_, b_, c_ = (t.float().double() for t in O.cov_inverse_closed(d["scales"], d["rotations"]))
+    _, ref_g = O.operator_autograd(d["x_grid"], d["y_grid"], d["positions"], a_, b_, c_, d["alphas"], d["colors"],
+                                   d["grad_out"])
+    assert_grad(gx_f, ref_g["x"], "x", "fused grid grads")
+    assert_grad(gy_f, ref_g["y"], "y", "fused grid grads")
+    assert_grad(lv["positions"].grad, ref_g["position"], "position", "fused grid grads")
+    # the same request on grids stored in full that are separable: the device-side classification
+    # gates the separable kernels plus the pixel-major grid kernel
+    xe = f(d["x_grid"])[:1, :, :1, :].expand(B, 1, H, W)
+    ye = f(d["y_grid"])[:1, :, :, :1].expand(B, 1, H, W)
+    res = []
+    for xx, yy in ((xe, ye), (xe.contiguous(), ye.contiguous())):
+        lv = {k: f(d[k]).requires_grad_(True) for k in names}
+        xx, yy = xx.detach().requires_grad_(True), yy.detach().requires_grad_(True)
+        igs.gaussian_splatting_2d(*(lv[k] for k in names), xx, yy).backward(f(d["grad_out"]))
+        res.append((xx.grad, yy.grad, lv["scales"].grad))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
