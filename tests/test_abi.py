@@ -106,6 +106,13 @@ def test_argument_errors_are_status_codes_not_crashes(lib):
     assert lib.igs_gs2d_pack_covinv(None, None, None, None, None, None, 1, 8, 3, None, None) == -1
     assert lib.igs_gs2d_finalize_covinv(None, 1, None, None, None, None, None, 1, 8, 4, 4, 3,
                                         None, None, None, None, None, None, None) == -1
+    assert lib.igs_gs2d_backward_with_grid(None, None, None, None, st, 1, None, None, None, None, 1, 8, 4, 4, 3, 1e-6,
+                                           None, 0, None, 0, None, 0, None, None, None) == -1
+    fake = ctypes.c_void_p(4096)
+    assert lib.igs_gs2d_grid_workspace_bytes(2, 3000, 10, 13, 3) == 2 * 3 * 132 * 8     # B x groups x roundup4(HW) x float2
+    assert lib.igs_gs2d_grid_workspace_bytes(2, 3000, 10, 13, 5) == 0                   # not a compiled channel count
+    assert lib.igs_gs2d_backward_with_grid(fake, fake, fake, fake, st, 1, None, fake, fake, fake, 2, 3000, 10, 13, 3,
+                                           1e-6, fake, 1 << 30, fake, 1 << 30, fake, 8, fake, fake, None) == -4
     assert b"workspace" in lib.igs_status_string(-4)
     with pytest.raises(RuntimeError):
         _lib.check(-2, "x")
