@@ -12,6 +12,8 @@ it raises.
 """
 from __future__ import annotations
 
+import functools
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -241,6 +243,14 @@ def _cov_inverse_torch(scales, rotations, eps):
     return inv[..., 0, 0, None, None], inv[..., 0, 1, None, None], inv[..., 1, 1, None, None]
 
 
+@functools.lru_cache(maxsize=32)
+def _grid_vectors(h: int, w: int, device):
+    aspect_ratio = h / w
+    h_range = aspect_ratio ** 0.5
+    w_range = 1 / aspect_ratio ** 0.5
+    return torch.linspace(-w_range, w_range, w).to(device), torch.linspace(-h_range, h_range, h).to(device)
+
+
 class GaussianSplatting2D(nn.Module):
     """Drop-in for the reference module (src/igs/gs2d.py:479-689): a linear head producing
     `num_gaussians_per_emb` Gaussians (2 position, 2 log-scale, 1 rotation, 1 unused opacity
@@ -267,14 +277,11 @@ class GaussianSplatting2D(nn.Module):
     @staticmethod
     def xy_grid(size=None, device=None):
         """x in +-sqrt(w/h), y in +-sqrt(h/w) as stride-0 expanded [1,h,w] tensors
-        (src/igs/gs2d.py:503-522)."""
+        (src/igs/gs2d.py:503-522).  The two coordinate vectors are built once per (size, device)
+        and kept: the reference rebuilds them on the host and copies them over in every forward."""
         h, w = size
-        aspect_ratio = h / w
-        h_range = aspect_ratio ** 0.5
-        w_range = 1 / aspect_ratio ** 0.5
-        x_grid = torch.linspace(-w_range, w_range, w).to(device).view(1, 1, w).expand(1, h, w)
-        y_grid = torch.linspace(-h_range, h_range, h).to(device).view(1, h, 1).expand(1, h, w)
-        return x_grid, y_grid
+        xs, ys = _grid_vectors(int(h), int(w), None if device is None else torch.device(device))
+        return xs.view(1, 1, w).expand(1, h, w), ys.view(1, h, 1).expand(1, h, w)
 
     @staticmethod
     def render(positions, colors, scales, rotations, alphas, x_grid, y_grid, eps=1e-6, fused=True):
