@@ -42,6 +42,9 @@ def main() -> int:
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the JSON line, print the operator-level table of the reference's "
                          "scripts/profiling.py (B x N x H sweep, median of 32 timed calls after 4 warm-ups)")
+    ap.add_argument("--sweep-shape", default=None, metavar="BxNxH",
+                    help="with --sweep: this one shape only, forward+backward with all eight gradients (for profiling "
+                         "the general-grid kernels)")
     ap.add_argument("--all", action="store_true",
                     help="instead of the JSON line, print forward and forward+backward times of all five "
                          "configurations (c0-c4; c3 is the module, c2 also as the fused fit step)")
@@ -60,7 +63,7 @@ def main() -> int:
         return 2
 
     if args.sweep:
-        return sweep()
+        return sweep(args.sweep_shape)
     if args.all:
         return all_configs(args.steps, args.warmup)
     if args.koleo:
@@ -352,7 +355,7 @@ def koleo_table(no_cpu: bool, only: str = None) -> int:
     return 0
 
 
-def sweep() -> int:
+def sweep(only: str = None) -> int:
     """Operator-level sweep in the protocol of the reference's scripts/profiling.py:30-49, :69-151, :199-211:
     `.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors)` on randn/rand inputs (per-pixel
     random coordinates, so the general-grid kernels run), 4 warm-ups, 32 timed calls with events, median;
@@ -365,7 +368,10 @@ def sweep() -> int:
 
     dev = torch.device("cuda:0")
     rows = []
-    for B, N, H in itertools.product([4, 8], [4096, 8192, 16384], [128, 256]):
+    shapes = list(itertools.product([4, 8], [4096, 8192, 16384], [128, 256]))
+    if only:
+        shapes = [tuple(int(v) for v in only.split("x"))]
+    for B, N, H in shapes:
         W = H
         for mode in ("fwd", "fwd_bwd"):
             rg = mode == "fwd_bwd"

@@ -289,6 +289,16 @@ def require_gpu(t: Tensor):
     _lib.load()
 
 
+def require_same_device(dev, tensors: Sequence[Optional[Tensor]], what: str):
+    """Every tensor whose address goes to the kernels must live on `dev`: a host pointer (or one of
+    another GPU) handed to a launch is a memory fault, not an exception.  The reference raises
+    torch's device-mismatch RuntimeError for mixed arguments; so does this, before any launch."""
+    for t in tensors:
+        if t is not None and t.device != dev:
+            raise RuntimeError(f"Expected all tensors to be on the same device, but {what} has a tensor on "
+                               f"{t.device} while the Gaussian parameters are on {dev}")
+
+
 def run_forward(kind: int, params: Sequence[Tensor], x: Tensor, y: Tensor, eps: float):
     """pack + splat.  Returns (op, keep, packed, col, out, den): `keep` are the fp32 contiguous
     copies of the parameters that the finalize kernel of this kind reads again, `col` the colours
@@ -296,6 +306,7 @@ def run_forward(kind: int, params: Sequence[Tensor], x: Tensor, y: Tensor, eps: 
     require_gpu(params[0])
     B, N, C = problem_dims(kind, params)
     dev = params[0].device
+    require_same_device(dev, list(params) + [x, y], "the forward")
     with torch.cuda.device(dev):
         grid = Grid(x, y, B)
         op = Splat(B, N, C, grid, eps, dev)
@@ -325,6 +336,7 @@ def run_backward(kind: int, op: Splat, keep, packed, col, out, den, grad_result:
     of the kind's parameter list, fp32, None where `need` is False; colour gradients cut back to
     C channels; cov_inv gradients as [B,N]."""
     B, N, C, Cp, dev = op.B, op.N, op.C, op.Cp, op.device
+    require_same_device(dev, [grad_result, packed, col, out, den, *keep], "the backward")
     g_x = g_y = None
     grads: List[Optional[Tensor]] = [None] * len(need)
     with torch.cuda.device(dev):

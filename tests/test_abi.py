@@ -142,6 +142,20 @@ def test_fused_path_refuses_cpu_tensors():
         igs_amd.GaussianSplatting2DKernel.apply(d["x_grid"], d["y_grid"], d["positions"], a, a * 0, a, d["alphas"], d["colors"])
 
 
+def test_mixed_device_arguments_are_refused_before_any_launch():
+    """A host tensor among device tensors must raise, never reach a kernel as a host pointer (the
+    check itself needs no GPU: a torch.device is only a name)."""
+    import torch
+
+    from igs_amd import _splat
+
+    gpu = torch.device("cuda", 0)
+    host = torch.zeros(2)
+    with pytest.raises(RuntimeError, match="same device"):
+        _splat.require_same_device(gpu, [None, host], "the forward")
+    _splat.require_same_device(host.device, [host, None, host], "the forward")
+
+
 def test_host_api_surface_and_module_init():
     import torch
 

@@ -317,6 +317,29 @@ def test_error_paths(igs, dev):
                                   c["x_grid"], c["y_grid"])
 
 
+def test_mixed_devices_raise_instead_of_faulting(igs, dev):
+    """Device parameters with host grids (what `xy_grid(size)` returns without a device argument),
+    a host parameter among device ones, and a host grad_out: each must raise before a launch."""
+    d = to_dev(small_case(1, 8, 4, 4, 3, seed=1), dev)
+    names = ("positions", "colors", "scales", "rotations", "alphas")
+    xg, yg = igs.GaussianSplatting2D.xy_grid((4, 4))
+    assert xg.device.type == "cpu"
+    with pytest.raises(RuntimeError, match="same device"):
+        igs.gaussian_splatting_2d(*(d[k] for k in names), xg[None], yg[None])
+    with pytest.raises(RuntimeError, match="same device"):
+        igs.gaussian_splatting_2d(d["positions"], d["colors"].cpu(), d["scales"], d["rotations"], d["alphas"],
+                                  d["x_grid"], d["y_grid"])
+    a = torch.ones(1, 8, 1, 1, device=dev)
+    with pytest.raises(RuntimeError, match="same device"):
+        igs.GaussianSplatting2DKernel.apply(d["x_grid"], d["y_grid"].cpu(), d["positions"], a, a * 0, a,
+                                            d["alphas"], d["colors"])
+    lv = d["positions"].clone().requires_grad_(True)
+    out = igs.gaussian_splatting_2d(lv, d["colors"], d["scales"], d["rotations"], d["alphas"], d["x_grid"], d["y_grid"])
+    from igs_amd import _splat
+    with pytest.raises(RuntimeError, match="same device"):
+        _splat.require_same_device(out.device, [d["grad_out"].cpu()], "the backward")
+
+
 def test_random_small_shapes_against_oracle(igs, dev):
     """Thirty seeded random shapes (N, H, W around the tile and chunk sizes of the kernels, all
     compiled channel counts and some padded ones, dense to sparse scales, batch-1 grids): forward
