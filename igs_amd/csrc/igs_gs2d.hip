@@ -34,6 +34,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "igs_hip.h"
@@ -461,6 +462,7 @@ const char* igs_status_string(int status) {
         case IGS_ERR_BAD_MODE: return "unknown grid mode";
         case IGS_ERR_NO_DEVICE: return "no usable HIP device";
         case IGS_ERR_ALIGNMENT: return "buffer not 16-byte aligned";
+        case IGS_ERR_STATIC_SCRATCH: return "problem needs more scratch than the static array holds (IGS_STATIC_SCRATCH_BYTES)";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -515,10 +517,13 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
     return launch_status();
 }
 
-int igs_gs2d_forward(const float* packed, const float* x, const float* y,
-                     const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag, int B,
-                     int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
-                     size_t ws_bytes, igs_stream_t stream) {
+}  // extern "C"
+
+namespace {
+int forward_impl(const float* packed, const float* x, const float* y,
+                 const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag, int B,
+                 int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
+                 size_t ws_bytes, igs_stream_t stream) {
     if (!packed || !x || !y || !grid_strides || !out || !den) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
@@ -579,6 +584,63 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
         }
     }
     return IGS_OK;
+}
+}  // namespace
+
+// Scratch of igs_gs2d_forward_static_ws: one array per device, held from the load of the code
+// object to the end of the process.  In host code this name is only a handle for
+// hipGetSymbolAddress; the device address it yields is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[IGS_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each device, resolved once
+
+// The current device's copy of the static scratch array (resolved on the first call on that device).
+int static_scratch(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return IGS_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return IGS_ERR_NO_DEVICE;
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return IGS_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int igs_gs2d_forward(const float* packed, const float* x, const float* y,
+                     const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag, int B,
+                     int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
+                     size_t ws_bytes, igs_stream_t stream) {
+    return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
+                        ws_bytes, stream);
+}
+
+int igs_gs2d_forward_static_ws(const float* packed, const float* x, const float* y,
+                               const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                               int B, int N, int H, int W, int C, float eps, float* out, float* den,
+                               igs_stream_t stream) {
+    int rc = mode_ok(grid_mode, grid_flag);
+    if (rc) return rc;
+    igs_gs2d_plan_t total;
+    rc = make_plan(B, N, H, W, C, grid_mode, &total);
+    if (rc) return rc;
+    if (total.fwd_ws_bytes > (uint64_t)IGS_STATIC_SCRATCH_BYTES) return IGS_ERR_STATIC_SCRATCH;
+    void* ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc) return rc;
+    return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
+                        IGS_STATIC_SCRATCH_BYTES, stream);
 }
 
 }  // extern "C"

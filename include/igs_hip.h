@@ -24,8 +24,10 @@
 extern "C" {
 #endif
 
-#define IGS_ABI_VERSION 4
+#define IGS_ABI_VERSION 5
 #define IGS_MAX_CHANNELS 16
+/* Size of the per-device static scratch array behind igs_gs2d_forward_static_ws. */
+#define IGS_STATIC_SCRATCH_BYTES (64u << 20)
 
 typedef void *igs_stream_t; /* a hipStream_t */
 
@@ -38,7 +40,9 @@ typedef enum igs_status {
     IGS_ERR_WORKSPACE = -4,      /* a workspace is smaller than igs_gs2d_plan says */
     IGS_ERR_BAD_MODE = -5,       /* unknown grid mode */
     IGS_ERR_NO_DEVICE = -6,      /* no usable HIP device */
-    IGS_ERR_ALIGNMENT = -7       /* a buffer that must be 16-byte aligned is not */
+    IGS_ERR_ALIGNMENT = -7,      /* a buffer that must be 16-byte aligned is not */
+    IGS_ERR_STATIC_SCRATCH = -8  /* igs_gs2d_forward_static_ws: the plan's fwd_ws_bytes exceeds
+                                    IGS_STATIC_SCRATCH_BYTES */
 } igs_status;
 
 /* How the pixel coordinates are described.
@@ -140,6 +144,24 @@ int igs_gs2d_forward(const float *packed, const float *x, const float *y,
                      const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag, int B,
                      int N, int H, int W, int C, float eps, float *out, float *den, void *ws,
                      size_t ws_bytes, igs_stream_t stream);
+
+/* igs_gs2d_forward without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory around the
+ * call: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The forward's scratch (split partials, per-tile Gaussian lists) lives in a static device array
+ * of IGS_STATIC_SCRATCH_BYTES (64 MiB) that every GPU the library runs on holds until the process
+ * ends; problems whose plan.fwd_ws_bytes is larger are rejected with IGS_ERR_STATIC_SCRATCH
+ * (B=1, N=2048, 256x256, C=3 needs 32 MiB; the 16-image headline shape needs 136 MiB and must use
+ * igs_gs2d_forward).  Same kernels, same launch plan and bit-identical results as
+ * igs_gs2d_forward.  All calls on one GPU share that GPU's array: calls that overlap in time on
+ * one GPU (two streams, two threads) race on it; nothing in it has to start at zero and its
+ * contents mean nothing after the call.  The first call on a device resolves the array's device
+ * address (hipGetSymbolAddress, which may load the code object there): make that call outside
+ * graph capture, with that device current. */
+int igs_gs2d_forward_static_ws(const float *packed, const float *x, const float *y,
+                               const int64_t grid_strides[6], int grid_mode,
+                               const int32_t *grid_flag, int B, int N, int H, int W, int C,
+                               float eps, float *out, float *den, igs_stream_t stream);
 
 /* Backward, stage 1: per-pixel prologue, g^ = grad_out/(den+eps), s = <g^, out>, written
  * as one record per pixel into pix_ws (plan.pix_bytes).  Replaces the per-image pre-pass of
