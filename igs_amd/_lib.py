@@ -18,6 +18,9 @@ ABI_VERSION = 5  # IGS_ABI_VERSION of include/igs_hip.h this binding was written
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1
 IGS_GRID_AUTO = 2
+IGS_OPT_NO_CULL = 0x100
+IGS_OPT_BIN_LEVELS_1 = 0x200
+IGS_OPT_BIN_LEVELS_2 = 0x400
 IGS_MAX_CHANNELS = 16
 IGS_STATIC_SCRATCH_BYTES = 64 << 20
 COMPILED_CHANNELS = (1, 2, 3, 4, 8, 16)

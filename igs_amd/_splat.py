@@ -16,6 +16,7 @@ stream; every FLOP happens in libigs_hip.so.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from typing import List, Optional, Sequence, Tuple
 
@@ -29,6 +30,28 @@ Tensor = torch.Tensor
 KIND_COVINV = 0
 KIND_SCALE_ROT = 1
 KIND_FEATURE = 2
+
+
+# igs_option bits OR-ed into the grid_mode word of every Grid built while `library_options` is active
+_option_bits = 0
+
+
+@contextlib.contextmanager
+def library_options(no_cull: bool = False, bin_levels: Optional[int] = None):
+    """Testing aid: problems set up inside this context run with the given igs_option bits of
+    include/igs_hip.h -- `no_cull` lists every Gaussian for every pixel tile (the reference point
+    for "culling changes no bit"), `bin_levels` = 1 | 2 forces the one- or two-level construction
+    of the tile lists.  The bits travel as explicit arguments of each library call (in the
+    grid_mode word); the library itself holds no such state."""
+    global _option_bits
+    bits = _lib.IGS_OPT_NO_CULL if no_cull else 0
+    if bin_levels is not None:
+        bits |= {1: _lib.IGS_OPT_BIN_LEVELS_1, 2: _lib.IGS_OPT_BIN_LEVELS_2}[int(bin_levels)]
+    saved, _option_bits = _option_bits, _option_bits | bits   # nested contexts add up
+    try:
+        yield
+    finally:
+        _option_bits = saved
 
 
 def _ptr(t: Optional[Tensor]):
@@ -117,9 +140,9 @@ class Grid:
         # flag that the kernels read, so there is no host synchronisation either way.
         self.flag = None
         if self.sx[1] == 0 and self.sy[2] == 0:
-            self.mode = _lib.IGS_GRID_SEPARABLE
+            self.mode = _lib.IGS_GRID_SEPARABLE | _option_bits
         else:
-            self.mode = _lib.IGS_GRID_AUTO
+            self.mode = _lib.IGS_GRID_AUTO | _option_bits
             self.flag = torch.empty(1, dtype=torch.int32, device=x.device)
             _lib.check(_lib.load().igs_gs2d_grid_classify(_ptr(self.x), _ptr(self.y), self.strides, B, self.H,
                                                           self.W, _ptr(self.flag), _stream(x.device)),
@@ -198,8 +221,10 @@ class Splat:
         g, p = self.grid, self.plan
         pix = self._empty(p.pix_bytes)
         partial = self._empty(p.partial_bytes)
-        gws_bytes = int(self.lib.igs_gs2d_grid_workspace_bytes(self.B, self.N, g.H, g.W, self.Cp))
-        gws = self._empty(gws_bytes)
+        # host-proven separable grids run the pixel-major grid kernel, which needs no workspace
+        separable = (g.mode & 0xff) == _lib.IGS_GRID_SEPARABLE
+        gws_bytes = 0 if separable else int(self.lib.igs_gs2d_grid_workspace_bytes(self.B, self.N, g.H, g.W, self.Cp))
+        gws = None if separable else self._empty(gws_bytes)
         gx = self._new(self.B, g.H, g.W)
         gy = torch.empty_like(gx)
         _lib.check(self.lib.igs_gs2d_backward_with_grid(

@@ -119,7 +119,7 @@ inline size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
 // the finalize kernel adds the tiles in another order (super-tile by super-tile), so gradients
 // agree to rounding.  Space for the super-tile lists / tables is part of the plan whenever the
 // tile grid is large enough (a function of the shape only); whether a launch uses them depends
-// on the work, tiles x N, or on IGS_BIN_LEVELS=1|2 in the environment (read at every call).
+// on the work, tiles x N, or on the IGS_OPT_BIN_LEVELS_1|2 bit of the call's grid_mode argument.
 struct SuperGeometry {
     int x, y, count;  // super-tiles along x, along y, per image
     int chunk, K;     // Gaussians per first-level workgroup, workgroups per super-tile
@@ -139,17 +139,20 @@ inline SuperGeometry super_tiles(int tiles_x, int tiles_y, int B, int N) {
     return g;
 }
 inline bool super_reserved(int tiles_x, int tiles_y) { return tiles_x * tiles_y >= 32; }
-inline bool two_level(int N, int tiles_x, int tiles_y) {
+inline bool two_level(int N, int tiles_x, int tiles_y, int opts) {
     if (!super_reserved(tiles_x, tiles_y)) return false;
-    const char* e = getenv("IGS_BIN_LEVELS");
-    if (e && e[0] == '1') return false;
-    if (e && e[0] == '2') return true;
+    if (opts & IGS_OPT_BIN_LEVELS_1) return false;
+    if (opts & IGS_OPT_BIN_LEVELS_2) return true;
     return (long)N * tiles_x * tiles_y >= (1L << 25);  // measured break-even: N = 65536 on 256-512 tiles
 }
 // Super-tile lists of one launch: counts [B][stiles][kBinMaxChunks] then lists [B][stiles][Np].
 inline size_t super_bins_bytes(int B, int stiles, int Np) {
     return ((size_t)B * stiles * kBinMaxChunks + (size_t)B * stiles * Np) * sizeof(int);
 }
+
+// A grid_mode argument of the ABI: the igs_grid_mode in the low byte, IGS_OPT_* bits above it.
+inline int mode_of(int word) { return word & 0xff; }
+inline int opts_of(int word) { return word & ~0xff; }
 
 // Plan of one kernel variant (grid_mode is GENERAL or SEPARABLE here).
 int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
@@ -264,16 +267,10 @@ inline const float4* boxes_of(const float* packed, int B, int Np, int RS) {
     return reinterpret_cast<const float4*>(packed + (size_t)B * Np * RS);
 }
 
-// IGS_NO_CULL=1 in the environment makes every reach box unbounded (nothing is skipped): the
-// reference point for checking that culling changes no bit.  Read at every pack call.
-inline int culling_enabled() {
-    const char* e = getenv("IGS_NO_CULL");
-    return !(e && e[0] == '1');
-}
-
 // Public plan: AUTO reports the separable variant's geometry with the workspace sizes of
 // whichever variant needs more.
 int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* p) {
+    grid_mode = mode_of(grid_mode);  // the option bits change no size
     if (grid_mode != IGS_GRID_AUTO) return plan_one(B, N, H, W, C, grid_mode, p);
     igs_gs2d_plan_t g;
     int rc = plan_one(B, N, H, W, C, IGS_GRID_SEPARABLE, p);
@@ -340,6 +337,7 @@ struct Variant {
 };
 
 int variants_of(int grid_mode, const int32_t* grid_flag, Variant (&v)[2]) {
+    grid_mode = mode_of(grid_mode);
     if (grid_mode == IGS_GRID_AUTO) {
         v[0] = {IGS_GRID_SEPARABLE, grid_flag, 1};
         v[1] = {IGS_GRID_GENERAL, grid_flag, 0};
@@ -439,6 +437,10 @@ int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* col
 }
 
 int mode_ok(int grid_mode, const int32_t* grid_flag) {
+    const int opts = opts_of(grid_mode);
+    if (opts & ~(IGS_OPT_NO_CULL | IGS_OPT_BIN_LEVELS_1 | IGS_OPT_BIN_LEVELS_2)) return IGS_ERR_BAD_MODE;
+    if ((opts & IGS_OPT_BIN_LEVELS_1) && (opts & IGS_OPT_BIN_LEVELS_2)) return IGS_ERR_BAD_MODE;
+    grid_mode = mode_of(grid_mode);
     if (grid_mode != IGS_GRID_GENERAL && grid_mode != IGS_GRID_SEPARABLE && grid_mode != IGS_GRID_AUTO)
         return IGS_ERR_BAD_MODE;
     if (grid_mode == IGS_GRID_AUTO && !grid_flag) return IGS_ERR_NULL_POINTER;
@@ -498,7 +500,7 @@ int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const f
     hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
                        colors, N, Np, C, rec_stride_of(C), 0.0f, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))), culling_enabled());
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
@@ -513,7 +515,7 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
     hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
                        alphas, colors, N, Np, C, rec_stride_of(C), eps, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))), culling_enabled());
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
@@ -566,7 +568,8 @@ int forward_impl(const float* packed, const float* x, const float* y,
             ba.tiles_x = fg.tiles_x; ba.tiles_y = fg.tiles_y;
             ba.counts = bp.counts; ba.lists = bp.lists; ba.slots = nullptr;
             ba.flag = vs[i].flag; ba.want = vs[i].want;
-            const bool levels2 = two_level(N, fg.tiles_x, fg.tiles_y);
+            ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
+            const bool levels2 = two_level(N, fg.tiles_x, fg.tiles_y, opts_of(grid_mode));
             const BinPlace cp = levels2 ? super_bins_at(ws, split_bytes, B, plan.fwd_tiles, plan.n_padded,
                                                         super_tiles(fg.tiles_x, fg.tiles_y, B, N).count)
                                         : BinPlace{nullptr, nullptr};
@@ -797,7 +800,8 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
             ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists);
             ba.slots = slots_at(partial, B, a.T, 6 + C, N);
             ba.flag = a.flag; ba.want = a.want;
-            const bool levels2 = two_level(N, ba.tiles_x, ba.tiles_y);
+            ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
+            const bool levels2 = two_level(N, ba.tiles_x, ba.tiles_y, opts_of(grid_mode));
             BinPlace cp{nullptr, nullptr};
             int* cslots = nullptr;
             if (levels2) {
@@ -849,9 +853,12 @@ int igs_gs2d_backward_with_grid(const float* packed, const float* colors, const 
                                 int H, int W, int C, float eps, float* pix_ws, size_t pix_bytes, float* partial,
                                 size_t partial_bytes, void* grid_ws, size_t grid_ws_bytes, float* g_x,
                                 float* g_y, igs_stream_t stream) {
-    if (!x || !out || !den || !grad_out || !grid_ws || !g_x || !g_y) return IGS_ERR_NULL_POINTER;
-    if (grid_ws_bytes < igs_gs2d_grid_workspace_bytes(B, N, H, W, C)) return IGS_ERR_WORKSPACE;
-    if ((uintptr_t)grid_ws & 7) return IGS_ERR_ALIGNMENT;
+    if (!x || !out || !den || !grad_out || !g_x || !g_y) return IGS_ERR_NULL_POINTER;
+    if (mode_of(grid_mode) != IGS_GRID_SEPARABLE) {  // only the general-grid kernels use grid_ws
+        if (!grid_ws) return IGS_ERR_NULL_POINTER;
+        if (grid_ws_bytes < igs_gs2d_grid_workspace_bytes(B, N, H, W, C)) return IGS_ERR_WORKSPACE;
+        if ((uintptr_t)grid_ws & 7) return IGS_ERR_ALIGNMENT;
+    }
     int rc = igs_gs2d_backward_prologue(x, y, grid_strides, grid_mode, grid_flag, out, den, grad_out, B, N,
                                         H, W, C, eps, pix_ws, pix_bytes, stream);
     if (rc) return rc;
@@ -903,7 +910,7 @@ int igs_gs2d_backward_grid(const float* packed, const float* x, const float* y,
 
 // The slot tables that the separable backward left behind the partial sums (none on general grids).
 static const int* finalize_slots(const float* partial, int grid_mode, int B, int T, int NF, int N) {
-    if (grid_mode == IGS_GRID_GENERAL) return nullptr;
+    if (mode_of(grid_mode) == IGS_GRID_GENERAL) return nullptr;
     return slots_at(const_cast<float*>(partial), B, T, NF, N);
 }
 
@@ -911,6 +918,8 @@ static const int* finalize_slots(const float* partial, int grid_mode, int B, int
 // tables of the separable backward when it binned in two levels.
 static int finalize_tiles(int grid_mode, int B, int N, int H, int W, int C, int* T, int* T_alt,
                           const float* partial, SuperSlots* sup) {
+    const int opts = opts_of(grid_mode);
+    grid_mode = mode_of(grid_mode);
     igs_gs2d_plan_t plan;
     int rc = plan_one(B, N, H, W, C, grid_mode == IGS_GRID_AUTO ? IGS_GRID_SEPARABLE : grid_mode, &plan);
     if (rc) return rc;
@@ -919,7 +928,7 @@ static int finalize_tiles(int grid_mode, int B, int N, int H, int W, int C, int*
     *sup = SuperSlots{nullptr, 1, 1, 1, 1};
     if (grid_mode != IGS_GRID_GENERAL) {
         const int tiles_y = plan.bwd_tiles / plan.bwd_tiles_x;
-        if (two_level(N, plan.bwd_tiles_x, tiles_y)) {
+        if (two_level(N, plan.bwd_tiles_x, tiles_y, opts)) {
             const SuperGeometry sg = super_tiles(plan.bwd_tiles_x, tiles_y, B, N);
             sup->cslots = super_slots_at(const_cast<float*>(partial), B, plan.bwd_tiles, 6 + C, N, plan.n_padded);
             sup->tiles_x = plan.bwd_tiles_x;
@@ -950,7 +959,7 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
     if (rc) return rc;
     IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<false, kFT>),
-                       (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
+                       (hipStream_t)stream, partial, T, mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), sup, (N + 3) & ~3, cov_inv_00,
                        cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
                        g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
@@ -970,7 +979,7 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
     if (rc) return rc;
     IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<true, kFT>),
-                       (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
+                       (hipStream_t)stream, partial, T, mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), sup, (N + 3) & ~3, scales, rotations,
                        (const float*)nullptr, alphas, N, C, eps, g_positions,
                        g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
@@ -987,8 +996,7 @@ int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int 
     hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
                        rec_stride_of(C_kernel), eps, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out,
-                       culling_enabled());
+                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
     return launch_status();
 }
 
@@ -1004,7 +1012,7 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
     rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt, partial, &sup);
     if (rc) return rc;
     IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize_feature<kFT>),
-                       (hipStream_t)stream, partial, T, grid_mode == IGS_GRID_AUTO ? grid_flag : nullptr,
+                       (hipStream_t)stream, partial, T, mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr,
                        T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N), sup, (N + 3) & ~3, gs_feature,
                        N, C, C_kernel, eps, g_feature);
     return launch_status();

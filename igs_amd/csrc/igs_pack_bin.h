@@ -43,7 +43,7 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
                                                    const float* __restrict__ colors, int N,
                                                    int Np, int C, int RS, float eps,
                                                    float* __restrict__ packed,
-                                                   float4* __restrict__ boxes, int cull) {
+                                                   float4* __restrict__ boxes) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n >= Np) return;
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
     }
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
-    const float4 box = reach_box(px, py, sxx, syy, cull && bounded && fin);
+    const float4 box = reach_box(px, py, sxx, syy, bounded && fin);
     boxes[(size_t)b * Np + n] = box;
     if (RS >= 8 + C) {  // room in the record: the y range of the box travels with it
         r[6 + C] = box.z;
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
                                                            int Np, int C, int Cp, int RS, float eps,
                                                            float* __restrict__ packed,
                                                            float4* __restrict__ boxes,
-                                                           float* __restrict__ colors_out, int cull) {
+                                                           float* __restrict__ colors_out) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n >= Np) return;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
     }
     for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
     const float4 box = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
-                                 cull && fin && v0 > 0.0 && v1 > 0.0);
+                                 fin && v0 > 0.0 && v1 > 0.0);
     boxes[(size_t)b * Np + n] = box;
     if (RS >= 8 + Cp) {
         r[6 + Cp] = box.z;
@@ -199,6 +199,7 @@ struct BinArgs {
     int cand_K, cand_chunk, stiles_x, stiles;
     const int* flag;
     int want;
+    int no_cull;  // list every candidate (IGS_OPT_NO_CULL): the reference point for "culling changes no bit"
 };
 
 // Tiles per super-tile of the two-level binning (each way) and the most segments per list.
@@ -267,7 +268,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         ylo = fminf(ylo, v);
         yhi = fmaxf(yhi, v);
     }
-    if (bad) {  // a NaN coordinate: nothing may be culled for this tile
+    if (bad || a.no_cull) {  // a NaN coordinate, or culling switched off: nothing may be culled for this tile
         xlo = ylo = -inf;
         xhi = yhi = inf;
     }

@@ -61,12 +61,26 @@ typedef enum igs_status {
  *                        Workspace sizes are the larger of the two variants'.
  * Entry points take `grid_flag` (device int32, 1 = separable); it is only read in AUTO mode
  * and may be NULL otherwise.
+ *
+ * The `grid_mode` argument of an entry point carries the igs_grid_mode in its low byte and may
+ * have igs_option bits OR-ed in above it (testing aids; they change no buffer size, and unknown
+ * bits are rejected with IGS_ERR_BAD_MODE).  A backward and its finalize call must get the same
+ * IGS_OPT_BIN_LEVELS_* bits.
  */
 typedef enum igs_grid_mode {
     IGS_GRID_GENERAL = 0,
     IGS_GRID_SEPARABLE = 1,
     IGS_GRID_AUTO = 2
 } igs_grid_mode;
+
+typedef enum igs_option {
+    IGS_OPT_NO_CULL = 0x100,      /* separable grids: list every Gaussian for every pixel tile
+                                     (nothing is skipped): the reference point for checking that
+                                     skipping changes no bit */
+    IGS_OPT_BIN_LEVELS_1 = 0x200, /* build the per-tile Gaussian lists in one level ...           */
+    IGS_OPT_BIN_LEVELS_2 = 0x400  /* ... or through super-tiles of 4 x 4 tiles, whatever the size;
+                                     without either bit the library chooses by tiles x N          */
+} igs_option;
 
 /* Launch plan and workspace sizes for one problem shape (filled by igs_gs2d_plan).  In AUTO
  * mode the geometry fields describe the separable variant. */
@@ -119,13 +133,12 @@ int igs_gs2d_grid_classify(const float *x, const float *y, const int64_t grid_st
  * (plan.fwd_split == 1) and to fp32 rounding otherwise, where a tile's list rather than the
  * index range is cut into the splits (the reference evaluates every pair:
  * src/igs/gs_triton_chunked.py:100-200).  Records with a
- * non-finite field or a cov_inv that is not positive definite are never skipped.  Setting
- * IGS_NO_CULL=1 in the environment (read at each pack call) makes every box unbounded.
+ * non-finite field or a cov_inv that is not positive definite are never skipped; with
+ * IGS_OPT_NO_CULL in a forward / backward call's grid_mode nothing is.
  * Large problems (tiles x N >= 2^25) build the per-tile lists in two levels (super-tiles of
- * 4 x 4 tiles first); IGS_BIN_LEVELS=1|2 in the environment (read at each forward / backward /
- * finalize call; keep it fixed between a backward and its finalize) forces one or two.  The
- * lists and the forward do not depend on it; the finalize kernels add the tiles in another
- * order under two levels, so gradients agree to fp32 rounding. */
+ * 4 x 4 tiles first); IGS_OPT_BIN_LEVELS_1|2 forces one or two.  The lists and the forward do
+ * not depend on it; the finalize kernels add the tiles in another order under two levels, so
+ * gradients agree to fp32 rounding. */
 int igs_gs2d_pack_covinv(const float *position, const float *cov_inv_00, const float *cov_inv_01,
                          const float *cov_inv_11, const float *alphas, const float *colors,
                          int B, int N, int C, float *packed, igs_stream_t stream);
@@ -196,7 +209,8 @@ int igs_gs2d_backward(const float *packed, const float *colors, const float *x, 
  * them) in one call.  On general grids the per-pixel sums are formed inside the per-Gaussian
  * reduction (one exponential per pair instead of two) into grid_ws
  * (igs_gs2d_grid_workspace_bytes, 8-byte aligned) and added in a fixed order; on separable
- * grids this equals igs_gs2d_backward followed by igs_gs2d_backward_grid. */
+ * grids this equals igs_gs2d_backward followed by igs_gs2d_backward_grid, and with
+ * IGS_GRID_SEPARABLE grid_ws is not used and may be NULL. */
 size_t igs_gs2d_grid_workspace_bytes(int B, int N, int H, int W, int C);
 int igs_gs2d_backward_with_grid(const float *packed, const float *colors, const float *x,
                                 const float *y, const int64_t grid_strides[6], int grid_mode,

@@ -111,9 +111,22 @@ def test_argument_errors_are_status_codes_not_crashes(lib):
     fake = ctypes.c_void_p(4096)
     assert lib.igs_gs2d_grid_workspace_bytes(2, 3000, 10, 13, 3) == 2 * 3 * 132 * 8     # B x groups x roundup4(HW) x float2
     assert lib.igs_gs2d_grid_workspace_bytes(2, 3000, 10, 13, 5) == 0                   # not a compiled channel count
-    assert lib.igs_gs2d_backward_with_grid(fake, fake, fake, fake, st, 1, None, fake, fake, fake, 2, 3000, 10, 13, 3,
+    assert lib.igs_gs2d_backward_with_grid(fake, fake, fake, fake, st, 0, None, fake, fake, fake, 2, 3000, 10, 13, 3,
                                            1e-6, fake, 1 << 30, fake, 1 << 30, fake, 8, fake, fake, None) == -4
     assert b"workspace" in lib.igs_status_string(-4)
+    # host-proven separable grids need no grid workspace: the call gets past that check (and stops
+    # at the next one, the pixel workspace, here 0 bytes) ...
+    assert lib.igs_gs2d_backward_with_grid(fake, fake, fake, fake, st, 1, None, fake, fake, fake, 2, 3000, 10, 13, 3,
+                                           1e-6, fake, 0, fake, 1 << 30, None, 0, fake, fake, None) == -4
+    # ... while general grids insist on it
+    assert lib.igs_gs2d_backward_with_grid(fake, fake, fake, fake, st, 0, None, fake, fake, fake, 2, 3000, 10, 13, 3,
+                                           1e-6, fake, 1 << 30, fake, 1 << 30, None, 0, fake, fake, None) == -1
+    # option bits ride in the grid_mode word; unknown or contradictory ones are rejected
+    assert lib.igs_gs2d_forward(fake, fake, fake, st, 1 | 0x800, None, 1, 8, 4, 4, 3, 1e-6, fake, fake, fake, 1 << 30,
+                                None) == -5
+    assert lib.igs_gs2d_forward(fake, fake, fake, st, 1 | 0x200 | 0x400, None, 1, 8, 4, 4, 3, 1e-6, fake, fake, fake,
+                                1 << 30, None) == -5
+    assert lib.igs_gs2d_plan(1, 8, 4, 4, 3, 1 | 0x100 | 0x400, ctypes.byref(p)) == 0      # sizes ignore them
     with pytest.raises(RuntimeError):
         _lib.check(-2, "x")
 

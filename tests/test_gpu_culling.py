@@ -1,6 +1,6 @@
 """Culling on separable grids: a Gaussian is skipped for a pixel tile when its reach box (the
 bounding box of q <= 221.8, beyond which exp2 of the kernels' exponent is exactly 0) misses the
-tile.  The claim under test is that this drops only exact zeros: with IGS_NO_CULL=1 the
+tile.  The claim under test is that this drops only exact zeros: with IGS_OPT_NO_CULL the
 library makes every box unbounded, and both runs must agree exactly (one forward split) or to
 fp32 rounding (several, where the grouping of the terms changes); beside that, sparse scenes
 against the fp64 oracle, non-finite parameters, and grids whose coordinates are not monotone."""
@@ -47,13 +47,16 @@ def run(igs, g, x=None, y=None):
 
 @pytest.fixture
 def no_cull():
-    """Context that disables culling in the library (read at every pack call)."""
-    class Ctx:
+    """Context in which the library lists every Gaussian for every tile (IGS_OPT_NO_CULL)."""
+    from igs_amd._splat import library_options
+
+    class Ctx:  # re-enterable: a fresh context per `with`
         def __enter__(self):
-            os.environ["IGS_NO_CULL"] = "1"
+            self.ctx = library_options(no_cull=True)
+            return self.ctx.__enter__()
 
         def __exit__(self, *a):
-            os.environ.pop("IGS_NO_CULL", None)
+            return self.ctx.__exit__(*a)
 
     return Ctx()
 
@@ -88,15 +91,12 @@ def test_long_rotated_gaussians_bit_for_bit(igs, dev, no_cull):
         assert torch.equal(grads[k], grads0[k]), k
 
 
-class _Env:
-    def __init__(self, name, value):
-        self.name, self.value = name, value
+def _Env(name, value):
+    """The one- or two-level construction of the tile lists, forced (IGS_OPT_BIN_LEVELS_1 | _2)."""
+    from igs_amd._splat import library_options
 
-    def __enter__(self):
-        os.environ[self.name] = self.value
-
-    def __exit__(self, *a):
-        os.environ.pop(self.name, None)
+    assert name == "IGS_BIN_LEVELS"
+    return library_options(bin_levels=int(value))
 
 
 def _kernel_channels(C):
@@ -110,7 +110,7 @@ def _kernel_channels(C):
                                           ((1, 9000, 520, 1000, 3), (0.002, 0.02)), ((2, 20000, 256, 512, 3), (0.002, 0.01))],
                          ids=lambda v: "x".join(map(str, v)))
 def test_two_level_binning(igs, dev, shape, scales):
-    """IGS_BIN_LEVELS=2 lists the Gaussians per super-tile (4 x 4 tiles, several workgroups per
+    """IGS_OPT_BIN_LEVELS_2 lists the Gaussians per super-tile (4 x 4 tiles, several workgroups per
     super-tile, each filling its own segment) first and lets every tile scan those segments only.
     The tile lists are the same as with one level, hence the forward bit for bit; the finalize kernel
     then adds the tiles super-tile by super-tile, so the gradients agree to rounding."""

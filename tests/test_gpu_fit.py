@@ -192,10 +192,10 @@ def test_fit_converges_config2_reduced(igs, dev):
 
 
 def test_fused_step_under_two_level_binning(igs, dev):
-    """IGS_BIN_LEVELS=2 (the tile lists built through super-tiles) changes the order in which the
+    """IGS_OPT_BIN_LEVELS_2 (the tile lists built through super-tiles) changes the order in which the
     finalize kernel adds the tiles and nothing else: the first loss is bit-identical, the
     parameters after a few steps agree to rounding."""
-    import os
+    from igs_amd._splat import library_options
 
     B, N, H, W, C = 1, 3000, 256, 512, 3
     block0 = make_block(B, N, C, 5, dev)
@@ -204,13 +204,10 @@ def test_fused_step_under_two_level_binning(igs, dev):
     target = torch.rand(B, C, H, W, generator=torch.Generator().manual_seed(6)).to(dev)
     res = {}
     for levels in ("1", "2"):
-        os.environ["IGS_BIN_LEVELS"] = levels
-        try:
+        with library_options(bin_levels=int(levels)):
             fit = igs.GaussianImageFit(block0.clone(), target, xg, yg, lr=0.01)
             losses = [float(fit.step()) for _ in range(4)]
             res[levels] = (losses, fit.params.clone())
-        finally:
-            os.environ.pop("IGS_BIN_LEVELS", None)
     assert res["1"][0][0] == res["2"][0][0]
     assert res["1"][0][-1] < res["1"][0][0]
     torch.testing.assert_close(res["1"][1], res["2"][1], rtol=1e-4, atol=1e-5)
