@@ -381,13 +381,12 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
 }
 
 // General grid: the tile is a flat pixel range (multiple of 256); x and y come with the
-// pixel record.  Sums are flushed into the totals once per 128-pixel chunk.
-template <int C, int G, bool kGrid>
+// pixel record.  Sums are flushed into the totals once per chunk of pixel records.
+template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     constexpr int CP = pix_stride_gen(C), CP4 = CP / 4;
     constexpr int kPixChunk = pix_chunk(C);
     __shared__ float4 sh[2 * kPixChunk * CP4];
-    __shared__ float2 gacc[kGrid ? kThreads / 64 : 1][kGrid ? kPixChunk : 1];  // per wave and record of the chunk
     IGS_GATE(a);
     const int b = blockIdx.z, t = blockIdx.y;
     int n[G];
@@ -395,21 +394,6 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     for (int g = 0; g < G; ++g) n[g] = (blockIdx.x * G + g) * kThreads + threadIdx.x;
     float px[G], py[G], A[G], B2[G], D[G], col[G][C];
     bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
-    // Grid gradients (kGrid): d L / d x(pixel) = -sum_n G_n w_n (A dx + B dy), same with (B dx + D dy)
-    // for y.  With t1 = A'dx + (B2'/2) dy, t2 = (B2'/2) dx + D'dy the exponent is dx t1 + dy t2, and
-    // a lane adds alpha G e (t1, t2) of its G Gaussians per pixel record; the 64 lanes are summed
-    // by a butterfly, the four waves and the workgroups of the other Gaussians in a fixed order
-    // (LDS, then k_grid_reduce), which also applies the factor -1/k of t1 = k (A dx + B dy).
-    float hb[G], al[G];
-    if (kGrid) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            hb[g] = 0.5f * B2[g];
-            // unused lane slots (n >= N) must add nothing
-            al[g] = n[g] < a.N ? a.packed[((size_t)b * a.Np + n[g]) * rec_stride_of(C) + 5] : 0.0f;
-        }
-    }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     float M[G][6], CG[G][C], R[G][6], RC[G][C];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -431,58 +415,55 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
             pv[4 * q4 + 2] = tq.z;
             pv[4 * q4 + 3] = tq.w;
         }
-        float dxs[G], dys[G], ee[G], t1[G], t2[G];
+        // every step runs over the G Gaussians before the next one starts, so that neighbouring
+        // instructions are independent (a wave issues a dependent fp32 op only every ~8 cycles, an
+        // independent one every ~4.5)
+        float dx[G], dy[G], ee[G], tt[G], v[G];
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const float dx = pv[0] - px[g];
-            const float dy = pv[1] - py[g];
-            if (kGrid) {
-                t1[g] = fmaf(A[g], dx, hb[g] * dy);
-                t2[g] = fmaf(D[g], dy, hb[g] * dx);
-                ee[g] = fmaf(dx, t1[g], dy * t2[g]);
-            } else {
-                float tt = A[g] * dx;
-                tt = fmaf(B2[g], dy, tt);
-                const float v = D[g] * dy;
-                float q = tt * dx;
-                ee[g] = fmaf(v, dy, q);
-            }
-            dxs[g] = dx;
-            dys[g] = dy;
-        }
+        for (int g = 0; g < G; ++g) dx[g] = pv[0] - px[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) dy[g] = pv[1] - py[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) tt[g] = A[g] * dx[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) v[g] = D[g] * dy[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) tt[g] = fmaf(B2[g], dy[g], tt[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) v[g] = v[g] * dy[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) ee[g] = fmaf(tt[g], dx[g], v[g]);
 #pragma unroll
         for (int g = 0; g < G; ++g) ee[g] = hw_exp2(ee[g]);
-        float gxl = 0.0f, gyl = 0.0f;
+        float Gv[G], ge[G], m1[G], m2[G];
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const float e = ee[g], dx = dxs[g], dy = dys[g];
-            float Gv = pv[2 + C];  // -s
+        for (int g = 0; g < G; ++g) Gv[g] = fmaf(pv[2], col[g][0], pv[2 + C]);  // <g^, c> - s
 #pragma unroll
-            for (int c = 0; c < C; ++c) Gv = fmaf(pv[2 + c], col[g][c], Gv);
-            const float ge = Gv * e;
-            R[g][0] += ge;
-            const float m1 = ge * dx, m2 = ge * dy;
-            R[g][1] += m1;
-            R[g][2] += m2;
-            R[g][3] = fmaf(m1, dx, R[g][3]);
-            R[g][4] = fmaf(m1, dy, R[g][4]);
-            R[g][5] = fmaf(m2, dy, R[g][5]);
+        for (int c = 1; c < C; ++c)
 #pragma unroll
-            for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[2 + c], RC[g][c]);
-            if (kGrid) {
-                const float gw = ge * al[g];
-                gxl = fmaf(gw, t1[g], gxl);
-                gyl = fmaf(gw, t2[g], gyl);
-            }
-        }
-        if (kGrid) {
+            for (int g = 0; g < G; ++g) Gv[g] = fmaf(pv[2 + c], col[g][c], Gv[g]);
 #pragma unroll
-            for (int k = 32; k > 0; k >>= 1) {
-                gxl += __shfl_xor(gxl, k);
-                gyl += __shfl_xor(gyl, k);
-            }
-            if (lane == 0) gacc[kGrid ? wave : 0][kGrid ? (seen & (kPixChunk - 1)) : 0] = make_float2(gxl, gyl);
-        }
+        for (int g = 0; g < G; ++g) ge[g] = Gv[g] * ee[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) m1[g] = ge[g] * dx[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) m2[g] = ge[g] * dy[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][0] += ge[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][1] += m1[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][2] += m2[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][3] = fmaf(m1[g], dx[g], R[g][3]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][4] = fmaf(m1[g], dy[g], R[g][4]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][5] = fmaf(m2[g], dy[g], R[g][5]);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int g = 0; g < G; ++g) RC[g][c] = fmaf(ee[g], pv[2 + c], RC[g][c]);
         if ((++seen & (kPixChunk - 1)) == 0) {  // two-level summation
 #pragma unroll
             for (int g = 0; g < G; ++g) {
@@ -497,20 +478,6 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
                     RC[g][c] = 0.0f;
                 }
             }
-            if (kGrid) {  // the chunk's records are complete in all four waves: add them in wave order
-                __syncthreads();
-                const int p = p0 + seen - kPixChunk + (int)threadIdx.x;
-                if ((int)threadIdx.x < kPixChunk && p < p1) {
-                    float2 sum = gacc[0][kGrid ? threadIdx.x : 0];
-#pragma unroll
-                    for (int w = 1; w < kThreads / 64; ++w) {
-                        sum.x += gacc[kGrid ? w : 0][kGrid ? threadIdx.x : 0].x;
-                        sum.y += gacc[kGrid ? w : 0][kGrid ? threadIdx.x : 0].y;
-                    }
-                    a.grid_part[((size_t)b * gridDim.x + blockIdx.x) * a.HWp + p] = sum;
-                }
-                __syncthreads();
-            }
         }
     });
 #pragma unroll
@@ -519,6 +486,293 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
         for (int f = 0; f < 6; ++f) M[g][f] += R[g][f];
 #pragma unroll
         for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+    }
+    bwd_store<C, G>(a, b, t, n, M, CG);
+}
+
+// ---- cross-lane sums of the fused grid gradients
+// A lane of the general backward owns Gaussians, so the per-pixel sums of the grid gradients run
+// across the lanes.  Instead of one 64-lane butterfly per pixel record, the records are summed in
+// a transposed fashion: two records' values are merged into one register in which half of the
+// lanes carry the first record's pair sums and the other half the second's, so that each level of
+// the tree halves the number of live registers and a block of 64 records costs 63 merges (one per
+// record) instead of 64 x 6.  Level by level the partner lane differs in bit 5, 3, 2 (within a
+// group of 8 records), then 4, 0, 1 (over 8 groups): the lane whose bits are L5..L0 ends up with
+// the wave's complete sum of record  (L4 + 2 L0 + 4 L1) * 8 + (L5 + 2 L3 + 4 L2)  of the block.
+// The order of the additions is fixed by the lane numbers, so results are reproducible.
+__device__ __forceinline__ float xl_merge32(float a, float b) {
+    // v_permlane32_swap: lanes 32..63 of the first register <-> lanes 0..31 of the second
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xl_merge16(float a, float b) {
+    // v_permlane16_swap: the odd rows (of 16 lanes) of the first <-> the even rows of the second
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+template <int kCtrl, int kBanks>
+__device__ __forceinline__ float xl_dpp(float old, float src) {  // lanes outside kBanks keep `old`
+    return __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(old), __float_as_uint(src), kCtrl, 0xf,
+                                                       kBanks, false));
+}
+__device__ __forceinline__ float xl_merge8(float a, float b) {
+    // row_ror:8 = partner lane ^ 8; banks 0,1 (bit 3 clear) take a, banks 2,3 take b
+    return xl_dpp<0x128, 0x3>(b, a) + xl_dpp<0x128, 0xc>(a, b);
+}
+__device__ __forceinline__ float xl_merge4(float a, float b) {
+    // banks 0,2 (bit 2 clear) read lane + 4 (row_shl:4) of a, banks 1,3 read lane - 4 (row_shr:4) of b
+    return xl_dpp<0x104, 0x5>(b, a) + xl_dpp<0x114, 0xa>(a, b);
+}
+template <int kQuadPerm>
+__device__ __forceinline__ float xl_merge_quad(float a, float b, bool second) {
+    const float keep = second ? b : a, send = second ? a : b;
+    return keep + __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(send), kQuadPerm, 0xf, 0xf, true));
+}
+
+// General grid with the gradients w.r.t. the grids fused in:
+// d L / d x(pixel) = -sum_n G_n w_n (A dx + B dy), same with (B dx + D dy) for y.  With
+// t1 = A'dx + (B2'/2) dy, t2 = (B2'/2) dx + D'dy the exponent is dx t1 + dy t2, and a lane adds
+// alpha G e (t1, t2) of its G Gaussians per pixel record; the 64 lanes are summed by the
+// transposed tree above, the four waves through LDS in wave order once per chunk, and the
+// workgroups of the other Gaussians by k_grid_reduce, which also applies the factor -1/k of
+// t1 = k (A dx + B dy).
+#ifndef IGS_GRID_WAVES
+#define IGS_GRID_WAVES 3
+#endif
+template <int C, int G>
+__global__ __launch_bounds__(kThreads, C <= 8 ? IGS_GRID_WAVES : 2) void k_bwd_gen_grid(const BwdArgs a) {
+    constexpr int CP = pix_stride_gen(C), CP4 = CP / 4;
+    constexpr int CH = pix_chunk(C);
+    constexpr int E = CH * CP4, PRE = (E + kThreads - 1) / kThreads;
+    constexpr int kWaves = kThreads / 64;
+    static_assert(CH % 64 == 0 && CH <= kThreads, "a chunk is whole 64-record blocks, one thread per record at the flush");
+    __shared__ float4 sh[2 * E];
+    __shared__ float2 wsum[2][kWaves][CH];  // per chunk parity, wave, record: the wave's grid sums
+    IGS_GATE(a);
+    const int b = blockIdx.z, t = blockIdx.y;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    int n[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) n[g] = (blockIdx.x * G + g) * kThreads + tid;
+    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
+    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+    float hb[G], al[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        hb[g] = 0.5f * B2[g];
+        // unused lane slots (n >= N) must add nothing
+        al[g] = n[g] < a.N ? a.packed[((size_t)b * a.Np + n[g]) * rec_stride_of(C) + 5] : 0.0f;
+    }
+    float M[G][6], CG[G][C], R[G][6], RC[G][C];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int f = 0; f < 6; ++f) M[g][f] = R[g][f] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) CG[g][c] = RC[g][c] = 0.0f;
+    }
+    // the record of a 64-record block whose wave sum the tree leaves in this lane
+    const int my_rec = (((lane >> 4) & 1) | ((lane & 1) << 1) | (((lane >> 1) & 1) << 2)) * 8 +
+                       (((lane >> 5) & 1) | (((lane >> 3) & 1) << 1) | (((lane >> 2) & 1) << 2));
+    const bool bit0 = lane & 1, bit1 = lane & 2;
+
+    const int p0 = t * a.per_tile, p1 = min(a.HWp, p0 + a.per_tile);
+    const int total = (p1 - p0) * CP4, chunks = (p1 - p0 + CH - 1) / CH;
+    const float4* src = reinterpret_cast<const float4*>(a.pixrec + ((size_t)b * a.HWp + p0) * CP);
+    const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float4 pre[PRE];
+    auto load_records = [&](int chunk) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int e = i * kThreads + tid, ge = chunk * E + e;
+            pre[i] = (e < E && ge < total) ? src[ge] : zero;   // records past the tile are zero: they add 0
+        }
+    };
+    load_records(0);
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int e = i * kThreads + tid;
+        if (e < E) sh[e] = pre[i];
+    }
+    __syncthreads();
+
+    // One pixel record against the lane's G Gaussians; returns this lane's grid-gradient terms.
+    // Every step runs over the G Gaussians before the next step starts, so that neighbouring
+    // instructions are independent: a wave issues a dependent fp32 op only every ~8 cycles but an
+    // independent one every ~4.5, and at three waves per SIMD that difference is not hidden.
+    auto record = [&](const float4 (&r)[CP4], float& gxl, float& gyl) {
+        float pv[CP];
+#pragma unroll
+        for (int q4 = 0; q4 < CP4; ++q4) {
+            pv[4 * q4] = r[q4].x;
+            pv[4 * q4 + 1] = r[q4].y;
+            pv[4 * q4 + 2] = r[q4].z;
+            pv[4 * q4 + 3] = r[q4].w;
+        }
+        float dx[G], dy[G], ee[G], t1[G], t2[G], u[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) dx[g] = pv[0] - px[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) dy[g] = pv[1] - py[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) t1[g] = hb[g] * dy[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) t2[g] = hb[g] * dx[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) t1[g] = fmaf(A[g], dx[g], t1[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) t2[g] = fmaf(D[g], dy[g], t2[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) u[g] = dy[g] * t2[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) ee[g] = fmaf(dx[g], t1[g], u[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) ee[g] = hw_exp2(ee[g]);
+        float Gv[G], ge[G], m1[G], m2[G], gw[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) Gv[g] = fmaf(pv[2], col[g][0], pv[2 + C]);  // <g^, c> - s
+#pragma unroll
+        for (int c = 1; c < C; ++c)
+#pragma unroll
+            for (int g = 0; g < G; ++g) Gv[g] = fmaf(pv[2 + c], col[g][c], Gv[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) ge[g] = Gv[g] * ee[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) m1[g] = ge[g] * dx[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) m2[g] = ge[g] * dy[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) gw[g] = ge[g] * al[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][0] += ge[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][1] += m1[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][2] += m2[g];
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][3] = fmaf(m1[g], dx[g], R[g][3]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][4] = fmaf(m1[g], dy[g], R[g][4]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) R[g][5] = fmaf(m2[g], dy[g], R[g][5]);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int g = 0; g < G; ++g) RC[g][c] = fmaf(ee[g], pv[2 + c], RC[g][c]);
+        // the lane's grid terms: two chains each (even / odd Gaussians), joined at the end
+        float gx0 = gw[0] * t1[0], gy0 = gw[0] * t2[0];
+        float gx1 = G > 1 ? gw[G > 1 ? 1 : 0] * t1[G > 1 ? 1 : 0] : 0.0f, gy1 = G > 1 ? gw[G > 1 ? 1 : 0] * t2[G > 1 ? 1 : 0] : 0.0f;
+#pragma unroll
+        for (int g = 2; g < G; g += 2) {
+            gx0 = fmaf(gw[g], t1[g], gx0);
+            gy0 = fmaf(gw[g], t2[g], gy0);
+            if (g + 1 < G) {
+                gx1 = fmaf(gw[g + 1], t1[g + 1], gx1);
+                gy1 = fmaf(gw[g + 1], t2[g + 1], gy1);
+            }
+        }
+        gxl = gx0 + gx1;
+        gyl = gy0 + gy1;
+    };
+
+    for (int k = 0; k < chunks; ++k) {
+        if (k + 1 < chunks) load_records(k + 1);
+        const float4* cur = sh + (k & 1) * E;
+        float x3 = 0.0f, y3 = 0.0f, x4 = 0.0f, y4 = 0.0f, x5 = 0.0f, y5 = 0.0f;  // pending partners, tree levels 3..5
+#pragma unroll 1
+        for (int grp = 0; grp < CH / 8; ++grp) {
+            float gx[8], gy[8];
+#pragma unroll
+            for (int h = 0; h < 8; h += 2) {
+                // the LDS reads of two records are issued together, above the work
+                float4 rr[2][CP4];
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int i = 0; i < CP4; ++i) rr[u][i] = cur[(grp * 8 + h + u) * CP4 + i];
+                __builtin_amdgcn_sched_barrier(0);
+                record(rr[0], gx[h], gy[h]);
+                __builtin_amdgcn_sched_barrier(0);
+                record(rr[1], gx[h + 1], gy[h + 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // The running sums are complete here: without this the compiler sinks their updates
+            // below the branches that follow and keeps every record's terms alive until then.
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+#pragma unroll
+                for (int f = 0; f < 6; ++f) asm volatile("" : "+v"(R[g][f]));
+#pragma unroll
+                for (int c = 0; c < C; ++c) asm volatile("" : "+v"(RC[g][c]));
+            }
+            // levels 1-3: the 8 records of the group -> one register (lane bits 5, 3, 2)
+            // (x and y alternate so that neighbouring instructions are independent)
+            float ax[4], ay[4], bx[2], by[2];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                ax[i] = xl_merge32(gx[2 * i], gx[2 * i + 1]);
+                ay[i] = xl_merge32(gy[2 * i], gy[2 * i + 1]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                bx[i] = xl_merge8(ax[2 * i], ax[2 * i + 1]);
+                by[i] = xl_merge8(ay[2 * i], ay[2 * i + 1]);
+            }
+            const float fx = xl_merge4(bx[0], bx[1]);
+            const float fy = xl_merge4(by[0], by[1]);
+            // levels 4-6 over the 8 groups of a block (lane bits 4, 0, 1); the branches are wave-uniform
+            if (!(grp & 1)) {
+                x3 = fx; y3 = fy;
+            } else {
+                const float wx4 = xl_merge16(x3, fx), wy4 = xl_merge16(y3, fy);
+                if (!(grp & 2)) {
+                    x4 = wx4; y4 = wy4;
+                } else {
+                    const float wx5 = xl_merge_quad<0xb1>(x4, wx4, bit0), wy5 = xl_merge_quad<0xb1>(y4, wy4, bit0);
+                    if (!(grp & 4)) {
+                        x5 = wx5; y5 = wy5;
+                    } else {
+                        const float wx6 = xl_merge_quad<0x4e>(x5, wx5, bit1), wy6 = xl_merge_quad<0x4e>(y5, wy5, bit1);
+                        wsum[k & 1][wave][(grp >> 3) * 64 + my_rec] = make_float2(wx6, wy6);
+                    }
+                }
+            }
+        }
+        // two-level summation of the per-Gaussian sums
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int f = 0; f < 6; ++f) {
+                M[g][f] += R[g][f];
+                R[g][f] = 0.0f;
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                CG[g][c] += RC[g][c];
+                RC[g][c] = 0.0f;
+            }
+        }
+        if (k + 1 < chunks) {
+            float4* nxt = sh + ((k + 1) & 1) * E;
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int e = i * kThreads + tid;
+                if (e < E) nxt[e] = pre[i];
+            }
+        }
+        __syncthreads();
+        // the chunk's grid sums are complete in all waves: add them in wave order.  wsum[k & 1] is
+        // written again in chunk k + 2, behind the barrier that ends chunk k + 1.
+        const int p = p0 + k * CH + tid;
+        if (tid < CH && p < p1) {
+            float2 sum = wsum[k & 1][0][tid];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) {
+                sum.x += wsum[k & 1][w][tid].x;
+                sum.y += wsum[k & 1][w][tid].y;
+            }
+            a.grid_part[((size_t)b * gridDim.x + blockIdx.x) * a.HWp + p] = sum;
+        }
     }
     bwd_store<C, G>(a, b, t, n, M, CG);
 }

@@ -28,7 +28,10 @@ __host__ __device__ constexpr int fwd_sep_p(int C) { return C <= 3 ? IGS_FWD_SEP
 // pixels per lane, general forward
 __host__ __device__ constexpr int fwd_gen_p(int C) { return C <= 4 ? 8 : 4; }
 // Gaussians per lane, general backward (more independent chains per pixel record)
-__host__ __device__ constexpr int bwd_gen_g(int C) { return C <= 4 ? 4 : 2; }
+#ifndef IGS_BWD_GEN_G
+#define IGS_BWD_GEN_G 4
+#endif
+__host__ __device__ constexpr int bwd_gen_g(int C) { return C <= 4 ? IGS_BWD_GEN_G : 2; }
 constexpr int kBwdG = IGS_BWD_G;  // Gaussians per lane, backward
 
 __host__ __device__ constexpr int rec_stride_of(int C) { return (6 + C + 3) & ~3; }

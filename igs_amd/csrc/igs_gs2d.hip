@@ -403,9 +403,9 @@ int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     } else {
         const dim3 grid(bwd_gen_groups(a.N, C), a.T, B);
         if (a.grid_part != nullptr)
-            hipLaunchKernelGGL((k_bwd_gen<C, bwd_gen_g(C), true>), grid, dim3(kThreads), 0, st, a);
+            hipLaunchKernelGGL((k_bwd_gen_grid<C, bwd_gen_g(C)>), grid, dim3(kThreads), 0, st, a);
         else
-            hipLaunchKernelGGL((k_bwd_gen<C, bwd_gen_g(C), false>), grid, dim3(kThreads), 0, st, a);
+            hipLaunchKernelGGL((k_bwd_gen<C, bwd_gen_g(C)>), grid, dim3(kThreads), 0, st, a);
     }
     return launch_status();
 }
