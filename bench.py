@@ -27,6 +27,25 @@ sys.path.insert(0, ROOT)
 FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) peak
 
 
+# Per-launch counter readings of the two hot kernels at c1, taken from the committed rocprofv3 summary
+# (profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md): wave-level instruction counts and HBM KiB.
+# executed FLOPs = (2 FMA + MUL + ADD + TRANS) x 64 lanes; HBM bytes = FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
+# (factors from the plain-copy calibration of the same profile run).
+C1_PROFILE = {
+    "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
+    "bwd": {"fma": 1.321e9, "mul": 2.47e8, "add": 1.33e8, "trans": 1.196e8, "fetch_kib": 48242, "write_kib": 141887},
+    "fwd": {"fma": 7.38e8, "mul": 2.3e7, "add": 1.31e8, "trans": 1.230e8, "fetch_kib": 9920, "write_kib": 139170},
+}
+
+
+def executed_flops(k):
+    return (2 * k["fma"] + k["mul"] + k["add"] + k["trans"]) * 64
+
+
+def hbm_bytes(k):
+    return (k["fetch_kib"] * 2.0 + k["write_kib"] * 1.0) * 1024
+
+
 def flops_per_pair(C: int):
     """Algorithmic FLOPs per Gaussian-pixel pair (FMA = 2, exp = 1)."""
     return 12 + 2 * C, 30 + 4 * C
@@ -39,6 +58,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--cpu-full", action="store_true",
+                    help="time the CPU baseline on the whole batch of the configuration (c1: about two minutes on 16 "
+                         "threads) instead of the bounded sample")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the JSON line, print the operator-level table of the reference's "
                          "scripts/profiling.py (B x N x H sweep, median of 32 timed calls after 4 warm-ups)")
@@ -101,6 +123,20 @@ def main() -> int:
         out.backward(d["grad_out"])
         for v in leaves.values():
             v.grad = None
+
+    # ---- the timed path must be the correct one: image 0 of its output against the fp64 oracle
+    with torch.no_grad():
+        chk = forward()[:1].double()
+    g64 = {k: d[k][:1].double() for k in names + ("x_grid", "y_grid")}
+    ca, cb, cd = O.cov_inverse_closed(g64["scales"], g64["rotations"])
+    ref, _ = O.forward_strips(g64["x_grid"], g64["y_grid"], g64["positions"], ca, cb, cd, g64["alphas"], g64["colors"],
+                              rows=8)
+    err = (chk - ref).abs()
+    if not bool((err <= 1e-6 + 1e-5 * ref.abs()).all()):
+        print(f"bench.py: output differs from the oracle (max err {float(err.max()):.3e}); not timing a wrong result",
+              file=sys.stderr)
+        return 1
+    del chk, ref, err, g64
 
     if args.copy_calibration:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
@@ -171,7 +207,18 @@ def main() -> int:
     t_bwd_kernel = event_time(reduce_kernel, args.steps)
     t_fwd_kernel = event_time(fwd_kernel, args.steps)
     f_fwd, f_bwd = flops_per_pair(C)
-    achieved = pairs * f_bwd / t_bwd_kernel / 1e12
+
+    # Pairs the backward kernel evaluated: its per-tile Gaussian lists (behind the pixel records in the
+    # workspace; written by the k_bin launch inside the bracket) times the pixels of each tile.  Pairs
+    # that are not listed are exact zeros and are skipped.
+    plan = op.plan
+    scratch = (B * H * plan.w_padded * plan.pix_stride + B * plan.w_padded) * 4
+    counts = pix.view(torch.int32)[(scratch + 15) // 16 * 4:][: B * plan.bwd_tiles].view(B, -1, plan.bwd_tiles_x).cpu()
+    rows = torch.tensor([min(H, (i + 1) * plan.bwd_per_tile) - i * plan.bwd_per_tile for i in range(counts.shape[1])])
+    cols = torch.tensor([min(W, (i + 1) * 64) - i * 64 for i in range(plan.bwd_tiles_x)])
+    evaluated = int((counts.long() * (rows[:, None] * cols[None, :])[None]).sum())
+    achieved = evaluated * f_bwd / t_bwd_kernel / 1e12
+    prof = C1_PROFILE if (args.config == "c1" and C == 3) else None
 
     result = {
         "metric": "gaussian_pixel_evals_per_sec_fwd_bwd",
@@ -194,27 +241,39 @@ def main() -> int:
         "step_frac_of_fp32_vector_peak": pairs * (f_fwd + f_bwd) / t_step / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
         "roofline": {
             "bound": "valu",
-            "kernel": "k_bwd_sep<3,2> (backward per-Gaussian reduction)" if C == 3 else f"k_bwd_sep<{C},2>",
+            "kernel": f"k_bwd_sep<{C},2> (backward per-Gaussian reduction)",
             "achieved": achieved,
             "peak": FP32_VECTOR_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / FP32_VECTOR_PEAK_TFLOPS,
             "flops_per_pair": f_bwd,
             "pairs_per_launch": pairs,
+            "pairs_evaluated_per_launch": evaluated,
+            "frac_counting_all_pairs": pairs * f_bwd / t_bwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
             "launch_ms": t_bwd_kernel * 1e3,
-            "traffic": (94.2 + 138.6) * 1024 * 1024 if args.config == "c1" and C == 3 else None,
+            "executed_frac": executed_flops(prof["bwd"]) / t_bwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS if prof else None,
+            "traffic": hbm_bytes(prof["bwd"]) if prof else None,
             "forward_kernel": {"launch_ms": t_fwd_kernel * 1e3, "flops_per_pair": f_fwd,
                                "achieved": pairs * f_fwd / t_fwd_kernel / 1e12,
-                               "frac": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS},
-            "traffic_note": "HBM bytes per launch from rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (copy-calibrated), "
-                            "from the committed rocprofv3 counter summary; valid for the c1 workload only",
-            "note": "launch_ms brackets igs_gs2d_backward_reduce = k_bin (tile lists, ~33 us) + k_bwd_sep; peak = published fp32 vector peak; the kernels use plain (non-packed) fp32 VALU ops with "
-                    "VGPR-only operands, v_exp_f32 counted as 1 FLOP",
+                               "frac": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+                               "executed_frac": executed_flops(prof["fwd"]) / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS
+                               if prof else None,
+                               "traffic": hbm_bytes(prof["fwd"]) if prof else None},
+            "counter_source": prof["source"] if prof else None,
+            "note": "achieved / frac: the 30+4C FLOP model of one backward pair x the pairs the kernel evaluated (the tile "
+                    "lists skip pairs whose weight is exactly 0; frac_counting_all_pairs uses all B N H W as the metric "
+                    "does) / launch_ms, measured live with HIP events around igs_gs2d_backward_reduce = k_bin (~33 us) + "
+                    "k_bwd_sep.  executed_frac: the arithmetic the hardware ran, (2 FMA + MUL + ADD + TRANS) x 64 per "
+                    "launch from the rocprofv3 counters of counter_source (separable grids hoist the row/column part of "
+                    "the model's operations, so it is below frac) / the live launch_ms.  traffic: HBM bytes per launch "
+                    "from FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of the same summary (copy-calibrated); c1 only.  peak: "
+                    "published fp32 vector peak at 2.4 GHz; the kernels use plain fp32 VALU ops with VGPR-only operands, "
+                    "v_exp_f32 counted as 1 FLOP.",
         },
     }
 
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(args.config, O)
+        result["cpu_baseline"] = cpu_baseline(args.config, O, full=args.cpu_full)
     print(json.dumps(result), flush=True)
     return 0
 
@@ -406,17 +465,39 @@ def sweep(only: str = None) -> int:
     return 0
 
 
-def cpu_baseline(config: str, O):
+def host_cpu():
+    """(model name, physical cores) of the host, from /proc/cpuinfo."""
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "model name":
+                model = v
+            elif k == "physical id":
+                phys = v
+            elif k == "core id":
+                core = v
+            elif not k and phys is not None:
+                cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    return model, len(cores) or (os.cpu_count() or 0)
+
+
+def cpu_baseline(config: str, O, full: bool = False):
     """Chunked torch autograd path on the host cores, on a bounded sample of the same workload
-    (a few images of it; cost is linear in the number of images)."""
+    (a few images of it; cost is linear in the number of images) or, with `full`, on all of it."""
     import torch
 
     from oracle.chunked_cpu import render_chunked_cpu
 
     threads = torch.get_num_threads()
-    full = O.CONFIGS[config]
-    nb = {"c0": 1, "c1": 4, "c2": 1, "c4": 1}[config]
-    N = full["N"] // 8 if config == "c4" else full["N"]
+    cfg = O.CONFIGS[config]
+    nb = cfg["B"] if full else {"c0": 1, "c1": 4, "c2": 1, "c4": 1}[config]
+    N = cfg["N"] // 8 if (config == "c4" and not full) else cfg["N"]
     d = O.make_config_inputs(config, B=nb, N=N)
     B, N, C = d["colors"].shape
     H, W = d["x_grid"].shape[-2:]
@@ -439,9 +520,12 @@ def cpu_baseline(config: str, O):
     run()
     t = time.perf_counter() - t0
     pairs = B * N * H * W
+    model, physical = host_cpu()
+    what = "the whole batch" if (B == cfg["B"] and N == cfg["N"]) else "a bounded sample"
     return {"value": pairs / t, "unit": "pairs/s", "cores": threads, "kind": "port",
-            "sample": f"{B} image(s) of {config} (B={B}, N={N}, {H}x{W}, C={C}), fwd+bwd once, {t:.1f} s, "
-                      f"eager torch fp32 with {threads} threads"}
+            "cpu_model": model, "physical_cores": physical,
+            "sample": f"{what}: {B} image(s) of {config} (B={B}, N={N}, {H}x{W}, C={C}), fwd+bwd once, {t:.1f} s, "
+                      f"eager torch fp32 with {threads} threads on {model} ({physical} physical cores visible)"}
 
 
 if __name__ == "__main__":
