@@ -104,6 +104,7 @@ SIGNATURES = {
     "igs_gs2d_backward_prologue_mse": (c_int, [_FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int,
                                                c_int, c_int, c_int, c_float, _FP, c_size_t, _FP, c_size_t, _FP,
                                                c_void_p]),
+    "igs_gs2d_position_penalty": (c_int, [_FP, c_int64, c_int, c_float, c_int64, _FP, _FP, c_void_p]),
     "igs_adamw_step": (c_int, [_FP, _FP, _FP, _FP, c_int64, _FP, c_float, c_float, c_float, c_float, c_void_p]),
     "igs_koleo_plan": (c_int, [c_int, c_int, c_int, POINTER(KoleoPlan)]),
     "igs_koleo_forward": (c_int, [_FP, c_int, c_int, c_int, _FP, _FP, c_size_t, _FP, c_size_t, c_void_p]),

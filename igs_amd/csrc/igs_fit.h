@@ -36,3 +36,36 @@ __global__ __launch_bounds__(kThreads) void k_adamw(float* __restrict__ param,
     exp_avg[i] = m;
     exp_avg_sq[i] = v;
 }
+
+// ----------------------------------------------------------------------------- position penalty
+// Regulariser of the fit loop (scripts/2dgs_img_comp.py:224-228): weight * mean(relu(|p| - 1)) over
+// the position columns (the first two floats of every row of `rows` x `stride` floats).  Every
+// thread adds the gradient weight * sign(p) [|p| > 1] / count of its row to g_feature; workgroup 0
+// also sums the penalty over all rows in a fixed order and adds it to loss[0].
+__global__ __launch_bounds__(kThreads) void k_position_penalty(const float* __restrict__ feature, long rows,
+                                                               int stride, float weight, float inv_count,
+                                                               float* __restrict__ g_feature,
+                                                               float* __restrict__ loss) {
+    const long r = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (r < rows) {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const float p = feature[r * stride + k];
+            if (fabsf(p) > 1.0f) g_feature[r * stride + k] += copysignf(weight * inv_count, p);
+        }
+    }
+    if (blockIdx.x != 0 || loss == nullptr) return;  // workgroup-uniform
+    __shared__ float red[kThreads];
+    float s = 0.0f;
+    for (long i = threadIdx.x; i < rows; i += kThreads) {
+        s += fmaxf(fabsf(feature[i * stride]) - 1.0f, 0.0f);
+        s += fmaxf(fabsf(feature[i * stride + 1]) - 1.0f, 0.0f);
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int k = kThreads / 2; k > 0; k >>= 1) {
+        if ((int)threadIdx.x < k) red[threadIdx.x] += red[threadIdx.x + k];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) loss[0] += weight * inv_count * red[0];
+}

@@ -716,6 +716,16 @@ int igs_gs2d_backward_prologue_mse(const float* x, const float* y, const int64_t
                              C, eps, pix_ws, pix_bytes, stream);
 }
 
+int igs_gs2d_position_penalty(const float* gs_feature, int64_t rows, int row_floats, float weight,
+                              int64_t count, float* g_feature, float* loss, igs_stream_t stream) {
+    if (!gs_feature || !g_feature) return IGS_ERR_NULL_POINTER;
+    if (rows < 1 || rows > (int64_t)kThreads * 0x7fffffff || row_floats < 2 || count < 1) return IGS_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(k_position_penalty, dim3((unsigned)((rows + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                       (hipStream_t)stream, gs_feature, (long)rows, row_floats, weight, (float)(1.0 / (double)count),
+                       g_feature, loss);
+    return launch_status();
+}
+
 int igs_adamw_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int64_t count,
                    float* state, float beta1, float beta2, float eps, float weight_decay,
                    igs_stream_t stream) {

@@ -15,6 +15,13 @@ No torch op and no allocation happens inside a step, so it can be captured in a 
 (`capture()`), which removes the host launch cost from small problems; the step counter and the
 learning rate live in device memory so that replays advance.
 
+Two things of the script's loop beyond the mean-squared error are covered as well: its position
+regulariser `0.01 * mean(relu(|position| - 1))` (scripts/2dgs_img_comp.py:224-228;
+`position_penalty=`) is added to the gradient and the loss inside the step, and any other image
+loss -- the script mixes SSIM-type terms, :133-142 -- can be supplied as `step(loss_fn=...)`: the
+image goes to `loss_fn` as a torch leaf, torch differentiates the loss down to the image, and the
+splat backward, the chain rule and AdamW run fused from that upstream gradient.
+
 The parameters are one block `[B, N, 6+C]` in the layout of the module's `gs_feature`
 (src/igs/gs2d.py:638-644): position (2), log-scale (2), rotation (1), an unused column,
 colours (C) -- the same parameterisation as the fit script's `ProgressiveGaussianSplatter`
@@ -45,11 +52,14 @@ class GaussianImageFit:
     lr, betas, adam_eps, weight_decay  AdamW hyper-parameters (defaults: those of
              scripts/2dgs_img_comp.py:186-193 with lr for 4096 Gaussians).
     eps      the splat's eps (covariance regulariser and denominator guard).
+    position_penalty  weight of `mean(relu(|position| - 1))` in the loss (the script uses 0.01; the
+             mean runs over the positions of all B*N Gaussians, also in a prefix step, which moves
+             only the active ones).
     """
 
     def __init__(self, params: Tensor, target: Tensor, x_grid: Tensor, y_grid: Tensor, lr: float = 0.03,
                  betas: Tuple[float, float] = (0.9, 0.995), adam_eps: float = 1e-6, weight_decay: float = 1e-4,
-                 eps: float = 1e-6):
+                 eps: float = 1e-6, position_penalty: float = 0.0):
         if params.device.type != "cuda":
             raise RuntimeError("GaussianImageFit runs on the GPU only (HIP kernels)")
         if params.dim() != 3 or params.shape[-1] < 7:
@@ -63,6 +73,7 @@ class GaussianImageFit:
         self.eps = float(eps)
         self.betas = (float(betas[0]), float(betas[1]))
         self.adam_eps, self.weight_decay = float(adam_eps), float(weight_decay)
+        self.position_penalty = float(position_penalty)
         with torch.cuda.device(self.device):
             self.exp_avg = torch.zeros_like(self.params)
             self.exp_avg_sq = torch.zeros_like(self.params)
@@ -145,18 +156,23 @@ class GaussianImageFit:
                                         H, W, Cp, self.eps, _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]),
                                         int(p.fwd_ws_bytes), st), "igs_gs2d_forward")
 
-    def _enqueue_step(self, n: int):
-        lib, g = self.lib, self.grid
-        ws = self._workspace(n)
-        p = ws["plan"]
+    def _enqueue_backward(self, n: int, ws: dict, st, grad_out: Optional[Tensor]):
+        """Everything after the render: per-pixel prologue (from `grad_out` [B,Cp,H,W], or with the
+        mean-squared-error gradient and loss formed in place when it is None), per-Gaussian
+        reduction, chain rule, position penalty, AdamW."""
+        lib, g, p = self.lib, self.grid, ws["plan"]
         B, C, Cp, H, W = self.B, self.C, self.Cp, g.H, g.W
-        st = _stream(self.device)
-        self._enqueue_render(n, ws, st)
-        _lib.check(lib.igs_gs2d_backward_prologue_mse(_ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag),
-                                                      _ptr(ws["out"]), _ptr(ws["den"]), _ptr(self.target), C, B, n, H,
-                                                      W, Cp, self.eps, _ptr(ws["pix"]), int(p.pix_bytes),
-                                                      _ptr(ws["loss_ws"]), ws["loss_bytes"], _ptr(self.loss), st),
-                   "igs_gs2d_backward_prologue_mse")
+        if grad_out is None:
+            _lib.check(lib.igs_gs2d_backward_prologue_mse(_ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag),
+                                                          _ptr(ws["out"]), _ptr(ws["den"]), _ptr(self.target), C, B, n,
+                                                          H, W, Cp, self.eps, _ptr(ws["pix"]), int(p.pix_bytes),
+                                                          _ptr(ws["loss_ws"]), ws["loss_bytes"], _ptr(self.loss), st),
+                       "igs_gs2d_backward_prologue_mse")
+        else:
+            _lib.check(lib.igs_gs2d_backward_prologue(_ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag),
+                                                      _ptr(ws["out"]), _ptr(ws["den"]), _ptr(grad_out), B, n, H, W, Cp,
+                                                      self.eps, _ptr(ws["pix"]), int(p.pix_bytes), st),
+                       "igs_gs2d_backward_prologue")
         _lib.check(lib.igs_gs2d_backward_reduce(_ptr(ws["packed"]), _ptr(ws["col"]), _ptr(g.y), g.strides, g.mode,
                                                 _ptr(g.flag), B, n, H, W, Cp, _ptr(ws["pix"]), int(p.pix_bytes),
                                                 _ptr(ws["partial"]), int(p.partial_bytes), st),
@@ -164,17 +180,52 @@ class GaussianImageFit:
         _lib.check(lib.igs_gs2d_finalize_feature(_ptr(ws["partial"]), g.mode, _ptr(g.flag), _ptr(self.params), B, n, H,
                                                  W, C, Cp, self.eps, _ptr(ws["g_feat"]), st),
                    "igs_gs2d_finalize_feature")
+        if self.position_penalty != 0.0:
+            _lib.check(lib.igs_gs2d_position_penalty(_ptr(self.params), B * n, 6 + C, self.position_penalty,
+                                                     2 * B * self.N, _ptr(ws["g_feat"]), _ptr(self.loss), st),
+                       "igs_gs2d_position_penalty")
         # B == 1 or n == N: the active prefix is the first B*n*(6+C) floats of every block
         _lib.check(lib.igs_adamw_step(_ptr(self.params), _ptr(ws["g_feat"]), _ptr(self.exp_avg), _ptr(self.exp_avg_sq),
                                       B * n * (6 + C), _ptr(self.state), self.betas[0], self.betas[1], self.adam_eps,
                                       self.weight_decay, st), "igs_adamw_step")
 
-    def step(self, num_active: Optional[int] = None) -> Tensor:
+    def _enqueue_step(self, n: int):
+        ws = self._workspace(n)
+        st = _stream(self.device)
+        self._enqueue_render(n, ws, st)
+        self._enqueue_backward(n, ws, st, None)
+
+    def _step_with_loss_fn(self, n: int, loss_fn):
+        ws = self._workspace(n)
+        st = _stream(self.device)
+        self._enqueue_render(n, ws, st)
+        image = ws["out"][:, :self.C].detach().requires_grad_(True)       # a view: no copy
+        with torch.enable_grad():
+            loss = loss_fn(image)
+            if loss.dim() != 0:
+                raise ValueError("loss_fn must return a scalar tensor")
+            (g,) = torch.autograd.grad(loss, image)
+        g = g.to(torch.float32)
+        if self.Cp != self.C:
+            g = F.pad(g, (0, 0, 0, 0, 0, self.Cp - self.C))
+        self.loss.copy_(loss.detach())
+        self._enqueue_backward(n, ws, st, g.contiguous())
+
+    def step(self, num_active: Optional[int] = None, loss_fn=None) -> Tensor:
         """One iteration on the first `num_active` Gaussians (default all; the progressive
         schedule of scripts/2dgs_img_comp.py:107-111).  Returns the loss of the image rendered
         *before* the update as a 0-dim device tensor that the next step overwrites; nothing
-        synchronises.  Replays the captured graph when `capture()` was called for this count."""
+        synchronises.  Replays the captured graph when `capture()` was called for this count.
+
+        With `loss_fn` (image [B,C,H,W] -> scalar tensor, differentiable torch code; the target is
+        the caller's business) that loss replaces the mean-squared error: torch differentiates it
+        down to the image and the fused backward starts from that gradient.  Such a step is not
+        replayed from a graph (the loss runs in torch)."""
         n = self._active(num_active)
+        if loss_fn is not None:
+            with torch.cuda.device(self.device):
+                self._step_with_loss_fn(n, loss_fn)
+            return self.loss
         graph = self._graphs.get(n)
         if graph is not None:
             graph.replay()

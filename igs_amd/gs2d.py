@@ -245,10 +245,14 @@ def _cov_inverse_torch(scales, rotations, eps):
 
 @functools.lru_cache(maxsize=32)
 def _grid_vectors(h: int, w: int, device):
+    """The two coordinate vectors of xy_grid, kept per (size, device) for the module's forward.
+    Built outside inference mode so that a first call under torch.inference_mode() does not leave
+    inference tensors behind for later training calls."""
     aspect_ratio = h / w
     h_range = aspect_ratio ** 0.5
     w_range = 1 / aspect_ratio ** 0.5
-    return torch.linspace(-w_range, w_range, w).to(device), torch.linspace(-h_range, h_range, h).to(device)
+    with torch.inference_mode(False):
+        return torch.linspace(-w_range, w_range, w).to(device), torch.linspace(-h_range, h_range, h).to(device)
 
 
 class GaussianSplatting2D(nn.Module):
@@ -277,8 +281,17 @@ class GaussianSplatting2D(nn.Module):
     @staticmethod
     def xy_grid(size=None, device=None):
         """x in +-sqrt(w/h), y in +-sqrt(h/w) as stride-0 expanded [1,h,w] tensors
-        (src/igs/gs2d.py:503-522).  The two coordinate vectors are built once per (size, device)
-        and kept: the reference rebuilds them on the host and copies them over in every forward."""
+        (src/igs/gs2d.py:503-522).  Like the reference, every call returns tensors of its own (the
+        caller may write into what they view); the module's forward uses vectors kept per
+        (size, device) instead, see `_shared_xy_grid`."""
+        h, w = size
+        xs, ys = _grid_vectors(int(h), int(w), None if device is None else torch.device(device))
+        return xs.clone().view(1, 1, w).expand(1, h, w), ys.clone().view(1, h, 1).expand(1, h, w)
+
+    @staticmethod
+    def _shared_xy_grid(size, device):
+        """xy_grid without the copy: read-only views of the kept coordinate vectors (the reference
+        rebuilds them on the host and copies them over in every forward)."""
         h, w = size
         xs, ys = _grid_vectors(int(h), int(w), None if device is None else torch.device(device))
         return xs.view(1, 1, w).expand(1, h, w), ys.view(1, h, 1).expand(1, h, w)
@@ -306,7 +319,7 @@ class GaussianSplatting2D(nn.Module):
         b = gs_feature.shape[0]
 
         if grid is None:
-            x_grid, y_grid = self.xy_grid(size, feature.device)
+            x_grid, y_grid = self._shared_xy_grid(size, feature.device)
             # kept expanded (stride 0) instead of the reference's .repeat: same values, and
             # the kernels then take the separable-grid path
             x_grid = x_grid[None].expand(b, 1, -1, -1)

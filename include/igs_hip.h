@@ -283,6 +283,16 @@ int igs_gs2d_backward_prologue_mse(const float *x, const float *y, const int64_t
                                    float *loss_ws, size_t loss_ws_bytes, float *loss,
                                    igs_stream_t stream);
 
+/* Position regulariser of the fit loop, scripts/2dgs_img_comp.py:224-228:
+ * position_penalty = mean(relu(|position| - 1)), added to the loss with a weight (0.01 there).
+ * gs_feature is `rows` rows of `row_floats` floats whose first two are the position; `count` is
+ * the number of position elements the mean runs over (2 x the number of all Gaussians of the
+ * model, also when only a prefix of them is passed).  Adds weight * sign(p) [|p| > 1] / count to
+ * the position columns of g_feature (same layout; call after igs_gs2d_finalize_feature, before
+ * igs_adamw_step) and, when loss is not NULL, weight * mean to loss[0] (device; fixed-order sum). */
+int igs_gs2d_position_penalty(const float *gs_feature, int64_t rows, int row_floats, float weight,
+                              int64_t count, float *g_feature, float *loss, igs_stream_t stream);
+
 /* One torch.optim.AdamW step (amsgrad off; the optimiser of scripts/2dgs_img_comp.py:186-193)
  * over a flat block of `count` floats, in place:
  *   p *= 1 - lr wd;  m += (g - m)(1 - beta1);  v = beta2 v + (1 - beta2) g^2;

@@ -213,3 +213,106 @@ def test_fused_step_under_two_level_binning(igs, dev):
     torch.testing.assert_close(res["1"][1], res["2"][1], rtol=1e-4, atol=1e-5)
     for a, b in zip(res["1"][0], res["2"][0]):
         assert a == pytest.approx(b, rel=1e-5)
+
+
+def _oracle_loss_and_grad(block, target, xg, yg, penalty=0.0, loss_fn=None):
+    """fp64 truth of one iteration's loss and d loss / d block: the naive expression of the oracle
+    under autograd (no HIP code on this side), the script's activations exp(log_scale) + eps and
+    alpha = 1 (src/igs/gs2d.py:673-675), F.mse_loss (or `loss_fn`) and the position regulariser of
+    scripts/2dgs_img_comp.py:224-228."""
+    C = block.shape[-1] - 6
+    p = block.detach().double().cpu().requires_grad_(True)
+    pos, ls, rot, _, col = p.split([2, 2, 1, 1, C], dim=-1)
+    img = O.render_naive(pos, col, torch.exp(ls) + 1e-6, rot[..., 0], torch.ones_like(rot[..., 0]),
+                         xg.double().cpu(), yg.double().cpu(), 1e-6)
+    t = target.double().cpu()
+    loss = F.mse_loss(img, t) if loss_fn is None else loss_fn(img, t)
+    if penalty:
+        loss = loss + penalty * torch.mean(F.relu(pos.abs() - 1.0))
+    (g,) = torch.autograd.grad(loss, p)
+    return float(loss.detach()), g
+
+
+@pytest.mark.parametrize("penalty", [0.0, 0.01], ids=["mse", "mse+position-penalty"])
+def test_first_fused_step_against_the_fp64_oracle(igs, dev, penalty):
+    """Step-0 loss, d block and the updated parameters against the fp64 oracle and AdamW's closed
+    form for the first step, p1 = p0 (1 - lr wd) - lr g / (|g| + eps): no HIP render on the
+    reference side."""
+    from igs_amd.fit import GaussianImageFit
+
+    B, N, H, W, C = 2, 300, 40, 56, 3
+    block = make_block(B, N, C, 11, dev)
+    block[..., 0:2] *= 1.3                                  # some positions beyond +-1: the penalty is active
+    xg, yg = grids(igs, B, H, W, dev)
+    target = torch.rand(B, C, H, W, generator=torch.Generator().manual_seed(12)).to(dev)
+    lr, wd, aeps = 0.02, HYPER["weight_decay"], HYPER["eps"]
+    ref_loss, g64 = _oracle_loss_and_grad(block, target, xg, yg, penalty)
+    fit = GaussianImageFit(block.clone(), target, xg, yg, lr=lr, adam_eps=aeps, betas=HYPER["betas"], weight_decay=wd,
+                           position_penalty=penalty)
+    loss0 = float(fit.step())
+    assert loss0 == pytest.approx(ref_loss, rel=1e-5)
+    g = fit._ws[N]["g_feat"].double().cpu()
+    for name, sl in (("position", slice(0, 2)), ("log_scale", slice(2, 4)), ("rotation", slice(4, 5)),
+                     ("color", slice(6, 6 + C))):
+        d, r = g[..., sl] - g64[..., sl], g64[..., sl]
+        assert float(d.abs().max()) <= 1e-4 * float(r.abs().max()), name
+        assert float(d.norm()) <= 1e-4 * float(r.norm()), name
+    assert float(g[..., 5].abs().max()) == 0.0 and float(g64[..., 5].abs().max()) == 0.0    # the unused column
+    if penalty:   # the regulariser's own part: weight * sign(p) / (2 B N) where |p| > 1
+        outside = block[..., 0:2].abs().cpu() > 1.0
+        assert int(outside.sum()) > 20
+    p0 = block.double().cpu()
+    p1 = p0 * (1 - lr * wd) - lr * g64 / (g64.abs() + aeps)
+    # where |g| is not far above AdamW's eps the update depends on g to first order: compare there
+    # only up to the gradient's own tolerance
+    big = g64.abs() > 1e-3 * g64.abs().max()
+    err = (fit.params.double().cpu() - p1).abs()
+    assert float(err[big].max()) <= 2e-6 + 1e-6 * float(p1.abs().max())
+    assert float(err.max()) <= lr * 1.01                     # every update is bounded by lr
+
+
+def test_step_with_an_external_image_loss(igs, dev):
+    """`step(loss_fn=...)`: torch differentiates the caller's loss down to the image, the fused
+    backward takes that gradient.  Checked against the fp64 oracle for the first step and against
+    the torch iteration over four steps; with F.mse_loss as `loss_fn` it equals the built-in
+    mean-squared-error step to rounding."""
+    from igs_amd.fit import GaussianImageFit
+
+    B, N, H, W, C = 1, 260, 36, 52, 3
+    block = make_block(B, N, C, 21, dev)
+    xg, yg = grids(igs, B, H, W, dev)
+    target = O.smooth_noise_target(H, W, seed=22, C=C).to(dev)
+    mixed = lambda img, t: F.l1_loss(img, t) + 0.25 * F.mse_loss(img, t) + 0.1 * (img[..., 1:] - img[..., :-1]).abs().mean()
+    lr = 0.02
+    ref_loss, g64 = _oracle_loss_and_grad(block, target, xg, yg, loss_fn=mixed)
+    fit = GaussianImageFit(block.clone(), target, xg, yg, lr=lr, adam_eps=HYPER["eps"], betas=HYPER["betas"],
+                           weight_decay=HYPER["weight_decay"])
+    loss0 = float(fit.step(loss_fn=lambda img: mixed(img, target)))
+    assert loss0 == pytest.approx(ref_loss, rel=1e-5)
+    g = fit._ws[N]["g_feat"].double().cpu()
+    assert float((g - g64).abs().max()) <= 1e-4 * float(g64.abs().max())
+    assert float((g - g64).norm()) <= 1e-4 * float(g64.norm())
+    # four steps against the torch iteration with the same loss
+    p = block.clone().requires_grad_(True)
+    opt = torch.optim.AdamW([p], lr=lr, **HYPER)
+    fit2 = GaussianImageFit(block.clone(), target, xg, yg, lr=lr, adam_eps=HYPER["eps"], betas=HYPER["betas"],
+                            weight_decay=HYPER["weight_decay"])
+    for _ in range(4):
+        pos, ls, rot, _, col = p.split([2, 2, 1, 1, C], dim=-1)
+        img = igs.gaussian_splatting_2d(pos, col, torch.exp(ls) + 1e-6, rot[..., 0], torch.ones_like(rot[..., 0]), xg, yg)
+        loss = mixed(img, target)
+        loss.backward()
+        opt.step()
+        opt.zero_grad()
+        l2 = fit2.step(loss_fn=lambda im: mixed(im, target))
+        assert float(l2) == pytest.approx(float(loss), rel=1e-5)
+    # |d l1 / d image| is a constant 1/n: gradients of many parameters sit near AdamW's eps, where the
+    # update amplifies rounding; bound by a small multiple of lr there
+    close(fit2.params, p.detach(), "parameters after 4 steps with an external loss", rtol=1e-4, atol=2e-4)
+    # F.mse_loss as the external loss == the built-in step
+    fa = GaussianImageFit(block.clone(), target, xg, yg, lr=lr)
+    fb = GaussianImageFit(block.clone(), target, xg, yg, lr=lr)
+    for _ in range(3):
+        la, lb = fa.step(), fb.step(loss_fn=lambda im: F.mse_loss(im, target))
+        assert float(la) == pytest.approx(float(lb), rel=1e-6)
+    close(fa.params, fb.params, "mse as external loss", rtol=1e-5, atol=1e-6)

@@ -30,12 +30,22 @@ def igs():
     return igs_amd
 
 
+# how often a bound wider than the stated one was needed: (tag, elements beyond the strict bound,
+# elements, worst excess) -- printed by test_zzz_report_loosened_tolerances at the end of this file
+LOOSENED = []
+
+
 def assert_fwd(out, ref, tag="", atol=1e-6):
     ref = ref.to(out.device)
     err = (out.double() - ref).abs()
     tol = atol + 1e-5 * ref.abs()
     bad = err > tol
     assert not bad.any(), f"{tag}: {int(bad.sum())} of {bad.numel()} outside tol, max err {float(err.max()):.3e}"
+    if atol > 1e-6:  # a scaled absolute part was allowed: record what the strict bound would have refused
+        strict = err > 1e-6 + 1e-5 * ref.abs()
+        if strict.any():
+            LOOSENED.append((f"fwd {tag}", int(strict.sum()), strict.numel(),
+                             float((err - (1e-6 + 1e-5 * ref.abs())).max())))
 
 
 def assert_grad(g, ref, name, tag="", rtol=1e-4, atol=0.0):
@@ -45,6 +55,9 @@ def assert_grad(g, ref, name, tag="", rtol=1e-4, atol=0.0):
     l2 = float(ref.norm())
     assert float(d.abs().max()) <= rtol * mx + atol + 1e-30, f"{tag} {name}: max err {float(d.abs().max()):.3e} vs max ref {mx:.3e}"
     assert float(d.norm()) <= rtol * l2 + atol * math.sqrt(d.numel()) + 1e-30, f"{tag} {name}: l2 err {float(d.norm()):.3e} vs {l2:.3e}"
+    if atol > 0.0 and (float(d.abs().max()) > rtol * mx or float(d.norm()) > rtol * l2):
+        LOOSENED.append((f"grad {name} {tag}", int((d.abs() > rtol * mx).sum()), d.numel(),
+                         float(d.abs().max()) - rtol * mx))
 
 
 def small_case(B, N, H, W, C, seed, smin=0.05, smax=0.5, general=False):
@@ -419,3 +432,15 @@ def test_grid_gradients_fused_into_the_general_backward(igs, dev, C):
         res.append((xx.grad, yy.grad, lv["scales"].grad))
     for a, b in zip(*res):
         assert torch.equal(a, b)
+
+
+def test_zzz_report_loosened_tolerances():
+    """Runs last in this file: where a test above allowed more than the stated bounds (absolute part of
+    the forward bound scaled by the colour magnitude for signed colours; an absolute 1e-6 on gradients
+    of problems with at most five Gaussians), says how many elements needed it and by how much."""
+    if not LOOSENED:
+        print("no element needed a loosened tolerance")
+    for tag, n, total, excess in LOOSENED:
+        print(f"loosened tolerance used: {tag}: {n} of {total} elements beyond the strict bound, worst by {excess:.2e}")
+    total = sum(n for _, n, _, _ in LOOSENED)
+    assert total <= 200, f"{total} elements needed the loosened bounds; that is no longer a corner case"
