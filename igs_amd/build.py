@@ -22,6 +22,9 @@ HIPCC_FLAGS = [
     "-fPIC",
     "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix-core results land in ordinary VGPRs (the vector ALU reads them without a copy out of
+    # the accumulation registers); only the diversity-loss kernel uses the matrix cores
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-I", os.path.join(ROOT, "include"),
 ]
 

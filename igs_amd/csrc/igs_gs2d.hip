@@ -1058,20 +1058,32 @@ int koleo_plan(int B, int N, int D, igs_koleo_plan_t* p) {
     const int Dp = (D + 3) & ~3;
     if ((long)B * N > (1L << 28) || (long)B * N * Dp > (1L << 31)) return IGS_ERR_BAD_SHAPE;
     const int cus = device_cus() > 0 ? device_cus() : 256;
-    // similarity tiles of 128x64, unless one column tile per workgroup would leave most of the
-    // device idle (then 64x64, then 32x32); after that enough workgroups for two per compute
-    // unit, by splitting the columns
-    const long t128 = ceil_div(N, 128), t64 = ceil_div(N, 64);
-    // (128 rows pay only where the row tile is re-read from LDS at every step, Dp > kKoleoRegK)
-    const int tile_rows = (Dp > kKoleoRegK && t128 * t64 * B >= 2L * cus) ? 128
-                          : (t64 * t64 * B >= 2L * cus ? 64 : 32);
-    const int tile = tile_rows == 32 ? 32 : 64;
-    const int tiles = ceil_div(N, tile);
-    const int row_tiles = ceil_div(N, tile_rows);
-    int S = ceil_div(2L * cus, (long)row_tiles * B);
-    S = S < 1 ? 1 : (S > tiles ? tiles : S);
-    const int per = ceil_div(tiles, S);
-    S = ceil_div(tiles, per);
+    int tile_rows, tile, S, per;
+    if (Dp <= kKoleoMfmaMaxD) {
+        // matrix-core kernel: a workgroup owns 128 query rows (32 per wave) and streams candidate tiles
+        // of 32 rows; the candidates are split until there are four workgroups per compute unit
+        tile_rows = 128;
+        tile = 32;
+        const int tiles = ceil_div(N, tile);
+        S = ceil_div((long)IGS_KOLEO_WGS_PER_CU * cus, (long)ceil_div(N, tile_rows) * B);
+        S = S < 1 ? 1 : (S > tiles ? tiles : S);
+        per = ceil_div(tiles, S);
+        S = ceil_div(tiles, per);
+    } else {
+        // similarity tiles of 128x64, unless one column tile per workgroup would leave most of the
+        // device idle (then 64x64, then 32x32); after that enough workgroups for two per compute
+        // unit, by splitting the columns
+        const long t128 = ceil_div(N, 128), t64 = ceil_div(N, 64);
+        // (128 rows pay only where the row tile is re-read from LDS at every step, Dp > kKoleoRegK)
+        tile_rows = (Dp > kKoleoRegK && t128 * t64 * B >= 2L * cus) ? 128 : (t64 * t64 * B >= 2L * cus ? 64 : 32);
+        tile = tile_rows == 32 ? 32 : 64;
+        const int tiles = ceil_div(N, tile);
+        const int row_tiles = ceil_div(N, tile_rows);
+        S = ceil_div(2L * cus, (long)row_tiles * B);
+        S = S < 1 ? 1 : (S > tiles ? tiles : S);
+        per = ceil_div(tiles, S);
+        S = ceil_div(tiles, per);
+    }
     const long rows = (long)B * N;
     p->B = B;
     p->N = N;
@@ -1118,6 +1130,9 @@ int igs_koleo_forward(const float* features, int B, int N, int D, float* loss, v
     hipLaunchKernelGGL(k_koleo_normalize, dim3(ceil_div(rows, kThreads / 64)), dim3(kThreads), 0, st,
                        features, rows, D, p.d_padded, sv.fn, sv.norm);
     const dim3 nn_grid(ceil_div(N, p.tile_rows), p.splits, B);
+#define IGS_KOLEO_MFMA(KH)                                                                             \
+    hipLaunchKernelGGL((k_koleo_nn_mfma<KH>), nn_grid, dim3(kThreads), 0, st, (const float*)sv.fn, N,   \
+                       p.d_padded, p.tiles_per_split, part_val, part_idx)
 #define IGS_KOLEO_NN(MR, MC, KN)                                                                       \
     hipLaunchKernelGGL((k_koleo_nn<MR, MC, KN>), nn_grid, dim3(kThreads), 0, st, (const float*)sv.fn, N, \
                        p.d_padded, p.tiles_per_split, part_val, part_idx)
@@ -1127,6 +1142,17 @@ int igs_koleo_forward(const float* features, int B, int N, int D, float* loss, v
         else if (p.tile_rows == 64) IGS_KOLEO_NN(4, 4, KN);          \
         else IGS_KOLEO_NN(2, 2, KN);                                 \
     } while (0)
+    if (p.d_padded <= kKoleoMfmaMaxD) {  // MFMAs per candidate tile: half the (padded) row length, rounded up
+        const int kh = p.d_padded / 2;
+        if (kh <= 2) IGS_KOLEO_MFMA(2);
+        else if (kh <= 4) IGS_KOLEO_MFMA(4);
+        else if (kh <= 6) IGS_KOLEO_MFMA(6);
+        else if (kh <= 8) IGS_KOLEO_MFMA(8);
+        else if (kh <= 12) IGS_KOLEO_MFMA(12);
+        else if (kh <= 16) IGS_KOLEO_MFMA(16);
+        else if (kh <= 24) IGS_KOLEO_MFMA(24);
+        else IGS_KOLEO_MFMA(32);
+    } else
     switch (p.d_padded <= kKoleoRegK ? p.d_padded : 0) {
         case 4: IGS_KOLEO_NN_K(4); break;
         case 8: IGS_KOLEO_NN_K(8); break;
@@ -1134,6 +1160,7 @@ int igs_koleo_forward(const float* features, int B, int N, int D, float* loss, v
         case 16: IGS_KOLEO_NN_K(16); break;
         default: IGS_KOLEO_NN_K(0); break;
     }
+#undef IGS_KOLEO_MFMA
 #undef IGS_KOLEO_NN_K
 #undef IGS_KOLEO_NN
     hipLaunchKernelGGL(k_koleo_combine, dim3(blocks), dim3(kThreads), 0, st, (const float*)part_val,

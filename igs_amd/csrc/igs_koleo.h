@@ -3,14 +3,20 @@
 // that the reference materialises.  Included by igs_gs2d.hip inside its anonymous namespace.
 //
 //   k_koleo_normalize : fn = x / max(||x||, 1e-12), rows zero-padded to a multiple of 4 floats
-//   k_koleo_nn        : register-tiled fn fn^T (128x64, 64x64 or 32x32 per workgroup, K through LDS),
-//                       reduced on the fly to (max, argmax) per row and column split
+//   k_koleo_nn_mfma   : fn fn^T on the matrix cores (fp32 MFMA), reduced on the fly to (max, argmax) per
+//                       row and column split; for rows of up to 64 (padded) dimensions
+//   k_koleo_nn        : the same with register-tiled vector FMAs (128x64, 64x64 or 32x32 per workgroup,
+//                       K through LDS); any row length
 //   k_koleo_combine   : splits -> nearest neighbour per row, relu(. + 1), per-workgroup sums
 //   k_koleo_sum       : fixed-order sum of those -> loss
 //   k_koleo_bwd       : d x_i from the neighbour of row i and from the rows whose neighbour is i
 // No atomics: equal similarities resolve to the lowest column index, every sum has a fixed order.
 #pragma once
 
+#ifndef IGS_KOLEO_WGS_PER_CU
+#define IGS_KOLEO_WGS_PER_CU 4
+#endif
+constexpr int kKoleoMfmaMaxD = 64;    // up to this many (padded) dimensions the similarities run on the matrix cores
 constexpr int kKoleoRegK = 16;        // up to this many (padded) dimensions the row tile stays in registers
 constexpr float kKoleoNormEps = 1e-12f;   // torch.nn.functional.normalize's default (src/igs/reg.py:22)
 constexpr int kKoleoBwdMaxRows = 64;  // rows per wave in the backward, at most
@@ -252,6 +258,175 @@ __global__ __launch_bounds__(kThreads) void k_koleo_nn(const float* __restrict__
             part_val[((size_t)b * S + s) * N + grow] = best[r];
             part_idx[((size_t)b * S + s) * N + grow] = bidx[r];
         }
+    }
+}
+
+// ---- the same search on the matrix cores, for Dp <= 64
+// fp32 MFMA (v_mfma_f32_32x32x2_f32) forms the similarities; the vector ALU only keeps the running
+// maximum.  A wave owns 32 query rows (the B operand, in registers for the whole kernel) and
+// streams candidate rows in tiles of 32 (the A operand, from a double-buffered LDS window that the
+// workgroup's four waves share): after KH = Dp/2 accumulating MFMAs lane l holds, for query
+// q0 + l % 32, the similarities to the 16 candidates  c0 + 8 (r/4) + 4 (l/32) + r % 4,  r = 0..15.
+// The feature index of MFMA step t is  (l/32) KH + t  for both operands (any pairing of the k
+// index works as long as both agree), so a lane reads one contiguous run of KH floats per row.
+// On this hardware a SIMD does not run vector instructions while its matrix core works, so every
+// vector instruction per tile is paid in matrix time: the common case (a whole window of tiles
+// with nothing to mask) is unrolled with immediate LDS offsets and costs 8 v_max3 and one compare
+// per tile; the tiles that need masking -- the last one (candidates >= N) and the one that holds
+// the wave's own queries -- take a plain loop.  Same outputs and tie rule as k_koleo_nn (lowest
+// candidate index; the two half-waves of a query are merged with koleo_better at the end).
+typedef float koleo_v16f __attribute__((ext_vector_type(16)));
+
+__host__ __device__ constexpr int koleo_mfma_ld(int KH) { return ((2 * KH / 4) & 1) ? 2 * KH : 2 * KH + 4; }  // LD/4 odd
+__host__ __device__ constexpr int koleo_mfma_rows(int KH) { return KH <= 6 ? 256 : (KH <= 16 ? 128 : 64); }
+
+template <int KH>
+__global__ __launch_bounds__(kThreads, 3) void k_koleo_nn_mfma(const float* __restrict__ fn, int N, int Dp,
+                                                            int tiles_per_split, float* __restrict__ part_val,
+                                                            int* __restrict__ part_idx) {
+    constexpr int LD = koleo_mfma_ld(KH), CR = koleo_mfma_rows(KH), TPC = CR / 32;
+    __shared__ __align__(16) float cs[2][CR * LD];
+    const int b = blockIdx.z, s = blockIdx.y, S = gridDim.y;
+    const int tid = threadIdx.x, lane = tid & 63, j = lane & 31, h = lane >> 5;
+    const int q0 = blockIdx.x * 128 + __builtin_amdgcn_readfirstlane(tid >> 6) * 32;  // the wave's first query
+    const int q = q0 + j;                                                              // this lane's query
+    const float* img = fn + (size_t)b * N * Dp;
+    const float ninf = -__builtin_inff();
+    // columns of the window beyond Dp stay zero
+    for (int i = tid; i < 2 * CR * LD; i += kThreads) (&cs[0][0])[i] = 0.0f;
+    float bq[KH];
+#pragma unroll
+    for (int t = 0; t < KH; ++t) bq[t] = (q < N && h * KH + t < Dp) ? img[(size_t)q * Dp + h * KH + t] : 0.0f;
+    // The query values are used here, before the loop: their loads are then known to be complete,
+    // and the MFMAs inside the loop do not wait for the memory counter, which would also make them
+    // wait for the prefetch of the next window issued just before them.
+#pragma unroll
+    for (int t = 0; t < KH; ++t) asm volatile("" : "+v"(bq[t]));
+    const int ntiles = (N + 31) / 32;
+    const int t0 = s * tiles_per_split, t1 = min(ntiles, t0 + tiles_per_split);
+    const int row_begin = t0 * 32, row_end = min(N, t1 * 32);
+    const int nchunks = (t1 - t0 + TPC - 1) / TPC;
+    const int d4 = Dp / 4;                                   // float4 per row in memory
+    // Staging slots of this thread: float4 number e = i kThreads + tid of a window is columns
+    // 4 c4 .. 4 c4 + 3 of row r = e / d4.  The split into (r, c4) is done once, here: a division per
+    // slot and window would cost more vector time than the window's MFMAs leave room for.
+    constexpr int PRE = (CR * (2 * KH / 4) + kThreads - 1) / kThreads;
+    float4 pre[PRE];
+    int srow[PRE], scol[PRE], slds[PRE];   // row in the window (CR: no slot), first column, offset in LDS
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int e = i * kThreads + tid, r = e / d4, c4 = e - r * d4;
+        srow[i] = e < CR * d4 ? r : CR;
+        scol[i] = 4 * c4;
+        slds[i] = r * LD + 4 * c4;
+    }
+    // (the load is unconditional, from a clamped row, and the value is selected afterwards: a load
+    // behind a select of addresses would go through a flat access and a scratch copy)
+    auto gload = [&](int chunk) __attribute__((always_inline)) {
+        const int r0 = row_begin + chunk * CR;
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int r = r0 + srow[i];
+            const float4 v = *reinterpret_cast<const float4*>(img + (size_t)min(r, N - 1) * Dp + scol[i]);
+            const bool ok = srow[i] < CR && r < row_end;   // (component-wise: selecting whole float4 objects
+            pre[i].x = ok ? v.x : 0.0f;                      //  makes the compiler select between their addresses)
+            pre[i].y = ok ? v.y : 0.0f;
+            pre[i].z = ok ? v.z : 0.0f;
+            pre[i].w = ok ? v.w : 0.0f;
+        }
+    };
+    auto lstore = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i)
+            if (srow[i] < CR) *reinterpret_cast<float4*>(&cs[buf][slds[i]]) = pre[i];
+    };
+    __syncthreads();  // the zero fill is complete
+    if (nchunks > 0) {
+        gload(0);
+        lstore(0);
+    }
+    __syncthreads();
+    float best = ninf;
+    int bidx = -1;
+    // similarities of the tile whose row for this lane starts at `row`: KH accumulating MFMAs
+    auto tile_mfma = [&](const float* row) __attribute__((always_inline)) {
+        float a[KH];
+        if (KH % 4 == 0) {
+#pragma unroll
+            for (int t = 0; t < KH; t += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(row + t);
+                a[t] = v.x; a[t + 1] = v.y; a[t + 2] = v.z; a[t + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < KH; t += 2) {
+                const float2 v = *reinterpret_cast<const float2*>(row + t);
+                a[t] = v.x; a[t + 1] = v.y;
+            }
+        }
+        koleo_v16f acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < KH; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], bq[t], acc, 0, 0, 0);
+        return acc;
+    };
+    // fold a finished tile (candidates c0 .. c0 + 31) into the lane's running maximum
+    auto tile_max = [&](const koleo_v16f& acc, int c0) __attribute__((always_inline)) {
+        float m = acc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) m = fmaxf(m, acc[r]);
+        // A lane's maximum improves ever more rarely as the scan goes on (about 1/t at tile t), so
+        // the search for its position sits behind a branch that the whole wave takes together.
+        if (__builtin_amdgcn_ballot_w64(m > best) != 0ull) {
+            if (m > best) {  // candidates come in increasing order: the first maximum stays
+                int ri = 15;
+#pragma unroll
+                for (int r = 14; r >= 0; --r) ri = acc[r] == m ? r : ri;
+                best = m;
+                bidx = c0 + 8 * (ri >> 2) + 4 * h + (ri & 3);
+            }
+        }
+    };
+    for (int k = 0; k < nchunks; ++k) {
+        if (k + 1 < nchunks) gload(k + 1);
+        const int c_first = row_begin + k * CR;
+        const int tiles = min(TPC, t1 - t0 - k * TPC);
+        const float* row0 = cs[k & 1] + j * LD + h * KH;      // this lane's row of the window's first tile
+        // scalar: a whole window, all candidates < N, and the wave's own queries are not in it
+        if (tiles == TPC && c_first + CR <= N && (q0 < c_first || q0 >= c_first + CR)) {
+#pragma unroll
+            for (int t = 0; t < TPC; t += 2) {
+                const koleo_v16f a0 = tile_mfma(row0 + t * 32 * LD);
+                const koleo_v16f a1 = tile_mfma(row0 + (t + 1) * 32 * LD);
+                tile_max(a0, c_first + t * 32);
+                tile_max(a1, c_first + (t + 1) * 32);
+            }
+        } else {
+            for (int t = 0; t < tiles; ++t) {
+                const int c0 = c_first + t * 32;
+                koleo_v16f acc = tile_mfma(row0 + t * 32 * LD);
+                if (c0 + 32 > N || c0 == q0) {  // scalar
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int cand = c0 + 8 * (r >> 2) + 4 * h + (r & 3);
+                        if (cand >= N || cand == q) acc[r] = ninf;
+                    }
+                }
+                tile_max(acc, c0);
+            }
+        }
+        if (k + 1 < nchunks) lstore((k + 1) & 1);
+        __syncthreads();
+    }
+    // the two half-waves hold disjoint candidates of the same query
+    const float ov = __shfl_xor(best, 32);
+    const int oi = __shfl_xor(bidx, 32);
+    if (koleo_better(ov, oi, best, bidx)) {
+        best = ov;
+        bidx = oi;
+    }
+    if (h == 0 && q < N) {
+        part_val[((size_t)b * S + s) * N + q] = best;
+        part_idx[((size_t)b * S + s) * N + q] = bidx;
     }
 }
 

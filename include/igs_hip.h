@@ -314,8 +314,8 @@ int igs_adamw_step(float *param, const float *grad, float *exp_avg, float *exp_a
 typedef struct igs_koleo_plan_t {
     int32_t B, N, D;
     int32_t d_padded;        /* floats per normalised row (D rounded up to 4)                 */
-    int32_t tile_rows;       /* rows of a similarity tile: 128, 64 or 32 (by problem size)    */
-    int32_t tile;            /* columns of a similarity tile: 64 or 32                         */
+    int32_t tile_rows;       /* rows a workgroup searches for: 128, 64 or 32 (by problem size) */
+    int32_t tile;            /* candidate rows per similarity tile: 64 or 32                   */
     int32_t splits;          /* column splits of the similarity tiles (>= 1)                  */
     int32_t tiles_per_split; /* column tiles per split                                         */
     int32_t bwd_rows;        /* rows per wave of the backward                                  */
