@@ -282,7 +282,9 @@ def all_configs(steps: int, warmup: int) -> int:
     """Forward and forward+backward wall time of the five configurations through the public API
     (allocation included), pairs/s counting all B N H W pairs as scripts/profiling.py:199-211 does,
     and the fraction of the fp32 vector peak by the 42 + 6 C FLOP/pair model (above 1 is possible
-    where culling skips pairs)."""
+    where culling skips pairs).  The "fit step" rows are the graph-replayed fused iteration of
+    igs_amd.fit on the same problem: at c0 the public call is bound by the host's per-call cost
+    (Python, torch allocation, autograd: 0.13-0.25 ms depending on the box), the replay is not."""
     import torch
 
     import igs_amd
@@ -347,13 +349,14 @@ def all_configs(steps: int, warmup: int) -> int:
                     v.grad = None
         n = max(3, steps // 3) if cfg == "c4" else steps
         rows.append((cfg, B, N, H, W, C, timeit(fwd, n), timeit(step, n)))
-        if cfg == "c2":   # the fused fit iteration (render, MSE, backward, AdamW) on the same problem
+        if cfg in ("c0", "c2"):   # the fused fit iteration (render, MSE, backward, AdamW) on the same problem,
+            # replayed from a HIP graph: the step without the host's per-call cost
             block = torch.cat([d["positions"], d["scales"].log(), d["rotations"][..., None],
                                torch.zeros_like(d["rotations"])[..., None], d["colors"]], -1)
             fit = GaussianImageFit(block, O.smooth_noise_target(H, W, seed=1002).to(dev), d["x_grid"], d["y_grid"],
                                    lr=min(0.05 * 4096 / N, 0.03))
             fit.capture()
-            rows.append(("c2 fit step", B, N, H, W, C, float("nan"), timeit(fit.step, n)))
+            rows.append((cfg + " fit step", B, N, H, W, C, float("nan"), timeit(fit.step, n)))
     print("%-12s %3s %6s %4s %4s %3s %10s %12s %14s %10s" % ("config", "B", "N", "H", "W", "C", "fwd ms", "fwd+bwd ms",
                                                            "pairs/s", "of peak"))
     for cfg, B, N, H, W, C, tf, t in rows:
