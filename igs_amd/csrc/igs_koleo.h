@@ -445,13 +445,23 @@ __global__ __launch_bounds__(kThreads) void k_koleo_combine(const float* __restr
         const int b = (int)(row / N), n = (int)(row - (long)b * N);
         float v = -__builtin_inff();
         int idx = -1;
-        for (int s = 0; s < S; ++s) {
-            const float ov = part_val[((size_t)b * S + s) * N + n];
-            const int oi = part_idx[((size_t)b * S + s) * N + n];
-            if (koleo_better(ov, oi, v, idx)) {
-                v = ov;
-                idx = oi;
+        // eight splits' loads in flight at a time (the comparisons are a short dependent chain,
+        // the loads are what takes the time when few workgroups run)
+        for (int s0 = 0; s0 < S; s0 += 8) {
+            float ov[8];
+            int oi[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int s = min(s0 + k, S - 1);
+                ov[k] = part_val[((size_t)b * S + s) * N + n];
+                oi[k] = part_idx[((size_t)b * S + s) * N + n];
             }
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (s0 + k < S && koleo_better(ov[k], oi[k], v, idx)) {
+                    v = ov[k];
+                    idx = oi[k];
+                }
         }
         if (norm[row] != norm[row]) v = norm[row];  // non-finite row: NaN, which the sum below spreads
         const float t = v + 1.0f;
