@@ -67,6 +67,9 @@ def main() -> int:
     ap.add_argument("--sweep-shape", default=None, metavar="BxNxH",
                     help="with --sweep: this one shape only, forward+backward with all eight gradients (for profiling "
                          "the general-grid kernels)")
+    ap.add_argument("--sweep-no-grid-grads", action="store_true",
+                    help="with --sweep: the two coordinate grids do not require gradients (six gradients instead of "
+                         "the eight of the reference's protocol)")
     ap.add_argument("--all", action="store_true",
                     help="instead of the JSON line, print forward and forward+backward times of all five "
                          "configurations (c0-c4; c3 is the module, c2 also as the fused fit step)")
@@ -96,7 +99,7 @@ def main() -> int:
             return 1
         return subprocess.run([exe]).returncode
     if args.sweep:
-        return sweep(args.sweep_shape)
+        return sweep(args.sweep_shape, not args.sweep_no_grid_grads)
     if args.all:
         return all_configs(args.steps, args.warmup)
     if args.koleo:
@@ -438,7 +441,7 @@ def koleo_table(no_cpu: bool, only: str = None) -> int:
     return 0
 
 
-def sweep(only: str = None) -> int:
+def sweep(only: str = None, grid_grads: bool = True) -> int:
     """Operator-level sweep in the protocol of the reference's scripts/profiling.py:30-49, :69-151, :199-211:
     `.apply(x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors)` on randn/rand inputs (per-pixel
     random coordinates, so the general-grid kernels run), 4 warm-ups, 32 timed calls with events, median;
@@ -459,7 +462,8 @@ def sweep(only: str = None) -> int:
         for mode in ("fwd", "fwd_bwd"):
             rg = mode == "fwd_bwd"
             mk = lambda *sh, fn=torch.randn: fn(*sh, device=dev).requires_grad_(rg)
-            inputs = (mk(B, 1, H, W), mk(B, 1, H, W), mk(B, N, 2), mk(B, N, 1, 1), mk(B, N, 1, 1), mk(B, N, 1, 1),
+            mkg = (lambda *sh: mk(*sh)) if grid_grads else (lambda *sh: torch.randn(*sh, device=dev))
+            inputs = (mkg(B, 1, H, W), mkg(B, 1, H, W), mk(B, N, 2), mk(B, N, 1, 1), mk(B, N, 1, 1), mk(B, N, 1, 1),
                       mk(B, N, fn=torch.rand), mk(B, N, 3, fn=torch.rand))
 
             def call():
