@@ -13,6 +13,7 @@
 //              zero every KH steps (a tile loop), and the same with the 16 results consumed by
 //              v_max_f32 (what a nearest-neighbour search does per tile)
 //   section 4  matrix-core and vector instructions sharing a SIMD
+//   section 5  v_fmac_f32 with its three operands in distinct / shared register banks
 //
 // Build: hipcc -O3 --offload-arch=gfx950 -Xclang -target-feature -Xclang -packed-fp32-ops issue_rates.hip
 #include <hip/hip_runtime.h>
@@ -236,6 +237,104 @@ void run_mix(int waves, float* out, const float* in, long long* clk) {
                 waves, t.ms, t.mhz, t.ms * 1e-3 * t.mhz * 1e6 / n);
 }
 
+
+// ----------------------------------------------------------------------------- section 5
+// Register banks.  The accumulation phase of the separable forward is 64 x `v_fmac_f32 acc, e, coef`
+// per record: 16 weights e (each used four times in a row), 4 coefficients, 64 accumulators.  A VGPR's
+// bank is its index mod 4.  The same 64 instructions with three register assignments (all below v120,
+// so four waves fit a SIMD): no two operands of an instruction in one bank; the two sources (e, coef) of
+// every instruction in one bank; and the assignment the compiler chose for k_fwd_sep<3,16> (its
+// registers renumbered, banks kept: 16 instructions with both sources in one bank, 26 more with the
+// accumulator in the bank of a source).
+#define FM(acc, e, c) "v_fmac_f32 v" #acc ", v" #e ", v" #c "\n"
+#define BANKS_FREE \
+    FM(5, 3, 0) FM(6, 3, 1) FM(8, 3, 2) FM(9, 3, 4) \
+    FM(10, 7, 0) FM(12, 7, 1) FM(13, 7, 2) FM(14, 7, 4) \
+    FM(17, 11, 0) FM(16, 11, 1) FM(20, 11, 2) FM(18, 11, 4) \
+    FM(21, 15, 0) FM(22, 15, 1) FM(24, 15, 2) FM(25, 15, 4) \
+    FM(26, 19, 0) FM(28, 19, 1) FM(29, 19, 2) FM(30, 19, 4) \
+    FM(33, 23, 0) FM(32, 23, 1) FM(36, 23, 2) FM(34, 23, 4) \
+    FM(37, 27, 0) FM(38, 27, 1) FM(40, 27, 2) FM(41, 27, 4) \
+    FM(42, 31, 0) FM(44, 31, 1) FM(45, 31, 2) FM(46, 31, 4) \
+    FM(49, 35, 0) FM(48, 35, 1) FM(52, 35, 2) FM(50, 35, 4) \
+    FM(53, 39, 0) FM(54, 39, 1) FM(56, 39, 2) FM(57, 39, 4) \
+    FM(58, 43, 0) FM(60, 43, 1) FM(61, 43, 2) FM(62, 43, 4) \
+    FM(65, 47, 0) FM(64, 47, 1) FM(68, 47, 2) FM(66, 47, 4) \
+    FM(69, 51, 0) FM(70, 51, 1) FM(72, 51, 2) FM(73, 51, 4) \
+    FM(74, 55, 0) FM(76, 55, 1) FM(77, 55, 2) FM(78, 55, 4) \
+    FM(81, 59, 0) FM(80, 59, 1) FM(84, 59, 2) FM(82, 59, 4) \
+    FM(85, 63, 0) FM(86, 63, 1) FM(88, 63, 2) FM(89, 63, 4)
+#define BANKS_SOURCES_COLLIDE \
+    FM(0, 3, 67) FM(1, 3, 71) FM(2, 3, 75) FM(4, 3, 79) \
+    FM(5, 7, 67) FM(6, 7, 71) FM(8, 7, 75) FM(9, 7, 79) \
+    FM(10, 11, 67) FM(12, 11, 71) FM(13, 11, 75) FM(14, 11, 79) \
+    FM(16, 15, 67) FM(17, 15, 71) FM(18, 15, 75) FM(20, 15, 79) \
+    FM(21, 19, 67) FM(22, 19, 71) FM(24, 19, 75) FM(25, 19, 79) \
+    FM(26, 23, 67) FM(28, 23, 71) FM(29, 23, 75) FM(30, 23, 79) \
+    FM(32, 27, 67) FM(33, 27, 71) FM(34, 27, 75) FM(36, 27, 79) \
+    FM(37, 31, 67) FM(38, 31, 71) FM(40, 31, 75) FM(41, 31, 79) \
+    FM(42, 35, 67) FM(44, 35, 71) FM(45, 35, 75) FM(46, 35, 79) \
+    FM(48, 39, 67) FM(49, 39, 71) FM(50, 39, 75) FM(52, 39, 79) \
+    FM(53, 43, 67) FM(54, 43, 71) FM(56, 43, 75) FM(57, 43, 79) \
+    FM(58, 47, 67) FM(60, 47, 71) FM(61, 47, 75) FM(62, 47, 79) \
+    FM(64, 51, 67) FM(65, 51, 71) FM(66, 51, 75) FM(68, 51, 79) \
+    FM(69, 55, 67) FM(70, 55, 71) FM(72, 55, 75) FM(73, 55, 79) \
+    FM(74, 59, 67) FM(76, 59, 71) FM(77, 59, 75) FM(78, 59, 79) \
+    FM(80, 63, 67) FM(81, 63, 71) FM(82, 63, 75) FM(84, 63, 79)
+#define BANKS_COMPILER \
+    FM(2, 0, 1) FM(5, 0, 6) FM(4, 0, 3) FM(7, 0, 8) \
+    FM(10, 9, 1) FM(13, 9, 6) FM(11, 9, 3) FM(14, 9, 8) \
+    FM(12, 15, 1) FM(16, 15, 6) FM(19, 15, 3) FM(17, 15, 8) \
+    FM(23, 20, 1) FM(27, 20, 6) FM(18, 20, 3) FM(21, 20, 8) \
+    FM(22, 25, 1) FM(26, 25, 6) FM(29, 25, 3) FM(31, 25, 8) \
+    FM(33, 30, 1) FM(24, 30, 6) FM(35, 30, 3) FM(34, 30, 8) \
+    FM(37, 28, 1) FM(32, 28, 6) FM(39, 28, 3) FM(38, 28, 8) \
+    FM(41, 45, 1) FM(36, 45, 6) FM(43, 45, 3) FM(42, 45, 8) \
+    FM(49, 46, 1) FM(40, 46, 6) FM(47, 46, 3) FM(50, 46, 8) \
+    FM(53, 51, 1) FM(44, 51, 6) FM(55, 51, 3) FM(54, 51, 8) \
+    FM(57, 48, 1) FM(52, 48, 6) FM(59, 48, 3) FM(58, 48, 8) \
+    FM(61, 56, 1) FM(63, 56, 6) FM(62, 56, 3) FM(65, 56, 8) \
+    FM(67, 69, 1) FM(66, 69, 6) FM(73, 69, 3) FM(60, 69, 8) \
+    FM(70, 74, 1) FM(77, 74, 6) FM(64, 74, 3) FM(71, 74, 8) \
+    FM(81, 75, 1) FM(68, 75, 6) FM(79, 75, 3) FM(85, 75, 8) \
+    FM(72, 78, 1) FM(82, 78, 6) FM(89, 78, 3) FM(76, 78, 8)
+#define CLOBBER_V0_V119                                                                                        \
+    "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", \
+        "v17", "v18", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", \
+        "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", \
+        "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", \
+        "v62", "v63", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", \
+        "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", \
+        "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105",  \
+        "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118",  \
+        "v119"
+
+// The loop runs kIters times inside one asm statement (registers hold whatever they held: the
+// timing of v_fmac_f32 does not depend on the values).
+#define BANK_KERNEL(NAME, BODY)                                                                            \
+    __global__ __launch_bounds__(256) void NAME(float* out, long long* clk) {                              \
+        extern __shared__ float lds[];                                                                     \
+        const long long t0 = clock64(), w0 = wall_clock64();                                               \
+        asm volatile("s_mov_b32 s20, 2048\n"                                                               \
+                     "1:\n" BODY "s_sub_u32 s20, s20, 1\n"                                                 \
+                     "s_cmp_lg_u32 s20, 0\n"                                                               \
+                     "s_cbranch_scc1 1b\n" ::                                                              \
+                         : CLOBBER_V0_V119, "s20", "scc");                                                 \
+        stamp(clk, t0, w0);                                                                                \
+        out[blockIdx.x * 256 + threadIdx.x] = lds[0];                                                      \
+    }
+BANK_KERNEL(k_banks_free, BANKS_FREE)
+BANK_KERNEL(k_banks_sources, BANKS_SOURCES_COLLIDE)
+BANK_KERNEL(k_banks_compiler, BANKS_COMPILER)
+
+template <class K>
+void run_banks(K kernel, const char* name, int waves, float* out, long long* clk) {
+    const Timing t = timed(kernel, kCus * waves, lds_for(waves), clk, out);
+    const double n = (double)kIters * 64 * waves;
+    std::printf("%-44s waves/SIMD %d  %7.3f ms  clock %4.0f MHz  %5.2f cycles per v_fmac_f32 and SIMD\n", name, waves, t.ms,
+                t.mhz, t.ms * 1e-3 * t.mhz * 1e6 / n);
+}
+
 }  // namespace
 
 int main() {
@@ -289,6 +388,12 @@ int main() {
         run_mix<4>(w, out, in, clk);
         run_mix<8>(w, out, in, clk);
         run_mix<16>(w, out, in, clk);
+    }
+    std::printf("\n== 5. register banks: 64 x v_fmac_f32 acc, e, coef per step\n");
+    for (int w : {2, 3, 4}) {
+        run_banks(k_banks_free, "no two operands in one bank", w, out, clk);
+        run_banks(k_banks_compiler, "the compiler's assignment in k_fwd_sep<3,16>", w, out, clk);
+        run_banks(k_banks_sources, "both sources in one bank", w, out, clk);
     }
     CK(hipFree(out));
     CK(hipFree(in));
