@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
         }
 }
 
-// Grid gradients of the general backward with the grid sums fused in (k_bwd_gen<.., true>): adds
+// Grid gradients of the general backward with the grid sums fused in (k_bwd_gen_grid): adds
 // the `groups` workgroup partials of every pixel in order and applies the factor -1/k.
 __global__ __launch_bounds__(kThreads) void k_grid_reduce(const float2* __restrict__ part, int groups, int HW,
                                                           int HWp, float* __restrict__ gx, float* __restrict__ gy,
