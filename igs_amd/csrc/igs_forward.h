@@ -150,8 +150,10 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
         // (the compiler would otherwise sink each read next to its first use and wait for it
         // there); each record's body then only waits for its own reads, so one LDS latency is
         // exposed per group instead of per record.
+        // (the last chunk stops after its last record's group; the slots behind it hold zeros)
+        const int lim = min(CH, (count - k * CH + kStreamUnroll - 1) / kStreamUnroll * kStreamUnroll);
 #pragma unroll 1
-        for (int n = 0; n < CH; n += kStreamUnroll) {
+        for (int n = 0; n < lim; n += kStreamUnroll) {
             float4 rr[kStreamUnroll][R4];
 #pragma unroll
             for (int u = 0; u < kStreamUnroll; ++u)
