@@ -33,8 +33,8 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 # (factors from the plain-copy calibration of the same profile run).
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
-    "bwd": {"fma": 1.321e9, "mul": 2.47e8, "add": 1.33e8, "trans": 1.196e8, "fetch_kib": 48242, "write_kib": 141887},
-    "fwd": {"fma": 7.38e8, "mul": 2.3e7, "add": 1.31e8, "trans": 1.230e8, "fetch_kib": 9920, "write_kib": 139170},
+    "bwd": {"fma": 1.321e9, "mul": 2.47e8, "add": 1.33e8, "trans": 1.196e8, "fetch_kib": 48216, "write_kib": 141629},
+    "fwd": {"fma": 7.095e8, "mul": 2.22e7, "add": 1.256e8, "trans": 1.183e8, "fetch_kib": 9886, "write_kib": 139251},
 }
 
 
