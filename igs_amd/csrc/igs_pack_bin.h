@@ -244,7 +244,7 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
 
 __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     if (a.flag != nullptr && *a.flag != a.want) return;
-    __shared__ float red[4][kBinThreads];
+    __shared__ float red[4][kBinWaves];
     __shared__ int wsum[kBinWaves];
     __shared__ int seg_first[kBinMaxChunks + 1];  // second level: first candidate index of each segment
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -272,19 +272,24 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         xlo = ylo = -inf;
         xhi = yhi = inf;
     }
-    red[0][tid] = xlo;
-    red[1][tid] = -xhi;
-    red[2][tid] = ylo;
-    red[3][tid] = -yhi;
-    __syncthreads();
-    for (int k = kBinThreads / 2; k > 0; k >>= 1) {
-        if (tid < k) {
+    // minima of (xlo, -xhi, ylo, -yhi) over the workgroup: within each wave by lane exchanges, then
+    // over the 16 waves' results through LDS (fminf drops NaN, which `bad` has already handled)
+    float rv[4] = {xlo, -xhi, ylo, -yhi};
 #pragma unroll
-            for (int f = 0; f < 4; ++f) red[f][tid] = fminf(red[f][tid], red[f][tid + k]);
-        }
-        __syncthreads();
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int k = 32; k > 0; k >>= 1) rv[f] = fminf(rv[f], __shfl_xor(rv[f], k));
+    if (lane == 0)
+#pragma unroll
+        for (int f = 0; f < 4; ++f) red[f][wave] = rv[f];
+    __syncthreads();
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+        rv[f] = red[f][lane & (kBinWaves - 1)];
+#pragma unroll
+        for (int k = kBinWaves / 2; k > 0; k >>= 1) rv[f] = fminf(rv[f], __shfl_xor(rv[f], k));
     }
-    const float txlo = red[0][0], txhi = -red[1][0], tylo = red[2][0], tyhi = -red[3][0];
+    const float txlo = rv[0], txhi = -rv[1], tylo = rv[2], tyhi = -rv[3];
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     const float4* boxes = a.boxes + (size_t)b * a.Np;
