@@ -14,7 +14,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 LIB_PATH = os.environ.get("IGS_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "libigs_hip.so")
 
-ABI_VERSION = 5  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
+ABI_VERSION = 6  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1
 IGS_GRID_AUTO = 2
@@ -74,8 +74,10 @@ SIGNATURES = {
     "igs_abi_version": (c_int, []),
     "igs_status_string": (c_char_p, [c_int]),
     "igs_gs2d_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, POINTER(Plan)]),
-    "igs_gs2d_pack_covinv": (c_int, [_FP, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, _FP, c_void_p]),
-    "igs_gs2d_pack_scale_rot": (c_int, [_FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, _FP, c_void_p]),
+    "igs_gs2d_skip_weight": (c_float, [c_int, c_float, c_float]),
+    "igs_gs2d_pack_covinv": (c_int, [_FP, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, _FP, c_void_p]),
+    "igs_gs2d_pack_scale_rot": (c_int, [_FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, c_float, _FP,
+                                        c_void_p]),
     "igs_gs2d_grid_classify": (c_int, [_FP, _FP, _STRIDES, c_int, c_int, c_int, _FP, c_void_p]),
     "igs_gs2d_forward": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
                                  c_float, _FP, _FP, c_void_p, c_size_t, c_void_p]),
@@ -97,7 +99,7 @@ SIGNATURES = {
                                          _FP, _FP, _FP, _FP, _FP, _FP, c_void_p]),
     "igs_gs2d_finalize_scale_rot": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                             c_float, _FP, _FP, _FP, _FP, _FP, c_void_p]),
-    "igs_gs2d_pack_feature": (c_int, [_FP, _FP, c_int, c_int, c_int, c_int, c_float, _FP, _FP, c_void_p]),
+    "igs_gs2d_pack_feature": (c_int, [_FP, _FP, c_int, c_int, c_int, c_int, c_float, c_float, _FP, _FP, c_void_p]),
     "igs_gs2d_finalize_feature": (c_int, [_FP, c_int, _FP, _FP, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                           _FP, c_void_p]),
     "igs_gs2d_mse_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

@@ -35,23 +35,43 @@ KIND_FEATURE = 2
 # igs_option bits OR-ed into the grid_mode word of every Grid built while `library_options` is active
 _option_bits = 0
 
+# Bound on what skipping far-away (Gaussian, pixel) pairs may change in an output element, as a
+# fraction of the largest colour magnitude: the pack calls get the skip weight
+# igs_gs2d_skip_weight(N, eps, SKIP_TOLERANCE) = SKIP_TOLERANCE * eps / (2 N).  The forward is held to
+# 1e-6 + 1e-5 |ref| against the plain expression; 1e-7 leaves that budget to the fp32 rounding.
+# 0 skips exact zeros only (bit-identical to evaluating every pair).
+SKIP_TOLERANCE = 1e-7
+_skip_tolerance = SKIP_TOLERANCE
+
 
 @contextlib.contextmanager
-def library_options(no_cull: bool = False, bin_levels: Optional[int] = None):
-    """Testing aid: problems set up inside this context run with the given igs_option bits of
+def library_options(no_cull: bool = False, bin_levels: Optional[int] = None,
+                    skip_tolerance: Optional[float] = None):
+    """Problems set up inside this context run with the given igs_option bits of
     include/igs_hip.h -- `no_cull` lists every Gaussian for every pixel tile (the reference point
-    for "culling changes no bit"), `bin_levels` = 1 | 2 forces the one- or two-level construction
-    of the tile lists.  The bits travel as explicit arguments of each library call (in the
-    grid_mode word); the library itself holds no such state."""
-    global _option_bits
+    for what culling changes), `bin_levels` = 1 | 2 forces the one- or two-level construction
+    of the tile lists -- and with the given `skip_tolerance` (see SKIP_TOLERANCE; 0 = only pairs
+    whose weight is exactly zero are skipped).  The bits and the skip weight travel as explicit
+    arguments of each library call; the library itself holds no such state."""
+    global _option_bits, _skip_tolerance
     bits = _lib.IGS_OPT_NO_CULL if no_cull else 0
     if bin_levels is not None:
         bits |= {1: _lib.IGS_OPT_BIN_LEVELS_1, 2: _lib.IGS_OPT_BIN_LEVELS_2}[int(bin_levels)]
-    saved, _option_bits = _option_bits, _option_bits | bits   # nested contexts add up
+    saved = (_option_bits, _skip_tolerance)
+    _option_bits |= bits   # nested contexts add up
+    if skip_tolerance is not None:
+        if not 0.0 <= float(skip_tolerance) < 1.0:
+            raise ValueError("skip_tolerance must be in [0, 1)")
+        _skip_tolerance = float(skip_tolerance)
     try:
         yield
     finally:
-        _option_bits = saved
+        _option_bits, _skip_tolerance = saved
+
+
+def skip_weight(N: int, eps: float) -> float:
+    """The skip weight the pack calls of a problem get under the current skip tolerance."""
+    return float(_lib.load().igs_gs2d_skip_weight(int(N), float(eps), float(_skip_tolerance)))
 
 
 def _ptr(t: Optional[Tensor]):
@@ -95,9 +115,9 @@ def round_up(v, m):
 
 def packed_numel(B, N, Cp):
     """float32 elements of the packed buffer: per image roundup4(N) records of roundup4(6+Cp)
-    floats plus a 4-float reach box each (the `packed_bytes` of igs_gs2d_plan, restated so that
-    shape inference under torch.compile needs no library call)."""
-    return B * round_up(N, 4) * (round_up(6 + Cp, 4) + 4)
+    floats plus a 4-float reach box each, then 4 floats for the skip limit (the `packed_bytes` of
+    igs_gs2d_plan, restated so that shape inference under torch.compile needs no library call)."""
+    return B * round_up(N, 4) * (round_up(6 + Cp, 4) + 4) + 4
 
 
 class Grid:
@@ -158,6 +178,7 @@ class Splat:
         self.Cp = padded_channels(C)
         self.grid, self.eps, self.device = grid, float(eps), device
         self.plan = _lib.plan(B, N, grid.H, grid.W, self.Cp, grid.mode)
+        self.skip_weight = skip_weight(N, self.eps)
         self.stream = None
         self.use_current_stream()
 
@@ -175,22 +196,23 @@ class Splat:
     def pack_covinv(self, position, a, b, d, alphas, colors_p) -> Tensor:
         packed = self._empty(self.plan.packed_bytes)
         _lib.check(self.lib.igs_gs2d_pack_covinv(_ptr(position), _ptr(a), _ptr(b), _ptr(d), _ptr(alphas),
-                                                 _ptr(colors_p), self.B, self.N, self.Cp, _ptr(packed),
-                                                 self.stream), "igs_gs2d_pack_covinv")
+                                                 _ptr(colors_p), self.B, self.N, self.Cp, self.skip_weight,
+                                                 _ptr(packed), self.stream), "igs_gs2d_pack_covinv")
         return packed
 
     def pack_scale_rot(self, positions, scales, rotations, alphas, colors_p) -> Tensor:
         packed = self._empty(self.plan.packed_bytes)
         _lib.check(self.lib.igs_gs2d_pack_scale_rot(_ptr(positions), _ptr(scales), _ptr(rotations), _ptr(alphas),
                                                     _ptr(colors_p), self.B, self.N, self.Cp, self.eps,
-                                                    _ptr(packed), self.stream), "igs_gs2d_pack_scale_rot")
+                                                    self.skip_weight, _ptr(packed), self.stream),
+                   "igs_gs2d_pack_scale_rot")
         return packed
 
     def pack_feature(self, feat, off) -> Tuple[Tensor, Tensor]:
         packed = self._empty(self.plan.packed_bytes)
         col = self._new(self.B, self.N, self.Cp)
         _lib.check(self.lib.igs_gs2d_pack_feature(_ptr(feat), _ptr(off), self.B, self.N, self.C, self.Cp, self.eps,
-                                                  _ptr(packed), _ptr(col), self.stream),
+                                                  self.skip_weight, _ptr(packed), _ptr(col), self.stream),
                    "igs_gs2d_pack_feature")
         return packed, col
 

@@ -203,8 +203,8 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     p->bwd_tiles = (int)T;
     p->fwd_tiles = sep ? fg.tiles_x * fg.tiles_y : 0;
     p->pix_stride = sep ? pix_stride_sep(C) : pix_stride_gen(C);
-    // records, then one reach box (4 floats) per record
-    p->packed_bytes = (uint64_t)B * p->n_padded * (p->rec_stride + 4) * sizeof(float);
+    // records, then one reach box (4 floats) per record, then the call's skip limit (4 floats)
+    p->packed_bytes = ((uint64_t)B * p->n_padded * (p->rec_stride + 4) + 4) * sizeof(float);
     p->fwd_ws_bytes = S > 1 ? (uint64_t)S * B * (C + 1) * H * W * sizeof(float) : 0;
     p->pix_bytes = sep ? ((uint64_t)B * H * p->w_padded * p->pix_stride + (uint64_t)B * p->w_padded) * sizeof(float)
                        : (uint64_t)B * p->hw_padded * p->pix_stride * sizeof(float);
@@ -265,6 +265,17 @@ inline int* super_slots_at(float* partial, int B, int T, int NF, int N, int Np) 
 
 inline const float4* boxes_of(const float* packed, int B, int Np, int RS) {
     return reinterpret_cast<const float4*>(packed + (size_t)B * Np * RS);
+}
+// The skip limit the pack kernel left behind the boxes.
+inline const float* limit_of(const float* packed, int B, int Np, int RS) {
+    return packed + (size_t)B * Np * (RS + 4);
+}
+// Skip weight of a pack call -> limit in units of the kernels' exponent (see reach_box); a weight of
+// 0 (or one too small to matter) is the exact limit.
+inline int limit_from_skip_weight(float skip_weight, float* limit) {
+    if (!(skip_weight >= 0.0f) || skip_weight >= 1.0f) return IGS_ERR_BAD_SKIP_WEIGHT;
+    *limit = skip_weight > 0.0f ? -log2f(skip_weight) : 1e30f;
+    return IGS_OK;
 }
 
 // Public plan: AUTO reports the separable variant's geometry with the workspace sizes of
@@ -464,6 +475,7 @@ const char* igs_status_string(int status) {
         case IGS_ERR_BAD_MODE: return "unknown grid mode";
         case IGS_ERR_NO_DEVICE: return "no usable HIP device";
         case IGS_ERR_ALIGNMENT: return "buffer not 16-byte aligned";
+        case IGS_ERR_BAD_SKIP_WEIGHT: return "skip weight outside [0, 1)";
         case IGS_ERR_STATIC_SCRATCH: return "problem needs more scratch than the static array holds (IGS_STATIC_SCRATCH_BYTES)";
         default: break;
     }
@@ -475,6 +487,12 @@ int igs_gs2d_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_pla
     const int rc = make_plan(B, N, H, W, C, grid_mode, plan);
     if (rc) return rc;
     return channels_compiled(C) ? IGS_OK : IGS_ERR_BAD_CHANNELS;
+}
+
+float igs_gs2d_skip_weight(int N, float eps, float tolerance) {
+    if (!(tolerance > 0.0f) || !(eps > 0.0f) || N <= 0) return 0.0f;
+    const double w = (double)tolerance * (double)eps / (2.0 * (double)N);
+    return w < 0.5 ? (float)w : 0.5f;
 }
 
 int igs_gs2d_grid_classify(const float* x, const float* y, const int64_t grid_strides[6], int B,
@@ -491,30 +509,34 @@ int igs_gs2d_grid_classify(const float* x, const float* y, const int64_t grid_st
 
 int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const float* cov_inv_01,
                          const float* cov_inv_11, const float* alphas, const float* colors, int B,
-                         int N, int C, float* packed, igs_stream_t stream) {
+                         int N, int C, float skip_weight, float* packed, igs_stream_t stream) {
     if (!position || !cov_inv_00 || !cov_inv_01 || !cov_inv_11 || !alphas || !colors || !packed)
         return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
     if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    float limit;
+    if (const int rc = limit_from_skip_weight(skip_weight, &limit)) return rc;
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
-                       colors, N, Np, C, rec_stride_of(C), 0.0f, packed,
+                       colors, N, Np, C, rec_stride_of(C), 0.0f, limit, packed,
                        const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
 int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const float* rotations,
                             const float* alphas, const float* colors, int B, int N, int C, float eps,
-                            float* packed, igs_stream_t stream) {
+                            float skip_weight, float* packed, igs_stream_t stream) {
     if (!positions || !scales || !rotations || !alphas || !colors || !packed)
         return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
     if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
+    float limit;
+    if (const int rc = limit_from_skip_weight(skip_weight, &limit)) return rc;
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
-                       alphas, colors, N, Np, C, rec_stride_of(C), eps, packed,
+                       alphas, colors, N, Np, C, rec_stride_of(C), eps, limit, packed,
                        const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
@@ -560,6 +582,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
             const BinPlace bp = bins_at(ws, split_bytes, B, plan.fwd_tiles);
             BinArgs ba;
             ba.boxes = boxes_of(packed, B, plan.n_padded, plan.rec_stride);
+            ba.limit = limit_of(packed, B, plan.n_padded, plan.rec_stride);
             ba.packed = packed; ba.RS = plan.rec_stride;
             ba.x = x; ba.y = y;
             ba.sxb = a.sxb; ba.sxw = a.sxw; ba.syb = a.syb; ba.syh = a.syh;
@@ -801,6 +824,7 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
         if (sep) {
             BinArgs ba;
             ba.boxes = boxes_of(packed, B, a.Np, rec_stride_of(C));
+            ba.limit = limit_of(packed, B, a.Np, rec_stride_of(C));
             ba.packed = packed; ba.RS = rec_stride_of(C);
             ba.x = a.xs; ba.y = y;               // the prologue's compact column coordinates
             ba.sxb = a.Wp; ba.sxw = 1; ba.syb = a.syb; ba.syh = a.syh;
@@ -997,15 +1021,17 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
 }
 
 int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int B, int N, int C,
-                          int C_kernel, float eps, float* packed, float* colors_out,
+                          int C_kernel, float eps, float skip_weight, float* packed, float* colors_out,
                           igs_stream_t stream) {
     if (!gs_feature || !packed || !colors_out) return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
     if (C < 1 || C > C_kernel || !channels_compiled(C_kernel)) return IGS_ERR_BAD_CHANNELS;
+    float limit;
+    if (const int rc = limit_from_skip_weight(skip_weight, &limit)) return rc;
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
-                       rec_stride_of(C_kernel), eps, packed,
+                       rec_stride_of(C_kernel), eps, limit, packed,
                        const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
     return launch_status();
 }

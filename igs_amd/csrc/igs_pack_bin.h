@@ -3,24 +3,38 @@
 #pragma once
 
 // ----------------------------------------------------------------------------- pack
-// Reach box of a Gaussian: the axis-aligned bounding box of the ellipse q <= kReachQ, outside
-// of which its weight is exactly zero in these kernels: there the exponent
-// q' = -0.5 log2(e) q is below -160, ten binades under the -149/-150 at which exp2 returns 0
-// in fp32 whatever the denormal mode (the margin covers the rounding of q' itself, which is
-// a few ulp of its largest term).  Pixels outside the box therefore receive exactly +0 from
-// this Gaussian and give exactly 0 to its gradient sums, so skipping them changes no bit.
-// Half extents: sqrt(kReachQ Sigma_xx), sqrt(kReachQ Sigma_yy) with Sigma the covariance that
-// (A, B, D) invert.  A record with a non-finite field or a non-positive-definite (A, B, D)
-// gets an unbounded box (its NaN/inf must propagate as without culling); padding records get
-// an empty one.  Stored as (xlo, xhi, ylo, yhi).
-constexpr double kReachQ = 160.0 / 0.72134752044448170368;
+// Reach box of a Gaussian: the axis-aligned bounding box of the ellipse q <= Q, outside of which
+// the kernels skip it.  Q comes from the skip limit L of the call (in units of the kernels'
+// exponent q' = -0.5 log2(e) q, so that e = 2^q'):
+//   * L = kExactLimit (skip weight 0): the box bounds q' >= -160, ten binades under the -149/-150
+//     at which exp2 returns 0 in fp32 whatever the denormal mode (the margin covers the rounding of
+//     q' itself, which is a few ulp of its largest term).  Pixels outside the box receive exactly +0
+//     from this Gaussian and give exactly 0 to its gradient sums, so skipping them changes no bit.
+//   * L < kExactLimit (skip weight w > 0, L = -log2 w): a pair is skipped only where
+//     e < w / max(1, |alpha|), i.e. where both the weight alpha e and the bare exponential (which is
+//     what the gradient of alpha sums) are below w.  The limit of Gaussian n is
+//     L_n = min(kExactLimit, L + log2 max(1, |alpha_n|)).
+// The box is five binades wider than the tile test of k_bin (ellipse_reaches), as in the exact case.
+// Half extents: sqrt(Q Sigma_xx), sqrt(Q Sigma_yy) with Sigma the covariance that (A, B, D) invert.
+// A record with a non-finite field or a non-positive-definite (A, B, D) gets an unbounded box (its
+// NaN/inf must propagate as without culling); padding records get an empty one.  Stored as
+// (xlo, xhi, ylo, yhi).
+constexpr float kExactLimit = 155.0f;
+constexpr double kHalfLog2e = 0.72134752044448170368;
 
-__device__ __forceinline__ float4 reach_box(float px, float py, double sxx, double syy, bool bounded) {
+// limit of one Gaussian from the call's limit and its alpha (finite alpha)
+__device__ __forceinline__ float skip_limit(float limit, float alpha) {
+    return fminf(kExactLimit, limit + __log2f(fmaxf(1.0f, fabsf(alpha))));
+}
+
+__device__ __forceinline__ float4 reach_box(float px, float py, double sxx, double syy, bool bounded,
+                                            float limit_n) {
     const float inf = __builtin_inff();
     if (!bounded || !(sxx >= 0.0) || !(syy >= 0.0) || !isfinite(px) || !isfinite(py))
         return make_float4(-inf, inf, -inf, inf);
+    const double Q = ((double)limit_n + 5.0) / kHalfLog2e;
     // rounded outwards: one part in 1e5 is far more than the fp32 rounding of the bounds
-    const double hx = sqrt(kReachQ * sxx) * 1.00001, hy = sqrt(kReachQ * syy) * 1.00001;
+    const double hx = sqrt(Q * sxx) * 1.00001, hy = sqrt(Q * syy) * 1.00001;
     const double ax = fabs((double)px) * 1e-6 + 1e-30, ay = fabs((double)py) * 1e-6 + 1e-30;
     return make_float4((float)((double)px - hx - ax), (float)((double)px + hx + ax),
                        (float)((double)py - hy - ay), (float)((double)py + hy + ay));
@@ -29,6 +43,12 @@ __device__ __forceinline__ float4 reach_box(float px, float py, double sxx, doub
 __device__ __forceinline__ float4 empty_box() {
     const float inf = __builtin_inff();
     return make_float4(inf, -inf, inf, -inf);
+}
+
+// The call's skip limit travels behind the reach boxes [B][Np] in the packed buffer (4 floats, the
+// first one used), where k_bin reads it: the forward and the backward then need no argument for it.
+__device__ __forceinline__ void write_skip_limit(float4* boxes, int B, int Np, float limit) {
+    boxes[(size_t)B * Np] = make_float4(fminf(limit, kExactLimit), 0.0f, 0.0f, 0.0f);
 }
 
 // One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
@@ -42,10 +62,11 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
                                                    const float* __restrict__ alphas,
                                                    const float* __restrict__ colors, int N,
                                                    int Np, int C, int RS, float eps,
-                                                   float* __restrict__ packed,
+                                                   float limit, float* __restrict__ packed,
                                                    float4* __restrict__ boxes) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
+    if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit);
     if (n >= Np) return;
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {  // padding: alpha = 0 and e = exp2(0) = 1, so it contributes exactly 0
@@ -95,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
     }
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
-    const float4 box = reach_box(px, py, sxx, syy, bounded && fin);
+    const float4 box = reach_box(px, py, sxx, syy, bounded && fin, skip_limit(limit, al));
     boxes[(size_t)b * Np + n] = box;
     if (RS >= 8 + C) {  // room in the record: the y range of the box travels with it
         r[6 + C] = box.z;
@@ -111,11 +132,12 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
 __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restrict__ feat,
                                                            const float* __restrict__ pos_off, int N,
                                                            int Np, int C, int Cp, int RS, float eps,
-                                                           float* __restrict__ packed,
+                                                           float limit, float* __restrict__ packed,
                                                            float4* __restrict__ boxes,
                                                            float* __restrict__ colors_out) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
+    if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit);
     if (n >= Np) return;
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {
@@ -154,7 +176,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
     }
     for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
     const float4 box = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
-                                 fin && v0 > 0.0 && v1 > 0.0);
+                                 fin && v0 > 0.0 && v1 > 0.0, skip_limit(limit, 1.0f));
     boxes[(size_t)b * Np + n] = box;
     if (RS >= 8 + Cp) {
         r[6 + Cp] = box.z;
@@ -197,6 +219,7 @@ struct BinArgs {
     const int* cand_counts;  // [B][stiles][cand_K]
     const int* cand_lists;   // [B][stiles][Np], segment k at offset k cand_chunk
     int cand_K, cand_chunk, stiles_x, stiles;
+    const float* limit;  // the call's skip limit, written by the pack kernel behind the boxes
     const int* flag;
     int want;
     int no_cull;  // list every candidate (IGS_OPT_NO_CULL): the reference point for "culling changes no bit"
@@ -213,11 +236,13 @@ constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads i
 // P over the rectangle is 0 when it holds the centre and else lies on an edge, where P is a
 // parabola in one variable.  The kernels' weight is exactly 0 where their fp32 q' is below -150;
 // both their q' and the P evaluated here differ from the exact value by a few ulp of the largest
-// term, bounded over the rectangle by T below.  The tile is dropped only if min P - 4e-6 T > 155: the same margin
-// against rounding as the reach box has, so dropping it changes no bit either.  A
-// non-positive-definite or NaN record fails the comparison and stays listed.
+// term, bounded over the rectangle by T below.  The tile is dropped only if min P - 4e-6 T > L_n, the
+// Gaussian's skip limit (see reach_box): with the exact limit 155 this is the same margin against
+// rounding as the reach box has, so dropping it changes no bit either; with a skip weight w every
+// pair of a dropped tile has e < w / max(1, |alpha|).  A non-positive-definite or NaN record fails
+// the comparison and stays listed.
 __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, float txlo, float txhi,
-                                                float tylo, float tyhi) {
+                                                float tylo, float tyhi, float limit) {
     const float4 h = *reinterpret_cast<const float4*>(rec);  // px, py, A', B2'
     const float a = -h.z, b2 = -h.w, d = -rec[4];
     const float x0 = txlo - h.x, x1 = txhi - h.x, y0 = tylo - h.y, y1 = tyhi - h.y;
@@ -239,7 +264,7 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
     const float pmin = fminf(pv, ph);
     const float mx = fmaxf(fabsf(x0), fabsf(x1)), my = fmaxf(fabsf(y0), fabsf(y1));
     const float T = a * mx * mx + fabsf(b2) * mx * my + d * my * my;
-    return !(pmin - 4e-6f * T > 155.0f);
+    return !(pmin - 4e-6f * T > skip_limit(limit, rec[5]));
 }
 
 __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
@@ -290,6 +315,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         for (int k = kBinWaves / 2; k > 0; k >>= 1) rv[f] = fminf(rv[f], __shfl_xor(rv[f], k));
     }
     const float txlo = rv[0], txhi = -rv[1], tylo = rv[2], tyhi = -rv[3];
+    const float limit = *a.limit;
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     const float4* boxes = a.boxes + (size_t)b * a.Np;
@@ -345,7 +371,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             listed[u] = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
             // bounded box (unbounded ones mark records that must never be skipped): refine
             if (listed[u] && bb[u].x > -inf)
-                listed[u] = ellipse_reaches(recs + (size_t)n[u] * a.RS, txlo, txhi, tylo, tyhi);
+                listed[u] = ellipse_reaches(recs + (size_t)n[u] * a.RS, txlo, txhi, tylo, tyhi, limit);
         }
     };
     // the first pass keeps its verdicts (one bit per box of this lane) for the second one when

@@ -36,7 +36,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib
-from ._splat import Grid, _ptr, _stream, padded_channels
+from ._splat import Grid, _ptr, _stream, padded_channels, skip_weight
 
 Tensor = torch.Tensor
 
@@ -138,7 +138,8 @@ class GaussianImageFit:
             with torch.cuda.device(self.device):
                 buf = lambda nbytes: torch.empty(max(int(nbytes) // 4, 1), dtype=torch.float32, device=self.device)
                 new = lambda *s: torch.empty(*s, dtype=torch.float32, device=self.device)
-                ws = dict(plan=plan, packed=buf(plan.packed_bytes), col=new(self.B, n, self.Cp),
+                ws = dict(plan=plan, skip_weight=skip_weight(n, self.eps), packed=buf(plan.packed_bytes),
+                          col=new(self.B, n, self.Cp),
                           out=new(self.B, self.Cp, g.H, g.W), den=new(self.B, g.H, g.W),
                           fwd_ws=buf(plan.fwd_ws_bytes) if plan.fwd_ws_bytes else None, pix=buf(plan.pix_bytes),
                           partial=buf(plan.partial_bytes), loss_ws=buf(loss_bytes), loss_bytes=loss_bytes,
@@ -150,8 +151,8 @@ class GaussianImageFit:
     def _enqueue_render(self, n: int, ws: dict, st):
         lib, g, p = self.lib, self.grid, ws["plan"]
         B, C, Cp, H, W = self.B, self.C, self.Cp, g.H, g.W
-        _lib.check(lib.igs_gs2d_pack_feature(_ptr(self.params), None, B, n, C, Cp, self.eps, _ptr(ws["packed"]),
-                                             _ptr(ws["col"]), st), "igs_gs2d_pack_feature")
+        _lib.check(lib.igs_gs2d_pack_feature(_ptr(self.params), None, B, n, C, Cp, self.eps, ws["skip_weight"],
+                                             _ptr(ws["packed"]), _ptr(ws["col"]), st), "igs_gs2d_pack_feature")
         _lib.check(lib.igs_gs2d_forward(_ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n,
                                         H, W, Cp, self.eps, _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]),
                                         int(p.fwd_ws_bytes), st), "igs_gs2d_forward")

@@ -241,14 +241,46 @@ def operator_autograd(x, y, position, a, b_, d, alphas, colors, grad_out, eps=1e
 REACH_Q = 160.0 / (0.5 * math.log2(math.e))   # q beyond which the fp32 kernels' exp2 argument is < -160
 
 
-def reach_box(position, a, b_, d, q_max: float = REACH_Q):
+EXACT_LIMIT = 155.0                           # tile-test limit (in units of -q') when only exact zeros are skipped
+
+
+def skip_weight(N: int, eps: float, tolerance: float) -> float:
+    """Weight below which a (Gaussian, pixel) pair may be skipped so that no output element moves by
+    more than tolerance * max|colors|: with every skipped |alpha e| <= w, a pixel's numerator loses
+    at most N w max|c| and its denominator at most N w, hence
+    |d out| <= N w (max|c| + |out|) / (den + eps) <= 2 N w max|c| / eps  (den >= 0, |out| <= max|c|),
+    which is the tolerance for w = tolerance eps / (2 N).  Test infrastructure's restatement of
+    igs_gs2d_skip_weight (no counterpart in the reference, which evaluates every pair:
+    src/igs/gs_triton_chunked.py:100-200)."""
+    if not (tolerance > 0 and eps > 0 and N > 0):
+        return 0.0
+    return min(tolerance * eps / (2.0 * N), 0.5)
+
+
+def skip_limit(alphas, w: float):
+    """Per-Gaussian limit L_n on -q' = 0.5 log2(e) q beyond which the kernels may skip a pair:
+    e = 2^q' < w / max(1, |alpha_n|)  <=>  -q' > -log2 w + log2 max(1, |alpha_n|), capped at the
+    exact-zero limit; w = 0 is that cap."""
+    if w <= 0:
+        return torch.full_like(alphas, EXACT_LIMIT)
+    return torch.clamp(-math.log2(w) + torch.log2(torch.clamp(alphas.abs(), min=1.0)), max=EXACT_LIMIT)
+
+
+def reach_q(alphas, w: float):
+    """q_max of each Gaussian's reach box under skip weight w: five binades beyond its skip limit
+    (the exact-zero case gives REACH_Q)."""
+    return (skip_limit(alphas, w) + 5.0) / (0.5 * math.log2(math.e))
+
+
+def reach_box(position, a, b_, d, q_max=REACH_Q):
     """Axis-aligned bounding box of the ellipse q(dx, dy) = a dx^2 + 2 b dx dy + d dy^2 <= q_max
     around each Gaussian, as (xlo, xhi, ylo, yhi) [...,4].  Textbook result: the extreme of dx on
     the ellipse is sqrt(q_max * Sigma_xx) with Sigma = [[a, b], [b, d]]^-1, i.e.
     Sigma_xx = d / (a d - b^2), Sigma_yy = a / (a d - b^2).  This is the test infrastructure's
     restatement of the culling bound of the HIP pack kernels (no counterpart in the reference,
     which evaluates every pair: src/igs/gs_triton_chunked.py:100-200); pixels outside the box
-    have q > q_max and therefore a weight of exactly zero in the fp32 kernels."""
+    have q > q_max and therefore a weight of exactly zero in the fp32 kernels (q_max = REACH_Q) or
+    one below the call's skip weight (q_max = reach_q(alphas, w), a tensor per Gaussian)."""
     a, b_, d = (t.reshape(position.shape[:-1]) for t in (a, b_, d))
     det = a * d - b_ * b_
     hx = torch.sqrt(q_max * d / det)

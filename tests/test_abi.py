@@ -69,7 +69,7 @@ def test_plan_arithmetic(lib, mode):
         assert p.n_padded % 4 == 0 and p.n_padded >= N
         assert p.fwd_n_per_split % 4 == 0 and p.fwd_split * p.fwd_n_per_split >= p.n_padded
         assert (p.fwd_split - 1) * p.fwd_n_per_split < p.n_padded          # no empty split
-        assert p.packed_bytes == B * p.n_padded * (p.rec_stride + 4) * 4    # records + reach boxes
+        assert p.packed_bytes == (B * p.n_padded * (p.rec_stride + 4) + 4) * 4    # records + reach boxes + skip limit
         assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
         assert p.bwd_tiles >= 1 and p.partial_bytes >= B * p.bwd_tiles * (6 + C) * N * 4
         if mode != 0:
@@ -101,14 +101,24 @@ def test_argument_errors_are_status_codes_not_crashes(lib):
     assert lib.igs_gs2d_plan(1, 1 << 24, 64, 64, 3, 1, ctypes.byref(p)) == 0
     assert lib.igs_gs2d_plan(1, 8, 1 << 14, 1 << 14, 3, 1, ctypes.byref(p)) == 0
     # null pointers are rejected before anything is launched
+    fake = ctypes.c_void_p(4096)
     st = _lib.strides6((0, 0, 1), (0, 4, 0))
     assert lib.igs_gs2d_forward(None, None, None, st, 1, None, 1, 8, 4, 4, 3, 1e-6, None, None, None, 0, None) == -1
-    assert lib.igs_gs2d_pack_covinv(None, None, None, None, None, None, 1, 8, 3, None, None) == -1
+    assert lib.igs_gs2d_pack_covinv(None, None, None, None, None, None, 1, 8, 3, 0.0, None, None) == -1
+    # the skip weight of a pack call: 0 <= w < 1
+    for bad in (-1e-9, 1.0, float("nan")):
+        assert lib.igs_gs2d_pack_covinv(fake, fake, fake, fake, fake, fake, 1, 8, 3, bad, fake, None) == -9
+        assert lib.igs_gs2d_pack_scale_rot(fake, fake, fake, fake, fake, 1, 8, 3, 1e-6, bad, fake, None) == -9
+        assert lib.igs_gs2d_pack_feature(fake, None, 1, 8, 3, 3, 1e-6, bad, fake, fake, None) == -9
+    assert b"skip weight" in lib.igs_status_string(-9)
+    # tolerance * eps / (2 N); nothing may be skipped without an eps to measure against
+    assert lib.igs_gs2d_skip_weight(8192, 1e-6, 1e-7) == pytest.approx(1e-13 / 16384, rel=1e-6)
+    assert lib.igs_gs2d_skip_weight(8192, 0.0, 1e-7) == 0.0 and lib.igs_gs2d_skip_weight(8192, 1e-6, 0.0) == 0.0
+    assert lib.igs_gs2d_skip_weight(1, 1.0, 0.9) < 1.0
     assert lib.igs_gs2d_finalize_covinv(None, 1, None, None, None, None, None, 1, 8, 4, 4, 3,
                                         None, None, None, None, None, None, None) == -1
     assert lib.igs_gs2d_backward_with_grid(None, None, None, None, st, 1, None, None, None, None, 1, 8, 4, 4, 3, 1e-6,
                                            None, 0, None, 0, None, 0, None, None, None) == -1
-    fake = ctypes.c_void_p(4096)
     assert lib.igs_gs2d_grid_workspace_bytes(2, 3000, 10, 13, 3) == 2 * 3 * 132 * 8     # B x groups x roundup4(HW) x float2
     assert lib.igs_gs2d_grid_workspace_bytes(2, 3000, 10, 13, 5) == 0                   # not a compiled channel count
     assert lib.igs_gs2d_backward_with_grid(fake, fake, fake, fake, st, 0, None, fake, fake, fake, 2, 3000, 10, 13, 3,
@@ -255,7 +265,7 @@ def test_plan_invariants_over_random_shapes(lib):
             Np = p.n_padded
             assert Np % 4 == 0 and N <= Np < N + 4
             assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
-            assert p.packed_bytes == B * Np * (p.rec_stride + 4) * 4
+            assert p.packed_bytes == (B * Np * (p.rec_stride + 4) + 4) * 4
             assert 1 <= p.fwd_split <= 64 and p.fwd_n_per_split % 4 == 0
             assert p.fwd_split * p.fwd_n_per_split >= Np > (p.fwd_split - 1) * p.fwd_n_per_split
             assert p.bwd_tiles >= 1 and p.bwd_per_tile >= 1

@@ -1,9 +1,12 @@
-"""Culling on separable grids: a Gaussian is skipped for a pixel tile when its reach box (the
-bounding box of q <= 221.8, beyond which exp2 of the kernels' exponent is exactly 0) misses the
-tile.  The claim under test is that this drops only exact zeros: with IGS_OPT_NO_CULL the
-library makes every box unbounded, and both runs must agree exactly (one forward split) or to
-fp32 rounding (several, where the grouping of the terms changes); beside that, sparse scenes
-against the fp64 oracle, non-finite parameters, and grids whose coordinates are not monotone."""
+"""Culling on separable grids: a Gaussian is skipped for a pixel tile when its reach box misses the
+tile or its ellipse does not reach the tile's rectangle.  Two claims are under test.  With a skip
+weight of 0 (`library_options(skip_tolerance=0)`; the box bounds q <= 221.8, beyond which exp2 of
+the kernels' exponent is exactly 0) only exact zeros are dropped: with IGS_OPT_NO_CULL the library
+lists everything, and both runs must agree exactly (one forward split) or to fp32 rounding (several,
+where the grouping of the terms changes).  With the default skip tolerance only pairs below the
+skip weight are dropped: the run stays within the stated bound of the run that lists everything.
+Beside that: sparse scenes against the fp64 oracle, non-finite parameters, grids whose coordinates
+are not monotone, and the boxes and tile lists themselves against the oracle's restatement."""
 import os
 
 import pytest
@@ -61,6 +64,13 @@ def no_cull():
     return Ctx()
 
 
+def exact():
+    """Context in which only pairs whose weight is exactly zero are skipped (skip weight 0)."""
+    from igs_amd._splat import library_options
+
+    return library_options(skip_tolerance=0.0)
+
+
 @pytest.mark.parametrize("shape", [(2, 120, 70, 150, 3), (1, 100, 200, 64, 16), (3, 64, 33, 257, 1)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_culled_equals_unculled_bit_for_bit(igs, dev, no_cull, shape):
@@ -68,7 +78,8 @@ def test_culled_equals_unculled_bit_for_bit(igs, dev, no_cull, shape):
     the same order and the skipped ones are exact zeros."""
     B, N, H, W, C = shape
     _, g = sparse_case(dev, B, N, H, W, C, seed=sum(shape))
-    out, grads = run(igs, g)
+    with exact():
+        out, grads = run(igs, g)
     with no_cull:
         out0, grads0 = run(igs, g)
     assert float(out.abs().max()) > 0
@@ -82,7 +93,8 @@ def test_long_rotated_gaussians_bit_for_bit(igs, dev, no_cull):
     ellipse-against-tile test of the binning decides; it must drop exact zeros only."""
     B, N, H, W, C = 2, 120, 192, 320, 3
     _, g = sparse_case(dev, B, N, H, W, C, seed=77, smin=0.002, smax=0.2)
-    out, grads = run(igs, g)
+    with exact():
+        out, grads = run(igs, g)
     with no_cull:
         out0, grads0 = run(igs, g)
     assert float(out.abs().max()) > 0
@@ -170,7 +182,8 @@ def test_two_level_binning_culled_equals_unculled(igs, dev, no_cull):
     B, N, H, W, C = 2, 120, 256, 512, 3
     _, g = sparse_case(dev, B, N, H, W, C, seed=21, smin=0.002, smax=0.2)
     with _Env("IGS_BIN_LEVELS", "2"):
-        out, grads = run(igs, g)
+        with exact():
+            out, grads = run(igs, g)
         with no_cull:
             out0, grads0 = run(igs, g)
     assert torch.equal(out, out0)
@@ -220,7 +233,8 @@ def test_culled_equals_unculled_with_several_forward_splits(igs, dev, no_cull):
     B, N, H, W, C = 1, 3000, 96, 160, 3
     assert _lib.plan(B, N, H, W, C, 1).fwd_split > 1
     _, g = sparse_case(dev, B, N, H, W, C, seed=5)
-    out, grads = run(igs, g)
+    with exact():
+        out, grads = run(igs, g)
     with no_cull:
         out0, grads0 = run(igs, g)
     torch.testing.assert_close(out, out0, rtol=0, atol=1e-6)
@@ -259,7 +273,8 @@ def test_non_monotone_separable_grid(igs, dev, no_cull):
     yg = ys.view(1, 1, H, 1).expand(B, 1, H, W)
     g2 = dict(g)
     g2["grad_out"] = g["grad_out"][:, :, pr][:, :, :, pc].contiguous()
-    out, grads = run(igs, g2, xg, yg)
+    with exact():
+        out, grads = run(igs, g2, xg, yg)
     with no_cull:
         out0, grads0 = run(igs, g2, xg, yg)
     assert torch.equal(out, out0)
@@ -285,12 +300,18 @@ def test_non_finite_parameters_propagate_as_without_culling(igs, dev, no_cull):
         h = {k: v.clone() for k, v in g.items()}
         h[field][index] = value
         with torch.no_grad():
-            got = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"])
+            with exact():
+                got = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"])
+            dflt = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"])
             with no_cull:
                 ref = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"])
             want = igs.gaussian_splatting_2d(*(h[k] for k in NAMES), g["x_grid"], g["y_grid"], fused=False)
         assert torch.equal(torch.isnan(got), torch.isnan(ref)), field
         assert torch.equal(torch.nan_to_num(got, nan=7.0), torch.nan_to_num(ref, nan=7.0)), field
+        # under the default skip weight such a record is never skipped either
+        assert torch.equal(torch.isfinite(dflt), torch.isfinite(ref)), field
+        fin = torch.isfinite(ref)
+        torch.testing.assert_close(dflt[fin], ref[fin], rtol=1e-6, atol=2e-7)
         if all_nan:
             assert bool(torch.isnan(want).all()) and bool(torch.isnan(got).all()), field
         else:   # the other channels are untouched
@@ -311,10 +332,15 @@ def test_operator_level_with_indefinite_cov_inverse(igs, dev, no_cull):
     K = igs.GaussianSplatting2DKernel
     args = (g["x_grid"], g["y_grid"], g["positions"], a, b, d, g["alphas"], g["colors"])
     with torch.no_grad():
-        out = K.apply(*args)
+        with exact():
+            out = K.apply(*args)
+        dflt = K.apply(*args)
         with no_cull:
             out0 = K.apply(*args)
         want = igs.naive_gaussian_2d(g["x_grid"], g["y_grid"], g["positions"], a, b, d, g["alphas"], g["colors"])
+    assert torch.equal(torch.isnan(dflt), torch.isnan(out0))
+    fin = torch.isfinite(out0)
+    torch.testing.assert_close(dflt[fin], out0[fin], rtol=1e-6, atol=2e-7)
     # the saddle overflows where it grows (inf / inf): same places, same values elsewhere
     assert torch.equal(torch.isnan(out), torch.isnan(out0))
     assert torch.equal(torch.nan_to_num(out, nan=7.0), torch.nan_to_num(out0, nan=7.0))
@@ -323,34 +349,44 @@ def test_operator_level_with_indefinite_cov_inverse(igs, dev, no_cull):
     torch.testing.assert_close(out[ok], want[ok], rtol=1e-4, atol=1e-5)
 
 
-def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev):
+@pytest.mark.parametrize("tolerance", [0.0, 1e-7, 1e-3], ids=lambda t: f"tol{t:g}")
+def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev, tolerance):
     """The boxes behind the packed records (scale/rotation, cov-inverse and module-feature
-    packing) against the oracle's restatement: never inside it, and no more than the stated
-    outward rounding (1e-5 relative on the half extent) beyond it."""
-    from igs_amd._splat import Grid, Splat, _f32c
+    packing) against the oracle's restatement, for the exact-zero limit and for two skip weights,
+    with alphas on both sides of 1: never inside it, and no more than the stated outward rounding
+    (1e-5 relative on the half extent) beyond it.  The skip limit itself sits behind the boxes."""
+    import math
+
+    from igs_amd._splat import Grid, Splat, _f32c, library_options
 
     B, N, C = 2, 257, 3
     d64, g = sparse_case(dev, B, N, 40, 72, C, seed=2, smin=0.003, smax=0.4)
+    g["alphas"] = (g["alphas"] * 6).contiguous()                       # a third of them above 1
     grid = Grid(g["x_grid"], g["y_grid"], B)
-    op = Splat(B, N, C, grid, 1e-6, dev)
+    with library_options(skip_tolerance=tolerance):
+        op = Splat(B, N, C, grid, 1e-6, dev)
+    w = O.skip_weight(N, 1e-6, tolerance)
+    assert op.skip_weight == pytest.approx(w, rel=1e-6)
     a, b, dd = O.cov_inverse_closed(d64["scales"].float().double(), d64["rotations"].float().double())
-    want = O.reach_box(d64["positions"].float().double(), a, b, dd).to(dev)
+    pos = d64["positions"].float().double()
 
     def boxes(packed):
         p = op.plan
-        return packed[B * p.n_padded * p.rec_stride:].view(B, p.n_padded, 4)
+        return packed[B * p.n_padded * p.rec_stride:][:B * p.n_padded * 4].view(B, p.n_padded, 4)
 
     col = _f32c(g["colors"])
-    cases = {"scale_rot": op.pack_scale_rot(_f32c(g["positions"]), _f32c(g["scales"]), _f32c(g["rotations"]),
-                                            _f32c(g["alphas"]), col)}
+    cases = {"scale_rot": (op.pack_scale_rot(_f32c(g["positions"]), _f32c(g["scales"]), _f32c(g["rotations"]),
+                                             _f32c(g["alphas"]), col), g["alphas"].cpu().double())}
     f = lambda t: t.to(dev, torch.float32).reshape(B, N).contiguous()
-    cases["covinv"] = op.pack_covinv(_f32c(g["positions"]), f(a), f(b), f(dd), _f32c(g["alphas"]), col)
+    cases["covinv"] = (op.pack_covinv(_f32c(g["positions"]), f(a), f(b), f(dd), _f32c(g["alphas"]), col),
+                       g["alphas"].cpu().double())
     feat = torch.cat([g["positions"], (g["scales"] - 1e-6).log(), g["rotations"][..., None],
                       torch.zeros_like(g["rotations"])[..., None], g["colors"]], dim=-1).contiguous()
-    cases["feature"] = op.pack_feature(feat, None)[0]
-    half = torch.stack([want[..., 1] - want[..., 0], want[..., 3] - want[..., 2]], -1).repeat_interleave(2, -1) / 2
+    cases["feature"] = (op.pack_feature(feat, None)[0], torch.ones(B, N, dtype=torch.float64))   # the module's alpha
     sign = torch.tensor([-1.0, 1.0, -1.0, 1.0], device=dev, dtype=torch.float64)
-    for name, packed in cases.items():
+    for name, (packed, alphas) in cases.items():
+        want = O.reach_box(pos, a, b, dd, O.reach_q(alphas, w)).to(dev)
+        half = torch.stack([want[..., 1] - want[..., 0], want[..., 3] - want[..., 2]], -1).repeat_interleave(2, -1) / 2
         got = boxes(packed)[:, :N].double()
         out = (got - want) * sign                      # how far outside the exact box each edge lies
         # cov-inverse / feature inputs are fp32 roundings of the fp64 route: allow their error too
@@ -359,6 +395,106 @@ def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev):
         assert bool((out <= slack * half + 1e-6).all()), (name, float((out / half).max()))
         pad = boxes(packed)[:, N:]
         assert bool((pad[..., 0] > pad[..., 1]).all())  # padding records: empty boxes
+        limit = float(packed[B * op.plan.n_padded * (op.plan.rec_stride + 4)])
+        assert limit == pytest.approx(O.EXACT_LIMIT if w == 0 else min(O.EXACT_LIMIT, -math.log2(w)), rel=1e-6)
+    if tolerance > 0:    # smaller boxes than the exact-zero ones, by sqrt of the limits' ratio
+        ratio = math.sqrt((-math.log2(w) + 5) / (O.EXACT_LIMIT + 5))
+        exact_box = O.reach_box(pos, a, b, dd)
+        got = boxes(cases["feature"][0])[:, :N].double().cpu()
+        r = (got[..., 1] - got[..., 0]) / (exact_box[..., 1] - exact_box[..., 0])
+        assert float((r - ratio).abs().max()) < 1e-4
+
+
+def _tile_counts(op, packed, dev):
+    """Per-tile list lengths [B, tiles_y, tiles_x] of the separable backward for `packed` (read back
+    from the workspace behind the pixel records, where the binning of the reduce call writes them)."""
+    from igs_amd import _lib
+    from igs_amd._splat import _ptr
+
+    g, p = op.grid, op.plan
+    B, H, W = op.B, g.H, g.W
+    pix = op._empty(p.pix_bytes)
+    partial = op._empty(p.partial_bytes)
+    out, den = op.forward(packed)
+    go = torch.ones(B, op.Cp, H, W, device=dev)
+    col = torch.zeros(B, op.N, op.Cp, device=dev)
+    _lib.check(op.lib.igs_gs2d_backward(_ptr(packed), _ptr(col), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag),
+                                        _ptr(out), _ptr(den), _ptr(go), B, op.N, H, W, op.Cp, op.eps, _ptr(pix),
+                                        int(p.pix_bytes), _ptr(partial), int(p.partial_bytes), op.stream), "backward")
+    scratch = (B * H * p.w_padded * p.pix_stride + B * p.w_padded) * 4
+    return pix.view(torch.int32)[(scratch + 15) // 16 * 4:][: B * p.bwd_tiles].view(B, -1, p.bwd_tiles_x).cpu()
+
+
+@pytest.mark.parametrize("tolerance", [0.0, 1e-7], ids=lambda t: f"tol{t:g}")
+def test_tile_lists_against_the_oracle_s_rectangle_minimum(igs, dev, tolerance):
+    """What the binning lists for each backward tile against the oracle: a Gaussian whose minimum
+    of -q' over the tile's coordinate rectangle (`min_q_over_rect`) is below its skip limit must be
+    listed; one whose minimum is beyond the limit by more than the kernel's rounding allowance must
+    not (aspect ratios stay far below the 1:600 beyond which the kernel lists an ellipse anyway).
+    Counted per tile: must <= listed <= may."""
+    from igs_amd._splat import Grid, Splat, _f32c, library_options
+
+    B, N, H, W, C = 2, 900, 96, 200, 3
+    d64, g = sparse_case(dev, B, N, H, W, C, seed=19, smin=0.004, smax=0.15)
+    g["alphas"] = (g["alphas"] * 3).contiguous()
+    with library_options(skip_tolerance=tolerance):
+        op = Splat(B, N, C, Grid(g["x_grid"], g["y_grid"], B), 1e-6, dev)
+    packed = op.pack_scale_rot(_f32c(g["positions"]), _f32c(g["scales"]), _f32c(g["rotations"]), _f32c(g["alphas"]),
+                               _f32c(g["colors"]))
+    counts = _tile_counts(op, packed, dev)
+    p = op.plan
+    a, b, dd = (t.reshape(B, N) for t in O.cov_inverse_closed(d64["scales"].float().double(),
+                                                               d64["rotations"].float().double()))
+    pos = d64["positions"].float().double()
+    lim = O.skip_limit(g["alphas"].cpu().double(), O.skip_weight(N, 1e-6, tolerance))
+    xs, ys = g["x_grid"][0, 0, 0, :].cpu().double(), g["y_grid"][0, 0, :, 0].cpu().double()
+    k = 0.5 * 1.4426950408889634
+    saw_less = False
+    for ty in range(counts.shape[1]):
+        for tx in range(counts.shape[2]):
+            r0, r1 = ty * p.bwd_per_tile, min(H, (ty + 1) * p.bwd_per_tile)
+            c0, c1 = tx * 64, min(W, (tx + 1) * 64)
+            m = k * O.min_q_over_rect(pos[..., 0], pos[..., 1], a, b, dd, xs[c0], xs[c1 - 1], ys[r0], ys[r1 - 1])
+            # the kernel's allowance for the fp32 rounding of its own evaluation: 4e-6 of the largest
+            # term of the form over the rectangle (here with a little room for its rounding)
+            mx = torch.maximum((xs[c0] - pos[..., 0]).abs(), (xs[c1 - 1] - pos[..., 0]).abs())
+            my = torch.maximum((ys[r0] - pos[..., 1]).abs(), (ys[r1 - 1] - pos[..., 1]).abs())
+            T = k * (a * mx * mx + 2 * b.abs() * mx * my + dd * my * my)
+            must = (m <= lim * (1 - 1e-4)).sum(1)
+            may = (m - 5e-6 * T <= lim * (1 + 1e-4) + 1e-3).sum(1)
+            got = counts[:, ty, tx]
+            assert bool((must <= got).all()) and bool((got <= may).all()), (ty, tx, must, got, may)
+            saw_less = saw_less or bool((got < N).any())
+    assert saw_less
+
+
+@pytest.mark.parametrize("alpha_scale", [1.0, 25.0])
+def test_default_skip_tolerance_stays_within_its_bound(igs, dev, alpha_scale):
+    """The default skip weight against the run that lists every Gaussian for every tile, on sparse
+    scenes where most pixels have a denominator far below eps (the worst case of the bound): every
+    output element within 1e-7 max|colors| (plus the rounding of sums that now miss their smallest
+    terms), every gradient within 1e-5 of the unculled one in norm."""
+    from igs_amd._splat import SKIP_TOLERANCE
+
+    B, N, H, W, C = 2, 120, 160, 192, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=23, smin=0.003, smax=0.03)
+    g["alphas"] = (g["alphas"] * alpha_scale).contiguous()
+    out, grads = run(igs, g)
+    with no_cull_ctx():
+        out0, grads0 = run(igs, g)
+    cmax = float(g["colors"].abs().max())
+    assert SKIP_TOLERANCE == 1e-7
+    err = (out - out0).abs()
+    assert bool((err <= SKIP_TOLERANCE * cmax + 3e-7 * out0.abs()).all()), float(err.max())
+    for k in NAMES:
+        d = (grads[k] - grads0[k]).double()
+        assert float(d.norm()) <= 1e-5 * float(grads0[k].double().norm()), k
+
+
+def no_cull_ctx():
+    from igs_amd._splat import library_options
+
+    return library_options(no_cull=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.bfloat16, torch.float16])

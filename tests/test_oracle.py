@@ -342,3 +342,60 @@ def test_min_q_over_rect_against_dense_sampling():
     ddx = torch.clamp(torch.maximum(xlo - px, px - xhi), min=0)
     ddy = torch.clamp(torch.maximum(ylo - py, py - yhi), min=0)
     torch.testing.assert_close(m0, a * ddx * ddx + d * ddy * ddy, rtol=1e-12, atol=1e-15)
+
+
+def test_skip_weight_bound_by_brute_force():
+    """Pins the claim behind the skip weight, not its formula: evaluate the plain expression in
+    fp64 with and without the pairs that `skip_limit` allows to drop (e < w / max(1, |alpha|)) on
+    scenes built to be the worst case -- sparse small Gaussians, so that many pixels have a
+    denominator far below eps and nearly everything they see is below the weight, alphas of either
+    magnitude -- and check |d out| <= tolerance max|c| with w = skip_weight(N, eps, tolerance), that
+    the bound is not vacuous (a constructed pixel comes within a factor 2.1 of it) and that each per-Gaussian sum of exponentials, which is what the gradient of
+    alpha adds up, loses less than w per pixel.  A missing factor N, eps or 2, or a limit that
+    ignores |alpha| > 1, fails the first check."""
+    g = torch.Generator().manual_seed(3)
+    N, H, W, C, eps = 60, 48, 64, 3, 1e-6
+    for tol, amax in ((1e-7, 1.0), (1e-3, 1.0), (1e-3, 30.0), (0.3, 5.0)):
+        pos = torch.rand(1, N, 2, generator=g, dtype=F64) * 2 - 1
+        sc = torch.rand(1, N, 2, generator=g, dtype=F64) * 0.03 + 0.004
+        rot = torch.rand(1, N, generator=g, dtype=F64) * 2 * math.pi
+        al = torch.rand(1, N, generator=g, dtype=F64) * amax
+        col = torch.rand(1, N, C, generator=g, dtype=F64) * 2 - 1
+        a, b, d = (t.reshape(1, N, 1, 1) for t in O.cov_inverse_closed(sc, rot, eps))
+        x = torch.linspace(-1, 1, W, dtype=F64).view(1, 1, 1, W)
+        y = torch.linspace(-1, 1, H, dtype=F64).view(1, 1, H, 1)
+        dx, dy = x - pos[..., 0, None, None], y - pos[..., 1, None, None]
+        q = a * dx * dx + 2 * b * dx * dy + d * dy * dy
+        e = torch.exp(-0.5 * q)                                                  # [1,N,H,W]
+        w = O.skip_weight(N, eps, tol)
+        assert w == tol * eps / (2 * N)
+        lim = O.skip_limit(al, w).view(1, N, 1, 1)
+        drop = 0.5 * math.log2(math.e) * q > lim
+        assert bool(drop.any()) and bool((e[drop] * torch.clamp(al.abs(), min=1).view(1, N, 1, 1).expand_as(e)[drop]
+                                          <= w * (1 + 1e-12)).all())
+
+        def image(ee):
+            wgt = ee * al.view(1, N, 1, 1)
+            return torch.einsum("bnhw,bnc->bchw", wgt, col) / (wgt.sum(1, keepdim=True) + eps)
+
+        full, kept = image(e), image(torch.where(drop, torch.zeros_like(e), e))
+        err = float((full - kept).abs().max())
+        assert err <= tol * float(col.abs().max()), (tol, amax, err)
+        assert float((e * drop).max()) <= w
+    # the bound is attained to within a factor of 2.1 when all N Gaussians coincide, carry the same
+    # colour and a pixel sees each of them just below the weight: out = N e / (N e + eps) ~ tol / 2
+    tol = 1e-3
+    w = O.skip_weight(N, eps, tol)
+    r = math.sqrt(-2 * math.log(w * 0.999))                       # distance in sigma at which e = 0.999 w
+    sig = 0.05
+    xs = torch.tensor([0.0, r * sig], dtype=F64)
+    e = torch.exp(-0.5 * (xs / sig) ** 2)
+    assert float(e[1]) < w and bool(0.5 * math.log2(math.e) * (xs[1] / sig) ** 2 > O.skip_limit(torch.ones(1, dtype=F64), w))
+    full = N * e[1] / (N * e[1] + eps)
+    assert tol / 2.1 <= float(full) <= tol                         # kept: 0
+    assert O.skip_weight(100, 0.0, 1e-7) == 0.0 and O.skip_weight(100, 1e-6, 0.0) == 0.0
+    assert bool((O.skip_limit(torch.tensor([0.5, 4.0]), 0.0) == O.EXACT_LIMIT).all())
+    assert math.isclose(float(O.reach_q(torch.tensor([1.0], dtype=F64), 0.0)[0]), O.REACH_Q, rel_tol=1e-12)
+    # |alpha| = 4 moves the limit by two binades, |alpha| < 1 by nothing
+    l = O.skip_limit(torch.tensor([0.25, 1.0, 4.0], dtype=F64), 2.0 ** -50)
+    assert l.tolist() == [50.0, 50.0, 52.0]
