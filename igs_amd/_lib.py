@@ -75,9 +75,10 @@ SIGNATURES = {
     "igs_status_string": (c_char_p, [c_int]),
     "igs_gs2d_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, POINTER(Plan)]),
     "igs_gs2d_skip_weight": (c_float, [c_int, c_float, c_float]),
-    "igs_gs2d_pack_covinv": (c_int, [_FP, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, _FP, c_void_p]),
-    "igs_gs2d_pack_scale_rot": (c_int, [_FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, c_float, _FP,
-                                        c_void_p]),
+    "igs_gs2d_pack_covinv": (c_int, [_FP, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, c_float, _FP,
+                                     c_void_p]),
+    "igs_gs2d_pack_scale_rot": (c_int, [_FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_float, c_float, c_float,
+                                        _FP, c_void_p]),
     "igs_gs2d_grid_classify": (c_int, [_FP, _FP, _STRIDES, c_int, c_int, c_int, _FP, c_void_p]),
     "igs_gs2d_forward": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
                                  c_float, _FP, _FP, c_void_p, c_size_t, c_void_p]),
@@ -99,7 +100,8 @@ SIGNATURES = {
                                          _FP, _FP, _FP, _FP, _FP, _FP, c_void_p]),
     "igs_gs2d_finalize_scale_rot": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                             c_float, _FP, _FP, _FP, _FP, _FP, c_void_p]),
-    "igs_gs2d_pack_feature": (c_int, [_FP, _FP, c_int, c_int, c_int, c_int, c_float, c_float, _FP, _FP, c_void_p]),
+    "igs_gs2d_pack_feature": (c_int, [_FP, _FP, c_int, c_int, c_int, c_int, c_float, c_float, c_float, _FP, _FP,
+                                      c_void_p]),
     "igs_gs2d_finalize_feature": (c_int, [_FP, c_int, _FP, _FP, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                           _FP, c_void_p]),
     "igs_gs2d_mse_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

@@ -37,7 +37,8 @@ _option_bits = 0
 
 # Bound on what skipping far-away (Gaussian, pixel) pairs may change in an output element, as a
 # fraction of the largest colour magnitude: the pack calls get the skip weight
-# igs_gs2d_skip_weight(N, eps, SKIP_TOLERANCE) = SKIP_TOLERANCE * eps / (2 N).  The forward is held to
+# igs_gs2d_skip_weight(N, eps, SKIP_TOLERANCE) = SKIP_TOLERANCE * eps / (2 N) and the skip fraction
+# SKIP_TOLERANCE / (2 N) of a pixel tile's smallest denominator.  The forward is held to
 # 1e-6 + 1e-5 |ref| against the plain expression; 1e-7 leaves that budget to the fp32 rounding.
 # 0 skips exact zeros only (bit-identical to evaluating every pair).
 SKIP_TOLERANCE = 1e-7
@@ -69,9 +70,10 @@ def library_options(no_cull: bool = False, bin_levels: Optional[int] = None,
         _option_bits, _skip_tolerance = saved
 
 
-def skip_weight(N: int, eps: float) -> float:
-    """The skip weight the pack calls of a problem get under the current skip tolerance."""
-    return float(_lib.load().igs_gs2d_skip_weight(int(N), float(eps), float(_skip_tolerance)))
+def skip_weight(N: int, eps: float) -> Tuple[float, float]:
+    """(skip_weight, skip_fraction) the pack calls of a problem get under the current skip tolerance."""
+    f = _lib.load().igs_gs2d_skip_weight
+    return float(f(int(N), float(eps), float(_skip_tolerance))), float(f(int(N), 1.0, float(_skip_tolerance)))
 
 
 def _ptr(t: Optional[Tensor]):
@@ -196,7 +198,7 @@ class Splat:
     def pack_covinv(self, position, a, b, d, alphas, colors_p) -> Tensor:
         packed = self._empty(self.plan.packed_bytes)
         _lib.check(self.lib.igs_gs2d_pack_covinv(_ptr(position), _ptr(a), _ptr(b), _ptr(d), _ptr(alphas),
-                                                 _ptr(colors_p), self.B, self.N, self.Cp, self.skip_weight,
+                                                 _ptr(colors_p), self.B, self.N, self.Cp, *self.skip_weight,
                                                  _ptr(packed), self.stream), "igs_gs2d_pack_covinv")
         return packed
 
@@ -204,7 +206,7 @@ class Splat:
         packed = self._empty(self.plan.packed_bytes)
         _lib.check(self.lib.igs_gs2d_pack_scale_rot(_ptr(positions), _ptr(scales), _ptr(rotations), _ptr(alphas),
                                                     _ptr(colors_p), self.B, self.N, self.Cp, self.eps,
-                                                    self.skip_weight, _ptr(packed), self.stream),
+                                                    *self.skip_weight, _ptr(packed), self.stream),
                    "igs_gs2d_pack_scale_rot")
         return packed
 
@@ -212,7 +214,7 @@ class Splat:
         packed = self._empty(self.plan.packed_bytes)
         col = self._new(self.B, self.N, self.Cp)
         _lib.check(self.lib.igs_gs2d_pack_feature(_ptr(feat), _ptr(off), self.B, self.N, self.C, self.Cp, self.eps,
-                                                  self.skip_weight, _ptr(packed), _ptr(col), self.stream),
+                                                  *self.skip_weight, _ptr(packed), _ptr(col), self.stream),
                    "igs_gs2d_pack_feature")
         return packed, col
 

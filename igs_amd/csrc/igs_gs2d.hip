@@ -272,8 +272,9 @@ inline const float* limit_of(const float* packed, int B, int Np, int RS) {
 }
 // Skip weight of a pack call -> limit in units of the kernels' exponent (see reach_box); a weight of
 // 0 (or one too small to matter) is the exact limit.
-inline int limit_from_skip_weight(float skip_weight, float* limit) {
+inline int limit_from_skip_weight(float skip_weight, float skip_fraction, float* limit) {
     if (!(skip_weight >= 0.0f) || skip_weight >= 1.0f) return IGS_ERR_BAD_SKIP_WEIGHT;
+    if (!(skip_fraction >= 0.0f) || skip_fraction >= 1.0f) return IGS_ERR_BAD_SKIP_WEIGHT;
     *limit = skip_weight > 0.0f ? -log2f(skip_weight) : 1e30f;
     return IGS_OK;
 }
@@ -509,34 +510,35 @@ int igs_gs2d_grid_classify(const float* x, const float* y, const int64_t grid_st
 
 int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const float* cov_inv_01,
                          const float* cov_inv_11, const float* alphas, const float* colors, int B,
-                         int N, int C, float skip_weight, float* packed, igs_stream_t stream) {
+                         int N, int C, float skip_weight, float skip_fraction, float* packed,
+                         igs_stream_t stream) {
     if (!position || !cov_inv_00 || !cov_inv_01 || !cov_inv_11 || !alphas || !colors || !packed)
         return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
     if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
     float limit;
-    if (const int rc = limit_from_skip_weight(skip_weight, &limit)) return rc;
+    if (const int rc = limit_from_skip_weight(skip_weight, skip_fraction, &limit)) return rc;
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
-                       colors, N, Np, C, rec_stride_of(C), 0.0f, limit, packed,
+                       colors, N, Np, C, rec_stride_of(C), 0.0f, limit, skip_fraction, packed,
                        const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
 int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const float* rotations,
                             const float* alphas, const float* colors, int B, int N, int C, float eps,
-                            float skip_weight, float* packed, igs_stream_t stream) {
+                            float skip_weight, float skip_fraction, float* packed, igs_stream_t stream) {
     if (!positions || !scales || !rotations || !alphas || !colors || !packed)
         return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
     if (!channels_compiled(C)) return IGS_ERR_BAD_CHANNELS;
     float limit;
-    if (const int rc = limit_from_skip_weight(skip_weight, &limit)) return rc;
+    if (const int rc = limit_from_skip_weight(skip_weight, skip_fraction, &limit)) return rc;
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
-                       alphas, colors, N, Np, C, rec_stride_of(C), eps, limit, packed,
+                       alphas, colors, N, Np, C, rec_stride_of(C), eps, limit, skip_fraction, packed,
                        const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
@@ -1021,17 +1023,18 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
 }
 
 int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int B, int N, int C,
-                          int C_kernel, float eps, float skip_weight, float* packed, float* colors_out,
+                          int C_kernel, float eps, float skip_weight, float skip_fraction, float* packed,
+                          float* colors_out,
                           igs_stream_t stream) {
     if (!gs_feature || !packed || !colors_out) return IGS_ERR_NULL_POINTER;
     if (!shape_ok(B, N, 1, 1)) return IGS_ERR_BAD_SHAPE;
     if (C < 1 || C > C_kernel || !channels_compiled(C_kernel)) return IGS_ERR_BAD_CHANNELS;
     float limit;
-    if (const int rc = limit_from_skip_weight(skip_weight, &limit)) return rc;
+    if (const int rc = limit_from_skip_weight(skip_weight, skip_fraction, &limit)) return rc;
     const int Np = (N + 3) & ~3;
     hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
-                       rec_stride_of(C_kernel), eps, limit, packed,
+                       rec_stride_of(C_kernel), eps, limit, skip_fraction, packed,
                        const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
     return launch_status();
 }

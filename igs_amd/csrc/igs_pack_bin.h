@@ -14,6 +14,9 @@
 //     e < w / max(1, |alpha|), i.e. where both the weight alpha e and the bare exponential (which is
 //     what the gradient of alpha sums) are below w.  The limit of Gaussian n is
 //     L_n = min(kExactLimit, L + log2 max(1, |alpha_n|)).
+//   The boxes are made for the call's skip weight; k_bin may use a larger weight for a tile whose
+//   denominators it can bound from below (tile_weight_sum), which only removes more of what the box
+//   lets through.
 // The box is five binades wider than the tile test of k_bin (ellipse_reaches), as in the exact case.
 // Half extents: sqrt(Q Sigma_xx), sqrt(Q Sigma_yy) with Sigma the covariance that (A, B, D) invert.
 // A record with a non-finite field or a non-positive-definite (A, B, D) gets an unbounded box (its
@@ -45,10 +48,11 @@ __device__ __forceinline__ float4 empty_box() {
     return make_float4(inf, -inf, inf, -inf);
 }
 
-// The call's skip limit travels behind the reach boxes [B][Np] in the packed buffer (4 floats, the
-// first one used), where k_bin reads it: the forward and the backward then need no argument for it.
-__device__ __forceinline__ void write_skip_limit(float4* boxes, int B, int Np, float limit) {
-    boxes[(size_t)B * Np] = make_float4(fminf(limit, kExactLimit), 0.0f, 0.0f, 0.0f);
+// The call's skip limit and skip fraction travel behind the reach boxes [B][Np] in the packed buffer
+// (4 floats, the first two used), where k_bin reads them: the forward and the backward then need no
+// argument for them.
+__device__ __forceinline__ void write_skip_limit(float4* boxes, int B, int Np, float limit, float fraction) {
+    boxes[(size_t)B * Np] = make_float4(fminf(limit, kExactLimit), fraction, 0.0f, 0.0f);
 }
 
 // One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
@@ -62,11 +66,12 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
                                                    const float* __restrict__ alphas,
                                                    const float* __restrict__ colors, int N,
                                                    int Np, int C, int RS, float eps,
-                                                   float limit, float* __restrict__ packed,
+                                                   float limit, float fraction,
+                                                   float* __restrict__ packed,
                                                    float4* __restrict__ boxes) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
-    if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit);
+    if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit, fraction);
     if (n >= Np) return;
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {  // padding: alpha = 0 and e = exp2(0) = 1, so it contributes exactly 0
@@ -132,12 +137,13 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
 __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restrict__ feat,
                                                            const float* __restrict__ pos_off, int N,
                                                            int Np, int C, int Cp, int RS, float eps,
-                                                           float limit, float* __restrict__ packed,
+                                                           float limit, float fraction,
+                                                           float* __restrict__ packed,
                                                            float4* __restrict__ boxes,
                                                            float* __restrict__ colors_out) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
-    if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit);
+    if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit, fraction);
     if (n >= Np) return;
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {
@@ -219,7 +225,7 @@ struct BinArgs {
     const int* cand_counts;  // [B][stiles][cand_K]
     const int* cand_lists;   // [B][stiles][Np], segment k at offset k cand_chunk
     int cand_K, cand_chunk, stiles_x, stiles;
-    const float* limit;  // the call's skip limit, written by the pack kernel behind the boxes
+    const float* limit;  // the call's skip limit and fraction, written by the pack kernel behind the boxes
     const int* flag;
     int want;
     int no_cull;  // list every candidate (IGS_OPT_NO_CULL): the reference point for "culling changes no bit"
@@ -265,6 +271,21 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
     const float mx = fmaxf(fabsf(x0), fabsf(x1)), my = fmaxf(fabsf(y0), fabsf(y1));
     const float T = a * mx * mx + fabsf(b2) * mx * my + d * my * my;
     return !(pmin - 4e-6f * T > skip_limit(limit, rec[5]));
+}
+
+// A Gaussian's smallest weight over the tile's coordinate rectangle: alpha 2^(-max P), P = -q' being
+// convex, its maximum over the rectangle is at a corner.  Summed over Gaussians with alpha >= 0 this
+// bounds every denominator of the tile from below.  Rounded down by 1e-3 against the fp32 rounding
+// of P at the corners (a few 1e-6 of its largest term, which matters only while 2^-P does).
+__device__ __forceinline__ float least_weight(const float* __restrict__ rec, float txlo, float txhi,
+                                              float tylo, float tyhi) {
+    const float4 h = *reinterpret_cast<const float4*>(rec);  // px, py, A', B2'
+    const float a = -h.z, b2 = -h.w, d = -rec[4];
+    const float x0 = txlo - h.x, x1 = txhi - h.x, y0 = tylo - h.y, y1 = tyhi - h.y;
+    auto form = [&](float x, float y) { return fmaf(fmaf(b2, x, d * y), y, a * x * x); };
+    const float pmax = fmaxf(fmaxf(form(x0, y0), form(x0, y1)), fmaxf(form(x1, y0), form(x1, y1)));
+    const float w = rec[5] * hw_exp2(-pmax) * 0.999f;
+    return w > 0.0f ? w : 0.0f;  // NaN, inf - inf and the like count as nothing
 }
 
 __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
@@ -315,7 +336,8 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         for (int k = kBinWaves / 2; k > 0; k >>= 1) rv[f] = fminf(rv[f], __shfl_xor(rv[f], k));
     }
     const float txlo = rv[0], txhi = -rv[1], tylo = rv[2], tyhi = -rv[3];
-    const float limit = *a.limit;
+    float limit = a.limit[0];
+    const float fraction = a.limit[1];
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     const float4* boxes = a.boxes + (size_t)b * a.Np;
@@ -358,6 +380,52 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     const unsigned long long below = (1ull << lane) - 1ull;
     // kU boxes per lane are loaded together, so that kU loads are in flight instead of one
     constexpr int kU = 8;
+    // Skip fraction f > 0: a tile whose denominators are all at least S (the sum of the least
+    // weights of the candidates whose box meets it; only if none of them has a negative or
+    // non-finite alpha) may skip pairs up to the weight w + f S instead of the call's w.  Not at the
+    // first level of a two-level binning (its lists must hold what any of its tiles may list), nor
+    // where nothing is culled.
+    if (fraction > 0.0f && a.chunk == 0 && txlo > -inf && !a.no_cull) {  // workgroup-uniform
+        float sum = 0.0f;
+        bool negative = false;
+        for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
+            int n[kU];
+            float4 bb[kU];
+#pragma unroll
+            for (int u = 0; u < kU; ++u) n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));
+#pragma unroll
+            for (int u = 0; u < kU; ++u) bb[u] = boxes[n[u]];
+#pragma unroll
+            for (int u = 0; u < kU; ++u) {
+                if (n0 + u * 64 + lane >= ne) continue;
+                if (bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi) continue;
+                const float* rec = recs + (size_t)n[u] * a.RS;
+                negative = negative || !(rec[5] >= 0.0f);
+                // (records that are never skipped have unbounded boxes: NaN fields or a form that is
+                // not positive definite; with alpha >= 0 they can only raise a denominator)
+                if (bb[u].x > -inf) sum += least_weight(rec, txlo, txhi, tylo, tyhi);
+            }
+        }
+#pragma unroll
+        for (int k = 32; k > 0; k >>= 1) sum += __shfl_xor(sum, k);  // fixed order: the lists are reproducible
+        const bool wneg = __ballot(negative) != 0ull;
+        __syncthreads();  // red[] was read above
+        if (lane == 0) {
+            red[0][wave] = sum;
+            red[1][wave] = wneg ? 1.0f : 0.0f;
+        }
+        __syncthreads();
+        float total = 0.0f, anyneg = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kBinWaves; ++w) {
+            total += red[0][w];
+            anyneg += red[1][w];
+        }
+        if (anyneg == 0.0f && total > 0.0f) {
+            const float w0 = limit < kExactLimit ? hw_exp2(-limit) : 0.0f;
+            limit = fminf(limit, -__log2f(w0 + fraction * total));
+        }
+    }
     auto classify = [&](int n0, bool (&listed)[kU], bool (&in)[kU], int (&n)[kU]) {
         float4 bb[kU];
 #pragma unroll

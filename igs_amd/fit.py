@@ -151,7 +151,7 @@ class GaussianImageFit:
     def _enqueue_render(self, n: int, ws: dict, st):
         lib, g, p = self.lib, self.grid, ws["plan"]
         B, C, Cp, H, W = self.B, self.C, self.Cp, g.H, g.W
-        _lib.check(lib.igs_gs2d_pack_feature(_ptr(self.params), None, B, n, C, Cp, self.eps, ws["skip_weight"],
+        _lib.check(lib.igs_gs2d_pack_feature(_ptr(self.params), None, B, n, C, Cp, self.eps, *ws["skip_weight"],
                                              _ptr(ws["packed"]), _ptr(ws["col"]), st), "igs_gs2d_pack_feature")
         _lib.check(lib.igs_gs2d_forward(_ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n,
                                         H, W, Cp, self.eps, _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]),

@@ -43,7 +43,8 @@ typedef enum igs_status {
     IGS_ERR_ALIGNMENT = -7,      /* a buffer that must be 16-byte aligned is not */
     IGS_ERR_STATIC_SCRATCH = -8, /* igs_gs2d_forward_static_ws: the plan's fwd_ws_bytes exceeds
                                     IGS_STATIC_SCRATCH_BYTES */
-    IGS_ERR_BAD_SKIP_WEIGHT = -9 /* a pack call's skip_weight is negative, NaN or >= 1 */
+    IGS_ERR_BAD_SKIP_WEIGHT = -9 /* a pack call's skip_weight or skip_fraction is negative, NaN
+                                    or >= 1 */
 } igs_status;
 
 /* How the pixel coordinates are described.
@@ -97,7 +98,7 @@ typedef struct igs_gs2d_plan_t {
     int32_t bwd_per_tile;    /* rows (separable) or pixels (general) per backward tile     */
     int32_t pix_stride;      /* floats per pixel record of the backward prologue           */
     uint64_t packed_bytes;   /* packed Gaussian buffer: records, then one reach box (4
-                                floats) per record, then the call's skip limit (4 floats):
+                                floats) per record, then the call's skip settings (4 floats):
                                 (B*n_padded*(rec_stride+4) + 4)*4                          */
     uint64_t fwd_ws_bytes;   /* forward scratch: split partials (fwd_split > 1) and, on
                                 separable grids, the per-tile Gaussian lists (plus those
@@ -123,12 +124,11 @@ int igs_gs2d_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_pla
 int igs_gs2d_grid_classify(const float *x, const float *y, const int64_t grid_strides[6], int B,
                            int H, int W, int32_t *grid_flag, igs_stream_t stream);
 
-/* Skip weight for a problem of N Gaussians per image whose forward will run with `eps`:
- * tolerance * eps / (2 N) (0 when eps <= 0 or tolerance <= 0).  With it, what the kernels skip
- * changes every output element by at most tolerance * max|colors| (see igs_gs2d_pack_covinv);
- * the host side of this build passes tolerance = 1e-7 against the 1e-6 + 1e-5 |ref| that the
- * forward is held to.  Pure host arithmetic; no counterpart in the reference, which evaluates
- * every pair. */
+/* tolerance * eps / (2 N) (0 when eps <= 0 or tolerance <= 0), capped at 0.5: the skip_weight, and
+ * with eps = 1 the skip_fraction, with which what the kernels skip changes every output element
+ * by at most tolerance * max|colors| (see igs_gs2d_pack_covinv).  The host side of this build
+ * passes tolerance = 1e-7 against the 1e-6 + 1e-5 |ref| that the forward is held to.  Pure host
+ * arithmetic; no counterpart in the reference, which evaluates every pair. */
 float igs_gs2d_skip_weight(int N, float eps, float tolerance);
 
 /* Pack per-Gaussian parameters for the kernels (operator level: the caller already has
@@ -139,17 +139,22 @@ float igs_gs2d_skip_weight(int N, float eps, float tolerance);
  * limit.  On separable grids the forward and the backward skip, per pixel tile (and the forward
  * per wave of rows), the Gaussians whose box misses the tile or whose ellipse does not reach the
  * tile's coordinate rectangle (the reference evaluates every pair:
- * src/igs/gs_triton_chunked.py:100-200).  What may be skipped is set by skip_weight, 0 <= w < 1:
- *   w = 0: only pairs whose exponential is exactly 0 in fp32.  The order of the other terms is
- *     kept, so results equal those of not skipping bit for bit while the forward runs one
+ * src/igs/gs_triton_chunked.py:100-200).  What may be skipped is set by skip_weight w and
+ * skip_fraction f, both in [0, 1):
+ *   w = f = 0: only pairs whose exponential is exactly 0 in fp32.  The order of the other terms
+ *     is kept, so results equal those of not skipping bit for bit while the forward runs one
  *     Gaussian split (plan.fwd_split == 1), and to fp32 rounding otherwise, where a tile's list
  *     rather than the index range is cut into the splits.
- *   w > 0: only pairs with exp(-q/2) < w / max(1, |alpha|), so that both the weight alpha e and
- *     the bare exponential (which the gradient of alpha sums) are below w.  Per pixel the skipped
- *     weights then add up to at most N w: den changes by at most N w and an output element by at
- *     most N w (max|colors| + |out|) / (den + eps) <= 2 N w max|colors| / eps for den >= 0; every
- *     per-Gaussian gradient sum misses terms of at most w |G| |moment| per pixel.
- *     igs_gs2d_skip_weight gives the w for a wanted bound.
+ *   otherwise: only pairs with exp(-q/2) max(1, |alpha|) < w + f S, so that both the weight
+ *     alpha e and the bare exponential (which the gradient of alpha sums) are below that.  S is
+ *     a lower bound of the denominators of the pixel tile the pair is skipped for: the sum, over
+ *     the Gaussians whose box meets the tile, of the least weight each has on it (0 if one of
+ *     them has a negative or non-finite alpha).  Per pixel the skipped weights then add up to at
+ *     most N (w + f S): den changes by at most that and an output element by at most
+ *     N (w + f S) (max|colors| + |out|) / (den + eps) <= 2 N max|colors| max(w / eps, f) for
+ *     den >= S; every per-Gaussian gradient sum misses terms of at most (w + f S) |G| |moment|
+ *     per pixel, |G| <= 2 max|colors| |grad_out| / (den + eps).  igs_gs2d_skip_weight gives w
+ *     and f for a wanted bound.
  * Records with a non-finite field or a cov_inv that is not positive definite are never skipped;
  * with IGS_OPT_NO_CULL in a forward / backward call's grid_mode nothing is.
  * Large problems (tiles x N >= 2^25) build the per-tile lists in two levels (super-tiles of
@@ -158,14 +163,15 @@ float igs_gs2d_skip_weight(int N, float eps, float tolerance);
  * gradients agree to fp32 rounding. */
 int igs_gs2d_pack_covinv(const float *position, const float *cov_inv_00, const float *cov_inv_01,
                          const float *cov_inv_11, const float *alphas, const float *colors,
-                         int B, int N, int C, float skip_weight, float *packed,
-                         igs_stream_t stream);
+                         int B, int N, int C, float skip_weight, float skip_fraction,
+                         float *packed, igs_stream_t stream);
 
 /* Same, from scales [B,N,2] and rotations [B,N]: closed form of
  * (R S S^T R^T + eps I)^-1, replacing src/igs/gs2d.py:548-580. */
 int igs_gs2d_pack_scale_rot(const float *positions, const float *scales, const float *rotations,
                             const float *alphas, const float *colors, int B, int N, int C,
-                            float eps, float skip_weight, float *packed, igs_stream_t stream);
+                            float eps, float skip_weight, float skip_fraction, float *packed,
+                            igs_stream_t stream);
 
 /* Forward: out [B,C,H,W] = sum_n w_n c_n / (sum_n w_n + eps), den [B,H,W] = sum_n w_n.
  * Replaces the forward of src/igs/gs2d.py:68-144 / src/igs/gs_triton_chunked.py:551-680.
@@ -276,11 +282,11 @@ int igs_gs2d_finalize_scale_rot(const float *partial, int grid_mode, const int32
  * NULL (pos_map_offset, src/igs/gs2d.py:654-667).  C_kernel is the compiled channel count
  * (>= C) the other calls are made with; colors_out [B,N,C_kernel] receives the zero-padded raw
  * colours for igs_gs2d_backward.  g_feature [B,N,6+C] gets d L / d gs_feature (0 for the
- * opacity logit); d L / d pos_offset equals its first two columns.  skip_weight: as in
- * igs_gs2d_pack_covinv. */
+ * opacity logit); d L / d pos_offset equals its first two columns.  skip_weight, skip_fraction:
+ * as in igs_gs2d_pack_covinv. */
 int igs_gs2d_pack_feature(const float *gs_feature, const float *pos_offset, int B, int N, int C,
-                          int C_kernel, float eps, float skip_weight, float *packed,
-                          float *colors_out, igs_stream_t stream);
+                          int C_kernel, float eps, float skip_weight, float skip_fraction,
+                          float *packed, float *colors_out, igs_stream_t stream);
 int igs_gs2d_finalize_feature(const float *partial, int grid_mode, const int32_t *grid_flag,
                               const float *gs_feature, int B, int N, int H, int W, int C,
                               int C_kernel, float eps, float *g_feature, igs_stream_t stream);

@@ -266,6 +266,30 @@ def skip_limit(alphas, w: float):
     return torch.clamp(-math.log2(w) + torch.log2(torch.clamp(alphas.abs(), min=1.0)), max=EXACT_LIMIT)
 
 
+def tile_weight_floor(px, py, a, b_, d, alphas, xlo, xhi, ylo, yhi):
+    """Lower bound of the denominator sum_n alpha_n exp(-q_n / 2) at every point of the rectangle
+    [xlo, xhi] x [ylo, yhi], for alphas >= 0 (else 0): q_n is convex, so its maximum over the
+    rectangle is at a corner and exp(-max q_n / 2) is the least weight Gaussian n has on it.
+    Sums over the last dimension of the Gaussian tensors.  Test infrastructure's restatement of the
+    per-tile bound of the HIP binning kernel (no counterpart in the reference)."""
+    if bool((alphas < 0).any()) or not bool(torch.isfinite(alphas).all()):
+        return torch.zeros(alphas.shape[:-1], dtype=alphas.dtype)
+    qmax = None
+    for xe in (xlo, xhi):
+        for ye in (ylo, yhi):
+            dx, dy = xe - px, ye - py
+            q = a * dx * dx + 2 * b_ * dx * dy + d * dy * dy
+            qmax = q if qmax is None else torch.maximum(qmax, q)
+    return (alphas * torch.exp(-0.5 * qmax)).sum(-1)
+
+
+def tile_skip_weight(w: float, f: float, floor):
+    """Weight below which pairs of a tile may be skipped: the call's skip weight plus the skip
+    fraction of the tile's denominator floor.  With w = tolerance eps / (2 N), f = tolerance / (2 N):
+    N (w + f S) (max|c| + |out|) / (den + eps) <= tolerance max|c| wherever den >= S."""
+    return w + f * floor
+
+
 def reach_q(alphas, w: float):
     """q_max of each Gaussian's reach box under skip weight w: five binades beyond its skip limit
     (the exact-zero case gives REACH_Q)."""

@@ -104,12 +104,13 @@ def test_argument_errors_are_status_codes_not_crashes(lib):
     fake = ctypes.c_void_p(4096)
     st = _lib.strides6((0, 0, 1), (0, 4, 0))
     assert lib.igs_gs2d_forward(None, None, None, st, 1, None, 1, 8, 4, 4, 3, 1e-6, None, None, None, 0, None) == -1
-    assert lib.igs_gs2d_pack_covinv(None, None, None, None, None, None, 1, 8, 3, 0.0, None, None) == -1
+    assert lib.igs_gs2d_pack_covinv(None, None, None, None, None, None, 1, 8, 3, 0.0, 0.0, None, None) == -1
     # the skip weight of a pack call: 0 <= w < 1
     for bad in (-1e-9, 1.0, float("nan")):
-        assert lib.igs_gs2d_pack_covinv(fake, fake, fake, fake, fake, fake, 1, 8, 3, bad, fake, None) == -9
-        assert lib.igs_gs2d_pack_scale_rot(fake, fake, fake, fake, fake, 1, 8, 3, 1e-6, bad, fake, None) == -9
-        assert lib.igs_gs2d_pack_feature(fake, None, 1, 8, 3, 3, 1e-6, bad, fake, fake, None) == -9
+        assert lib.igs_gs2d_pack_covinv(fake, fake, fake, fake, fake, fake, 1, 8, 3, bad, 0.0, fake, None) == -9
+        assert lib.igs_gs2d_pack_covinv(fake, fake, fake, fake, fake, fake, 1, 8, 3, 0.0, bad, fake, None) == -9
+        assert lib.igs_gs2d_pack_scale_rot(fake, fake, fake, fake, fake, 1, 8, 3, 1e-6, bad, 0.0, fake, None) == -9
+        assert lib.igs_gs2d_pack_feature(fake, None, 1, 8, 3, 3, 1e-6, 0.0, bad, fake, fake, None) == -9
     assert b"skip weight" in lib.igs_status_string(-9)
     # tolerance * eps / (2 N); nothing may be skipped without an eps to measure against
     assert lib.igs_gs2d_skip_weight(8192, 1e-6, 1e-7) == pytest.approx(1e-13 / 16384, rel=1e-6)

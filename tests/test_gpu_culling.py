@@ -366,7 +366,7 @@ def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev, tolerance):
     with library_options(skip_tolerance=tolerance):
         op = Splat(B, N, C, grid, 1e-6, dev)
     w = O.skip_weight(N, 1e-6, tolerance)
-    assert op.skip_weight == pytest.approx(w, rel=1e-6)
+    assert op.skip_weight == pytest.approx((w, O.skip_weight(N, 1.0, tolerance)), rel=1e-6)
     a, b, dd = O.cov_inverse_closed(d64["scales"].float().double(), d64["rotations"].float().double())
     pos = d64["positions"].float().double()
 
@@ -395,8 +395,9 @@ def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev, tolerance):
         assert bool((out <= slack * half + 1e-6).all()), (name, float((out / half).max()))
         pad = boxes(packed)[:, N:]
         assert bool((pad[..., 0] > pad[..., 1]).all())  # padding records: empty boxes
-        limit = float(packed[B * op.plan.n_padded * (op.plan.rec_stride + 4)])
+        limit, fraction = packed[B * op.plan.n_padded * (op.plan.rec_stride + 4):][:2].tolist()
         assert limit == pytest.approx(O.EXACT_LIMIT if w == 0 else min(O.EXACT_LIMIT, -math.log2(w)), rel=1e-6)
+        assert fraction == pytest.approx(O.skip_weight(N, 1.0, tolerance), rel=1e-6)
     if tolerance > 0:    # smaller boxes than the exact-zero ones, by sqrt of the limits' ratio
         ratio = math.sqrt((-math.log2(w) + 5) / (O.EXACT_LIMIT + 5))
         exact_box = O.reach_box(pos, a, b, dd)
@@ -425,17 +426,21 @@ def _tile_counts(op, packed, dev):
     return pix.view(torch.int32)[(scratch + 15) // 16 * 4:][: B * p.bwd_tiles].view(B, -1, p.bwd_tiles_x).cpu()
 
 
-@pytest.mark.parametrize("tolerance", [0.0, 1e-7], ids=lambda t: f"tol{t:g}")
-def test_tile_lists_against_the_oracle_s_rectangle_minimum(igs, dev, tolerance):
+@pytest.mark.parametrize("tolerance,scales", [(0.0, (0.004, 0.15)), (1e-7, (0.004, 0.15)), (1e-7, (0.03, 0.3))],
+                         ids=["exact-sparse", "default-sparse", "default-dense"])
+def test_tile_lists_against_the_oracle_s_rectangle_minimum(igs, dev, tolerance, scales):
     """What the binning lists for each backward tile against the oracle: a Gaussian whose minimum
     of -q' over the tile's coordinate rectangle (`min_q_over_rect`) is below its skip limit must be
     listed; one whose minimum is beyond the limit by more than the kernel's rounding allowance must
     not (aspect ratios stay far below the 1:600 beyond which the kernel lists an ellipse anyway).
+    The limit of a tile comes from the call's skip weight plus the skip fraction of the tile's
+    denominator floor (`tile_weight_floor`; the kernel rounds its floor down by 1e-3 and sums only
+    the Gaussians whose box meets the tile, which differ by less than that).
     Counted per tile: must <= listed <= may."""
     from igs_amd._splat import Grid, Splat, _f32c, library_options
 
     B, N, H, W, C = 2, 900, 96, 200, 3
-    d64, g = sparse_case(dev, B, N, H, W, C, seed=19, smin=0.004, smax=0.15)
+    d64, g = sparse_case(dev, B, N, H, W, C, seed=19, smin=scales[0], smax=scales[1])
     g["alphas"] = (g["alphas"] * 3).contiguous()
     with library_options(skip_tolerance=tolerance):
         op = Splat(B, N, C, Grid(g["x_grid"], g["y_grid"], B), 1e-6, dev)
@@ -446,26 +451,34 @@ def test_tile_lists_against_the_oracle_s_rectangle_minimum(igs, dev, tolerance):
     a, b, dd = (t.reshape(B, N) for t in O.cov_inverse_closed(d64["scales"].float().double(),
                                                                d64["rotations"].float().double()))
     pos = d64["positions"].float().double()
-    lim = O.skip_limit(g["alphas"].cpu().double(), O.skip_weight(N, 1e-6, tolerance))
+    al = g["alphas"].cpu().double()
+    w, f = O.skip_weight(N, 1e-6, tolerance), O.skip_weight(N, 1.0, tolerance)
     xs, ys = g["x_grid"][0, 0, 0, :].cpu().double(), g["y_grid"][0, 0, :, 0].cpu().double()
     k = 0.5 * 1.4426950408889634
     saw_less = False
+    floors = []
     for ty in range(counts.shape[1]):
         for tx in range(counts.shape[2]):
             r0, r1 = ty * p.bwd_per_tile, min(H, (ty + 1) * p.bwd_per_tile)
             c0, c1 = tx * 64, min(W, (tx + 1) * 64)
             m = k * O.min_q_over_rect(pos[..., 0], pos[..., 1], a, b, dd, xs[c0], xs[c1 - 1], ys[r0], ys[r1 - 1])
+            S = O.tile_weight_floor(pos[..., 0], pos[..., 1], a, b, dd, al, xs[c0], xs[c1 - 1], ys[r0], ys[r1 - 1])
+            floors.append(S)
+            lim_lo = torch.stack([O.skip_limit(al[i], float(O.tile_skip_weight(w, f, S[i]))) for i in range(B)])
+            lim_hi = torch.stack([O.skip_limit(al[i], float(O.tile_skip_weight(w, f, 0.997 * S[i]))) for i in range(B)])
             # the kernel's allowance for the fp32 rounding of its own evaluation: 4e-6 of the largest
             # term of the form over the rectangle (here with a little room for its rounding)
             mx = torch.maximum((xs[c0] - pos[..., 0]).abs(), (xs[c1 - 1] - pos[..., 0]).abs())
             my = torch.maximum((ys[r0] - pos[..., 1]).abs(), (ys[r1 - 1] - pos[..., 1]).abs())
             T = k * (a * mx * mx + 2 * b.abs() * mx * my + dd * my * my)
-            must = (m <= lim * (1 - 1e-4)).sum(1)
-            may = (m - 5e-6 * T <= lim * (1 + 1e-4) + 1e-3).sum(1)
+            must = (m <= lim_lo * (1 - 1e-4)).sum(1)
+            may = (m - 5e-6 * T <= lim_hi * (1 + 1e-4) + 1e-3).sum(1)
             got = counts[:, ty, tx]
             assert bool((must <= got).all()) and bool((got <= may).all()), (ty, tx, must, got, may)
             saw_less = saw_less or bool((got < N).any())
     assert saw_less
+    if scales[0] > 0.01:    # the scene is dense enough for the floors to matter: they beat the call's weight
+        assert float(torch.stack(floors).median()) * f > 10 * w
 
 
 @pytest.mark.parametrize("alpha_scale", [1.0, 25.0])

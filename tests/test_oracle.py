@@ -349,7 +349,8 @@ def test_skip_weight_bound_by_brute_force():
     fp64 with and without the pairs that `skip_limit` allows to drop (e < w / max(1, |alpha|)) on
     scenes built to be the worst case -- sparse small Gaussians, so that many pixels have a
     denominator far below eps and nearly everything they see is below the weight, alphas of either
-    magnitude -- and check |d out| <= tolerance max|c| with w = skip_weight(N, eps, tolerance), that
+    magnitude -- and check |d out| <= tolerance max|c| with w = skip_weight(N, eps, tolerance) (then
+    also on a dense scene with the per-tile weight w + f S, S the tile's denominator floor), that
     the bound is not vacuous (a constructed pixel comes within a factor 2.1 of it) and that each per-Gaussian sum of exponentials, which is what the gradient of
     alpha adds up, loses less than w per pixel.  A missing factor N, eps or 2, or a limit that
     ignores |alpha| > 1, fails the first check."""
@@ -393,6 +394,40 @@ def test_skip_weight_bound_by_brute_force():
     assert float(e[1]) < w and bool(0.5 * math.log2(math.e) * (xs[1] / sig) ** 2 > O.skip_limit(torch.ones(1, dtype=F64), w))
     full = N * e[1] / (N * e[1] + eps)
     assert tol / 2.1 <= float(full) <= tol                         # kept: 0
+    # With the skip fraction: a dense scene cut into tiles, each tile skipping up to
+    # w + f S (S = tile_weight_floor, which must bound the tile's denominators from below).
+    N, H, W = 300, 48, 64
+    tol = 1e-3
+    pos = torch.rand(1, N, 2, generator=g, dtype=F64) * 2 - 1
+    sc = torch.rand(1, N, 2, generator=g, dtype=F64) * 0.25 + 0.02
+    rot = torch.rand(1, N, generator=g, dtype=F64) * 2 * math.pi
+    al = torch.rand(1, N, generator=g, dtype=F64)
+    col = torch.rand(1, N, C, generator=g, dtype=F64) * 2 - 1
+    a, b, d = (t.reshape(1, N) for t in O.cov_inverse_closed(sc, rot, eps))
+    xs, ys = torch.linspace(-1, 1, W, dtype=F64), torch.linspace(-1, 1, H, dtype=F64)
+    dx, dy = xs.view(1, 1, 1, W) - pos[..., 0, None, None], ys.view(1, 1, H, 1) - pos[..., 1, None, None]
+    q = a[..., None, None] * dx * dx + 2 * b[..., None, None] * dx * dy + d[..., None, None] * dy * dy
+    e = torch.exp(-0.5 * q)
+    den = (e * al[..., None, None]).sum(1)
+    w, f = O.skip_weight(N, eps, tol), O.skip_weight(N, 1.0, tol)
+    assert f == tol / (2 * N)
+    drop = torch.zeros_like(e, dtype=torch.bool)
+    gained = 0
+    for r0 in range(0, H, 16):
+        for c0 in range(0, W, 16):
+            S = O.tile_weight_floor(pos[..., 0], pos[..., 1], a, b, d, al, xs[c0], xs[c0 + 15], ys[r0], ys[r0 + 15])
+            assert bool((den[:, r0:r0 + 16, c0:c0 + 16] >= S[:, None, None] * (1 - 1e-12)).all())     # a floor indeed
+            assert float(S) > 100 * eps                                                              # and not a vacuous one
+            wt = O.tile_skip_weight(w, f, S)
+            et = e[:, :, r0:r0 + 16, c0:c0 + 16]
+            drop[:, :, r0:r0 + 16, c0:c0 + 16] = et < wt
+            gained += int((et < wt).sum()) - int((et < w).sum())
+    assert gained > 0.05 * e.numel()                                 # the fraction is what skips most here
+    full = torch.einsum("bnhw,bnc->bchw", e * al[..., None, None], col) / (den[:, None] + eps)
+    ek = torch.where(drop, torch.zeros_like(e), e) * al[..., None, None]
+    kept = torch.einsum("bnhw,bnc->bchw", ek, col) / (ek.sum(1)[:, None] + eps)
+    assert float((full - kept).abs().max()) <= tol * float(col.abs().max())
+    assert float(O.tile_weight_floor(pos[..., 0], pos[..., 1], a, b, d, -al, xs[0], xs[5], ys[0], ys[5])) == 0.0
     assert O.skip_weight(100, 0.0, 1e-7) == 0.0 and O.skip_weight(100, 1e-6, 0.0) == 0.0
     assert bool((O.skip_limit(torch.tensor([0.5, 4.0]), 0.0) == O.EXACT_LIMIT).all())
     assert math.isclose(float(O.reach_q(torch.tensor([1.0], dtype=F64), 0.0)[0]), O.REACH_Q, rel_tol=1e-12)
