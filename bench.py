@@ -229,7 +229,8 @@ def main() -> int:
     scratch = (B * H * plan.w_padded * plan.pix_stride + B * plan.w_padded) * 4
     counts = pix.view(torch.int32)[(scratch + 15) // 16 * 4:][: B * plan.bwd_tiles].view(B, -1, plan.bwd_tiles_x).cpu()
     rows = torch.tensor([min(H, (i + 1) * plan.bwd_per_tile) - i * plan.bwd_per_tile for i in range(counts.shape[1])])
-    cols = torch.tensor([min(W, (i + 1) * 64) - i * 64 for i in range(plan.bwd_tiles_x)])
+    tw = plan.bwd_tile_w
+    cols = torch.tensor([min(W, (i + 1) * tw) - i * tw for i in range(plan.bwd_tiles_x)])
     evaluated = int((counts.long() * (rows[:, None] * cols[None, :])[None]).sum())
     achieved = evaluated * f_bwd / t_bwd_kernel / 1e12
     prof = C1_PROFILE if (args.config == "c1" and C == 3) else None

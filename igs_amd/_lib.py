@@ -46,6 +46,7 @@ class Plan(ctypes.Structure):
         ("partial_bytes", c_uint64),
         ("fwd_tiles", c_int32),
         ("bwd_tiles_x", c_int32),
+        ("bwd_tile_w", c_int32),
     ]
 
 

@@ -191,7 +191,7 @@ constexpr int kBwdMaxRows = IGS_BWD_MAX_ROWS;
 #endif
 constexpr int kBwdMinRows = IGS_BWD_MIN_ROWS;
 #ifndef IGS_BWD_TILE_W
-#define IGS_BWD_TILE_W 64
+#define IGS_BWD_TILE_W 32
 #endif
 constexpr int kBwdTileW = IGS_BWD_TILE_W;
 

@@ -37,11 +37,18 @@ template <int C>
 struct GRec {
     float px, py, A, B2, D, al;
     float ac[C];
-    float ylo, yhi;  // y range of the reach box (records with two spare floats only)
+    float ylo, yhi;  // y range of the reach box (records with two spare floats only); in the separable
+                     // forward's LDS copy ylo holds the wave mask of the tile's list entry instead
 };
 
 // whether a record of C channels has room for the y range of the reach box
 __host__ __device__ constexpr bool rec_has_yrange(int C) { return rec_stride_of(C) >= 8 + C; }
+// List entries of the separable forward: Gaussian index in the low 24 bits, wave mask above (k_bin).
+constexpr int kListIndexMask = 0xffffff;
+// Wave masks are built for the variants whose waves hold 16 rows (C <= 3); with fewer rows per wave
+// the tile is small already and the four extra ellipse tests per Gaussian cost the binning more than
+// the forward gains: those variants test the reach box's y range against the wave's rows instead.
+__host__ __device__ constexpr bool fwd_wave_masks(int C) { return rec_has_yrange(C) && fwd_sep_p(C) >= 16; }
 
 // Unpacks one record held in R4 float4 registers (read from a wave-uniform LDS address).
 template <int C>
@@ -98,8 +105,9 @@ constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
 // once per record with a wave-uniform LDS pointer.  Records past `count` in the last chunk
 // read as all-zero (for a Gaussian record: alpha = 0, adds exactly 0).  Must be called by all
 // kThreads threads of the workgroup (it contains barriers).
-// With kGather, record i of the stream is src record index[i] (a tile's Gaussian list).
-template <int R4, int CH, bool kGather = false, class Body>
+// With kGather, record i of the stream is src record (index[i] & kListIndexMask) (a tile's Gaussian
+// list); kMaskSlot >= 0 then puts the entry's bits 24.. into float kMaskSlot of the record's LDS copy.
+template <int R4, int CH, bool kGather = false, int kMaskSlot = -1, class Body>
 __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
                                                    float4* sh, Body&& body,
                                                    const int* __restrict__ index = nullptr) {
@@ -125,10 +133,18 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
         for (int i = 0; i < PRE; ++i) {
             const int e = i * kThreads + tid, ge = chunk * E + e;
             const bool valid = e < E && ge < total;
-            if (kGather)
-                pre[i] = valid ? src[(size_t)idx[i] * R4 + (ge % R4)] : zero;
-            else
+            if (kGather) {
+                pre[i] = valid ? src[(size_t)(idx[i] & kListIndexMask) * R4 + (ge % R4)] : zero;
+                if (kMaskSlot >= 0 && ge % R4 == kMaskSlot / 4) {
+                    const float m = __int_as_float(idx[i] >> 24);
+                    if (kMaskSlot % 4 == 0) pre[i].x = m;
+                    if (kMaskSlot % 4 == 1) pre[i].y = m;
+                    if (kMaskSlot % 4 == 2) pre[i].z = m;
+                    if (kMaskSlot % 4 == 3) pre[i].w = m;
+                }
+            } else {
                 pre[i] = valid ? src[ge] : zero;
+            }
         }
     };
     load_idx(0);
@@ -248,9 +264,14 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
     auto body = [&](auto wave_skip, const float4* r) {
         const GRec<C> g = lds_grec<C>(r);
-        // The tile list is per workgroup (4 waves of P rows each); a wave whose own rows the
-        // reach box misses skips the record (wave-uniform: the record is the same in all lanes).
-        if (decltype(wave_skip)::value && __ballot(!(g.yhi < wylo || g.ylo > wyhi)) == 0ull) return;
+        // The tile list is per workgroup (4 waves of 64 columns x P rows each); a wave that the entry's
+        // mask does not name, or whose rows the reach box misses, skips the record (wave-uniform: the
+        // record is the same in all lanes).
+        if (decltype(wave_skip)::value) {
+            if (fwd_wave_masks(C) ? __ballot((__float_as_int(g.ylo) >> wave) & 1) == 0ull
+                                  : __ballot(!(g.yhi < wylo || g.ylo > wyhi)) == 0ull)
+                return;
+        }
         const float dx = xv - g.px;
         const float adx = g.A * dx;
         const float c0 = adx * dx;
@@ -277,7 +298,7 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     // that fewer than 7/8 of the Gaussians reach (workgroup-uniform choice of the loop): there
     // some boxes are small against the image, and those are often small against the tile too.
     if (rec_has_yrange(C) && 8L * count < 7L * a.Np)
-        stream_records_lds<R4, kGaussChunk, true>(
+        stream_records_lds<R4, kGaussChunk, true, fwd_wave_masks(C) ? 6 + C : -1>(
             src, n1 - n0, sh, [&](const float4* r) { body(std::true_type{}, r); }, list);
     else
         stream_records_lds<R4, kGaussChunk, true>(

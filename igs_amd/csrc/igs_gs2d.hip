@@ -183,6 +183,7 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     const long groups = (long)B * ceil_div(N, kThreads * (sep ? kBwdG : bwd_gen_g(C))) * 4;  // waves per tile
     long T = ((long)cus * 4 * IGS_BWD_WAVES + groups - 1) / groups;     // backward: waves per SIMD wanted
     p->bwd_tiles_x = sep ? ceil_div(p->w_padded, kBwdTileW) : 1;
+    p->bwd_tile_w = sep ? kBwdTileW : 0;
     if (sep) {
         T = (T + p->bwd_tiles_x - 1) / p->bwd_tiles_x;                  // row bands
         // small tiles keep the tile lists short when the Gaussians are small (a tile is skipped
@@ -314,6 +315,7 @@ int launch_bins(BinArgs fine, int B, bool levels2, const BinPlace& coarse, int* 
     c.tiles_x = sg.x; c.tiles_y = sg.y;
     c.counts = coarse.counts; c.lists = coarse.lists; c.slots = coarse_slots;
     c.chunk = sg.chunk;
+    c.sub_nx = 0; c.sub_h = 0;  // wave masks belong to the tiles' own lists
     int rc = launch_bin(c, sg.K, B, st);
     if (rc) return rc;
     fine.cand_counts = coarse.counts; fine.cand_lists = coarse.lists;
@@ -594,6 +596,9 @@ int forward_impl(const float* packed, const float* x, const float* y,
             ba.counts = bp.counts; ba.lists = bp.lists; ba.slots = nullptr;
             ba.flag = vs[i].flag; ba.want = vs[i].want;
             ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
+            // which of the workgroup's four waves a Gaussian reaches travels in its list entry
+            ba.sub_nx = fwd_wave_masks(C) ? fg.wx : 0;
+            ba.sub_h = fwd_sep_p(C);
             const bool levels2 = two_level(N, fg.tiles_x, fg.tiles_y, opts_of(grid_mode));
             const BinPlace cp = levels2 ? super_bins_at(ws, split_bytes, B, plan.fwd_tiles, plan.n_padded,
                                                         super_tiles(fg.tiles_x, fg.tiles_y, B, N).count)
@@ -837,6 +842,7 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
             ba.slots = slots_at(partial, B, a.T, 6 + C, N);
             ba.flag = a.flag; ba.want = a.want;
             ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
+            ba.sub_nx = 0; ba.sub_h = 0;
             const bool levels2 = two_level(N, ba.tiles_x, ba.tiles_y, opts_of(grid_mode));
             BinPlace cp{nullptr, nullptr};
             int* cslots = nullptr;

@@ -229,6 +229,11 @@ struct BinArgs {
     const int* flag;
     int want;
     int no_cull;  // list every candidate (IGS_OPT_NO_CULL): the reference point for "culling changes no bit"
+    // Wave masks (the forward's lists; sub_nx = 0: none).  The tile is sub_nx x (4 / sub_nx) rectangles of
+    // 64 columns x sub_h rows, one per wave of the forward's workgroup (wave w: column block w % sub_nx,
+    // row block w / sub_nx).  A Gaussian is listed when its ellipse reaches at least one of them, and bits
+    // 24..27 of its list entry say which (N <= 2^24 leaves them free).
+    int sub_nx, sub_h;
 };
 
 // Tiles per super-tile of the two-level binning (each way) and the most segments per list.
@@ -252,10 +257,11 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
     const float4 h = *reinterpret_cast<const float4*>(rec);  // px, py, A', B2'
     const float a = -h.z, b2 = -h.w, d = -rec[4];
     const float x0 = txlo - h.x, x1 = txhi - h.x, y0 = tylo - h.y, y1 = tyhi - h.y;
-    if (x0 <= 0.0f && x1 >= 0.0f && y0 <= 0.0f && y1 >= 0.0f) return true;
+    // straight-line code (every path is taken by some lane of a wave anyway)
+    const bool inside = x0 <= 0.0f && x1 >= 0.0f && y0 <= 0.0f && y1 >= 0.0f;
     // the argument below needs a form that is positive definite beyond the rounding of its
     // (fp32) coefficients; ellipses thinner than about 1:600 simply stay listed
-    if (!(a > 0.0f && 4.0f * a * d - b2 * b2 > 4e-5f * a * d)) return true;
+    const bool definite = a > 0.0f && 4.0f * a * d - b2 * b2 > 4e-5f * a * d;
     auto form = [&](float x, float y) { return fmaf(fmaf(b2, x, d * y), y, a * x * x); };
     auto clamp = [](float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); };
     // Only the edges that face the centre can hold the minimum: P grows along every ray from the
@@ -270,7 +276,8 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
     const float pmin = fminf(pv, ph);
     const float mx = fmaxf(fabsf(x0), fabsf(x1)), my = fmaxf(fabsf(y0), fabsf(y1));
     const float T = a * mx * mx + fabsf(b2) * mx * my + d * my * my;
-    return !(pmin - 4e-6f * T > skip_limit(limit, rec[5]));
+    const bool beyond = pmin - 4e-6f * T > skip_limit(limit, rec[5]);
+    return inside || !definite || !beyond;
 }
 
 // A Gaussian's smallest weight over the tile's coordinate rectangle: alpha 2^(-max P), P = -q' being
@@ -302,17 +309,31 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     const float inf = __builtin_inff();
     float xlo = inf, xhi = -inf, ylo = inf, yhi = -inf;
     bool bad = false;
-    for (int c = c0 + tid; c < c1; c += kBinThreads) {
-        const float v = a.x[b * a.sxb + (long)c * a.sxw];
-        bad = bad || !(v == v);
-        xlo = fminf(xlo, v);
-        xhi = fmaxf(xhi, v);
-    }
-    for (int r = r0 + tid; r < r1; r += kBinThreads) {
-        const float v = a.y[b * a.syb + (long)r * a.syh];
-        bad = bad || !(v == v);
-        ylo = fminf(ylo, v);
-        yhi = fmaxf(yhi, v);
+    const bool masks = a.sub_nx > 0;
+    if (!masks) {
+        for (int c = c0 + tid; c < c1; c += kBinThreads) {
+            const float v = a.x[b * a.sxb + (long)c * a.sxw];
+            bad = bad || !(v == v);
+            xlo = fminf(xlo, v);
+            xhi = fmaxf(xhi, v);
+        }
+        for (int r = r0 + tid; r < r1; r += kBinThreads) {
+            const float v = a.y[b * a.syb + (long)r * a.syh];
+            bad = bad || !(v == v);
+            ylo = fminf(ylo, v);
+            yhi = fmaxf(yhi, v);
+        }
+    } else if (wave < 4) {  // wave w takes the rectangle of the forward's wave w: its range is this wave's result
+        const int c = c0 + (wave % a.sub_nx) * 64 + lane;
+        const int r = r0 + (wave / a.sub_nx) * a.sub_h + lane;
+        if (c < c1) {
+            xlo = xhi = a.x[b * a.sxb + (long)c * a.sxw];
+            bad = !(xlo == xlo);
+        }
+        if (lane < a.sub_h && r < r1) {
+            ylo = yhi = a.y[b * a.syb + (long)r * a.syh];
+            bad = bad || !(ylo == ylo);
+        }
     }
     if (bad || a.no_cull) {  // a NaN coordinate, or culling switched off: nothing may be culled for this tile
         xlo = ylo = -inf;
@@ -336,6 +357,17 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         for (int k = kBinWaves / 2; k > 0; k >>= 1) rv[f] = fminf(rv[f], __shfl_xor(rv[f], k));
     }
     const float txlo = rv[0], txhi = -rv[1], tylo = rv[2], tyhi = -rv[3];
+    // the four waves' rectangles (xlo, xhi, ylo, yhi); one that is empty along an axis holds no pixel
+    float sub[4][4];
+    bool sub_any[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        sub[w][0] = masks ? red[0][w] : 0.0f;
+        sub[w][1] = masks ? -red[1][w] : 0.0f;
+        sub[w][2] = masks ? red[2][w] : 0.0f;
+        sub[w][3] = masks ? -red[3][w] : 0.0f;
+        sub_any[w] = sub[w][0] <= sub[w][1] && sub[w][2] <= sub[w][3];
+    }
     float limit = a.limit[0];
     const float fraction = a.limit[1];
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
@@ -426,7 +458,8 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             limit = fminf(limit, -__log2f(w0 + fraction * total));
         }
     }
-    auto classify = [&](int n0, bool (&listed)[kU], bool (&in)[kU], int (&n)[kU]) {
+    // code: which of the forward's waves the Gaussian reaches (wave masks), or 1; 0 = not listed
+    auto classify = [&](int n0, int (&code)[kU], bool (&in)[kU], int (&n)[kU]) {
         float4 bb[kU];
 #pragma unroll
         for (int u = 0; u < kU; ++u) n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));  // M > 0 inside the loops
@@ -436,25 +469,49 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         for (int u = 0; u < kU; ++u) {
             in[u] = n0 + u * 64 + lane < ne;
             // "definitely outside" negated, so that NaN bounds count as inside
-            listed[u] = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
+            const bool meets = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
+            code[u] = meets ? (masks ? 15 : 1) : 0;
             // bounded box (unbounded ones mark records that must never be skipped): refine
-            if (listed[u] && bb[u].x > -inf)
-                listed[u] = ellipse_reaches(recs + (size_t)n[u] * a.RS, txlo, txhi, tylo, tyhi, limit);
+            if (meets && bb[u].x > -inf) {
+                const float* rec = recs + (size_t)n[u] * a.RS;
+                if (masks) {
+                    code[u] = 0;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w)
+                        if (sub_any[w] && ellipse_reaches(rec, sub[w][0], sub[w][1], sub[w][2], sub[w][3], limit))
+                            code[u] |= 1 << w;
+#ifdef IGS_DEBUG_SUB
+                    if (n[u] == 2 && t == 0 && b == 0) {
+                        list[a.Np - 32] = code[u];
+                        list[a.Np - 31] = sub_any[0];
+                        list[a.Np - 30] = ellipse_reaches(rec, sub[0][0], sub[0][1], sub[0][2], sub[0][3], limit);
+                        list[a.Np - 29] = __float_as_int(limit);
+                        list[a.Np - 28] = __float_as_int(rec[0]);
+                        list[a.Np - 27] = __float_as_int(rec[5]);
+                        list[a.Np - 26] = __float_as_int(txlo);
+                        list[a.Np - 25] = __float_as_int(tyhi);
+                    }
+#endif
+                } else {
+                    code[u] = ellipse_reaches(rec, txlo, txhi, tylo, tyhi, limit) ? 1 : 0;
+                }
+            }
         }
     };
-    // the first pass keeps its verdicts (one bit per box of this lane) for the second one when
-    // they fit in a register pair, i.e. up to 64 boxes per lane (65536 candidates)
-    const bool keep = per_wave <= 64 * 64;
+    // the first pass keeps its verdicts (one bit, or four with wave masks, per box of this lane) for
+    // the second one when they fit in a register pair, i.e. up to 64 (16) boxes per lane
+    const int vbits = masks ? 4 : 1;
+    const bool keep = per_wave * vbits <= 64 * 64;
     unsigned long long verdicts = 0ull;
     int cnt = 0, it = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
-        bool listed[kU], in[kU];
-        int n[kU];
-        classify(n0, listed, in, n);
+        bool in[kU];
+        int code[kU], n[kU];
+        classify(n0, code, in, n);
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
-            cnt += __popcll(__ballot(listed[u]));
-            if (listed[u]) verdicts |= 1ull << ((it * kU + u) & 63);
+            cnt += __popcll(__ballot(code[u] != 0));
+            verdicts |= (unsigned long long)code[u] << (((it * kU + u) * vbits) & 63);
         }
     }
     if (lane == 0) wsum[wave] = cnt;
@@ -467,28 +524,34 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     }
     it = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
-        bool listed[kU], in[kU];
-        int n[kU];
+        bool in[kU];
+        int code[kU], n[kU];
         if (keep) {
 #pragma unroll
             for (int u = 0; u < kU; ++u) {
                 in[u] = n0 + u * 64 + lane < ne;
-                listed[u] = (verdicts >> ((it * kU + u) & 63)) & 1ull;
+                code[u] = (int)((verdicts >> (((it * kU + u) * vbits) & 63)) & (unsigned long long)((1 << vbits) - 1));
                 n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));
             }
         } else {
-            classify(n0, listed, in, n);
+            classify(n0, code, in, n);
         }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
-            const unsigned long long m = __ballot(listed[u]);
+            const bool listed = code[u] != 0;
+            const unsigned long long m = __ballot(listed);
             const int pos = base + __popcll(m & below);
-            if (listed[u]) list[pos] = n[u];
+            if (listed) list[pos] = masks ? (n[u] | (code[u] << 24)) : n[u];
             // the slot of every candidate: its position (within the segment, at the first level,
             // where only the sign is used) or -1
-            if (slot != nullptr && in[u]) slot[n[u]] = listed[u] ? pos : -1;
+            if (slot != nullptr && in[u]) slot[n[u]] = listed ? pos : -1;
             base += __popcll(m);
         }
     }
     if (tid == 0) a.counts[((size_t)b * tiles + t) * K + kc] = total;
+#ifdef IGS_DEBUG_SUB
+    if (tid == 0 && masks)
+        for (int w = 0; w < 4; ++w)
+            for (int f = 0; f < 4; ++f) list[a.Np - 16 + w * 4 + f] = __float_as_int(sub[w][f]);
+#endif
 }

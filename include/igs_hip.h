@@ -108,7 +108,8 @@ typedef struct igs_gs2d_plan_t {
     uint64_t partial_bytes;  /* backward partial sums B*T*(6+C)*N*4 and, on separable
                                 grids, the slot tables of the tiles (and super-tiles)       */
     int32_t fwd_tiles;       /* separable: pixel tiles per image of the forward            */
-    int32_t bwd_tiles_x;     /* separable: column bands (64 columns) of the backward tiles */
+    int32_t bwd_tiles_x;     /* separable: column bands of the backward tiles              */
+    int32_t bwd_tile_w;      /* separable: columns per band                                */
 } igs_gs2d_plan_t;
 
 int igs_abi_version(void);

@@ -74,7 +74,7 @@ def test_plan_arithmetic(lib, mode):
         assert p.bwd_tiles >= 1 and p.partial_bytes >= B * p.bwd_tiles * (6 + C) * N * 4
         if mode != 0:
             assert p.w_padded % 8 == 0 and p.bwd_tiles % p.bwd_tiles_x == 0
-            assert (p.bwd_tiles // p.bwd_tiles_x) * p.bwd_per_tile >= H and p.bwd_tiles_x * 64 >= W
+            assert (p.bwd_tiles // p.bwd_tiles_x) * p.bwd_per_tile >= H and p.bwd_tiles_x * p.bwd_tile_w >= W
             # room for the per-tile Gaussian lists behind the other scratch
             assert p.fwd_tiles >= 1 and p.fwd_ws_bytes >= B * p.fwd_tiles * (p.n_padded + 1) * 4
             assert p.pix_bytes >= B * H * W * (C + 1) * 4 + B * p.bwd_tiles * (p.n_padded + 1) * 4
@@ -274,7 +274,7 @@ def test_plan_invariants_over_random_shapes(lib):
             if mode != 0:
                 rows = p.bwd_tiles // p.bwd_tiles_x
                 assert p.bwd_tiles == rows * p.bwd_tiles_x and rows * p.bwd_per_tile >= H > (rows - 1) * p.bwd_per_tile
-                assert p.bwd_tiles_x * 64 >= p.w_padded >= W and p.w_padded % 8 == 0
+                assert p.bwd_tiles_x * p.bwd_tile_w >= p.w_padded >= W and p.w_padded % 8 == 0
                 assert p.fwd_tiles >= 1
                 assert p.fwd_ws_bytes >= B * p.fwd_tiles * (Np + 1) * 4
                 assert p.pix_bytes >= (B * H * p.w_padded * p.pix_stride + B * p.w_padded) * 4 + B * p.bwd_tiles * (Np + 1) * 4

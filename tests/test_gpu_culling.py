@@ -460,7 +460,7 @@ def test_tile_lists_against_the_oracle_s_rectangle_minimum(igs, dev, tolerance, 
     for ty in range(counts.shape[1]):
         for tx in range(counts.shape[2]):
             r0, r1 = ty * p.bwd_per_tile, min(H, (ty + 1) * p.bwd_per_tile)
-            c0, c1 = tx * 64, min(W, (tx + 1) * 64)
+            c0, c1 = tx * p.bwd_tile_w, min(W, (tx + 1) * p.bwd_tile_w)
             m = k * O.min_q_over_rect(pos[..., 0], pos[..., 1], a, b, dd, xs[c0], xs[c1 - 1], ys[r0], ys[r1 - 1])
             S = O.tile_weight_floor(pos[..., 0], pos[..., 1], a, b, dd, al, xs[c0], xs[c1 - 1], ys[r0], ys[r1 - 1])
             floors.append(S)
