@@ -204,8 +204,8 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     p->bwd_tiles = (int)T;
     p->fwd_tiles = sep ? fg.tiles_x * fg.tiles_y : 0;
     p->pix_stride = sep ? pix_stride_sep(C) : pix_stride_gen(C);
-    // records, then one reach box (4 floats) per record, then the call's skip limit (4 floats)
-    p->packed_bytes = ((uint64_t)B * p->n_padded * (p->rec_stride + 4) + 4) * sizeof(float);
+    // records, then one bin record (8 floats) per record, then the call's skip settings (4 floats)
+    p->packed_bytes = ((uint64_t)B * p->n_padded * (p->rec_stride + 8) + 4) * sizeof(float);
     p->fwd_ws_bytes = S > 1 ? (uint64_t)S * B * (C + 1) * H * W * sizeof(float) : 0;
     p->pix_bytes = sep ? ((uint64_t)B * H * p->w_padded * p->pix_stride + (uint64_t)B * p->w_padded) * sizeof(float)
                        : (uint64_t)B * p->hw_padded * p->pix_stride * sizeof(float);
@@ -264,12 +264,12 @@ inline int* super_slots_at(float* partial, int B, int T, int NF, int N, int Np) 
     return reinterpret_cast<int*>(slots + align16((size_t)B * T * Np * sizeof(int)));
 }
 
-inline const float4* boxes_of(const float* packed, int B, int Np, int RS) {
+inline const float4* bins_of(const float* packed, int B, int Np, int RS) {
     return reinterpret_cast<const float4*>(packed + (size_t)B * Np * RS);
 }
 // The skip limit the pack kernel left behind the boxes.
 inline const float* limit_of(const float* packed, int B, int Np, int RS) {
-    return packed + (size_t)B * Np * (RS + 4);
+    return packed + (size_t)B * Np * (RS + 8);
 }
 // Skip weight of a pack call -> limit in units of the kernels' exponent (see reach_box); a weight of
 // 0 (or one too small to matter) is the exact limit.
@@ -524,7 +524,7 @@ int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const f
     hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
                        colors, N, Np, C, rec_stride_of(C), 0.0f, limit, skip_fraction, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
+                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
@@ -541,7 +541,7 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
     hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
                        alphas, colors, N, Np, C, rec_stride_of(C), eps, limit, skip_fraction, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C))));
+                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C))));
     return launch_status();
 }
 
@@ -585,9 +585,8 @@ int forward_impl(const float* packed, const float* x, const float* y,
             const size_t split_bytes = a.S > 1 ? (size_t)a.S * B * (C + 1) * H * W * sizeof(float) : 0;
             const BinPlace bp = bins_at(ws, split_bytes, B, plan.fwd_tiles);
             BinArgs ba;
-            ba.boxes = boxes_of(packed, B, plan.n_padded, plan.rec_stride);
+            ba.bins = bins_of(packed, B, plan.n_padded, plan.rec_stride);
             ba.limit = limit_of(packed, B, plan.n_padded, plan.rec_stride);
-            ba.packed = packed; ba.RS = plan.rec_stride;
             ba.x = x; ba.y = y;
             ba.sxb = a.sxb; ba.sxw = a.sxw; ba.syb = a.syb; ba.syh = a.syh;
             ba.N = N; ba.Np = plan.n_padded; ba.H = H; ba.W = W;
@@ -830,9 +829,8 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
         if (sep) {
             BinArgs ba;
-            ba.boxes = boxes_of(packed, B, a.Np, rec_stride_of(C));
+            ba.bins = bins_of(packed, B, a.Np, rec_stride_of(C));
             ba.limit = limit_of(packed, B, a.Np, rec_stride_of(C));
-            ba.packed = packed; ba.RS = rec_stride_of(C);
             ba.x = a.xs; ba.y = y;               // the prologue's compact column coordinates
             ba.sxb = a.Wp; ba.sxw = 1; ba.syb = a.syb; ba.syh = a.syh;
             ba.N = N; ba.Np = a.Np; ba.H = H; ba.W = W;
@@ -1041,7 +1039,7 @@ int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int 
     hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
                        rec_stride_of(C_kernel), eps, limit, skip_fraction, packed,
-                       const_cast<float4*>(boxes_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
+                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
     return launch_status();
 }
 

@@ -1,4 +1,4 @@
-// igs_pack_bin.h -- pack kernels (records + reach boxes) and the per-tile Gaussian lists (k_bin).
+// igs_pack_bin.h -- pack kernels (records + bin records) and the per-tile Gaussian lists (k_bin).
 // Included by igs_gs2d.hip inside its anonymous namespace (one translation unit).
 #pragma once
 
@@ -15,13 +15,18 @@
 //     what the gradient of alpha sums) are below w.  The limit of Gaussian n is
 //     L_n = min(kExactLimit, L + log2 max(1, |alpha_n|)).
 //   The boxes are made for the call's skip weight; k_bin may use a larger weight for a tile whose
-//   denominators it can bound from below (tile_weight_sum), which only removes more of what the box
+//   denominators it can bound from below (least_weight), which only removes more of what the box
 //   lets through.
 // The box is five binades wider than the tile test of k_bin (ellipse_reaches), as in the exact case.
 // Half extents: sqrt(Q Sigma_xx), sqrt(Q Sigma_yy) with Sigma the covariance that (A, B, D) invert.
 // A record with a non-finite field or a non-positive-definite (A, B, D) gets an unbounded box (its
-// NaN/inf must propagate as without culling); padding records get an empty one.  Stored as
-// (xlo, xhi, ylo, yhi).
+// NaN/inf must propagate as without culling); padding records get an empty one.
+//
+// What k_bin needs of a Gaussian sits in a "bin record" of its own, 8 floats, so that the binning
+// reads one contiguous stream instead of a box and then, for the boxes that meet the tile, the
+// Gaussian's record: (px, py, hx, hy) = centre and half extents of the box (+inf: unbounded, -inf:
+// empty) and (a, b2, d, alpha) = the quadratic form of -q' (the negated A', B2', D' of the record).
+// The bin records [B][Np] follow the records in the packed buffer.
 constexpr float kExactLimit = 155.0f;
 constexpr double kHalfLog2e = 0.72134752044448170368;
 
@@ -30,34 +35,38 @@ __device__ __forceinline__ float skip_limit(float limit, float alpha) {
     return fminf(kExactLimit, limit + __log2f(fmaxf(1.0f, fabsf(alpha))));
 }
 
-__device__ __forceinline__ float4 reach_box(float px, float py, double sxx, double syy, bool bounded,
-                                            float limit_n) {
+// half extents (hx, hy) of the reach box
+__device__ __forceinline__ float2 reach_extent(float px, float py, double sxx, double syy, bool bounded,
+                                               float limit_n) {
     const float inf = __builtin_inff();
-    if (!bounded || !(sxx >= 0.0) || !(syy >= 0.0) || !isfinite(px) || !isfinite(py))
-        return make_float4(-inf, inf, -inf, inf);
+    if (!bounded || !(sxx >= 0.0) || !(syy >= 0.0) || !isfinite(px) || !isfinite(py)) return make_float2(inf, inf);
     const double Q = ((double)limit_n + 5.0) / kHalfLog2e;
-    // rounded outwards: one part in 1e5 is far more than the fp32 rounding of the bounds
+    // rounded outwards: one part in 1e5 is far more than the fp32 rounding of the bounds px -+ hx
     const double hx = sqrt(Q * sxx) * 1.00001, hy = sqrt(Q * syy) * 1.00001;
     const double ax = fabs((double)px) * 1e-6 + 1e-30, ay = fabs((double)py) * 1e-6 + 1e-30;
-    return make_float4((float)((double)px - hx - ax), (float)((double)px + hx + ax),
-                       (float)((double)py - hy - ay), (float)((double)py + hy + ay));
+    return make_float2((float)(hx + ax), (float)(hy + ay));
 }
 
-__device__ __forceinline__ float4 empty_box() {
+__device__ __forceinline__ void write_bin_record(float4* bins, size_t i, float px, float py, float2 h,
+                                                 float A, float B2, float D, float alpha) {
+    bins[2 * i] = make_float4(px, py, h.x, h.y);
+    bins[2 * i + 1] = make_float4(-A, -B2, -D, alpha);
+}
+__device__ __forceinline__ void write_empty_bin_record(float4* bins, size_t i) {
     const float inf = __builtin_inff();
-    return make_float4(inf, -inf, inf, -inf);
+    bins[2 * i] = make_float4(0.0f, 0.0f, -inf, -inf);
+    bins[2 * i + 1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 }
 
-// The call's skip limit and skip fraction travel behind the reach boxes [B][Np] in the packed buffer
+// The call's skip limit and skip fraction travel behind the bin records in the packed buffer
 // (4 floats, the first two used), where k_bin reads them: the forward and the backward then need no
 // argument for them.
-__device__ __forceinline__ void write_skip_limit(float4* boxes, int B, int Np, float limit, float fraction) {
-    boxes[(size_t)B * Np] = make_float4(fminf(limit, kExactLimit), fraction, 0.0f, 0.0f);
+__device__ __forceinline__ void write_skip_limit(float4* bins, int B, int Np, float limit, float fraction) {
+    bins[(size_t)2 * B * Np] = make_float4(fminf(limit, kExactLimit), fraction, 0.0f, 0.0f);
 }
 
 // One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
 // with A' = k A, B2' = 2 k B, D' = k D, k = -0.5 log2 e.  Records N..Np-1 are zero.
-// The reach boxes [B][Np] follow the records in the packed buffer.
 template <bool kScaleRot>
 __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ position,
                                                    const float* __restrict__ p0,  // cov00 | scales
@@ -76,7 +85,7 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {  // padding: alpha = 0 and e = exp2(0) = 1, so it contributes exactly 0
         for (int c = 0; c < RS; ++c) r[c] = 0.0f;
-        boxes[(size_t)b * Np + n] = empty_box();
+        write_empty_bin_record(boxes, (size_t)b * Np + n);
         return;
     }
     const size_t i = (size_t)b * N + n;
@@ -121,11 +130,11 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
     }
     for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
-    const float4 box = reach_box(px, py, sxx, syy, bounded && fin, skip_limit(limit, al));
-    boxes[(size_t)b * Np + n] = box;
+    const float2 ext = reach_extent(px, py, sxx, syy, bounded && fin, skip_limit(limit, al));
+    write_bin_record(boxes, (size_t)b * Np + n, px, py, ext, r[2], r[3], r[4], al);
     if (RS >= 8 + C) {  // room in the record: the y range of the box travels with it
-        r[6 + C] = box.z;
-        r[7 + C] = box.w;
+        r[6 + C] = py - ext.y;
+        r[7 + C] = py + ext.y;
     }
 }
 
@@ -148,7 +157,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
     float* r = packed + ((size_t)b * Np + n) * RS;
     if (n >= N) {
         for (int c = 0; c < RS; ++c) r[c] = 0.0f;
-        boxes[(size_t)b * Np + n] = empty_box();
+        write_empty_bin_record(boxes, (size_t)b * Np + n);
         return;
     }
     const size_t i = (size_t)b * N + n;
@@ -181,12 +190,12 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
         fin = fin && isfinite(col);
     }
     for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
-    const float4 box = reach_box(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
-                                 fin && v0 > 0.0 && v1 > 0.0, skip_limit(limit, 1.0f));
-    boxes[(size_t)b * Np + n] = box;
+    const float2 ext = reach_extent(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
+                                    fin && v0 > 0.0 && v1 > 0.0, skip_limit(limit, 1.0f));
+    write_bin_record(boxes, (size_t)b * Np + n, px, py, ext, r[2], r[3], r[4], 1.0f);
     if (RS >= 8 + Cp) {
-        r[6 + Cp] = box.z;
-        r[7 + Cp] = box.w;
+        r[6 + Cp] = py - ext.y;
+        r[7 + Cp] = py + ext.y;
     }
 }
 
@@ -205,9 +214,7 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
 // Separable grids only: a tile is tile_w columns x tile_h rows and its coordinate range is
 // [min, max] of x over its columns and of y over its rows (no monotonicity assumed).
 struct BinArgs {
-    const float4* boxes;  // [B][Np]
-    const float* packed;  // [B][Np][RS] records (the refined test reads px, py, A', B2', D')
-    int RS;
+    const float4* bins;   // [B][Np][2] bin records
     const float* x;
     const float* y;
     long sxb, sxw, syb, syh;
@@ -225,7 +232,7 @@ struct BinArgs {
     const int* cand_counts;  // [B][stiles][cand_K]
     const int* cand_lists;   // [B][stiles][Np], segment k at offset k cand_chunk
     int cand_K, cand_chunk, stiles_x, stiles;
-    const float* limit;  // the call's skip limit and fraction, written by the pack kernel behind the boxes
+    const float* limit;  // the call's skip limit and fraction, written by the pack kernel behind the bin records
     const int* flag;
     int want;
     int no_cull;  // list every candidate (IGS_OPT_NO_CULL): the reference point for "culling changes no bit"
@@ -252,11 +259,10 @@ constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads i
 // rounding as the reach box has, so dropping it changes no bit either; with a skip weight w every
 // pair of a dropped tile has e < w / max(1, |alpha|).  A non-positive-definite or NaN record fails
 // the comparison and stays listed.
-__device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, float txlo, float txhi,
+__device__ __forceinline__ bool ellipse_reaches(float4 q0, float4 q1, float txlo, float txhi,
                                                 float tylo, float tyhi, float limit) {
-    const float4 h = *reinterpret_cast<const float4*>(rec);  // px, py, A', B2'
-    const float a = -h.z, b2 = -h.w, d = -rec[4];
-    const float x0 = txlo - h.x, x1 = txhi - h.x, y0 = tylo - h.y, y1 = tyhi - h.y;
+    const float a = q1.x, b2 = q1.y, d = q1.z;
+    const float x0 = txlo - q0.x, x1 = txhi - q0.x, y0 = tylo - q0.y, y1 = tyhi - q0.y;
     // straight-line code (every path is taken by some lane of a wave anyway)
     const bool inside = x0 <= 0.0f && x1 >= 0.0f && y0 <= 0.0f && y1 >= 0.0f;
     // the argument below needs a form that is positive definite beyond the rounding of its
@@ -276,7 +282,7 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
     const float pmin = fminf(pv, ph);
     const float mx = fmaxf(fabsf(x0), fabsf(x1)), my = fmaxf(fabsf(y0), fabsf(y1));
     const float T = a * mx * mx + fabsf(b2) * mx * my + d * my * my;
-    const bool beyond = pmin - 4e-6f * T > skip_limit(limit, rec[5]);
+    const bool beyond = pmin - 4e-6f * T > skip_limit(limit, q1.w);
     return inside || !definite || !beyond;
 }
 
@@ -284,14 +290,13 @@ __device__ __forceinline__ bool ellipse_reaches(const float* __restrict__ rec, f
 // convex, its maximum over the rectangle is at a corner.  Summed over Gaussians with alpha >= 0 this
 // bounds every denominator of the tile from below.  Rounded down by 1e-3 against the fp32 rounding
 // of P at the corners (a few 1e-6 of its largest term, which matters only while 2^-P does).
-__device__ __forceinline__ float least_weight(const float* __restrict__ rec, float txlo, float txhi,
-                                              float tylo, float tyhi) {
-    const float4 h = *reinterpret_cast<const float4*>(rec);  // px, py, A', B2'
-    const float a = -h.z, b2 = -h.w, d = -rec[4];
-    const float x0 = txlo - h.x, x1 = txhi - h.x, y0 = tylo - h.y, y1 = tyhi - h.y;
+__device__ __forceinline__ float least_weight(float4 q0, float4 q1, float txlo, float txhi, float tylo,
+                                              float tyhi) {
+    const float a = q1.x, b2 = q1.y, d = q1.z;
+    const float x0 = txlo - q0.x, x1 = txhi - q0.x, y0 = tylo - q0.y, y1 = tyhi - q0.y;
     auto form = [&](float x, float y) { return fmaf(fmaf(b2, x, d * y), y, a * x * x); };
     const float pmax = fmaxf(fmaxf(form(x0, y0), form(x0, y1)), fmaxf(form(x1, y0), form(x1, y1)));
-    const float w = rec[5] * hw_exp2(-pmax) * 0.999f;
+    const float w = q1.w * hw_exp2(-pmax) * 0.999f;
     return w > 0.0f ? w : 0.0f;  // NaN, inf - inf and the like count as nothing
 }
 
@@ -372,8 +377,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     const float fraction = a.limit[1];
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
-    const float4* boxes = a.boxes + (size_t)b * a.Np;
-    const float* recs = a.packed + (size_t)b * a.Np * a.RS;
+    const float4* bins = a.bins + (size_t)2 * b * a.Np;
     // The candidates, numbered 0..M-1: all Gaussians; or this workgroup's chunk of them (first
     // level); or the entries of the super-tile's list, segment after segment (second level).
     int first = 0, M = a.N;
@@ -410,8 +414,8 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     const int per_wave = ((M + kBinWaves - 1) / kBinWaves + 63) & ~63;
     const int nb = wave * per_wave, ne = min(M, nb + per_wave);
     const unsigned long long below = (1ull << lane) - 1ull;
-    // kU boxes per lane are loaded together, so that kU loads are in flight instead of one
-    constexpr int kU = 8;
+    // the bin records of kU candidates per lane are loaded together (2 kU loads in flight)
+    constexpr int kU = 4;
     // Skip fraction f > 0: a tile whose denominators are all at least S (the sum of the least
     // weights of the candidates whose box meets it; only if none of them has a negative or
     // non-finite alpha) may skip pairs up to the weight w + f S instead of the call's w.  Not at the
@@ -422,20 +426,24 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         bool negative = false;
         for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
             int n[kU];
-            float4 bb[kU];
+            float4 q0[kU], q1[kU];
 #pragma unroll
             for (int u = 0; u < kU; ++u) n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));
 #pragma unroll
-            for (int u = 0; u < kU; ++u) bb[u] = boxes[n[u]];
+            for (int u = 0; u < kU; ++u) {
+                q0[u] = bins[2 * n[u]];
+                q1[u] = bins[2 * n[u] + 1];
+            }
 #pragma unroll
             for (int u = 0; u < kU; ++u) {
-                if (n0 + u * 64 + lane >= ne) continue;
-                if (bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi) continue;
-                const float* rec = recs + (size_t)n[u] * a.RS;
-                negative = negative || !(rec[5] >= 0.0f);
+                const bool meets = n0 + u * 64 + lane < ne &&
+                                   !(q0[u].x + q0[u].z < txlo || q0[u].x - q0[u].z > txhi ||
+                                     q0[u].y + q0[u].w < tylo || q0[u].y - q0[u].w > tyhi);
+                negative = negative || (meets && !(q1[u].w >= 0.0f));
                 // (records that are never skipped have unbounded boxes: NaN fields or a form that is
                 // not positive definite; with alpha >= 0 they can only raise a denominator)
-                if (bb[u].x > -inf) sum += least_weight(rec, txlo, txhi, tylo, tyhi);
+                const float w = least_weight(q0[u], q1[u], txlo, txhi, tylo, tyhi);
+                sum += (meets && q0[u].z < inf) ? w : 0.0f;
             }
         }
 #pragma unroll
@@ -460,42 +468,32 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     }
     // code: which of the forward's waves the Gaussian reaches (wave masks), or 1; 0 = not listed
     auto classify = [&](int n0, int (&code)[kU], bool (&in)[kU], int (&n)[kU]) {
-        float4 bb[kU];
+        float4 q0[kU], q1[kU];
 #pragma unroll
         for (int u = 0; u < kU; ++u) n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));  // M > 0 inside the loops
 #pragma unroll
-        for (int u = 0; u < kU; ++u) bb[u] = boxes[n[u]];
+        for (int u = 0; u < kU; ++u) {
+            q0[u] = bins[2 * n[u]];
+            q1[u] = bins[2 * n[u] + 1];
+        }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             in[u] = n0 + u * 64 + lane < ne;
             // "definitely outside" negated, so that NaN bounds count as inside
-            const bool meets = in[u] && !(bb[u].y < txlo || bb[u].x > txhi || bb[u].w < tylo || bb[u].z > tyhi);
-            code[u] = meets ? (masks ? 15 : 1) : 0;
-            // bounded box (unbounded ones mark records that must never be skipped): refine
-            if (meets && bb[u].x > -inf) {
-                const float* rec = recs + (size_t)n[u] * a.RS;
-                if (masks) {
-                    code[u] = 0;
+            const bool meets = in[u] && !(q0[u].x + q0[u].z < txlo || q0[u].x - q0[u].z > txhi ||
+                                          q0[u].y + q0[u].w < tylo || q0[u].y - q0[u].w > tyhi);
+            // an unbounded box marks a record that must never be skipped; a bounded one is refined
+            const bool refine = q0[u].z < inf;
+            int reached = 0;
+            if (masks) {
 #pragma unroll
-                    for (int w = 0; w < 4; ++w)
-                        if (sub_any[w] && ellipse_reaches(rec, sub[w][0], sub[w][1], sub[w][2], sub[w][3], limit))
-                            code[u] |= 1 << w;
-#ifdef IGS_DEBUG_SUB
-                    if (n[u] == 2 && t == 0 && b == 0) {
-                        list[a.Np - 32] = code[u];
-                        list[a.Np - 31] = sub_any[0];
-                        list[a.Np - 30] = ellipse_reaches(rec, sub[0][0], sub[0][1], sub[0][2], sub[0][3], limit);
-                        list[a.Np - 29] = __float_as_int(limit);
-                        list[a.Np - 28] = __float_as_int(rec[0]);
-                        list[a.Np - 27] = __float_as_int(rec[5]);
-                        list[a.Np - 26] = __float_as_int(txlo);
-                        list[a.Np - 25] = __float_as_int(tyhi);
-                    }
-#endif
-                } else {
-                    code[u] = ellipse_reaches(rec, txlo, txhi, tylo, tyhi, limit) ? 1 : 0;
-                }
+                for (int w = 0; w < 4; ++w)
+                    reached |= (sub_any[w] && ellipse_reaches(q0[u], q1[u], sub[w][0], sub[w][1], sub[w][2],
+                                                              sub[w][3], limit)) ? 1 << w : 0;
+            } else {
+                reached = ellipse_reaches(q0[u], q1[u], txlo, txhi, tylo, tyhi, limit) ? 1 : 0;
             }
+            code[u] = !meets ? 0 : (refine ? reached : (masks ? 15 : 1));
         }
     };
     // the first pass keeps its verdicts (one bit, or four with wave masks, per box of this lane) for
@@ -549,9 +547,4 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         }
     }
     if (tid == 0) a.counts[((size_t)b * tiles + t) * K + kc] = total;
-#ifdef IGS_DEBUG_SUB
-    if (tid == 0 && masks)
-        for (int w = 0; w < 4; ++w)
-            for (int f = 0; f < 4; ++f) list[a.Np - 16 + w * 4 + f] = __float_as_int(sub[w][f]);
-#endif
 }

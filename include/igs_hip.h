@@ -97,9 +97,10 @@ typedef struct igs_gs2d_plan_t {
     int32_t bwd_tiles;       /* pixel tiles T per image of the backward partial buffer     */
     int32_t bwd_per_tile;    /* rows (separable) or pixels (general) per backward tile     */
     int32_t pix_stride;      /* floats per pixel record of the backward prologue           */
-    uint64_t packed_bytes;   /* packed Gaussian buffer: records, then one reach box (4
-                                floats) per record, then the call's skip settings (4 floats):
-                                (B*n_padded*(rec_stride+4) + 4)*4                          */
+    uint64_t packed_bytes;   /* packed Gaussian buffer: records, then one bin record (8
+                                floats: reach box and quadratic form, what the tile lists
+                                are built from) per record, then the call's skip settings
+                                (4 floats): (B*n_padded*(rec_stride+8) + 4)*4              */
     uint64_t fwd_ws_bytes;   /* forward scratch: split partials (fwd_split > 1) and, on
                                 separable grids, the per-tile Gaussian lists (plus those
                                 of the super-tiles when there are 32 tiles or more)         */
@@ -136,8 +137,8 @@ float igs_gs2d_skip_weight(int N, float eps, float tolerance);
  * the inverse covariance).  position [B,N,2]; cov_inv_00/01/11 [B,N]; alphas [B,N];
  * colors [B,N,C]; packed: plan.packed_bytes, 16-byte aligned.  Replaces nothing in the
  * reference (its kernels read the tensors directly); it exists so the hot loops read one
- * record.  Behind the records the buffer holds one "reach box" per Gaussian and the call's skip
- * limit.  On separable grids the forward and the backward skip, per pixel tile (and the forward
+ * record.  Behind the records the buffer holds one bin record per Gaussian (its "reach box" and
+ * quadratic form) and the call's skip settings.  On separable grids the forward and the backward skip, per pixel tile (and the forward
  * per wave of rows), the Gaussians whose box misses the tile or whose ellipse does not reach the
  * tile's coordinate rectangle (the reference evaluates every pair:
  * src/igs/gs_triton_chunked.py:100-200).  What may be skipped is set by skip_weight w and

@@ -371,8 +371,9 @@ def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev, tolerance):
     pos = d64["positions"].float().double()
 
     def boxes(packed):
-        p = op.plan
-        return packed[B * p.n_padded * p.rec_stride:][:B * p.n_padded * 4].view(B, p.n_padded, 4)
+        p = op.plan   # bin records (px, py, hx, hy | a, b2, d, alpha): the box is px -+ hx, py -+ hy
+        q = packed[B * p.n_padded * p.rec_stride:][:B * p.n_padded * 8].view(B, p.n_padded, 8)
+        return torch.stack([q[..., 0] - q[..., 2], q[..., 0] + q[..., 2], q[..., 1] - q[..., 3], q[..., 1] + q[..., 3]], -1)
 
     col = _f32c(g["colors"])
     cases = {"scale_rot": (op.pack_scale_rot(_f32c(g["positions"]), _f32c(g["scales"]), _f32c(g["rotations"]),
@@ -395,7 +396,7 @@ def test_reach_boxes_of_the_pack_kernels_match_the_oracle(igs, dev, tolerance):
         assert bool((out <= slack * half + 1e-6).all()), (name, float((out / half).max()))
         pad = boxes(packed)[:, N:]
         assert bool((pad[..., 0] > pad[..., 1]).all())  # padding records: empty boxes
-        limit, fraction = packed[B * op.plan.n_padded * (op.plan.rec_stride + 4):][:2].tolist()
+        limit, fraction = packed[B * op.plan.n_padded * (op.plan.rec_stride + 8):][:2].tolist()
         assert limit == pytest.approx(O.EXACT_LIMIT if w == 0 else min(O.EXACT_LIMIT, -math.log2(w)), rel=1e-6)
         assert fraction == pytest.approx(O.skip_weight(N, 1.0, tolerance), rel=1e-6)
     if tolerance > 0:    # smaller boxes than the exact-zero ones, by sqrt of the limits' ratio
