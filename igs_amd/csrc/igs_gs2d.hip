@@ -297,7 +297,10 @@ int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t*
 }
 
 int launch_bin(const BinArgs& a, int K, int B, hipStream_t st) {
-    hipLaunchKernelGGL(k_bin, dim3(a.tiles_x * a.tiles_y, K, B), dim3(kBinThreads), 0, st, a);
+    if (a.sub_nx > 0)
+        hipLaunchKernelGGL(k_bin<true>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(kBinThreads), 0, st, a);
+    else
+        hipLaunchKernelGGL(k_bin<false>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(kBinThreads), 0, st, a);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? IGS_OK : (int)e;
 }

@@ -300,6 +300,7 @@ __device__ __forceinline__ float least_weight(float4 q0, float4 q1, float txlo, 
     return w > 0.0f ? w : 0.0f;  // NaN, inf - inf and the like count as nothing
 }
 
+template <bool kMasks>
 __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     if (a.flag != nullptr && *a.flag != a.want) return;
     __shared__ float red[4][kBinWaves];
@@ -312,9 +313,72 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     const int c0 = tx * a.tile_w, c1 = min(a.W, c0 + a.tile_w);
     const int r0 = ty * a.tile_h, r1 = min(a.H, r0 + a.tile_h);
     const float inf = __builtin_inff();
+    const float4* bins = a.bins + (size_t)2 * b * a.Np;
+    // The candidates, numbered 0..M-1: all Gaussians; or this workgroup's chunk of them (first
+    // level); or the entries of the super-tile's list, segment after segment (second level).
+    int first = 0, M = a.N;
+    const int* cand = nullptr;
+    if (a.chunk > 0) {
+        first = kc * a.chunk;
+        M = max(0, min(a.N, first + a.chunk) - first);
+    }
+    if (a.cand_lists != nullptr) {
+        const size_t st = (size_t)b * a.stiles + (ty / kSuperY) * a.stiles_x + tx / kSuperX;
+        cand = a.cand_lists + st * a.Np;
+        if (tid == 0) {
+            int run = 0;
+            for (int j = 0; j < a.cand_K; ++j) {
+                seg_first[j] = run;
+                run += a.cand_counts[st * a.cand_K + j];
+            }
+            for (int j = a.cand_K; j <= kBinMaxChunks; ++j) seg_first[j] = run;
+        }
+        __syncthreads();
+        M = seg_first[kBinMaxChunks];
+    }
+    // candidate index -> Gaussian index
+    auto gaussian_of = [&](int i) {
+        if (cand == nullptr) return first + i;
+        int seg = 0;  // the last segment that starts at or before i (binary search over 64 entries)
+#pragma unroll
+        for (int step = kBinMaxChunks / 2; step > 0; step >>= 1)
+            if (seg_first[seg + step] <= i) seg += step;
+        return cand[(size_t)seg * a.cand_chunk + (i - seg_first[seg])];
+    };
+    // Each wave scans one contiguous share of the candidates, without barriers inside a scan: once
+    // for the tile's denominator floor (skip fraction only), once to classify and count, and once
+    // (from the kept verdicts, with the shares' counts prefixed in wave order) to write.
+    const int per_wave = ((M + kBinWaves - 1) / kBinWaves + 63) & ~63;
+    const int nb = wave * per_wave, ne = min(M, nb + per_wave);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    // The bin records of kU candidates per lane are loaded together (2 kU loads in flight).  The
+    // first batch of a wave is loaded before anything else, so that its latency overlaps with the
+    // tile's coordinate range, and is kept for both scans: small problems never load twice.
+    constexpr int kU = 4;
+    struct Batch {
+        int n[kU];
+        float4 q0[kU], q1[kU];
+    };
+    auto load_batch = [&](int n0, Batch& bt) {
+#pragma unroll
+        for (int u = 0; u < kU; ++u) bt.n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));  // M > 0 in the loops
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            bt.q0[u] = bins[2 * bt.n[u]];
+            bt.q1[u] = bins[2 * bt.n[u] + 1];
+        }
+    };
+    Batch head;
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+        head.n[u] = 0;
+        head.q0[u] = head.q1[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+    if (nb < ne) load_batch(nb, head);
+
     float xlo = inf, xhi = -inf, ylo = inf, yhi = -inf;
     bool bad = false;
-    const bool masks = a.sub_nx > 0;
+    constexpr bool masks = kMasks;  // a.sub_nx > 0
     if (!masks) {
         for (int c = c0 + tid; c < c1; c += kBinThreads) {
             const float v = a.x[b * a.sxb + (long)c * a.sxw];
@@ -377,45 +441,11 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     const float fraction = a.limit[1];
     int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
-    const float4* bins = a.bins + (size_t)2 * b * a.Np;
-    // The candidates, numbered 0..M-1: all Gaussians; or this workgroup's chunk of them (first
-    // level); or the entries of the super-tile's list, segment after segment (second level).
-    int first = 0, M = a.N;
-    const int* cand = nullptr;
-    if (a.chunk > 0) {
-        first = kc * a.chunk;
-        M = max(0, min(a.N, first + a.chunk) - first);
-    }
-    if (a.cand_lists != nullptr) {
-        const size_t st = (size_t)b * a.stiles + (ty / kSuperY) * a.stiles_x + tx / kSuperX;
-        cand = a.cand_lists + st * a.Np;
-        if (tid == 0) {
-            int run = 0;
-            for (int j = 0; j < a.cand_K; ++j) {
-                seg_first[j] = run;
-                run += a.cand_counts[st * a.cand_K + j];
-            }
-            for (int j = a.cand_K; j <= kBinMaxChunks; ++j) seg_first[j] = run;
-        }
-        __syncthreads();
-        M = seg_first[kBinMaxChunks];
-    }
-    // candidate index -> Gaussian index
-    auto gaussian_of = [&](int i) {
-        if (cand == nullptr) return first + i;
-        int seg = 0;  // the last segment that starts at or before i (binary search over 64 entries)
-#pragma unroll
-        for (int step = kBinMaxChunks / 2; step > 0; step >>= 1)
-            if (seg_first[seg + step] <= i) seg += step;
-        return cand[(size_t)seg * a.cand_chunk + (i - seg_first[seg])];
+    // "definitely outside" negated, so that NaN bounds count as inside
+    auto meets_tile = [&](const Batch& bt, int u) {
+        return !(bt.q0[u].x + bt.q0[u].z < txlo || bt.q0[u].x - bt.q0[u].z > txhi ||
+                 bt.q0[u].y + bt.q0[u].w < tylo || bt.q0[u].y - bt.q0[u].w > tyhi);
     };
-    // Each wave scans one contiguous share of the candidates twice, without barriers: first to
-    // count, then (with the shares' counts prefixed in wave order) to write.
-    const int per_wave = ((M + kBinWaves - 1) / kBinWaves + 63) & ~63;
-    const int nb = wave * per_wave, ne = min(M, nb + per_wave);
-    const unsigned long long below = (1ull << lane) - 1ull;
-    // the bin records of kU candidates per lane are loaded together (2 kU loads in flight)
-    constexpr int kU = 4;
     // Skip fraction f > 0: a tile whose denominators are all at least S (the sum of the least
     // weights of the candidates whose box meets it; only if none of them has a negative or
     // non-finite alpha) may skip pairs up to the weight w + f S instead of the call's w.  Not at the
@@ -424,26 +454,18 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     if (fraction > 0.0f && a.chunk == 0 && txlo > -inf && !a.no_cull) {  // workgroup-uniform
         float sum = 0.0f;
         bool negative = false;
-        for (int n0 = nb; n0 < ne; n0 += 64 * kU) {
-            int n[kU];
-            float4 q0[kU], q1[kU];
-#pragma unroll
-            for (int u = 0; u < kU; ++u) n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));
-#pragma unroll
-            for (int u = 0; u < kU; ++u) {
-                q0[u] = bins[2 * n[u]];
-                q1[u] = bins[2 * n[u] + 1];
-            }
+        int it = 0;
+        for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
+            Batch bt = head;
+            if (it > 0) load_batch(n0, bt);
 #pragma unroll
             for (int u = 0; u < kU; ++u) {
-                const bool meets = n0 + u * 64 + lane < ne &&
-                                   !(q0[u].x + q0[u].z < txlo || q0[u].x - q0[u].z > txhi ||
-                                     q0[u].y + q0[u].w < tylo || q0[u].y - q0[u].w > tyhi);
-                negative = negative || (meets && !(q1[u].w >= 0.0f));
+                const bool meets = n0 + u * 64 + lane < ne && meets_tile(bt, u);
+                negative = negative || (meets && !(bt.q1[u].w >= 0.0f));
                 // (records that are never skipped have unbounded boxes: NaN fields or a form that is
                 // not positive definite; with alpha >= 0 they can only raise a denominator)
-                const float w = least_weight(q0[u], q1[u], txlo, txhi, tylo, tyhi);
-                sum += (meets && q0[u].z < inf) ? w : 0.0f;
+                const float w = least_weight(bt.q0[u], bt.q1[u], txlo, txhi, tylo, tyhi);
+                sum += (meets && bt.q0[u].z < inf) ? w : 0.0f;
             }
         }
 #pragma unroll
@@ -467,45 +489,37 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         }
     }
     // code: which of the forward's waves the Gaussian reaches (wave masks), or 1; 0 = not listed
-    auto classify = [&](int n0, int (&code)[kU], bool (&in)[kU], int (&n)[kU]) {
-        float4 q0[kU], q1[kU];
-#pragma unroll
-        for (int u = 0; u < kU; ++u) n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));  // M > 0 inside the loops
-#pragma unroll
-        for (int u = 0; u < kU; ++u) {
-            q0[u] = bins[2 * n[u]];
-            q1[u] = bins[2 * n[u] + 1];
-        }
+    auto classify = [&](int n0, const Batch& bt, int (&code)[kU], bool (&in)[kU]) {
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             in[u] = n0 + u * 64 + lane < ne;
-            // "definitely outside" negated, so that NaN bounds count as inside
-            const bool meets = in[u] && !(q0[u].x + q0[u].z < txlo || q0[u].x - q0[u].z > txhi ||
-                                          q0[u].y + q0[u].w < tylo || q0[u].y - q0[u].w > tyhi);
+            const bool meets = in[u] && meets_tile(bt, u);
             // an unbounded box marks a record that must never be skipped; a bounded one is refined
-            const bool refine = q0[u].z < inf;
+            const bool refine = bt.q0[u].z < inf;
             int reached = 0;
             if (masks) {
 #pragma unroll
                 for (int w = 0; w < 4; ++w)
-                    reached |= (sub_any[w] && ellipse_reaches(q0[u], q1[u], sub[w][0], sub[w][1], sub[w][2],
+                    reached |= (sub_any[w] && ellipse_reaches(bt.q0[u], bt.q1[u], sub[w][0], sub[w][1], sub[w][2],
                                                               sub[w][3], limit)) ? 1 << w : 0;
             } else {
-                reached = ellipse_reaches(q0[u], q1[u], txlo, txhi, tylo, tyhi, limit) ? 1 : 0;
+                reached = ellipse_reaches(bt.q0[u], bt.q1[u], txlo, txhi, tylo, tyhi, limit) ? 1 : 0;
             }
             code[u] = !meets ? 0 : (refine ? reached : (masks ? 15 : 1));
         }
     };
-    // the first pass keeps its verdicts (one bit, or four with wave masks, per box of this lane) for
-    // the second one when they fit in a register pair, i.e. up to 64 (16) boxes per lane
+    // the classifying scan keeps its verdicts (one bit, or four with wave masks, per candidate of this
+    // lane) for the writing one when they fit in a register pair, i.e. up to 64 (16) candidates per lane
     const int vbits = masks ? 4 : 1;
     const bool keep = per_wave * vbits <= 64 * 64;
     unsigned long long verdicts = 0ull;
     int cnt = 0, it = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
+        Batch bt = head;
+        if (it > 0) load_batch(n0, bt);
         bool in[kU];
-        int code[kU], n[kU];
-        classify(n0, code, in, n);
+        int code[kU];
+        classify(n0, bt, code, in);
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             cnt += __popcll(__ballot(code[u] != 0));
@@ -532,7 +546,11 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
                 n[u] = gaussian_of(min(n0 + u * 64 + lane, M - 1));
             }
         } else {
-            classify(n0, code, in, n);
+            Batch bt = head;
+            if (it > 0) load_batch(n0, bt);
+            classify(n0, bt, code, in);
+#pragma unroll
+            for (int u = 0; u < kU; ++u) n[u] = bt.n[u];
         }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
