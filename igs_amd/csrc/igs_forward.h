@@ -5,6 +5,7 @@
 // ----------------------------------------------------------------------------- forward
 struct FwdArgs {
     const float* packed;  // [B][Np][RS]
+    const float* zero_rec;  // an all-zero record behind the packed buffer's skip settings
     const float* x;
     const float* y;
     long sxb, sxh, sxw, syb, syh, syw;
@@ -37,18 +38,18 @@ template <int C>
 struct GRec {
     float px, py, A, B2, D, al;
     float ac[C];
-    float ylo, yhi;  // y range of the reach box (records with two spare floats only); in the separable
-                     // forward's LDS copy ylo holds the wave mask of the tile's list entry instead
+    float ylo, yhi;  // y range of the reach box (records with two spare floats only)
 };
 
 // whether a record of C channels has room for the y range of the reach box
 __host__ __device__ constexpr bool rec_has_yrange(int C) { return rec_stride_of(C) >= 8 + C; }
-// List entries of the separable forward: Gaussian index in the low 24 bits, wave mask above (k_bin).
-constexpr int kListIndexMask = 0xffffff;
-// Wave masks are built for the variants whose waves hold 16 rows (C <= 3); with fewer rows per wave
-// the tile is small already and the four extra ellipse tests per Gaussian cost the binning more than
-// the forward gains: those variants test the reach box's y range against the wave's rows instead.
-__host__ __device__ constexpr bool fwd_wave_masks(int C) { return rec_has_yrange(C) && fwd_sep_p(C) >= 16; }
+// The separable forward variants whose waves hold 16 rows (C <= 3) give every wave a Gaussian list of
+// its own (64 columns x 16 rows) and run one wave per workgroup: no wave waits for another at a
+// chunk boundary, and none reads records it then skips.  With fewer rows per wave the tile of four
+// waves is small already (the lists of single waves would cost the binning more than the forward
+// gains): those variants stream one list to four waves, and a wave tests the reach box's y range
+// against its own rows.
+__host__ __device__ constexpr bool fwd_wave_lists(int C) { return fwd_sep_p(C) >= 16; }
 
 // Unpacks one record held in R4 float4 registers (read from a wave-uniform LDS address).
 template <int C>
@@ -104,15 +105,14 @@ constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
 // workgroup through the double-buffered LDS window sh[2][CH*R4]; body(const float4* rec) runs
 // once per record with a wave-uniform LDS pointer.  Records past `count` in the last chunk
 // read as all-zero (for a Gaussian record: alpha = 0, adds exactly 0).  Must be called by all
-// kThreads threads of the workgroup (it contains barriers).
-// With kGather, record i of the stream is src record (index[i] & kListIndexMask) (a tile's Gaussian
-// list); kMaskSlot >= 0 then puts the entry's bits 24.. into float kMaskSlot of the record's LDS copy.
-template <int R4, int CH, bool kGather = false, int kMaskSlot = -1, class Body>
+// NT threads of the workgroup (it contains barriers; with NT = 64, one wave, they cost nothing).
+// With kGather, record i of the stream is src record index[i] (a tile's Gaussian list).
+template <int R4, int CH, bool kGather = false, int NT = kThreads, class Body>
 __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
                                                    float4* sh, Body&& body,
                                                    const int* __restrict__ index = nullptr) {
     constexpr int E = CH * R4;                          // float4 per chunk
-    constexpr int PRE = (E + kThreads - 1) / kThreads;  // float4 per thread per chunk
+    constexpr int PRE = (E + NT - 1) / NT;              // float4 per thread per chunk
     const int total = count * R4;
     const int chunks = (count + CH - 1) / CH;
     const int tid = threadIdx.x;
@@ -123,7 +123,7 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
     auto load_idx = [&](int chunk) {
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
-            const int e = i * kThreads + tid, ge = chunk * E + e;
+            const int e = i * NT + tid, ge = chunk * E + e;
             idx[i] = (kGather && e < E && ge < total) ? index[ge / R4] : 0;
         }
     };
@@ -131,20 +131,12 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
     auto load_records = [&](int chunk) {
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
-            const int e = i * kThreads + tid, ge = chunk * E + e;
+            const int e = i * NT + tid, ge = chunk * E + e;
             const bool valid = e < E && ge < total;
-            if (kGather) {
-                pre[i] = valid ? src[(size_t)(idx[i] & kListIndexMask) * R4 + (ge % R4)] : zero;
-                if (kMaskSlot >= 0 && ge % R4 == kMaskSlot / 4) {
-                    const float m = __int_as_float(idx[i] >> 24);
-                    if (kMaskSlot % 4 == 0) pre[i].x = m;
-                    if (kMaskSlot % 4 == 1) pre[i].y = m;
-                    if (kMaskSlot % 4 == 2) pre[i].z = m;
-                    if (kMaskSlot % 4 == 3) pre[i].w = m;
-                }
-            } else {
+            if (kGather)
+                pre[i] = valid ? src[(size_t)idx[i] * R4 + (ge % R4)] : zero;
+            else
                 pre[i] = valid ? src[ge] : zero;
-            }
         }
     };
     load_idx(0);
@@ -152,7 +144,7 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
     load_idx(1);
 #pragma unroll
     for (int i = 0; i < PRE; ++i) {
-        const int e = i * kThreads + tid;
+        const int e = i * NT + tid;
         if (e < E) sh[e] = pre[i];
     }
     __syncthreads();
@@ -186,11 +178,93 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
             float4* nxt = sh + ((k + 1) & 1) * E;
 #pragma unroll
             for (int i = 0; i < PRE; ++i) {
-                const int e = i * kThreads + tid;
+                const int e = i * NT + tid;
                 if (e < E) nxt[e] = pre[i];
             }
         }
         __syncthreads();
+    }
+}
+
+// The same stream for a workgroup of one wave, without staging registers: the records of the next
+// chunk go from global memory straight into the other LDS buffer (global_load_lds_dwordx4: lane l
+// of the instruction writes 16 bytes at base + 16 l) while the current one is computed, and one
+// vmcnt wait per chunk separates the two.  Slots past `count` load the all-zero record `zero_rec`.
+// The two buffers are separate arrays and the chunk loop is unrolled by two, so that every LDS read
+// names the buffer it reads.
+template <int R4, int CH, class Body>
+__device__ __forceinline__ void stream_records_dma(const float4* __restrict__ src,
+                                                   const float4* __restrict__ zero_rec, int count,
+                                                   float4* sh0, float4* sh1, Body&& body,
+                                                   const int* __restrict__ index) {
+    constexpr int E = CH * R4;  // float4 per chunk
+    static_assert(E % 64 == 0 && CH % kStreamUnroll == 0, "a chunk is a whole number of wave loads");
+    constexpr int PRE = E / 64;
+    const int lane = threadIdx.x & 63;
+    const int total = count * R4;
+    const int chunks = (count + CH - 1) / CH;
+    int idx[PRE];
+    auto load_idx = [&](int chunk) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int ge = chunk * E + i * 64 + lane;
+            idx[i] = ge < total ? index[ge / R4] : -1;
+        }
+    };
+    auto issue = [&](float4* buf) {  // the records whose indices load_idx fetched last
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int part = (i * 64 + lane) % R4;  // E % R4 == 0: the same in every chunk
+            const float4* p = idx[i] >= 0 ? src + (size_t)idx[i] * R4 + part : zero_rec + part;
+            // Written as assembly: the compiler's wait-count pass, which follows the builtin form of
+            // this load, puts a vmcnt(0) in front of the LDS reads of whichever buffer sits at LDS
+            // address 0 (it no longer knows which array such a read belongs to), and the loads into
+            // the other buffer would not overlap with the compute.  The waits are `landed` below.
+            const unsigned lds = (unsigned)(__UINTPTR_TYPE__)(__attribute__((address_space(3))) float4*)(buf + i * 64);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :
+                         : "v"(p), "s"(lds)
+                         : "memory", "m0");
+        }
+    };
+    auto landed = [] { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    auto compute = [&](const float4* cur, int k) {
+        // (the last chunk stops after its last record's group; the slots behind it hold zeros)
+        const int lim = min(CH, (count - k * CH + kStreamUnroll - 1) / kStreamUnroll * kStreamUnroll);
+#pragma unroll 1
+        for (int n = 0; n < lim; n += kStreamUnroll) {
+            float4 rr[kStreamUnroll][R4];
+#pragma unroll
+            for (int u = 0; u < kStreamUnroll; ++u)
+#pragma unroll
+                for (int i = 0; i < R4; ++i) rr[u][i] = cur[(n + u) * R4 + i];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < kStreamUnroll; ++u) {
+                body(rr[u]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    if (chunks == 0) return;
+    load_idx(0);
+    issue(sh0);
+    load_idx(1);
+    landed();
+    for (int k = 0; k < chunks; k += 2) {
+        if (k + 1 < chunks) {
+            issue(sh1);
+            load_idx(k + 2);
+        }
+        compute(sh0, k);
+        landed();
+        if (k + 1 >= chunks) break;
+        if (k + 2 < chunks) {
+            issue(sh0);
+            load_idx(k + 3);
+        }
+        compute(sh1, k + 1);
+        landed();
     }
 }
 
@@ -211,29 +285,36 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
     }
 }
 
-// Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows;
-// workgroup = wx x (4/wx) waves, all four streaming the same Gaussians.  Per Gaussian and
-// lane: dx, A'dx^2, B2'dx once, then per pixel dy, 2 fma, exp2, 1 + C fma.
-template <int C, int P>
-__global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
+// Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows.  Per Gaussian
+// and lane: dx, A'dx^2, B2'dx once, then per pixel dy, 2 fma, exp2, 1 + C fma.
+// kWave = false: workgroup = wx x (4/wx) waves, all four streaming the tile's Gaussian list.
+// kWave = true (fwd_wave_lists): workgroup = one wave with a list of its own; four consecutive
+// workgroups are the four row blocks of one 64 x 4P tile of the binning.
+template <int C, int P, bool kWave>
+__global__ __launch_bounds__(kWave ? 64 : kThreads) void k_fwd_sep(const FwdArgs a) {
     constexpr int RS = rec_stride_of(C), R4 = RS / 4;
-    __shared__ float4 sh[2 * kGaussChunk * R4];
     IGS_GATE(a);
-    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
-    if (tile >= a.total_tiles) return;  // workgroup-uniform
+    const int units = kWave ? a.total_tiles * 4 : a.total_tiles;
+    const int unit = xcd_contiguous(blockIdx.x, units);
+    if (unit >= units) return;  // workgroup-uniform
+    const int tile = kWave ? unit >> 2 : unit;
     const int per_img = a.tiles_x * a.tiles_y;
     const int b = tile / per_img;
     const int tl = tile - b * per_img;
     const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
-    const int wave = threadIdx.x >> 6;
+    const int wave = kWave ? unit & 3 : (int)(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
-    const int wxi = wave % a.wx, wyi = wave / a.wx;
-    const int col = (tx * a.wx + wxi) * 64 + lane;
-    const int row0 = (ty * (4 / a.wx) + wyi) * P;
+    const int wx = kWave ? 1 : a.wx;
+    const int wxi = wave % wx, wyi = wave / wx;
+    const int col = (tx * wx + wxi) * 64 + lane;
+    const int row0 = (ty * (4 / wx) + wyi) * P;
     const float xv = a.x[b * a.sxb + (long)min(col, a.W - 1) * a.sxw];
     float yv[P];
+    // (all P loads first, then the pins: a pin right behind its load would wait for each load in turn)
 #pragma unroll
-    for (int p = 0; p < P; ++p) yv[p] = in_vgpr(a.y[b * a.syb + (long)min(row0 + p, a.H - 1) * a.syh]);
+    for (int p = 0; p < P; ++p) yv[p] = a.y[b * a.syb + (long)min(row0 + p, a.H - 1) * a.syh];
+#pragma unroll
+    for (int p = 0; p < P; ++p) yv[p] = in_vgpr(yv[p]);
 
     float dsum[P], num[P][C];
 #pragma unroll
@@ -254,24 +335,20 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
         wylo = -__builtin_inff();
         wyhi = __builtin_inff();
     }
-    // this tile's Gaussians (those whose reach box meets it), split S ways by list position
+    // this unit's Gaussians (those whose ellipse reaches it), split S ways by list position
     const int s = blockIdx.y;
-    const int count = a.counts[(size_t)b * per_img + tl];
+    const size_t li = kWave ? ((size_t)b * per_img + tl) * 4 + wave : (size_t)b * per_img + tl;
+    const int count = a.counts[li];
     const int per = ((count + a.S - 1) / a.S + 3) & ~3;
     const int n0 = min(count, s * per);
     const int n1 = min(count, n0 + per);
-    const int* list = a.lists + ((size_t)b * per_img + tl) * a.Np + n0;
+    const int* list = a.lists + li * a.Np + n0;
     const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
     auto body = [&](auto wave_skip, const float4* r) {
         const GRec<C> g = lds_grec<C>(r);
-        // The tile list is per workgroup (4 waves of 64 columns x P rows each); a wave that the entry's
-        // mask does not name, or whose rows the reach box misses, skips the record (wave-uniform: the
-        // record is the same in all lanes).
-        if (decltype(wave_skip)::value) {
-            if (fwd_wave_masks(C) ? __ballot((__float_as_int(g.ylo) >> wave) & 1) == 0ull
-                                  : __ballot(!(g.yhi < wylo || g.ylo > wyhi)) == 0ull)
-                return;
-        }
+        // A list shared by four waves of P rows each: a wave whose own rows the reach box misses
+        // skips the record (wave-uniform: the record is the same in all lanes).
+        if (decltype(wave_skip)::value && __ballot(!(g.yhi < wylo || g.ylo > wyhi)) == 0ull) return;
         const float dx = xv - g.px;
         const float adx = g.A * dx;
         const float c0 = adx * dx;
@@ -294,15 +371,24 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
             for (int c = 0; c < C; ++c) num[p][c] = fmaf(e[p], g.ac[c], num[p][c]);
         }
     };
-    // The per-wave test costs a few percent when it never fires, so it is used only for tiles
-    // that fewer than 7/8 of the Gaussians reach (workgroup-uniform choice of the loop): there
-    // some boxes are small against the image, and those are often small against the tile too.
-    if (rec_has_yrange(C) && 8L * count < 7L * a.Np)
-        stream_records_lds<R4, kGaussChunk, true, fwd_wave_masks(C) ? 6 + C : -1>(
-            src, n1 - n0, sh, [&](const float4* r) { body(std::true_type{}, r); }, list);
-    else
-        stream_records_lds<R4, kGaussChunk, true>(
-            src, n1 - n0, sh, [&](const float4* r) { body(std::false_type{}, r); }, list);
+    // The per-wave test of a shared list costs a few percent when it never fires, so it is used only
+    // for tiles that fewer than 7/8 of the Gaussians reach (workgroup-uniform choice of the loop):
+    // there some boxes are small against the image, and those are often small against the tile too.
+    if constexpr (kWave) {
+        __shared__ float4 sh0[kGaussChunk * R4];
+        __shared__ float4 sh1[kGaussChunk * R4];
+        stream_records_dma<R4, kGaussChunk>(
+            src, reinterpret_cast<const float4*>(a.zero_rec), n1 - n0, sh0, sh1,
+            [&](const float4* r) { body(std::false_type{}, r); }, list);
+    } else {
+        __shared__ float4 sh[2 * kGaussChunk * R4];
+        if (rec_has_yrange(C) && 8L * count < 7L * a.Np)
+            stream_records_lds<R4, kGaussChunk, true>(
+                src, n1 - n0, sh, [&](const float4* r) { body(std::true_type{}, r); }, list);
+        else
+            stream_records_lds<R4, kGaussChunk, true>(
+                src, n1 - n0, sh, [&](const float4* r) { body(std::false_type{}, r); }, list);
+    }
     if (col < a.W) {
 #pragma unroll
         for (int p = 0; p < P; ++p)

@@ -84,7 +84,8 @@ FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
         // on a tie the squarest tile (fewest Gaussians reach it)
         long best = -1;
         g.wx = 1;
-        for (int wx = 1; wx <= 4; wx <<= 1) {
+        // (variants with a list per wave stack their four waves: 64 columns x 4 P rows)
+        for (int wx = 1; wx <= (fwd_wave_lists(C) ? 1 : 4); wx <<= 1) {
             const long cols = (long)ceil_div(W, 64 * wx) * 64 * wx;
             const long rows = (long)ceil_div(H, kFwdSepP * (4 / wx)) * kFwdSepP * (4 / wx);
             const long area = cols * rows;
@@ -202,10 +203,11 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     }
     T = (long)ceil_div(sep ? H : p->hw_padded, p->bwd_per_tile) * p->bwd_tiles_x;
     p->bwd_tiles = (int)T;
-    p->fwd_tiles = sep ? fg.tiles_x * fg.tiles_y : 0;
+    p->fwd_tiles = sep ? fg.tiles_x * fg.tiles_y * (fwd_wave_lists(C) ? 4 : 1) : 0;
     p->pix_stride = sep ? pix_stride_sep(C) : pix_stride_gen(C);
     // records, then one bin record (8 floats) per record, then the call's skip settings (4 floats)
-    p->packed_bytes = ((uint64_t)B * p->n_padded * (p->rec_stride + 8) + 4) * sizeof(float);
+    // and an all-zero record
+    p->packed_bytes = ((uint64_t)B * p->n_padded * (p->rec_stride + 8) + 4 + kZeroRecFloats) * sizeof(float);
     p->fwd_ws_bytes = S > 1 ? (uint64_t)S * B * (C + 1) * H * W * sizeof(float) : 0;
     p->pix_bytes = sep ? ((uint64_t)B * H * p->w_padded * p->pix_stride + (uint64_t)B * p->w_padded) * sizeof(float)
                        : (uint64_t)B * p->hw_padded * p->pix_stride * sizeof(float);
@@ -318,7 +320,7 @@ int launch_bins(BinArgs fine, int B, bool levels2, const BinPlace& coarse, int* 
     c.tiles_x = sg.x; c.tiles_y = sg.y;
     c.counts = coarse.counts; c.lists = coarse.lists; c.slots = coarse_slots;
     c.chunk = sg.chunk;
-    c.sub_nx = 0; c.sub_h = 0;  // wave masks belong to the tiles' own lists
+    c.sub_nx = 0; c.sub_h = 0;  // a super-tile has one list
     int rc = launch_bin(c, sg.K, B, st);
     if (rc) return rc;
     fine.cand_counts = coarse.counts; fine.cand_lists = coarse.lists;
@@ -375,10 +377,11 @@ struct MseArgs {
 
 template <int C>
 int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
-    const int blocks = ((a.total_tiles + 7) / 8) * 8;
-    const dim3 grid(blocks, a.S, 1);
+    constexpr bool kWave = fwd_wave_lists(C);
+    const int units = sep && kWave ? a.total_tiles * 4 : a.total_tiles;  // one-wave workgroups: four per tile
+    const dim3 grid(((units + 7) / 8) * 8, a.S, 1);
     if (sep)
-        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C)>), grid, dim3(kThreads), 0, st, a);
+        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), kWave>), grid, dim3(kWave ? 64 : kThreads), 0, st, a);
     else
         hipLaunchKernelGGL((k_fwd_gen<C, fwd_gen_p(C)>), grid, dim3(kThreads), 0, st, a);
     return launch_status();
@@ -575,6 +578,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
         const FwdGeometry fg = fwd_geometry(B, H, W, C, sep);
         FwdArgs a;
         a.packed = packed; a.x = x; a.y = y;
+        a.zero_rec = limit_of(packed, B, plan.n_padded, plan.rec_stride) + 4;
         a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
         a.syb = grid_strides[3]; a.syh = grid_strides[4]; a.syw = grid_strides[5];
         a.B = B; a.Np = plan.n_padded; a.H = H; a.W = W;
@@ -598,8 +602,8 @@ int forward_impl(const float* packed, const float* x, const float* y,
             ba.counts = bp.counts; ba.lists = bp.lists; ba.slots = nullptr;
             ba.flag = vs[i].flag; ba.want = vs[i].want;
             ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
-            // which of the workgroup's four waves a Gaussian reaches travels in its list entry
-            ba.sub_nx = fwd_wave_masks(C) ? fg.wx : 0;
+            // a list per wave of the forward: four per tile of the binning
+            ba.sub_nx = fwd_wave_lists(C) ? fg.wx : 0;
             ba.sub_h = fwd_sep_p(C);
             const bool levels2 = two_level(N, fg.tiles_x, fg.tiles_y, opts_of(grid_mode));
             const BinPlace cp = levels2 ? super_bins_at(ws, split_bytes, B, plan.fwd_tiles, plan.n_padded,

@@ -60,9 +60,13 @@ __device__ __forceinline__ void write_empty_bin_record(float4* bins, size_t i) {
 
 // The call's skip limit and skip fraction travel behind the bin records in the packed buffer
 // (4 floats, the first two used), where k_bin reads them: the forward and the backward then need no
-// argument for them.
+// argument for them.  Behind them sits one all-zero record (kZeroRecFloats floats, the widest
+// record), which the forward's direct global-to-LDS loads read for the slots past a list's end.
+constexpr int kZeroRecFloats = 28;
 __device__ __forceinline__ void write_skip_limit(float4* bins, int B, int Np, float limit, float fraction) {
-    bins[(size_t)2 * B * Np] = make_float4(fminf(limit, kExactLimit), fraction, 0.0f, 0.0f);
+    float4* tail = bins + (size_t)2 * B * Np;
+    tail[0] = make_float4(fminf(limit, kExactLimit), fraction, 0.0f, 0.0f);
+    for (int i = 0; i < kZeroRecFloats / 4; ++i) tail[1 + i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 }
 
 // One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
@@ -236,10 +240,9 @@ struct BinArgs {
     const int* flag;
     int want;
     int no_cull;  // list every candidate (IGS_OPT_NO_CULL): the reference point for "culling changes no bit"
-    // Wave masks (the forward's lists; sub_nx = 0: none).  The tile is sub_nx x (4 / sub_nx) rectangles of
-    // 64 columns x sub_h rows, one per wave of the forward's workgroup (wave w: column block w % sub_nx,
-    // row block w / sub_nx).  A Gaussian is listed when its ellipse reaches at least one of them, and bits
-    // 24..27 of its list entry say which (N <= 2^24 leaves them free).
+    // Four lists per tile (the forward's wave lists; sub_nx = 0: one list).  The tile is sub_nx x
+    // (4 / sub_nx) rectangles of 64 columns x sub_h rows (rectangle w: column block w % sub_nx, row
+    // block w / sub_nx), each with a list of its own: list and count number 4 t + w of the image.
     int sub_nx, sub_h;
 };
 
@@ -304,7 +307,7 @@ template <bool kMasks>
 __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     if (a.flag != nullptr && *a.flag != a.want) return;
     __shared__ float red[4][kBinWaves];
-    __shared__ int wsum[kBinWaves];
+    __shared__ int wsum[kMasks ? 4 : 1][kBinWaves];
     __shared__ int seg_first[kBinMaxChunks + 1];  // second level: first candidate index of each segment
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tiles = a.tiles_x * a.tiles_y;
@@ -439,7 +442,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     }
     float limit = a.limit[0];
     const float fraction = a.limit[1];
-    int* list = a.lists + ((size_t)b * tiles + t) * a.Np + (size_t)kc * a.chunk;
+    int* list = a.lists + ((size_t)b * tiles + t) * (masks ? 4 : 1) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     // "definitely outside" negated, so that NaN bounds count as inside
     auto meets_tile = [&](const Batch& bt, int u) {
@@ -488,7 +491,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             limit = fminf(limit, -__log2f(w0 + fraction * total));
         }
     }
-    // code: which of the forward's waves the Gaussian reaches (wave masks), or 1; 0 = not listed
+    // code: which of the tile's four rectangles the Gaussian reaches (four lists), or 1; 0 = not listed
     auto classify = [&](int n0, const Batch& bt, int (&code)[kU], bool (&in)[kU]) {
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
@@ -508,12 +511,14 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             code[u] = !meets ? 0 : (refine ? reached : (masks ? 15 : 1));
         }
     };
-    // the classifying scan keeps its verdicts (one bit, or four with wave masks, per candidate of this
+    // the classifying scan keeps its verdicts (one bit, or four with four lists, per candidate of this
     // lane) for the writing one when they fit in a register pair, i.e. up to 64 (16) candidates per lane
-    const int vbits = masks ? 4 : 1;
+    constexpr int vbits = masks ? 4 : 1, kL = masks ? 4 : 1;  // kL lists per tile
     const bool keep = per_wave * vbits <= 64 * 64;
     unsigned long long verdicts = 0ull;
-    int cnt = 0, it = 0;
+    int cnt[kL], it = 0;
+#pragma unroll
+    for (int l = 0; l < kL; ++l) cnt[l] = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
         Batch bt = head;
         if (it > 0) load_batch(n0, bt);
@@ -522,17 +527,24 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         classify(n0, bt, code, in);
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
-            cnt += __popcll(__ballot(code[u] != 0));
+#pragma unroll
+            for (int l = 0; l < kL; ++l) cnt[l] += __popcll(__ballot((code[u] >> l) & 1));
             verdicts |= (unsigned long long)code[u] << (((it * kU + u) * vbits) & 63);
         }
     }
-    if (lane == 0) wsum[wave] = cnt;
-    __syncthreads();
-    int base = 0, total = 0;
+    if (lane == 0)
 #pragma unroll
-    for (int w = 0; w < kBinWaves; ++w) {
-        if (w < wave) base += wsum[w];
-        total += wsum[w];
+        for (int l = 0; l < kL; ++l) wsum[l][wave] = cnt[l];
+    __syncthreads();
+    int base[kL], total[kL];
+#pragma unroll
+    for (int l = 0; l < kL; ++l) {
+        base[l] = total[l] = 0;
+#pragma unroll
+        for (int w = 0; w < kBinWaves; ++w) {
+            if (w < wave) base[l] += wsum[l][w];
+            total[l] += wsum[l][w];
+        }
     }
     it = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
@@ -553,16 +565,20 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             for (int u = 0; u < kU; ++u) n[u] = bt.n[u];
         }
 #pragma unroll
-        for (int u = 0; u < kU; ++u) {
-            const bool listed = code[u] != 0;
-            const unsigned long long m = __ballot(listed);
-            const int pos = base + __popcll(m & below);
-            if (listed) list[pos] = masks ? (n[u] | (code[u] << 24)) : n[u];
-            // the slot of every candidate: its position (within the segment, at the first level,
-            // where only the sign is used) or -1
-            if (slot != nullptr && in[u]) slot[n[u]] = listed ? pos : -1;
-            base += __popcll(m);
-        }
+        for (int u = 0; u < kU; ++u)
+#pragma unroll
+            for (int l = 0; l < kL; ++l) {
+                const bool listed = (code[u] >> l) & 1;
+                const unsigned long long m = __ballot(listed);
+                const int pos = base[l] + __popcll(m & below);
+                if (listed) list[(size_t)l * a.Np + pos] = n[u];
+                // the slot of every candidate: its position (within the segment, at the first level,
+                // where only the sign is used) or -1
+                if (!masks && slot != nullptr && in[u]) slot[n[u]] = listed ? pos : -1;
+                base[l] += __popcll(m);
+            }
     }
-    if (tid == 0) a.counts[((size_t)b * tiles + t) * K + kc] = total;
+    if (tid == 0)
+#pragma unroll
+        for (int l = 0; l < kL; ++l) a.counts[(((size_t)b * tiles + t) * K + kc) * kL + l] = total[l];
 }

@@ -69,7 +69,7 @@ def test_plan_arithmetic(lib, mode):
         assert p.n_padded % 4 == 0 and p.n_padded >= N
         assert p.fwd_n_per_split % 4 == 0 and p.fwd_split * p.fwd_n_per_split >= p.n_padded
         assert (p.fwd_split - 1) * p.fwd_n_per_split < p.n_padded          # no empty split
-        assert p.packed_bytes == (B * p.n_padded * (p.rec_stride + 8) + 4) * 4    # records + bin records + skip settings
+        assert p.packed_bytes == (B * p.n_padded * (p.rec_stride + 8) + 32) * 4    # records + bin records + skip settings + zero record
         assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
         assert p.bwd_tiles >= 1 and p.partial_bytes >= B * p.bwd_tiles * (6 + C) * N * 4
         if mode != 0:
@@ -266,7 +266,7 @@ def test_plan_invariants_over_random_shapes(lib):
             Np = p.n_padded
             assert Np % 4 == 0 and N <= Np < N + 4
             assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
-            assert p.packed_bytes == (B * Np * (p.rec_stride + 8) + 4) * 4
+            assert p.packed_bytes == (B * Np * (p.rec_stride + 8) + 32) * 4
             assert 1 <= p.fwd_split <= 64 and p.fwd_n_per_split % 4 == 0
             assert p.fwd_split * p.fwd_n_per_split >= Np > (p.fwd_split - 1) * p.fwd_n_per_split
             assert p.bwd_tiles >= 1 and p.bwd_per_tile >= 1
