@@ -33,8 +33,8 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 # (factors from the plain-copy calibration of the same profile run).
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
-    "bwd": {"fma": 1.321e9, "mul": 2.47e8, "add": 1.33e8, "trans": 1.196e8, "fetch_kib": 48216, "write_kib": 141629},
-    "fwd": {"fma": 7.095e8, "mul": 2.22e7, "add": 1.256e8, "trans": 1.183e8, "fetch_kib": 9886, "write_kib": 139251},
+    "bwd": {"fma": 8.637e8, "mul": 1.655e8, "add": 9.489e7, "trans": 7.792e7, "fetch_kib": 50120, "write_kib": 191800},
+    "fwd": {"fma": 4.720e8, "mul": 1.477e7, "add": 8.358e7, "trans": 7.869e7, "fetch_kib": 13020, "write_kib": 131100},
 }
 
 
@@ -203,8 +203,13 @@ def main() -> int:
                                                 H, W, C, _ptr(pix), int(op.plan.pix_bytes), _ptr(partial),
                                                 int(op.plan.partial_bytes), st), "reduce")
 
+    fwd_ws = op._empty(op.plan.fwd_ws_bytes)
+    fwd_out, fwd_den = op._new(B, C, H, W), op._new(B, H, W)
+
     def fwd_kernel():
-        op.forward(packed)
+        _lib.check(lib.igs_gs2d_forward(_ptr(packed), _ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode,
+                                        _ptr(grid.flag), B, N, H, W, C, 1e-6, _ptr(fwd_out), _ptr(fwd_den), _ptr(fwd_ws),
+                                        int(op.plan.fwd_ws_bytes), st), "forward")
 
     def event_time(fn, reps):
         for _ in range(3):
@@ -234,6 +239,17 @@ def main() -> int:
     evaluated = int((counts.long() * (rows[:, None] * cols[None, :])[None]).sum())
     achieved = evaluated * f_bwd / t_bwd_kernel / 1e12
     prof = C1_PROFILE if (args.config == "c1" and C == 3) else None
+    # The same for the forward (C <= 3: one list per wave of 64 columns x 16 rows, four per 64 x 64 tile
+    # of the binning, behind the split partials in the forward's workspace).
+    fwd_evaluated = None
+    if C <= 3:
+        split = plan.fwd_split * B * (C + 1) * H * W * 4 if plan.fwd_split > 1 else 0
+        tx_n, ty_n = -(-W // 64), -(-H // 64)
+        fc = fwd_ws.view(torch.int32)[(split + 15) // 16 * 4:][: B * plan.fwd_tiles].view(B, ty_n, tx_n, 4).cpu()
+        frows = torch.tensor([[max(0, min(H, (4 * i + w + 1) * 16) - (4 * i + w) * 16) for w in range(4)]
+                              for i in range(ty_n)])
+        fcols = torch.tensor([min(W, (i + 1) * 64) - i * 64 for i in range(tx_n)])
+        fwd_evaluated = int((fc.long() * (frows[None, :, None, :] * fcols[None, None, :, None])).sum())
 
     result = {
         "metric": "gaussian_pixel_evals_per_sec_fwd_bwd",
@@ -254,6 +270,8 @@ def main() -> int:
         "fwd_ms": t_fwd * 1e3,
         "step_tflops": pairs * (f_fwd + f_bwd) / t_step / 1e12,
         "step_frac_of_fp32_vector_peak": pairs * (f_fwd + f_bwd) / t_step / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+        "step_frac_counting_evaluated_pairs": ((fwd_evaluated or pairs) * f_fwd + evaluated * f_bwd) / t_step / 1e12
+                                              / FP32_VECTOR_PEAK_TFLOPS,
         "roofline": {
             "bound": "valu",
             "kernel": f"k_bwd_sep<{C},2> (backward per-Gaussian reduction)",
@@ -269,16 +287,19 @@ def main() -> int:
             "executed_frac": executed_flops(prof["bwd"]) / t_bwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS if prof else None,
             "traffic": hbm_bytes(prof["bwd"]) if prof else None,
             "forward_kernel": {"launch_ms": t_fwd_kernel * 1e3, "flops_per_pair": f_fwd,
-                               "achieved": pairs * f_fwd / t_fwd_kernel / 1e12,
-                               "frac": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+                               "pairs_evaluated_per_launch": fwd_evaluated,
+                               "achieved": (fwd_evaluated or pairs) * f_fwd / t_fwd_kernel / 1e12,
+                               "frac": (fwd_evaluated or pairs) * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+                               "frac_counting_all_pairs": pairs * f_fwd / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
                                "executed_frac": executed_flops(prof["fwd"]) / t_fwd_kernel / 1e12 / FP32_VECTOR_PEAK_TFLOPS
                                if prof else None,
                                "traffic": hbm_bytes(prof["fwd"]) if prof else None},
             "counter_source": prof["source"] if prof else None,
             "note": "achieved / frac: the 30+4C FLOP model of one backward pair x the pairs the kernel evaluated (the tile "
-                    "lists skip pairs whose weight is exactly 0; frac_counting_all_pairs uses all B N H W as the metric "
-                    "does) / launch_ms, measured live with HIP events around igs_gs2d_backward_reduce = k_bin (~33 us) + "
-                    "k_bwd_sep.  executed_frac: the arithmetic the hardware ran, (2 FMA + MUL + ADD + TRANS) x 64 per "
+                    "lists skip pairs whose weight is below the skip weight, which bounds the change of every output "
+                    "element by 1e-7 max|colour|; frac_counting_all_pairs uses all B N H W as the metric does and can "
+                    "exceed 1) / launch_ms, measured live with HIP events around igs_gs2d_backward_reduce = k_bin "
+                    "(~65 us) + k_bwd_sep.  executed_frac: the arithmetic the hardware ran, (2 FMA + MUL + ADD + TRANS) x 64 per "
                     "launch from the rocprofv3 counters of counter_source (separable grids hoist the row/column part of "
                     "the model's operations, so it is below frac) / the live launch_ms.  traffic: HBM bytes per launch "
                     "from FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of the same summary (copy-calibrated); c1 only.  peak: "

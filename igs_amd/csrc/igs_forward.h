@@ -186,7 +186,8 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
     }
 }
 
-// The same stream for a workgroup of one wave, without staging registers: the records of the next
+// The same stream for one wave on its own (wave-uniform `count`, `index` and buffers; no barrier, so
+// the waves of a workgroup may run it with different lists), without staging registers: the records of the next
 // chunk go from global memory straight into the other LDS buffer (global_load_lds_dwordx4: lane l
 // of the instruction writes 16 bytes at base + 16 l) while the current one is computed, and one
 // vmcnt wait per chunk separates the two.  Slots past `count` load the all-zero record `zero_rec`.
@@ -220,7 +221,8 @@ __device__ __forceinline__ void stream_records_dma(const float4* __restrict__ sr
             // this load, puts a vmcnt(0) in front of the LDS reads of whichever buffer sits at LDS
             // address 0 (it no longer knows which array such a read belongs to), and the loads into
             // the other buffer would not overlap with the compute.  The waits are `landed` below.
-            const unsigned lds = (unsigned)(__UINTPTR_TYPE__)(__attribute__((address_space(3))) float4*)(buf + i * 64);
+            const unsigned lds = __builtin_amdgcn_readfirstlane(
+                (unsigned)(__UINTPTR_TYPE__)(__attribute__((address_space(3))) float4*)(buf + i * 64));
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                          :
                          : "v"(p), "s"(lds)
@@ -288,21 +290,20 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 // Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows.  Per Gaussian
 // and lane: dx, A'dx^2, B2'dx once, then per pixel dy, 2 fma, exp2, 1 + C fma.
 // kWave = false: workgroup = wx x (4/wx) waves, all four streaming the tile's Gaussian list.
-// kWave = true (fwd_wave_lists): workgroup = one wave with a list of its own; four consecutive
-// workgroups are the four row blocks of one 64 x 4P tile of the binning.
+// kWave = true (fwd_wave_lists): every wave has a list of its own and streams it independently of
+// the others (no barrier in the kernel); the four waves of a workgroup are the four row blocks of
+// one 64 x 4P tile of the binning.
 template <int C, int P, bool kWave>
-__global__ __launch_bounds__(kWave ? 64 : kThreads) void k_fwd_sep(const FwdArgs a) {
+__global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     constexpr int RS = rec_stride_of(C), R4 = RS / 4;
     IGS_GATE(a);
-    const int units = kWave ? a.total_tiles * 4 : a.total_tiles;
-    const int unit = xcd_contiguous(blockIdx.x, units);
-    if (unit >= units) return;  // workgroup-uniform
-    const int tile = kWave ? unit >> 2 : unit;
+    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
+    if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int per_img = a.tiles_x * a.tiles_y;
     const int b = tile / per_img;
     const int tl = tile - b * per_img;
     const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
-    const int wave = kWave ? unit & 3 : (int)(threadIdx.x >> 6);
+    const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int wx = kWave ? 1 : a.wx;
     const int wxi = wave % wx, wyi = wave / wx;
@@ -375,10 +376,10 @@ __global__ __launch_bounds__(kWave ? 64 : kThreads) void k_fwd_sep(const FwdArgs
     // for tiles that fewer than 7/8 of the Gaussians reach (workgroup-uniform choice of the loop):
     // there some boxes are small against the image, and those are often small against the tile too.
     if constexpr (kWave) {
-        __shared__ float4 sh0[kGaussChunk * R4];
-        __shared__ float4 sh1[kGaussChunk * R4];
+        __shared__ float4 sh0[4][kGaussChunk * R4];  // per wave: the two chunk buffers
+        __shared__ float4 sh1[4][kGaussChunk * R4];
         stream_records_dma<R4, kGaussChunk>(
-            src, reinterpret_cast<const float4*>(a.zero_rec), n1 - n0, sh0, sh1,
+            src, reinterpret_cast<const float4*>(a.zero_rec), n1 - n0, sh0[wave], sh1[wave],
             [&](const float4* r) { body(std::false_type{}, r); }, list);
     } else {
         __shared__ float4 sh[2 * kGaussChunk * R4];

@@ -377,11 +377,9 @@ struct MseArgs {
 
 template <int C>
 int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
-    constexpr bool kWave = fwd_wave_lists(C);
-    const int units = sep && kWave ? a.total_tiles * 4 : a.total_tiles;  // one-wave workgroups: four per tile
-    const dim3 grid(((units + 7) / 8) * 8, a.S, 1);
+    const dim3 grid(((a.total_tiles + 7) / 8) * 8, a.S, 1);
     if (sep)
-        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), kWave>), grid, dim3(kWave ? 64 : kThreads), 0, st, a);
+        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), fwd_wave_lists(C)>), grid, dim3(kThreads), 0, st, a);
     else
         hipLaunchKernelGGL((k_fwd_gen<C, fwd_gen_p(C)>), grid, dim3(kThreads), 0, st, a);
     return launch_status();
