@@ -298,11 +298,20 @@ int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t*
     return IGS_OK;
 }
 
+// Threads of a k_bin workgroup: four candidates per lane when there are few of them (the scans load
+// and test four at a time: more threads would only be more waves to start), 1024 otherwise.
+inline int bin_threads(long candidates) {
+    long t = ((candidates + 3) / 4 + 63) & ~63L;
+    return (int)(t < 256 ? 256 : (t > kBinThreads ? kBinThreads : t));
+}
+
 int launch_bin(const BinArgs& a, int K, int B, hipStream_t st) {
+    // (at the second level of a two-level binning the candidates are the super-tile's list: unknown here)
+    const int threads = bin_threads(a.cand_lists != nullptr ? kBinThreads * 4 : (a.chunk > 0 ? a.chunk : a.N));
     if (a.sub_nx > 0)
-        hipLaunchKernelGGL(k_bin<true>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(kBinThreads), 0, st, a);
+        hipLaunchKernelGGL(k_bin<true>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(threads), 0, st, a);
     else
-        hipLaunchKernelGGL(k_bin<false>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(kBinThreads), 0, st, a);
+        hipLaunchKernelGGL(k_bin<false>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(threads), 0, st, a);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? IGS_OK : (int)e;
 }

@@ -310,6 +310,15 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     __shared__ int wsum[kMasks ? 4 : 1][kBinWaves];
     __shared__ int seg_first[kBinMaxChunks + 1];  // second level: first candidate index of each segment
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // launched with 256 to kBinThreads threads (bin_threads): the reductions below run over kBinWaves
+    // slots, those of waves that do not exist hold the neutral element
+    const int nthreads = blockDim.x, nwaves = nthreads >> 6;
+    if (tid < kBinWaves && tid >= nwaves) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) red[f][tid] = __builtin_inff();
+#pragma unroll
+        for (int l = 0; l < (kMasks ? 4 : 1); ++l) wsum[l][tid] = 0;
+    }
     const int tiles = a.tiles_x * a.tiles_y;
     const int t = blockIdx.x, kc = blockIdx.y, K = gridDim.y, b = blockIdx.z;
     const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
@@ -351,7 +360,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     // Each wave scans one contiguous share of the candidates, without barriers inside a scan: once
     // for the tile's denominator floor (skip fraction only), once to classify and count, and once
     // (from the kept verdicts, with the shares' counts prefixed in wave order) to write.
-    const int per_wave = ((M + kBinWaves - 1) / kBinWaves + 63) & ~63;
+    const int per_wave = ((M + nwaves - 1) / nwaves + 63) & ~63;
     const int nb = wave * per_wave, ne = min(M, nb + per_wave);
     const unsigned long long below = (1ull << lane) - 1ull;
     // The bin records of kU candidates per lane are loaded together (2 kU loads in flight).  The
@@ -383,13 +392,13 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     bool bad = false;
     constexpr bool masks = kMasks;  // a.sub_nx > 0
     if (!masks) {
-        for (int c = c0 + tid; c < c1; c += kBinThreads) {
+        for (int c = c0 + tid; c < c1; c += nthreads) {
             const float v = a.x[b * a.sxb + (long)c * a.sxw];
             bad = bad || !(v == v);
             xlo = fminf(xlo, v);
             xhi = fmaxf(xhi, v);
         }
-        for (int r = r0 + tid; r < r1; r += kBinThreads) {
+        for (int r = r0 + tid; r < r1; r += nthreads) {
             const float v = a.y[b * a.syb + (long)r * a.syh];
             bad = bad || !(v == v);
             ylo = fminf(ylo, v);
@@ -483,8 +492,8 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         float total = 0.0f, anyneg = 0.0f;
 #pragma unroll
         for (int w = 0; w < kBinWaves; ++w) {
-            total += red[0][w];
-            anyneg += red[1][w];
+            total += w < nwaves ? red[0][w] : 0.0f;
+            anyneg += w < nwaves ? red[1][w] : 0.0f;
         }
         if (anyneg == 0.0f && total > 0.0f) {
             const float w0 = limit < kExactLimit ? hw_exp2(-limit) : 0.0f;
