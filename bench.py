@@ -78,6 +78,10 @@ def main() -> int:
                          "diversity loss (src/igs/reg.py of the reference) beside the plain torch expression")
     ap.add_argument("--koleo-shape", default=None, metavar="BxNxD",
                     help="with --koleo: time this one shape only, without the torch and CPU columns (for profiling)")
+    ap.add_argument("--skip-tolerance", type=float, default=None, metavar="T",
+                    help="bound on what skipped pairs may change in an output element, as a fraction of the largest "
+                         "colour (default: the library's 1e-7; 0 = skip exact zeros only)")
+    ap.add_argument("--no-cull", action="store_true", help="evaluate every pair (IGS_OPT_NO_CULL)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
@@ -98,6 +102,10 @@ def main() -> int:
             print("bench.py: %s is not built (python -m igs_amd.build)" % exe, file=sys.stderr)
             return 1
         return subprocess.run([exe]).returncode
+    # what the separable kernels may skip, for every mode below (explicit arguments of each library call)
+    from igs_amd._splat import library_options
+    culling = library_options(no_cull=args.no_cull, skip_tolerance=args.skip_tolerance)
+    culling.__enter__()   # (kept referenced to the end of main: a dropped context would restore at once)
     if args.sweep:
         return sweep(args.sweep_shape, not args.sweep_no_grid_grads)
     if args.all:

@@ -191,7 +191,7 @@ int igs_gs2d_forward(const float *packed, const float *x, const float *y,
  * The forward's scratch (split partials, per-tile Gaussian lists) lives in a static device array
  * of IGS_STATIC_SCRATCH_BYTES (64 MiB) that every GPU the library runs on holds until the process
  * ends; problems whose plan.fwd_ws_bytes is larger are rejected with IGS_ERR_STATIC_SCRATCH
- * (B=1, N=2048, 256x256, C=3 needs 32 MiB; the 16-image headline shape needs 136 MiB and must use
+ * (B=1, N=2048, 256x256, C=3 needs 32.5 MiB; the 16-image headline shape needs 160 MiB and must use
  * igs_gs2d_forward).  Same kernels, same launch plan and bit-identical results as
  * igs_gs2d_forward.  All calls on one GPU share that GPU's array: calls that overlap in time on
  * one GPU (two streams, two threads) race on it; nothing in it has to start at zero and its
