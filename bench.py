@@ -104,8 +104,11 @@ def main() -> int:
         return subprocess.run([exe]).returncode
     # what the separable kernels may skip, for every mode below (explicit arguments of each library call)
     from igs_amd._splat import library_options
-    culling = library_options(no_cull=args.no_cull, skip_tolerance=args.skip_tolerance)
-    culling.__enter__()   # (kept referenced to the end of main: a dropped context would restore at once)
+    with library_options(no_cull=args.no_cull, skip_tolerance=args.skip_tolerance):
+        return run(args)
+
+
+def run(args) -> int:
     if args.sweep:
         return sweep(args.sweep_shape, not args.sweep_no_grid_grads)
     if args.all:

@@ -223,10 +223,12 @@ __device__ __forceinline__ void stream_records_dma(const float4* __restrict__ sr
             // the other buffer would not overlap with the compute.  The waits are `landed` below.
             const unsigned lds = __builtin_amdgcn_readfirstlane(
                 (unsigned)(__UINTPTR_TYPE__)(__attribute__((address_space(3))) float4*)(buf + i * 64));
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                         :
+            unsigned m0_saved;  // M0 is put back: the compiler does not honour a clobber of it
+            asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\t"
+                         "s_nop 0\n\ts_mov_b32 m0, %0"
+                         : "=&s"(m0_saved)
                          : "v"(p), "s"(lds)
-                         : "memory", "m0");
+                         : "memory");
         }
     };
     auto landed = [] { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
