@@ -181,7 +181,7 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     S = ceil_div(p->n_padded, nps);
     p->fwd_split = (int)S;
     p->fwd_n_per_split = nps;
-    const long groups = (long)B * ceil_div(N, kThreads * (sep ? kBwdG : bwd_gen_g(C))) * 4;  // waves per tile
+    const long groups = (long)B * ceil_div(N, kThreads * (sep ? bwd_sep_g(C) : bwd_gen_g(C))) * 4;  // waves per tile
     long T = ((long)cus * 4 * IGS_BWD_WAVES + groups - 1) / groups;     // backward: waves per SIMD wanted
     p->bwd_tiles_x = sep ? ceil_div(p->w_padded, kBwdTileW) : 1;
     p->bwd_tile_w = sep ? kBwdTileW : 0;
@@ -425,8 +425,8 @@ template <int C>
 int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     if (sep) {
         // every list position up to Np is visited: listed Gaussians compute, the others store zeros
-        const dim3 grid(a.T, ceil_div(a.Np, kThreads * kBwdG), B);
-        hipLaunchKernelGGL((k_bwd_sep<C, kBwdG>), grid, dim3(kThreads), 0, st, a);
+        const dim3 grid(a.T, ceil_div(a.Np, kThreads * bwd_sep_g(C)), B);
+        hipLaunchKernelGGL((k_bwd_sep<C, bwd_sep_g(C)>), grid, dim3(kThreads), 0, st, a);
     } else {
         const dim3 grid(bwd_gen_groups(a.N, C), a.T, B);
         if (a.grid_part != nullptr)
