@@ -43,13 +43,16 @@ struct GRec {
 
 // whether a record of C channels has room for the y range of the reach box
 __host__ __device__ constexpr bool rec_has_yrange(int C) { return rec_stride_of(C) >= 8 + C; }
-// The separable forward variants whose waves hold 16 rows (C <= 3) give every wave a Gaussian list of
-// its own (64 columns x 16 rows) and run one wave per workgroup: no wave waits for another at a
-// chunk boundary, and none reads records it then skips.  With fewer rows per wave the tile of four
-// waves is small already (the lists of single waves would cost the binning more than the forward
-// gains): those variants stream one list to four waves, and a wave tests the reach box's y range
-// against its own rows.
-__host__ __device__ constexpr bool fwd_wave_lists(int C) { return fwd_sep_p(C) >= 16; }
+// The separable forward variants whose waves hold 16 or 8 rows (C <= 8) give every wave a Gaussian list
+// of its own (64 columns x P rows); the four waves of a workgroup stream theirs independently: no
+// wave waits for another at a chunk boundary, and none reads records it then skips.  With 4 rows per
+// wave (C = 16) the tile of four waves is small already and the lists of single waves cost the
+// binning more than the forward gains (B=4, N=32768, 384x640: 3.25 -> 3.73 ms): that variant streams
+// one list to four waves, and a wave tests the reach box's y range against its own rows.
+#ifndef IGS_FWD_WAVE_MIN_P
+#define IGS_FWD_WAVE_MIN_P 8
+#endif
+__host__ __device__ constexpr bool fwd_wave_lists(int C) { return fwd_sep_p(C) >= IGS_FWD_WAVE_MIN_P; }
 
 // Unpacks one record held in R4 float4 registers (read from a wave-uniform LDS address).
 template <int C>
