@@ -495,7 +495,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             total += w < nwaves ? red[0][w] : 0.0f;
             anyneg += w < nwaves ? red[1][w] : 0.0f;
         }
-        if (anyneg == 0.0f && total > 0.0f) {
+        if (anyneg == 0.0f && total > 0.0f && total < inf) {  // (an overflowed sum bounds nothing)
             const float w0 = limit < kExactLimit ? hw_exp2(-limit) : 0.0f;
             limit = fminf(limit, -__log2f(w0 + fraction * total));
         }

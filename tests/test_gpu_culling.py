@@ -482,7 +482,7 @@ def test_tile_lists_against_the_oracle_s_rectangle_minimum(igs, dev, tolerance, 
         assert float(torch.stack(floors).median()) * f > 10 * w
 
 
-@pytest.mark.parametrize("alpha_scale", [1.0, 25.0])
+@pytest.mark.parametrize("alpha_scale", [1.0, 25.0, 1e30])
 def test_default_skip_tolerance_stays_within_its_bound(igs, dev, alpha_scale):
     """The default skip weight against the run that lists every Gaussian for every tile, on sparse
     scenes where most pixels have a denominator far below eps (the worst case of the bound): every
@@ -492,10 +492,15 @@ def test_default_skip_tolerance_stays_within_its_bound(igs, dev, alpha_scale):
 
     B, N, H, W, C = 2, 120, 160, 192, 3
     _, g = sparse_case(dev, B, N, H, W, C, seed=23, smin=0.003, smax=0.03)
-    g["alphas"] = (g["alphas"] * alpha_scale).contiguous()
+    if alpha_scale > 1e20:   # one enormous alpha: its tiles' denominator floors are enormous too
+        g["alphas"] = g["alphas"].clone()
+        g["alphas"][:, 7] = alpha_scale
+    else:
+        g["alphas"] = (g["alphas"] * alpha_scale).contiguous()
     out, grads = run(igs, g)
     with no_cull_ctx():
         out0, grads0 = run(igs, g)
+    assert bool(torch.isfinite(out0).all())
     cmax = float(g["colors"].abs().max())
     assert SKIP_TOLERANCE == 1e-7
     err = (out - out0).abs()
