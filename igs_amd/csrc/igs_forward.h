@@ -16,8 +16,8 @@ struct FwdArgs {
     float* out;
     float* den;
     float* part;  // [S][B][C+1][HW] when S > 1
-    const int* counts;  // separable: Gaussians listed per tile [B][tiles]
-    const int* lists;   // separable: their indices [B][tiles][Np]
+    const int* counts;  // separable: Gaussians listed per tile [B][tiles], or per wave rectangle [B][4 tiles_y][tiles_x]
+    const int* lists;   // separable: their indices [B][lists][Np]
     const int* flag;  // AUTO grid mode: run only if *flag == want (nullptr: always run)
     int want;
 };
@@ -351,8 +351,9 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     }
     // this unit's Gaussians (those whose ellipse reaches it), split S ways by list position
     const int s = blockIdx.y;
-    const size_t li = kWave ? ((size_t)b * per_img + tl) * 4 + wave : (size_t)b * per_img + tl;
-    const int count = a.counts[li];
+    // (wave lists are numbered by rectangle, row after row; rows of rectangles below the image have none)
+    const size_t li = kWave ? ((size_t)b * 4 * a.tiles_y + (ty * 4 + wave)) * a.tiles_x + tx : (size_t)b * per_img + tl;
+    const int count = (!kWave || row0 < a.H) ? a.counts[li] : 0;
     // parts of decreasing length: part i has weight 1 + ramp - 2 ramp i / (S - 1), the sum is S
     auto cut = [&](int i) {  // first entry of part i, a multiple of 4
         const float f = a.S > 1 ? (float)i * (1.0f + kSplitRamp - kSplitRamp * (float)(i - 1) / (float)(a.S - 1)) / (float)a.S

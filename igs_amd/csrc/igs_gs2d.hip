@@ -34,6 +34,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -300,18 +301,49 @@ int make_plan(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t*
 
 // Threads of a k_bin workgroup: four candidates per lane when there are few of them (the scans load
 // and test four at a time: more threads would only be more waves to start), 1024 otherwise.
-inline int bin_threads(long candidates) {
+inline int bin_threads(long candidates, bool four_lists) {
+    const long most = four_lists ? kBinThreadsMasks : kBinThreads;
     long t = ((candidates + 3) / 4 + 63) & ~63L;
-    return (int)(t < 256 ? 256 : (t > kBinThreads ? kBinThreads : t));
+    return (int)(t < 256 ? 256 : (t > most ? most : t));
 }
+
+// Most workgroups of a forward binning with one workgroup per wave rectangle (see igs_gs2d_forward).
+#ifndef IGS_BIN_RECT_WORKGROUPS
+#define IGS_BIN_RECT_WORKGROUPS 512
+#endif
+
+// LDS for the weight classes of a tile's candidates: up to 48 KB fits, with the kernel's static LDS,
+// into the 64 KB that a launch gets by default; up to 128 KB (of a CU's 160) after raising the
+// kernel's limit on the device, which large problems only need.
+constexpr size_t kBinClassBytesDefault = 48 * 1024, kBinClassBytes = 128 * 1024;
 
 int launch_bin(const BinArgs& a, int K, int B, hipStream_t st) {
     // (at the second level of a two-level binning the candidates are the super-tile's list: unknown here)
-    const int threads = bin_threads(a.cand_lists != nullptr ? kBinThreads * 4 : (a.chunk > 0 ? a.chunk : a.N));
+    const int threads = bin_threads(a.cand_lists != nullptr ? kBinThreads * 4 : (a.chunk > 0 ? a.chunk : a.N), a.sub_nx > 0);
+    // LDS for the candidates' weight classes (a tile's candidates are at most all Gaussians); beyond
+    // kBinClassBytes the kernel evaluates them twice instead.  Not at the first level of a two-level
+    // binning, which skips by the call's skip weight alone.
+    BinArgs b = a;
+    const size_t class_bytes = (size_t)a.Np * (a.sub_nx > 0 ? 4 : 1);
+    b.store_classes = a.chunk == 0 && class_bytes <= kBinClassBytes;
+    const size_t lds = b.store_classes ? class_bytes : 0;
+    if (lds > kBinClassBytesDefault) {  // once per device and kernel (the call costs tens of microseconds)
+        static std::atomic<bool> raised[2][64];
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return (int)e;
+        const int which = a.sub_nx > 0 ? 1 : 0;
+        if (dev < 0 || dev >= 64 || !raised[which][dev].load(std::memory_order_acquire)) {
+            const void* f = which ? reinterpret_cast<const void*>(&k_bin<true>) : reinterpret_cast<const void*>(&k_bin<false>);
+            e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBinClassBytes);
+            if (e != hipSuccess) return (int)e;
+            if (dev >= 0 && dev < 64) raised[which][dev].store(true, std::memory_order_release);
+        }
+    }
     if (a.sub_nx > 0)
-        hipLaunchKernelGGL(k_bin<true>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(threads), 0, st, a);
+        hipLaunchKernelGGL(k_bin<true>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(threads), lds, st, b);
     else
-        hipLaunchKernelGGL(k_bin<false>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(threads), 0, st, a);
+        hipLaunchKernelGGL(k_bin<false>, dim3(a.tiles_x * a.tiles_y, K, B), dim3(threads), lds, st, b);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? IGS_OK : (int)e;
 }
@@ -329,7 +361,7 @@ int launch_bins(BinArgs fine, int B, bool levels2, const BinPlace& coarse, int* 
     c.tiles_x = sg.x; c.tiles_y = sg.y;
     c.counts = coarse.counts; c.lists = coarse.lists; c.slots = coarse_slots;
     c.chunk = sg.chunk;
-    c.sub_nx = 0; c.sub_h = 0;  // a super-tile has one list
+    c.sub_nx = 0; c.sub_h = 0; c.img_lists = 0;  // a super-tile has one list
     int rc = launch_bin(c, sg.K, B, st);
     if (rc) return rc;
     fine.cand_counts = coarse.counts; fine.cand_lists = coarse.lists;
@@ -612,7 +644,19 @@ int forward_impl(const float* packed, const float* x, const float* y,
             // a list per wave of the forward: four per tile of the binning
             ba.sub_nx = fwd_wave_lists(C) ? fg.wx : 0;
             ba.sub_h = fwd_sep_p(C);
+            ba.img_lists = 0;
             const bool levels2 = two_level(N, fg.tiles_x, fg.tiles_y, opts_of(grid_mode));
+            // Few tiles: a workgroup per wave rectangle instead of one per tile with four lists fills
+            // the device better (B=1 N=16384 512x512: 28 against 72 us) and bounds each rectangle's
+            // denominators by itself; with many tiles the four-list workgroups read the bin records
+            // a quarter as often (B=16 N=8192 256x256: 44 against 67 us).
+            const int rect_rows = ceil_div(H, fwd_sep_p(C));
+            if (ba.sub_nx > 0 && !levels2 && (long)B * fg.tiles_x * rect_rows <= IGS_BIN_RECT_WORKGROUPS) {
+                ba.img_lists = 4 * fg.tiles_y * fg.tiles_x;
+                ba.tile_h = fwd_sep_p(C);
+                ba.tiles_y = rect_rows;
+                ba.sub_nx = 0; ba.sub_h = 0;
+            }
             const BinPlace cp = levels2 ? super_bins_at(ws, split_bytes, B, plan.fwd_tiles, plan.n_padded,
                                                         super_tiles(fg.tiles_x, fg.tiles_y, B, N).count)
                                         : BinPlace{nullptr, nullptr};
@@ -854,7 +898,7 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
             ba.slots = slots_at(partial, B, a.T, 6 + C, N);
             ba.flag = a.flag; ba.want = a.want;
             ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
-            ba.sub_nx = 0; ba.sub_h = 0;
+            ba.sub_nx = 0; ba.sub_h = 0; ba.img_lists = 0;
             const bool levels2 = two_level(N, ba.tiles_x, ba.tiles_y, opts_of(grid_mode));
             BinPlace cp{nullptr, nullptr};
             int* cslots = nullptr;

@@ -244,49 +244,89 @@ struct BinArgs {
     // (4 / sub_nx) rectangles of 64 columns x sub_h rows (rectangle w: column block w % sub_nx, row
     // block w / sub_nx), each with a list of its own: list and count number 4 t + w of the image.
     int sub_nx, sub_h;
+    int img_lists;  // lists per image in `counts` and `lists` when that is not the launch's own number (0)
+    // The launch carries dynamic LDS for one byte (four with four lists) per candidate, in which the
+    // scan that settles what the tile skips leaves each candidate's weight class for the scan that
+    // lists; 0: that scan evaluates the rectangle test again.
+    int store_classes;
 };
 
 // Tiles per super-tile of the two-level binning (each way) and the most segments per list.
 constexpr int kSuperX = 4, kSuperY = 4, kBinMaxChunks = 64;
 
 constexpr int kBinThreads = 1024, kBinWaves = kBinThreads / 64;  // many loads in flight per tile
+// With four lists per tile a lane holds four rectangles' worth of intermediate values: at 1024 threads
+// (128 registers per lane) a third of them spilled to scratch memory.
+#ifndef IGS_BIN_THREADS_MASKS
+#define IGS_BIN_THREADS_MASKS 512
+#endif
+constexpr int kBinThreadsMasks = IGS_BIN_THREADS_MASKS;
 
 // Second test for a Gaussian whose reach box meets the tile: can its ellipse reach the tile's
-// coordinate rectangle at all (the box of a long, rotated ellipse is mostly empty)?  With
-// P = -q' = a dx^2 + b2 dx dy + d dy^2 (a, b2, d = -A', -B2', -D' of the record), the minimum of
-// P over the rectangle is 0 when it holds the centre and else lies on an edge, where P is a
-// parabola in one variable.  The kernels' weight is exactly 0 where their fp32 q' is below -150;
-// both their q' and the P evaluated here differ from the exact value by a few ulp of the largest
-// term, bounded over the rectangle by T below.  The tile is dropped only if min P - 4e-6 T > L_n, the
-// Gaussian's skip limit (see reach_box): with the exact limit 155 this is the same margin against
-// rounding as the reach box has, so dropping it changes no bit either; with a skip weight w every
-// pair of a dropped tile has e < w / max(1, |alpha|).  A non-positive-definite or NaN record fails
-// the comparison and stays listed.
-__device__ __forceinline__ bool ellipse_reaches(float4 q0, float4 q1, float txlo, float txhi,
-                                                float tylo, float tyhi, float limit) {
+// coordinate rectangle at all (the box of a long, rotated ellipse is mostly empty), and with what
+// weight at most?  With P = -q' = a dx^2 + b2 dx dy + d dy^2 (a, b2, d = -A', -B2', -D' of the
+// record), the minimum of P over the rectangle is 0 when it holds the centre and else lies on an
+// edge, where P is a parabola in one variable.  The kernels' weight is exactly 0 where their fp32 q'
+// is below -150; both their q' and the P evaluated here differ from the exact value by a few ulp of
+// the largest term, bounded over the rectangle by T below.  reach_p returns min P - 4e-6 T: every
+// weight of the Gaussian on the rectangle is at most 2^-reach_p, and exactly 0 in the kernels where
+// reach_p > kExactLimit (the same margin against rounding as the reach box has, so dropping such a
+// tile changes no bit).  -inf (never dropped) when the rectangle holds the centre or the form is
+// not safely positive definite; NaN for a NaN record, which fails every comparison and stays listed.
+// Evaluated twice per candidate (for the tile's histogram and for the verdict): without contraction
+// of multiplies and adds, so that both evaluations are the same arithmetic and agree bit for bit.
+__device__ __forceinline__ float reach_form(float a, float b2, float d, float x, float y) {
+#pragma clang fp contract(off)
+    return fmaf(fmaf(b2, x, d * y), y, (a * x) * x);
+}
+__device__ __forceinline__ float reach_p(float4 q0, float4 q1, float txlo, float txhi, float tylo, float tyhi) {
+#pragma clang fp contract(off)
     const float a = q1.x, b2 = q1.y, d = q1.z;
     const float x0 = txlo - q0.x, x1 = txhi - q0.x, y0 = tylo - q0.y, y1 = tyhi - q0.y;
     // straight-line code (every path is taken by some lane of a wave anyway)
     const bool inside = x0 <= 0.0f && x1 >= 0.0f && y0 <= 0.0f && y1 >= 0.0f;
     // the argument below needs a form that is positive definite beyond the rounding of its
     // (fp32) coefficients; ellipses thinner than about 1:600 simply stay listed
-    const bool definite = a > 0.0f && 4.0f * a * d - b2 * b2 > 4e-5f * a * d;
-    auto form = [&](float x, float y) { return fmaf(fmaf(b2, x, d * y), y, a * x * x); };
-    auto clamp = [](float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); };
+    const bool definite = a > 0.0f && (4.0f * a) * d - b2 * b2 > (4e-5f * a) * d;
     // Only the edges that face the centre can hold the minimum: P grows along every ray from the
     // centre, and the ray to a point of the rectangle enters it through such an edge.  The vertex
     // of an edge's parabola uses the hardware reciprocal (its error is of second order in P).
     const float inf = __builtin_inff();
     const bool vx = x0 > 0.0f || x1 < 0.0f, vy = y0 > 0.0f || y1 < 0.0f;
     const float xe = x0 > 0.0f ? x0 : x1, ye = y0 > 0.0f ? y0 : y1;
-    const float ky = -0.5f * b2 * __builtin_amdgcn_rcpf(d), kx = -0.5f * b2 * __builtin_amdgcn_rcpf(a);
-    const float pv = vx ? form(xe, clamp(ky * xe, y0, y1)) : inf;
-    const float ph = vy ? form(clamp(kx * ye, x0, x1), ye) : inf;
+    const float ky = (-0.5f * b2) * __builtin_amdgcn_rcpf(d), kx = (-0.5f * b2) * __builtin_amdgcn_rcpf(a);
+    const float pv = vx ? reach_form(a, b2, d, xe, fminf(fmaxf(ky * xe, y0), y1)) : inf;
+    const float ph = vy ? reach_form(a, b2, d, fminf(fmaxf(kx * ye, x0), x1), ye) : inf;
     const float pmin = fminf(pv, ph);
     const float mx = fmaxf(fabsf(x0), fabsf(x1)), my = fmaxf(fabsf(y0), fabsf(y1));
-    const float T = a * mx * mx + fabsf(b2) * mx * my + d * my * my;
-    const bool beyond = pmin - 4e-6f * T > skip_limit(limit, q1.w);
-    return inside || !definite || !beyond;
+    const float T = ((a * mx) * mx + (fabsf(b2) * mx) * my) + (d * my) * my;
+    const float p = pmin - 4e-6f * T;
+    return (inside || !definite) ? -inf : p;
+}
+
+// The weight classes of the binning: class k holds the (Gaussian, tile) pairs whose largest term of
+// a denominator, e max(1, |alpha|) <= 2^-(reach_p - log2 max(1, |alpha|)), lies in
+// (2^-((k + 1) / kBinRes), 2^-(k / kBinRes)].  -1: not classed (the bound exceeds 1, or NaN) and
+// never skipped.
+constexpr int kBinRes = 2;
+constexpr int kMaxSkipClasses = 253;  // (a class relative to the call's fits a byte)
+constexpr int kBinClasses = 320;  // >= kExactLimit kBinRes + 1, a multiple of 64
+static_assert(kBinClasses >= (int)kExactLimit * kBinRes + 1 && kBinClasses % 64 == 0, "weight classes");
+__device__ __forceinline__ int weight_class(float p, float alpha) {
+#pragma clang fp contract(off)
+    const float r = (p - __log2f(fmaxf(1.0f, fabsf(alpha)))) * (float)kBinRes;
+    return r >= 0.0f ? (int)fminf(r, (float)(kBinClasses - 1)) : -1;
+}
+// first class that the call's skip limit L (weights below 2^-L are skipped) lets skip entirely
+__device__ __forceinline__ int base_class(float limit) {
+    return limit < kExactLimit ? (int)ceilf(limit * (float)kBinRes) : 0x7fffffff;
+}
+// verdict for one rectangle: skipped when the weight is exactly zero there, or its class is one of
+// those the tile skips
+__device__ __forceinline__ bool ellipse_reaches(float4 q0, float4 q1, float txlo, float txhi, float tylo,
+                                                float tyhi, int first_skipped) {
+    const float p = reach_p(q0, q1, txlo, txhi, tylo, tyhi);
+    return !(p > kExactLimit || weight_class(p, q1.w) >= first_skipped);
 }
 
 // A Gaussian's smallest weight over the tile's coordinate rectangle: alpha 2^(-max P), P = -q' being
@@ -304,12 +344,16 @@ __device__ __forceinline__ float least_weight(float4 q0, float4 q1, float txlo, 
 }
 
 template <bool kMasks>
-__global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
+__global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin(const BinArgs a) {
     if (a.flag != nullptr && *a.flag != a.want) return;
     __shared__ float red[4][kBinWaves];
     __shared__ int wsum[kMasks ? 4 : 1][kBinWaves];
     __shared__ int seg_first[kBinMaxChunks + 1];  // second level: first candidate index of each segment
+    __shared__ int hist[kMasks ? 4 : 1][kBinClasses];  // candidates per weight class and list
+    __shared__ int first_skipped_s[kMasks ? 4 : 1];
+    extern __shared__ unsigned int class_store[];  // per candidate: kbase - class per list, 0 = skipped, 255 = listed
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < (kMasks ? 4 : 1) * kBinClasses; i += blockDim.x) (&hist[0][0])[i] = 0;
     // launched with 256 to kBinThreads threads (bin_threads): the reductions below run over kBinWaves
     // slots, those of waves that do not exist hold the neutral element
     const int nthreads = blockDim.x, nwaves = nthreads >> 6;
@@ -449,21 +493,39 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
         sub[w][3] = masks ? -red[3][w] : 0.0f;
         sub_any[w] = sub[w][0] <= sub[w][1] && sub[w][2] <= sub[w][3];
     }
-    float limit = a.limit[0];
+    const float limit = a.limit[0];
     const float fraction = a.limit[1];
-    int* list = a.lists + ((size_t)b * tiles + t) * (masks ? 4 : 1) * a.Np + (size_t)kc * a.chunk;
+    // The image's lists are numbered by tile; with four lists per tile by rectangle, row after row of
+    // rectangles (rectangle l of the tile lies in row 4 ty + l): the numbering that a binning with one
+    // workgroup per rectangle gives (which then sets img_lists, rows of rectangles past the image's
+    // last having no workgroup).
+    const size_t img_first = (size_t)b * (a.img_lists > 0 ? a.img_lists : tiles * (masks ? 4 : 1));
+    auto list_no = [&](int l) { return img_first + (masks ? (size_t)(ty * 4 + l) * a.tiles_x + tx : (size_t)t); };
+    int* list = a.lists + list_no(0) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     // "definitely outside" negated, so that NaN bounds count as inside
     auto meets_tile = [&](const Batch& bt, int u) {
         return !(bt.q0[u].x + bt.q0[u].z < txlo || bt.q0[u].x - bt.q0[u].z > txhi ||
                  bt.q0[u].y + bt.q0[u].w < tylo || bt.q0[u].y - bt.q0[u].w > tyhi);
     };
-    // Skip fraction f > 0: a tile whose denominators are all at least S (the sum of the least
-    // weights of the candidates whose box meets it; only if none of them has a negative or
-    // non-finite alpha) may skip pairs up to the weight w + f S instead of the call's w.  Not at the
-    // first level of a two-level binning (its lists must hold what any of its tiles may list), nor
-    // where nothing is culled.
-    if (fraction > 0.0f && a.chunk == 0 && txlo > -inf && !a.no_cull) {  // workgroup-uniform
+    // What a tile may skip.  Every Gaussian that is not listed for a tile changes the tile's
+    // denominators by at most its largest weight there, and the call allows N (w + f S) in total,
+    // w = 2^-limit the skip weight, f the skip fraction and S a lower bound of the tile's
+    // denominators (the sum of the least weights of the candidates whose box meets it; 0 if one of
+    // them has a negative or non-finite alpha).  Classes from kbase on hold weights of at most w: they
+    // are skipped, and so are the Gaussians that are no candidates here (their boxes miss the tile, or
+    // the first level of a two-level binning dropped them: below w as well); with n the number of
+    // classed candidates above w that leaves n w + N f S for them, which the lightest classes take up
+    // as far as it goes, each candidate counted with the upper end of its class.
+    // Not at the first level of a two-level binning (its lists must hold what any of its tiles may
+    // list), nor where nothing is culled.
+    const int kbase = base_class(limit);
+    constexpr int kL = kMasks ? 4 : 1;  // lists per tile
+    int first_skipped[kL];
+#pragma unroll
+    for (int l = 0; l < kL; ++l) first_skipped[l] = kbase;
+    const bool settle = fraction > 0.0f && a.chunk == 0 && txlo > -inf && !a.no_cull;  // workgroup-uniform
+    if (settle) {
         float sum = 0.0f;
         bool negative = false;
         int it = 0;
@@ -477,7 +539,26 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
                 // (records that are never skipped have unbounded boxes: NaN fields or a form that is
                 // not positive definite; with alpha >= 0 they can only raise a denominator)
                 const float w = least_weight(bt.q0[u], bt.q1[u], txlo, txhi, tylo, tyhi);
-                sum += (meets && bt.q0[u].z < inf) ? w : 0.0f;
+                const bool bounded = meets && bt.q0[u].z < inf;
+                sum += bounded ? w : 0.0f;
+                unsigned int stored = 0u;
+#pragma unroll
+                for (int l = 0; l < kL; ++l) {
+                    const float p = masks ? reach_p(bt.q0[u], bt.q1[u], sub[l][0], sub[l][1], sub[l][2], sub[l][3])
+                                          : reach_p(bt.q0[u], bt.q1[u], txlo, txhi, tylo, tyhi);
+                    const int k = weight_class(p, bt.q1[u].w);
+                    // classes further than kMaxSkipClasses above the call's are never skipped (nor counted)
+                    const bool classed = bounded && k >= 0 && k < kbase && kbase - k <= kMaxSkipClasses;
+                    const bool live = meets && (!masks || sub_any[l]);
+                    if (live && classed) atomicAdd(&hist[l][k], 1);
+                    const bool gone = !live || (bounded && (p > kExactLimit || k >= kbase));
+                    stored |= (gone ? 0u : (classed ? (unsigned int)(kbase - k) : 255u)) << (8 * l);
+                }
+                const int i = n0 + u * 64 + lane;
+                if (a.store_classes && i < ne) {
+                    if (masks) class_store[i] = stored;
+                    else reinterpret_cast<unsigned char*>(class_store)[i] = (unsigned char)stored;
+                }
             }
         }
 #pragma unroll
@@ -488,17 +569,52 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
             red[0][wave] = sum;
             red[1][wave] = wneg ? 1.0f : 0.0f;
         }
-        __syncthreads();
+        __syncthreads();  // (also: the histograms are complete)
         float total = 0.0f, anyneg = 0.0f;
 #pragma unroll
         for (int w = 0; w < kBinWaves; ++w) {
             total += w < nwaves ? red[0][w] : 0.0f;
             anyneg += w < nwaves ? red[1][w] : 0.0f;
         }
-        if (anyneg == 0.0f && total > 0.0f && total < inf) {  // (an overflowed sum bounds nothing)
-            const float w0 = limit < kExactLimit ? hw_exp2(-limit) : 0.0f;
-            limit = fminf(limit, -__log2f(w0 + fraction * total));
+        const float floor_sum = (anyneg == 0.0f && total > 0.0f && total < inf) ? total : 0.0f;  // (an overflowed sum bounds nothing)
+        if (wave < kL) {  // wave l settles list l: the first class k with (sum over classes >= k) <= budget
+            constexpr int per = kBinClasses / 64;
+            const float w0 = hw_exp2(-limit);
+            float v[per], s = 0.0f;
+            int n = 0;
+#pragma unroll
+            for (int j = 0; j < per; ++j) {
+                const int k = lane * per + j;
+                const int h = k < kbase ? hist[wave][k] : 0;
+                v[j] = (float)h * hw_exp2(-(float)k * (1.0f / (float)kBinRes));
+                s += v[j];
+                n += h;
+            }
+#pragma unroll
+            for (int k = 32; k > 0; k >>= 1) n += __shfl_xor(n, k);
+            float after = s;  // sum over this lane's classes and those of the lanes above
+#pragma unroll
+            for (int dlt = 1; dlt < 64; dlt <<= 1) {
+                const float o = __shfl_down(after, dlt);
+                after += lane + dlt < 64 ? o : 0.0f;
+            }
+            float run = __shfl_down(after, 1);
+            run = lane < 63 ? run : 0.0f;
+            // (one percent held back for the rounding of these sums)
+            const float budget = 0.99f * ((float)n * w0 + (float)a.N * fraction * floor_sum);
+            int best = 0x7fffffff;
+#pragma unroll
+            for (int j = per - 1; j >= 0; --j) {
+                run += v[j];
+                best = run <= budget ? lane * per + j : best;
+            }
+#pragma unroll
+            for (int k = 32; k > 0; k >>= 1) best = min(best, __shfl_xor(best, k));
+            if (lane == 0) first_skipped_s[wave] = max(min(best, kbase), kbase - kMaxSkipClasses);
         }
+        __syncthreads();
+#pragma unroll
+        for (int l = 0; l < kL; ++l) first_skipped[l] = first_skipped_s[l];
     }
     // code: which of the tile's four rectangles the Gaussian reaches (four lists), or 1; 0 = not listed
     auto classify = [&](int n0, const Batch& bt, int (&code)[kU], bool (&in)[kU]) {
@@ -513,27 +629,40 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
 #pragma unroll
                 for (int w = 0; w < 4; ++w)
                     reached |= (sub_any[w] && ellipse_reaches(bt.q0[u], bt.q1[u], sub[w][0], sub[w][1], sub[w][2],
-                                                              sub[w][3], limit)) ? 1 << w : 0;
+                                                              sub[w][3], first_skipped[masks ? w : 0])) ? 1 << w : 0;
             } else {
-                reached = ellipse_reaches(bt.q0[u], bt.q1[u], txlo, txhi, tylo, tyhi, limit) ? 1 : 0;
+                reached = ellipse_reaches(bt.q0[u], bt.q1[u], txlo, txhi, tylo, tyhi, first_skipped[0]) ? 1 : 0;
             }
             code[u] = !meets ? 0 : (refine ? reached : (masks ? 15 : 1));
         }
     };
     // the classifying scan keeps its verdicts (one bit, or four with four lists, per candidate of this
     // lane) for the writing one when they fit in a register pair, i.e. up to 64 (16) candidates per lane
-    constexpr int vbits = masks ? 4 : 1, kL = masks ? 4 : 1;  // kL lists per tile
+    constexpr int vbits = masks ? 4 : 1;
     const bool keep = per_wave * vbits <= 64 * 64;
     unsigned long long verdicts = 0ull;
     int cnt[kL], it = 0;
 #pragma unroll
     for (int l = 0; l < kL; ++l) cnt[l] = 0;
     for (int n0 = nb; n0 < ne; n0 += 64 * kU, ++it) {
-        Batch bt = head;
-        if (it > 0) load_batch(n0, bt);
         bool in[kU];
         int code[kU];
-        classify(n0, bt, code, in);
+        if (settle && a.store_classes) {  // the classes are known: a candidate is listed where its class is below the first skipped one
+#pragma unroll
+            for (int u = 0; u < kU; ++u) {
+                const int i = n0 + u * 64 + lane;
+                in[u] = i < ne;
+                const unsigned int stored = !in[u] ? 0u : (masks ? class_store[i] : (unsigned int)reinterpret_cast<unsigned char*>(class_store)[i]);
+                code[u] = 0;
+#pragma unroll
+                for (int l = 0; l < kL; ++l)
+                    code[u] |= (int)((stored >> (8 * l)) & 255u) > kbase - first_skipped[l] ? 1 << l : 0;
+            }
+        } else {
+            Batch bt = head;
+            if (it > 0) load_batch(n0, bt);
+            classify(n0, bt, code, in);
+        }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
 #pragma unroll
@@ -580,7 +709,7 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
                 const bool listed = (code[u] >> l) & 1;
                 const unsigned long long m = __ballot(listed);
                 const int pos = base[l] + __popcll(m & below);
-                if (listed) list[(size_t)l * a.Np + pos] = n[u];
+                if (listed) list[(size_t)l * a.tiles_x * a.Np + pos] = n[u];  // (l > 0 with four lists only: next row of rectangles)
                 // the slot of every candidate: its position (within the segment, at the first level,
                 // where only the sign is used) or -1
                 if (!masks && slot != nullptr && in[u]) slot[n[u]] = listed ? pos : -1;
@@ -589,5 +718,5 @@ __global__ __launch_bounds__(kBinThreads) void k_bin(const BinArgs a) {
     }
     if (tid == 0)
 #pragma unroll
-        for (int l = 0; l < kL; ++l) a.counts[(((size_t)b * tiles + t) * K + kc) * kL + l] = total[l];
+        for (int l = 0; l < kL; ++l) a.counts[masks ? list_no(l) : list_no(0) * K + kc] = total[l];
 }

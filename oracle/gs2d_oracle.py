@@ -290,6 +290,50 @@ def tile_skip_weight(w: float, f: float, floor):
     return w + f * floor
 
 
+WEIGHT_CLASSES_PER_BINADE = 2
+
+
+def weight_class(min_q, alphas):
+    """Weight class of each (Gaussian, tile) pair from the minimum of q over the tile's rectangle
+    (`min_q_over_rect`): the Gaussian's largest term of a denominator there is
+    max(1, |alpha|) exp(-min_q / 2) = 2^-p, p = 0.5 log2(e) min_q - log2 max(1, |alpha|), and the
+    class is floor(p R) with R classes per binade, i.e. the term lies in (2^-((k+1)/R), 2^-(k/R)].
+    -1 (never skipped) where the rectangle holds the centre (min_q = 0) or the bound exceeds 1."""
+    p = 0.5 * math.log2(math.e) * min_q - torch.log2(torch.clamp(alphas.abs(), min=1.0))
+    k = torch.floor(p * WEIGHT_CLASSES_PER_BINADE)
+    return torch.where((min_q > 0) & (p >= 0), k, torch.full_like(k, -1.0)).long()
+
+
+def tile_first_skipped_class(classes, N: int, w: float, f: float, floor: float):
+    """The per-tile rule of the HIP binning kernel, restated: which weight classes a tile leaves out
+    of its list.  Leaving out a set of Gaussians changes a denominator of the tile by at most the sum
+    of their largest terms there, and that sum may reach N (w + f S) (`tile_skip_weight` times N; S =
+    `floor` bounds the tile's denominators from below): then
+    |d out| <= N (w + f S) (max|c| + |out|) / (den + eps) <= tolerance max|c|.
+    Classes from kbase = ceil(-log2(w) R) on hold terms of at most w and are always left out; so are
+    the Gaussians that the kernel never examines for the tile (terms below w as well).  With n the
+    number of classed pairs below kbase these take at most (N - n) w of the allowance, which leaves
+    n w + N f S: the lightest classes below kbase are left out as long as the sum of (members x upper
+    end of the class) stays within that.  Returns the first class left out (kbase if none is);
+    `classes` is a 1-D integer tensor (-1 = never skipped).  w = 0: nothing but exact zeros is
+    skipped, returns None.  No counterpart in the reference, which evaluates every pair
+    (src/igs/gs_triton_chunked.py:100-200)."""
+    R = WEIGHT_CLASSES_PER_BINADE
+    if not w > 0 or -math.log2(w) >= EXACT_LIMIT:
+        return None
+    kbase = math.ceil(-math.log2(w) * R)
+    hi = classes[(classes >= 0) & (classes < kbase)]
+    budget = hi.numel() * w + N * f * floor
+    hist = torch.bincount(hi, minlength=kbase).tolist()
+    first, run = kbase, 0.0
+    for k in range(kbase - 1, -1, -1):
+        run += hist[k] * 2.0 ** (-k / R)
+        if run > budget:
+            break
+        first = k
+    return first
+
+
 def reach_q(alphas, w: float):
     """q_max of each Gaussian's reach box under skip weight w: five binades beyond its skip limit
     (the exact-zero case gives REACH_Q)."""

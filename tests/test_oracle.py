@@ -428,6 +428,54 @@ def test_skip_weight_bound_by_brute_force():
     kept = torch.einsum("bnhw,bnc->bchw", ek, col) / (ek.sum(1)[:, None] + eps)
     assert float((full - kept).abs().max()) <= tol * float(col.abs().max())
     assert float(O.tile_weight_floor(pos[..., 0], pos[..., 1], a, b, d, -al, xs[0], xs[5], ys[0], ys[5])) == 0.0
+    # The rule the binning kernel applies per tile (`tile_first_skipped_class`): whole weight classes
+    # are left out of a tile's list while the sum of their members' largest terms stays within
+    # N (w + f S).  Checked by brute force: the sum of the true maxima of the left-out Gaussians over
+    # the tile's pixels is within the allowance (and uses a good part of it), more is left out than
+    # by the per-pair weight w + f S, and the image stays within the tolerance.
+    drop2 = torch.zeros_like(e, dtype=torch.bool)
+    used, by_weight = [], 0
+    amax1 = torch.clamp(al.abs(), min=1.0)
+    for r0 in range(0, H, 16):
+        for c0 in range(0, W, 16):
+            S = float(O.tile_weight_floor(pos[..., 0], pos[..., 1], a, b, d, al, xs[c0], xs[c0 + 15], ys[r0], ys[r0 + 15]))
+            mq = O.min_q_over_rect(pos[..., 0], pos[..., 1], a, b, d, xs[c0], xs[c0 + 15], ys[r0], ys[r0 + 15])
+            cls = O.weight_class(mq, al)[0]
+            first = O.tile_first_skipped_class(cls, N, w, f, S)
+            out_n = cls >= first
+            et = e[0, :, r0:r0 + 16, c0:c0 + 16] * amax1[0, :, None, None]
+            true_max = et.amax((1, 2))
+            # the class bounds the Gaussian's terms on the tile from above
+            assert bool((true_max[cls >= 0] <= 2.0 ** (-cls[cls >= 0].double() / O.WEIGHT_CLASSES_PER_BINADE) * (1 + 1e-12)).all())
+            allowance = N * O.tile_skip_weight(w, f, S)
+            assert float(true_max[out_n].sum()) <= allowance
+            used.append(float(true_max[out_n].sum()) / allowance)
+            by_weight += 256 * int((amax1[0] * torch.exp(-0.5 * mq[0]) < O.tile_skip_weight(w, f, S)).sum())
+            drop2[0, :, r0:r0 + 16, c0:c0 + 16] = out_n[:, None, None]
+    assert int(drop2.sum()) > 1.05 * by_weight and sorted(used)[len(used) // 2] > 0.1, (int(drop2.sum()), by_weight, used)
+    ek = torch.where(drop2, torch.zeros_like(e), e) * al[..., None, None]
+    kept = torch.einsum("bnhw,bnc->bchw", ek, col) / (ek.sum(1)[:, None] + eps)
+    assert float((full - kept).abs().max()) <= tol * float(col.abs().max())
+    # N coincident Gaussians seen just beyond the class edge at w from the nearest pixel of a tile
+    # whose floor is ~0: all are left out and the pixel, out = N e / (N e + eps) ~ tolerance / 2,
+    # comes within a factor 2.1 sqrt(2) of the bound; one class nearer, none is left out.
+    kb = math.ceil(-math.log2(w) * O.WEIGHT_CLASSES_PER_BINADE)
+
+    def left_out(classes, floor):
+        first = O.tile_first_skipped_class(classes, N, w, f, floor)
+        return sorted(classes[(classes >= 0) & (classes >= first)].tolist())
+
+    assert left_out(torch.full((N,), kb), 0.0) == [kb] * N and left_out(torch.full((N,), kb - 1), 0.0) == []
+    e_edge = 2.0 ** (-kb / O.WEIGHT_CLASSES_PER_BINADE)
+    assert tol / (2.1 * math.sqrt(2)) <= N * e_edge / (N * e_edge + eps) <= tol
+    # with a floor, N (w + f S) is spent on the lightest classes first: ten classed members allow
+    # 10 w, which the three of class kb - 1 (at most sqrt(2) w each) fit into and the five of class
+    # kb - 9 (16 w each) do not; a floor of 1000 eps adds N f S = 1000 N w
+    few = torch.tensor([kb - 1] * 3 + [kb - 9] * 5 + [-1, 0, 1])
+    assert left_out(few, 0.0) == [kb - 1] * 3
+    assert left_out(few, 1e3 * eps) == [kb - 9] * 5 + [kb - 1] * 3
+    assert O.tile_first_skipped_class(few, N, 0.0, f, 1.0) is None
+    assert O.weight_class(torch.tensor([0.0, 4.0, 4.0]), torch.tensor([1.0, 1.0, 1e3])).tolist()[::2] == [-1, -1]
     assert O.skip_weight(100, 0.0, 1e-7) == 0.0 and O.skip_weight(100, 1e-6, 0.0) == 0.0
     assert bool((O.skip_limit(torch.tensor([0.5, 4.0]), 0.0) == O.EXACT_LIMIT).all())
     assert math.isclose(float(O.reach_q(torch.tensor([1.0], dtype=F64), 0.0)[0]), O.REACH_Q, rel_tol=1e-12)
