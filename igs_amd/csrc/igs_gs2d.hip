@@ -140,12 +140,17 @@ inline SuperGeometry super_tiles(int tiles_x, int tiles_y, int B, int N) {
     g.K = ceil_div(N, g.chunk);
     return g;
 }
+// Two binning levels from this many (Gaussian, tile) candidates per image on (measured: B=4 N=32768 on
+// 240 tiles gains 4 %, B=1 N=16384 on 256 tiles nothing).
+#ifndef IGS_BIN_TWO_LEVEL_FROM
+#define IGS_BIN_TWO_LEVEL_FROM 6000000L
+#endif
 inline bool super_reserved(int tiles_x, int tiles_y) { return tiles_x * tiles_y >= 32; }
 inline bool two_level(int N, int tiles_x, int tiles_y, int opts) {
     if (!super_reserved(tiles_x, tiles_y)) return false;
     if (opts & IGS_OPT_BIN_LEVELS_1) return false;
     if (opts & IGS_OPT_BIN_LEVELS_2) return true;
-    return (long)N * tiles_x * tiles_y >= (1L << 25);  // measured break-even: N = 65536 on 256-512 tiles
+    return (long)N * tiles_x * tiles_y >= IGS_BIN_TWO_LEVEL_FROM;
 }
 // Super-tile lists of one launch: counts [B][stiles][kBinMaxChunks] then lists [B][stiles][Np].
 inline size_t super_bins_bytes(int B, int stiles, int Np) {
