@@ -33,8 +33,8 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 # (factors from the plain-copy calibration of the same profile run).
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
-    "bwd": {"fma": 8.637e8, "mul": 1.655e8, "add": 9.489e7, "trans": 7.792e7, "fetch_kib": 50120, "write_kib": 191800},
-    "fwd": {"fma": 4.720e8, "mul": 1.477e7, "add": 8.358e7, "trans": 7.869e7, "fetch_kib": 13020, "write_kib": 131100},
+    "bwd": {"fma": 7.927e8, "mul": 1.519e8, "add": 8.709e7, "trans": 7.152e7, "fetch_kib": 48990, "write_kib": 173500},
+    "fwd": {"fma": 4.363e8, "mul": 1.372e7, "add": 7.724e7, "trans": 7.273e7, "fetch_kib": 12270, "write_kib": 131100},
 }
 
 
@@ -307,9 +307,9 @@ def run(args) -> int:
                                if prof else None,
                                "traffic": hbm_bytes(prof["fwd"]) if prof else None},
             "counter_source": prof["source"] if prof else None,
-            "note": "achieved / frac: the 30+4C FLOP model of one backward pair x the pairs the kernel evaluated (the tile "
-                    "lists skip pairs whose weight is below the skip weight, which bounds the change of every output "
-                    "element by 1e-7 max|colour|; frac_counting_all_pairs uses all B N H W as the metric does and can "
+            "note": "achieved / frac: the 30+4C FLOP model of one backward pair x the pairs the kernel evaluated (a tile's "
+                    "list leaves out the Gaussians with the smallest weights there as long as their sum stays within the "
+                    "call's allowance, which bounds the change of every output element by 1e-7 max|colour|; frac_counting_all_pairs uses all B N H W as the metric does and can "
                     "exceed 1) / launch_ms, measured live with HIP events around igs_gs2d_backward_reduce = k_bin "
                     "(~65 us) + k_bwd_sep.  executed_frac: the arithmetic the hardware ran, (2 FMA + MUL + ADD + TRANS) x 64 per "
                     "launch from the rocprofv3 counters of counter_source (separable grids hoist the row/column part of "

@@ -36,9 +36,10 @@ KIND_FEATURE = 2
 _option_bits = 0
 
 # Bound on what skipping far-away (Gaussian, pixel) pairs may change in an output element, as a
-# fraction of the largest colour magnitude: the pack calls get the skip weight
+# fraction of the largest colour magnitude: the pack calls get the skip weight w =
 # igs_gs2d_skip_weight(N, eps, SKIP_TOLERANCE) = SKIP_TOLERANCE * eps / (2 N) and the skip fraction
-# SKIP_TOLERANCE / (2 N) of a pixel tile's smallest denominator.  The forward is held to
+# f = SKIP_TOLERANCE / (2 N), and a pixel tile leaves out Gaussians whose largest weights on it add
+# up to at most N (w + f S), S bounding its denominators from below.  The forward is held to
 # 1e-6 + 1e-5 |ref| against the plain expression; 1e-7 leaves that budget to the fp32 rounding.
 # 0 skips exact zeros only (bit-identical to evaluating every pair).
 SKIP_TOLERANCE = 1e-7

@@ -14,8 +14,8 @@
 //     e < w / max(1, |alpha|), i.e. where both the weight alpha e and the bare exponential (which is
 //     what the gradient of alpha sums) are below w.  The limit of Gaussian n is
 //     L_n = min(kExactLimit, L + log2 max(1, |alpha_n|)).
-//   The boxes are made for the call's skip weight; k_bin may use a larger weight for a tile whose
-//   denominators it can bound from below (least_weight), which only removes more of what the box
+//   The boxes are made for the call's skip weight; k_bin may leave out heavier Gaussians for a
+//   tile (as far as the tile's allowance goes, see k_bin), which only removes more of what the box
 //   lets through.
 // The box is five binades wider than the tile test of k_bin (ellipse_reaches), as in the exact case.
 // Half extents: sqrt(Q Sigma_xx), sqrt(Q Sigma_yy) with Sigma the covariance that (A, B, D) invert.
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin
         return cand[(size_t)seg * a.cand_chunk + (i - seg_first[seg])];
     };
     // Each wave scans one contiguous share of the candidates, without barriers inside a scan: once
-    // for the tile's denominator floor (skip fraction only), once to classify and count, and once
+    // for what the tile may skip (skip fraction only), once to classify and count, and once
     // (from the kept verdicts, with the shares' counts prefixed in wave order) to write.
     const int per_wave = ((M + nwaves - 1) / nwaves + 63) & ~63;
     const int nb = wave * per_wave, ne = min(M, nb + per_wave);

@@ -148,22 +148,27 @@ float igs_gs2d_skip_weight(int N, float eps, float tolerance);
  *     is kept, so results equal those of not skipping bit for bit while the forward runs one
  *     Gaussian split (plan.fwd_split == 1), and to fp32 rounding otherwise, where a tile's list
  *     rather than the index range is cut into the splits.
- *   otherwise: only pairs with exp(-q/2) max(1, |alpha|) < w + f S, so that both the weight
- *     alpha e and the bare exponential (which the gradient of alpha sums) are below that.  S is
- *     a lower bound of the denominators of the pixel tile the pair is skipped for: the sum, over
- *     the Gaussians whose box meets the tile, of the least weight each has on it (0 if one of
- *     them has a negative or non-finite alpha).  Per pixel the skipped weights then add up to at
- *     most N (w + f S): den changes by at most that and an output element by at most
+ *   otherwise: per pixel tile (per wave rectangle in the forward), a set of Gaussians is left out
+ *     whose largest terms on the tile add up to at most N (w + f S).  A Gaussian's largest term
+ *     is exp(-q/2) max(1, |alpha|) at the point of the tile's coordinate rectangle where q is
+ *     smallest, so it bounds both its weight alpha e and the bare exponential (which the gradient
+ *     of alpha sums) on every pixel of the tile.  S is a lower bound of the tile's denominators:
+ *     the sum, over the Gaussians whose box meets the tile, of the least weight each has on it (0
+ *     if one of them has a negative or non-finite alpha).  Gaussians whose largest term is below w
+ *     are always left out; of the others the lightest are, by whole classes of half a binade of
+ *     weight, as far as what remains of the allowance goes.  Per pixel the skipped weights then add
+ *     up to at most N (w + f S): den changes by at most that and an output element by at most
  *     N (w + f S) (max|colors| + |out|) / (den + eps) <= 2 N max|colors| max(w / eps, f) for
- *     den >= S; every per-Gaussian gradient sum misses terms of at most (w + f S) |G| |moment|
- *     per pixel, |G| <= 2 max|colors| |grad_out| / (den + eps).  igs_gs2d_skip_weight gives w
- *     and f for a wanted bound.
+ *     den >= S; a per-Gaussian gradient sum misses, for a pixel of a tile the Gaussian is not
+ *     listed for, a term of at most N (w + f S) |G| |moment|, |G| <= 2 max|colors| |grad_out| /
+ *     (den + eps).  igs_gs2d_skip_weight gives w and f for a wanted bound.
  * Records with a non-finite field or a cov_inv that is not positive definite are never skipped;
  * with IGS_OPT_NO_CULL in a forward / backward call's grid_mode nothing is.
- * Large problems (tiles x N >= 2^25) build the per-tile lists in two levels (super-tiles of
- * 4 x 4 tiles first); IGS_OPT_BIN_LEVELS_1|2 forces one or two.  The lists and the forward do
- * not depend on it; the finalize kernels add the tiles in another order under two levels, so
- * gradients agree to fp32 rounding. */
+ * Large problems (tiles x N >= 6e6) build the per-tile lists in two levels (super-tiles of
+ * 4 x 4 tiles first); IGS_OPT_BIN_LEVELS_1|2 forces one or two.  With w = f = 0 the lists and
+ * the forward do not depend on it; otherwise a tile settles what it leaves out from the
+ * candidates it sees, so the lists may differ within the same bound.  The finalize kernels add
+ * the tiles in another order under two levels, so gradients agree to fp32 rounding. */
 int igs_gs2d_pack_covinv(const float *position, const float *cov_inv_00, const float *cov_inv_01,
                          const float *cov_inv_11, const float *alphas, const float *colors,
                          int B, int N, int C, float skip_weight, float skip_fraction,
