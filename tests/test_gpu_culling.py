@@ -583,6 +583,35 @@ def test_default_skip_tolerance_stays_within_its_bound(igs, dev, alpha_scale):
         assert float(d.norm()) <= 1e-5 * float(grads0[k].double().norm()), k
 
 
+@pytest.mark.parametrize("shape", [(1, 140000, 48, 48, 1), (33, 33000, 64, 256, 3)], ids=lambda v: "x".join(map(str, v)))
+def test_more_candidates_than_the_class_store_holds(igs, dev, no_cull, shape):
+    """The binning keeps each candidate's weight class in LDS between the scan that settles what a
+    tile skips and the scan that lists (one byte per candidate, four with the forward's four lists
+    per tile; 128 KB at most).  Beyond that -- N > 131072, or N > 32768 where the forward bins per
+    tile, i.e. with more than 512 wave rectangles in the batch -- the second scan evaluates the
+    rectangle test again, with the same arithmetic.  Both shapes: the default tolerance against the
+    run that lists everything (within its bound), and the exact mode against it (to rounding: the
+    forward cuts lists, not index ranges, into its splits)."""
+    from igs_amd._splat import SKIP_TOLERANCE
+
+    B, N, H, W, C = shape
+    _, g = sparse_case(dev, B, N, H, W, C, seed=sum(shape), smin=0.02, smax=0.3)
+    out, grads = run(igs, g)
+    with exact():
+        oute, gradse = run(igs, g)
+    with no_cull:
+        out0, grads0 = run(igs, g)
+    cmax = float(g["colors"].abs().max())
+    err = (out - out0).abs()
+    assert bool((err <= SKIP_TOLERANCE * cmax + 1e-6 * out0.abs().clamp(min=1.0)).all()), float(err.max())
+    torch.testing.assert_close(oute, out0, rtol=0, atol=2e-6)
+    assert not torch.equal(out, oute)          # the default did leave something out
+    for k in NAMES:
+        n0 = float(grads0[k].double().norm())
+        assert float((grads[k] - grads0[k]).double().norm()) <= 1e-5 * n0, k
+        assert float((gradse[k] - grads0[k]).double().norm()) <= 1e-5 * n0, k
+
+
 def no_cull_ctx():
     from igs_amd._splat import library_options
 
