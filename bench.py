@@ -250,17 +250,19 @@ def run(args) -> int:
     evaluated = int((counts.long() * (rows[:, None] * cols[None, :])[None]).sum())
     achieved = evaluated * f_bwd / t_bwd_kernel / 1e12
     prof = C1_PROFILE if (args.config == "c1" and C == 3) else None
-    # The same for the forward (C <= 8: one list per wave rectangle of 64 columns x P rows, P = 16 for
-    # C <= 3 and 8 above, numbered row after row of rectangles with 4 ceil(H / 4P) rows reserved per
-    # image; behind the split partials in the forward's workspace).
+    # The same for the forward (C <= 8: one list per wave rectangle of 32 columns x 2P rows, P = 16 for
+    # C <= 3 and 8 above, numbered row after row of rectangles over the 64 x 4P tiles' extent; behind the
+    # split partials in the forward's workspace).
     fwd_evaluated = None
     if C <= 8:
         P = 16 if C <= 3 else 8
         split = plan.fwd_split * B * (C + 1) * H * W * 4 if plan.fwd_split > 1 else 0
-        tx_n, rows_n = -(-W // 64), -(-H // P)
-        fc = fwd_ws.view(torch.int32)[(split + 15) // 16 * 4:][: B * plan.fwd_tiles].view(B, -1, tx_n)[:, :rows_n].cpu()
-        frows = torch.tensor([min(H, (i + 1) * P) - i * P for i in range(rows_n)])
-        fcols = torch.tensor([min(W, (i + 1) * 64) - i * 64 for i in range(tx_n)])
+        tx_n, ty_n = -(-W // 64), -(-H // (4 * P))
+        cols_n, rows_n = -(-W // 32), -(-H // (2 * P))
+        fc = fwd_ws.view(torch.int32)[(split + 15) // 16 * 4:][: B * plan.fwd_tiles].view(B, 2 * ty_n, 2 * tx_n)
+        fc = fc[:, :rows_n, :cols_n].cpu()
+        frows = torch.tensor([min(H, (i + 1) * 2 * P) - i * 2 * P for i in range(rows_n)])
+        fcols = torch.tensor([min(W, (i + 1) * 32) - i * 32 for i in range(cols_n)])
         fwd_evaluated = int((fc.long() * (frows[None, :, None] * fcols[None, None, :])).sum())
 
     result = {

@@ -16,7 +16,7 @@ struct FwdArgs {
     float* out;
     float* den;
     float* part;  // [S][B][C+1][HW] when S > 1
-    const int* counts;  // separable: Gaussians listed per tile [B][tiles], or per wave rectangle [B][4 tiles_y][tiles_x]
+    const int* counts;  // separable: Gaussians listed per tile [B][tiles], or per wave rectangle, row after row over the tiles' extent [B][4 tiles]
     const int* lists;   // separable: their indices [B][lists][Np]
     const int* flag;  // AUTO grid mode: run only if *flag == want (nullptr: always run)
     int want;
@@ -43,12 +43,20 @@ struct GRec {
 
 // whether a record of C channels has room for the y range of the reach box
 __host__ __device__ constexpr bool rec_has_yrange(int C) { return rec_stride_of(C) >= 8 + C; }
-// The separable forward variants whose waves hold 16 or 8 rows (C <= 8) give every wave a Gaussian list
-// of its own (64 columns x P rows); the four waves of a workgroup stream theirs independently: no
-// wave waits for another at a chunk boundary, and none reads records it then skips.  With 4 rows per
+// The separable forward variants whose lanes hold 16 or 8 rows (C <= 8) give every wave a Gaussian list
+// of its own (kWaveCols columns x 64 P / kWaveCols rows); the four waves of a workgroup stream theirs
+// independently: no wave waits for another at a chunk boundary, and none reads records it then skips.  With 4 rows per
 // wave (C = 16) the tile of four waves is small already and the lists of single waves cost the
 // binning more than the forward gains (B=4, N=32768, 384x640: 3.25 -> 3.73 ms): that variant streams
 // one list to four waves, and a wave tests the reach box's y range against its own rows.
+// Columns of a wave's rectangle where every wave has a list of its own: 32 columns x 2 P rows (32 x 32
+// pixels for C <= 3) are reached by fewer Gaussians than 64 x P (B=16 N=8192 256x256: forward 1.16 ->
+// 1.10 ms; B=1 N=16384 512x512: 0.209 -> 0.193 ms).
+#ifndef IGS_FWD_WAVE_COLS
+#define IGS_FWD_WAVE_COLS 32
+#endif
+constexpr int kWaveCols = IGS_FWD_WAVE_COLS;
+static_assert(kWaveCols == 64 || kWaveCols == 32, "wave rectangle");
 #ifndef IGS_FWD_WAVE_MIN_P
 #define IGS_FWD_WAVE_MIN_P 8
 #endif
@@ -300,12 +308,13 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
     }
 }
 
-// Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows.  Per Gaussian
+// Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows (kWave = false) or
+// kWaveCols columns x 64 / kWaveCols blocks of P rows (kWave = true).  Per Gaussian
 // and lane: dx, A'dx^2, B2'dx once, then per pixel dy, 2 fma, exp2, 1 + C fma.
 // kWave = false: workgroup = wx x (4/wx) waves, all four streaming the tile's Gaussian list.
 // kWave = true (fwd_wave_lists): every wave has a list of its own and streams it independently of
-// the others (no barrier in the kernel); the four waves of a workgroup are the four row blocks of
-// one 64 x 4P tile of the binning.
+// the others (no barrier in the kernel); the four waves of a workgroup are the rectangles of one
+// 64 x 4P tile of the binning.
 template <int C, int P, bool kWave>
 __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     constexpr int RS = rec_stride_of(C), R4 = RS / 4;
@@ -318,10 +327,14 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    const int wx = kWave ? 1 : a.wx;
+    // A wave with a list of its own covers kWaveCols columns x (64 / kWaveCols) P rows: lane l has
+    // column l % kWaveCols and the P rows of row block l / kWaveCols; the tile of four waves is 64
+    // columns x 4 P rows either way.
+    constexpr int kHalves = 64 / kWaveCols;
+    const int wx = kWave ? kHalves : a.wx;
     const int wxi = wave % wx, wyi = wave / wx;
-    const int col = (tx * wx + wxi) * 64 + lane;
-    const int row0 = (ty * (4 / wx) + wyi) * P;
+    const int col = kWave ? tx * 64 + wxi * kWaveCols + lane % kWaveCols : (tx * wx + wxi) * 64 + lane;
+    const int row0 = kWave ? (ty * 4 + wyi * kHalves + lane / kWaveCols) * P : (ty * (4 / wx) + wyi) * P;
     const float xv = a.x[b * a.sxb + (long)min(col, a.W - 1) * a.sxw];
     float yv[P];
     // (all P loads first, then the pins: a pin right behind its load would wait for each load in turn)
@@ -351,9 +364,11 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     }
     // this unit's Gaussians (those whose ellipse reaches it), split S ways by list position
     const int s = blockIdx.y;
-    // (wave lists are numbered by rectangle, row after row; rows of rectangles below the image have none)
-    const size_t li = kWave ? ((size_t)b * 4 * a.tiles_y + (ty * 4 + wave)) * a.tiles_x + tx : (size_t)b * per_img + tl;
-    const int count = (!kWave || row0 < a.H) ? a.counts[li] : 0;
+    // (wave lists are numbered by rectangle, row after row; rectangles outside the image have none)
+    const int rrow = ty * (4 / kHalves) + wyi, rcol = tx * kHalves + wxi;
+    const size_t li = kWave ? ((size_t)b * (4 / kHalves) * a.tiles_y + rrow) * (kHalves * a.tiles_x) + rcol
+                            : (size_t)b * per_img + tl;
+    const int count = (!kWave || (rrow * kHalves * P < a.H && rcol * kWaveCols < a.W)) ? a.counts[li] : 0;
     // parts of decreasing length: part i has weight 1 + ramp - 2 ramp i / (S - 1), the sum is S
     auto cut = [&](int i) {  // first entry of part i, a multiple of 4
         const float f = a.S > 1 ? (float)i * (1.0f + kSplitRamp - kSplitRamp * (float)(i - 1) / (float)(a.S - 1)) / (float)a.S

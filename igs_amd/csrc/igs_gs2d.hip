@@ -85,7 +85,7 @@ FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
         // on a tie the squarest tile (fewest Gaussians reach it)
         long best = -1;
         g.wx = 1;
-        // (variants with a list per wave stack their four waves: 64 columns x 4 P rows)
+        // (variants with a list per wave: the four waves' rectangles make a tile of 64 columns x 4 P rows)
         for (int wx = 1; wx <= (fwd_wave_lists(C) ? 1 : 4); wx <<= 1) {
             const long cols = (long)ceil_div(W, 64 * wx) * 64 * wx;
             const long rows = (long)ceil_div(H, kFwdSepP * (4 / wx)) * kFwdSepP * (4 / wx);
@@ -366,7 +366,7 @@ int launch_bins(BinArgs fine, int B, bool levels2, const BinPlace& coarse, int* 
     c.tiles_x = sg.x; c.tiles_y = sg.y;
     c.counts = coarse.counts; c.lists = coarse.lists; c.slots = coarse_slots;
     c.chunk = sg.chunk;
-    c.sub_nx = 0; c.sub_h = 0; c.img_lists = 0;  // a super-tile has one list
+    c.sub_nx = 0; c.sub_w = 0; c.sub_h = 0; c.img_lists = 0; c.row_lists = 0;  // a super-tile has one list
     int rc = launch_bin(c, sg.K, B, st);
     if (rc) return rc;
     fine.cand_counts = coarse.counts; fine.cand_lists = coarse.lists;
@@ -647,20 +647,24 @@ int forward_impl(const float* packed, const float* x, const float* y,
             ba.flag = vs[i].flag; ba.want = vs[i].want;
             ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
             // a list per wave of the forward: four per tile of the binning
-            ba.sub_nx = fwd_wave_lists(C) ? fg.wx : 0;
-            ba.sub_h = fwd_sep_p(C);
-            ba.img_lists = 0;
+            constexpr int kHalves = 64 / kWaveCols;
+            ba.sub_nx = fwd_wave_lists(C) ? kHalves : 0;
+            ba.sub_w = kWaveCols;
+            ba.sub_h = kHalves * fwd_sep_p(C);
+            ba.img_lists = 0; ba.row_lists = 0;
             const bool levels2 = two_level(N, fg.tiles_x, fg.tiles_y, opts_of(grid_mode));
             // Few tiles: a workgroup per wave rectangle instead of one per tile with four lists fills
-            // the device better (B=1 N=16384 512x512: 28 against 72 us) and bounds each rectangle's
-            // denominators by itself; with many tiles the four-list workgroups read the bin records
-            // a quarter as often (B=16 N=8192 256x256: 44 against 67 us).
-            const int rect_rows = ceil_div(H, fwd_sep_p(C));
-            if (ba.sub_nx > 0 && !levels2 && (long)B * fg.tiles_x * rect_rows <= IGS_BIN_RECT_WORKGROUPS) {
+            // the device better (B=1 N=16384 512x512: 28 against 72 us, measured with rectangles of
+            // 64 x 16 pixels) and bounds each rectangle's denominators by itself; with many tiles the
+            // four-list workgroups read the bin records a quarter as often (B=16 N=8192 256x256: 44
+            // against 67 us).
+            const int rect_rows = ceil_div(H, ba.sub_h), rect_cols = ceil_div(W, kWaveCols);
+            if (ba.sub_nx > 0 && !levels2 && (long)B * rect_cols * rect_rows <= IGS_BIN_RECT_WORKGROUPS) {
                 ba.img_lists = 4 * fg.tiles_y * fg.tiles_x;
-                ba.tile_h = fwd_sep_p(C);
-                ba.tiles_y = rect_rows;
-                ba.sub_nx = 0; ba.sub_h = 0;
+                ba.row_lists = kHalves * fg.tiles_x;
+                ba.tile_w = kWaveCols; ba.tile_h = ba.sub_h;
+                ba.tiles_x = rect_cols; ba.tiles_y = rect_rows;
+                ba.sub_nx = 0; ba.sub_w = 0; ba.sub_h = 0;
             }
             const BinPlace cp = levels2 ? super_bins_at(ws, split_bytes, B, plan.fwd_tiles, plan.n_padded,
                                                         super_tiles(fg.tiles_x, fg.tiles_y, B, N).count)
@@ -903,7 +907,7 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
             ba.slots = slots_at(partial, B, a.T, 6 + C, N);
             ba.flag = a.flag; ba.want = a.want;
             ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
-            ba.sub_nx = 0; ba.sub_h = 0; ba.img_lists = 0;
+            ba.sub_nx = 0; ba.sub_w = 0; ba.sub_h = 0; ba.img_lists = 0; ba.row_lists = 0;
             const bool levels2 = two_level(N, ba.tiles_x, ba.tiles_y, opts_of(grid_mode));
             BinPlace cp{nullptr, nullptr};
             int* cslots = nullptr;

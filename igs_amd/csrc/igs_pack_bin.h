@@ -241,10 +241,13 @@ struct BinArgs {
     int want;
     int no_cull;  // list every candidate (IGS_OPT_NO_CULL): the reference point for "culling changes no bit"
     // Four lists per tile (the forward's wave lists; sub_nx = 0: one list).  The tile is sub_nx x
-    // (4 / sub_nx) rectangles of 64 columns x sub_h rows (rectangle w: column block w % sub_nx, row
-    // block w / sub_nx), each with a list of its own: list and count number 4 t + w of the image.
-    int sub_nx, sub_h;
-    int img_lists;  // lists per image in `counts` and `lists` when that is not the launch's own number (0)
+    // (4 / sub_nx) rectangles of sub_w columns x sub_h rows (rectangle w: column block w % sub_nx, row
+    // block w / sub_nx), each with a list of its own; the image's lists are numbered by rectangle,
+    // row after row of rectangles.
+    int sub_nx, sub_w, sub_h;
+    // Where the numbering of `counts` and `lists` is not the launch's own (one list per tile, row
+    // after row of tiles_x tiles): lists per image and lists per row.  0: the launch's own.
+    int img_lists, row_lists;
     // The launch carries dynamic LDS for one byte (four with four lists) per candidate, in which the
     // scan that settles what the tile skips leaves each candidate's weight class for the scan that
     // lists; 0: that scan evaluates the rectangle test again.
@@ -449,9 +452,9 @@ __global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin
             yhi = fmaxf(yhi, v);
         }
     } else if (wave < 4) {  // wave w takes the rectangle of the forward's wave w: its range is this wave's result
-        const int c = c0 + (wave % a.sub_nx) * 64 + lane;
+        const int c = c0 + (wave % a.sub_nx) * a.sub_w + lane;
         const int r = r0 + (wave / a.sub_nx) * a.sub_h + lane;
-        if (c < c1) {
+        if (lane < a.sub_w && c < c1) {
             xlo = xhi = a.x[b * a.sxb + (long)c * a.sxw];
             bad = !(xlo == xlo);
         }
@@ -500,7 +503,11 @@ __global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin
     // workgroup per rectangle gives (which then sets img_lists, rows of rectangles past the image's
     // last having no workgroup).
     const size_t img_first = (size_t)b * (a.img_lists > 0 ? a.img_lists : tiles * (masks ? 4 : 1));
-    auto list_no = [&](int l) { return img_first + (masks ? (size_t)(ty * 4 + l) * a.tiles_x + tx : (size_t)t); };
+    const int row_lists = a.row_lists > 0 ? a.row_lists : a.tiles_x * (masks ? a.sub_nx : 1);
+    auto list_no = [&](int l) {
+        return img_first + (masks ? (size_t)(ty * (4 / a.sub_nx) + l / a.sub_nx) * row_lists + tx * a.sub_nx + l % a.sub_nx
+                                  : (size_t)ty * row_lists + tx);
+    };
     int* list = a.lists + list_no(0) * a.Np + (size_t)kc * a.chunk;
     int* slot = a.slots ? a.slots + ((size_t)b * tiles + t) * a.Np : nullptr;
     // "definitely outside" negated, so that NaN bounds count as inside
@@ -709,7 +716,7 @@ __global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin
                 const bool listed = (code[u] >> l) & 1;
                 const unsigned long long m = __ballot(listed);
                 const int pos = base[l] + __popcll(m & below);
-                if (listed) list[(size_t)l * a.tiles_x * a.Np + pos] = n[u];  // (l > 0 with four lists only: next row of rectangles)
+                if (listed) (masks ? a.lists + list_no(l) * a.Np : list)[pos] = n[u];
                 // the slot of every candidate: its position (within the segment, at the first level,
                 // where only the sign is used) or -1
                 if (!masks && slot != nullptr && in[u]) slot[n[u]] = listed ? pos : -1;
