@@ -11,7 +11,7 @@ struct FwdArgs {
     long sxb, sxh, sxw, syb, syh, syw;
     int B, Np, H, W;
     int n_per_split, S;  // n_per_split % 4 == 0
-    int tiles_x, tiles_y, total_tiles, wx;
+    int tiles_x, tiles_y, total_tiles, wx, wcols;  // shared lists: wx waves of wcols columns side by side
     float eps;
     float* out;
     float* den;
@@ -330,11 +330,14 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     // A wave with a list of its own covers kWaveCols columns x (64 / kWaveCols) P rows: lane l has
     // column l % kWaveCols and the P rows of row block l / kWaveCols; the tile of four waves is 64
     // columns x 4 P rows either way.
+    // With a shared list (kWave = false) the workgroup is wx waves of wcols columns side by side, 4 / wx
+    // down: 64 wx columns x (4 / wx) P rows, or 32 columns x 8 P rows.
     constexpr int kHalves = 64 / kWaveCols;
     const int wx = kWave ? kHalves : a.wx;
+    const int wcols = kWave ? kWaveCols : a.wcols;
     const int wxi = wave % wx, wyi = wave / wx;
-    const int col = kWave ? tx * 64 + wxi * kWaveCols + lane % kWaveCols : (tx * wx + wxi) * 64 + lane;
-    const int row0 = kWave ? (ty * 4 + wyi * kHalves + lane / kWaveCols) * P : (ty * (4 / wx) + wyi) * P;
+    const int col = (tx * wx + wxi) * wcols + lane % wcols;
+    const int row0 = ((ty * (4 / wx) + wyi) * (64 / wcols) + lane / wcols) * P;
     const float xv = a.x[b * a.sxb + (long)min(col, a.W - 1) * a.sxw];
     float yv[P];
     // (all P loads first, then the pins: a pin right behind its load would wait for each load in turn)

@@ -73,8 +73,11 @@ bool shape_ok(int B, int N, int H, int W) {
     return true;
 }
 
+#ifndef IGS_FWD_NARROW_TILES
+#define IGS_FWD_NARROW_TILES 1
+#endif
 struct FwdGeometry {
-    int wx, tiles_x, tiles_y, total_tiles;
+    int wx, wcols, tiles_x, tiles_y, total_tiles;  // wx waves of wcols columns side by side
 };
 
 FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
@@ -85,6 +88,7 @@ FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
         // on a tie the squarest tile (fewest Gaussians reach it)
         long best = -1;
         g.wx = 1;
+        g.wcols = 64;
         // (variants with a list per wave: the four waves' rectangles make a tile of 64 columns x 4 P rows)
         for (int wx = 1; wx <= (fwd_wave_lists(C) ? 1 : 4); wx <<= 1) {
             const long cols = (long)ceil_div(W, 64 * wx) * 64 * wx;
@@ -95,10 +99,19 @@ FwdGeometry fwd_geometry(int B, int H, int W, int C, bool sep) {
                 g.wx = wx;
             }
         }
-        g.tiles_x = ceil_div(W, 64 * g.wx);
-        g.tiles_y = ceil_div(H, kFwdSepP * (4 / g.wx));
+        if (!fwd_wave_lists(C)) {
+            // four waves of 32 columns x 2 P rows stacked: 32 columns x 8 P rows, the squarest tile
+            const long area = (long)ceil_div(W, 32) * 32 * ceil_div(H, 8 * kFwdSepP) * 8 * kFwdSepP;
+            if (IGS_FWD_NARROW_TILES && area <= best) {
+                g.wx = 1;
+                g.wcols = 32;
+            }
+        }
+        g.tiles_x = ceil_div(W, g.wcols * g.wx);
+        g.tiles_y = ceil_div(H, kFwdSepP * (64 / g.wcols) * (4 / g.wx));
     } else {
         g.wx = 4;
+        g.wcols = 64;
         g.tiles_x = ceil_div((long)H * W, kThreads * fwd_gen_p(C));
         g.tiles_y = 1;
     }
@@ -628,7 +641,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
         a.B = B; a.Np = plan.n_padded; a.H = H; a.W = W;
         a.S = plan.fwd_split;
         a.n_per_split = plan.fwd_n_per_split;
-        a.tiles_x = fg.tiles_x; a.tiles_y = fg.tiles_y; a.total_tiles = fg.total_tiles; a.wx = fg.wx;
+        a.tiles_x = fg.tiles_x; a.tiles_y = fg.tiles_y; a.total_tiles = fg.total_tiles; a.wx = fg.wx; a.wcols = fg.wcols;
         a.eps = eps; a.out = out; a.den = den; a.part = (float*)ws;
         a.counts = nullptr; a.lists = nullptr;
         a.flag = vs[i].flag; a.want = vs[i].want;
@@ -641,7 +654,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
             ba.x = x; ba.y = y;
             ba.sxb = a.sxb; ba.sxw = a.sxw; ba.syb = a.syb; ba.syh = a.syh;
             ba.N = N; ba.Np = plan.n_padded; ba.H = H; ba.W = W;
-            ba.tile_w = 64 * fg.wx; ba.tile_h = fwd_sep_p(C) * (4 / fg.wx);
+            ba.tile_w = fg.wcols * fg.wx; ba.tile_h = fwd_sep_p(C) * (64 / fg.wcols) * (4 / fg.wx);
             ba.tiles_x = fg.tiles_x; ba.tiles_y = fg.tiles_y;
             ba.counts = bp.counts; ba.lists = bp.lists; ba.slots = nullptr;
             ba.flag = vs[i].flag; ba.want = vs[i].want;
