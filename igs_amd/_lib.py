@@ -14,13 +14,14 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 LIB_PATH = os.environ.get("IGS_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "libigs_hip.so")
 
-ABI_VERSION = 6  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
+ABI_VERSION = 7  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1
 IGS_GRID_AUTO = 2
 IGS_OPT_NO_CULL = 0x100
 IGS_OPT_BIN_LEVELS_1 = 0x200
 IGS_OPT_BIN_LEVELS_2 = 0x400
+IGS_OPT_LISTS_BUILT = 0x800
 IGS_MAX_CHANNELS = 16
 IGS_STATIC_SCRATCH_BYTES = 64 << 20
 COMPILED_CHANNELS = (1, 2, 3, 4, 8, 16)
@@ -47,6 +48,7 @@ class Plan(ctypes.Structure):
         ("fwd_tiles", c_int32),
         ("bwd_tiles_x", c_int32),
         ("bwd_tile_w", c_int32),
+        ("lists_shared", c_int32),
     ]
 
 
@@ -83,6 +85,9 @@ SIGNATURES = {
     "igs_gs2d_grid_classify": (c_int, [_FP, _FP, _STRIDES, c_int, c_int, c_int, _FP, c_void_p]),
     "igs_gs2d_forward": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
                                  c_float, _FP, _FP, c_void_p, c_size_t, c_void_p]),
+    "igs_gs2d_forward_shared_lists": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
+                                              c_float, _FP, _FP, c_void_p, c_size_t, _FP, c_size_t, _FP, c_size_t,
+                                              c_void_p]),
     "igs_gs2d_forward_static_ws": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
                                            c_float, _FP, _FP, c_void_p]),
     "igs_gs2d_backward_prologue": (c_int, [_FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int,

@@ -182,6 +182,7 @@ class Splat:
         self.grid, self.eps, self.device = grid, float(eps), device
         self.plan = _lib.plan(B, N, grid.H, grid.W, self.Cp, grid.mode)
         self.skip_weight = skip_weight(N, self.eps)
+        self.shared = None   # (pix, partial) with the tile lists in place, after forward_shared_lists
         self.stream = None
         self.use_current_stream()
 
@@ -230,11 +231,34 @@ class Splat:
                                              int(p.fwd_ws_bytes), self.stream), "igs_gs2d_forward")
         return out, den
 
-    def backward_partials(self, packed, colors_p, out, den, grad_out_p) -> Tensor:
+    def forward_shared_lists(self, packed: Tensor) -> Tuple[Tensor, Tensor]:
+        """The forward of a step whose backward will follow, where the plan says that both passes can
+        run over one set of tile lists (`plan.lists_shared`): the lists are built once, in the
+        backward's workspaces, which this object keeps for `backward_partials*`."""
         g, p = self.grid, self.plan
+        out = self._new(self.B, self.Cp, g.H, g.W)
+        den = self._new(self.B, g.H, g.W)
+        ws = self._empty(p.fwd_ws_bytes) if p.fwd_ws_bytes else None
         pix = self._empty(p.pix_bytes)
         partial = self._empty(p.partial_bytes)
-        _lib.check(self.lib.igs_gs2d_backward(_ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, g.mode,
+        _lib.check(self.lib.igs_gs2d_forward_shared_lists(
+            _ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), self.B, self.N, g.H, g.W, self.Cp,
+            self.eps, _ptr(out), _ptr(den), _ptr(ws), int(p.fwd_ws_bytes), _ptr(pix), int(p.pix_bytes), _ptr(partial),
+            int(p.partial_bytes), self.stream), "igs_gs2d_forward_shared_lists")
+        self.shared = (pix, partial)
+        return out, den
+
+    def _backward_workspaces(self):
+        """(pix, partial, grid_mode): the workspaces that hold the tile lists already, if the forward
+        built them, else fresh ones."""
+        if self.shared is not None:
+            return (*self.shared, self.grid.mode | _lib.IGS_OPT_LISTS_BUILT)
+        return self._empty(self.plan.pix_bytes), self._empty(self.plan.partial_bytes), self.grid.mode
+
+    def backward_partials(self, packed, colors_p, out, den, grad_out_p) -> Tensor:
+        g, p = self.grid, self.plan
+        pix, partial, mode = self._backward_workspaces()
+        _lib.check(self.lib.igs_gs2d_backward(_ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, mode,
                                               _ptr(g.flag), _ptr(out), _ptr(den), _ptr(grad_out_p), self.B, self.N, g.H, g.W,
                                               self.Cp, self.eps, _ptr(pix), int(p.pix_bytes), _ptr(partial),
                                               int(p.partial_bytes), self.stream), "igs_gs2d_backward")
@@ -244,8 +268,7 @@ class Splat:
         """The per-Gaussian partial sums and d L / d x_grid, d L / d y_grid from one call (on general
         grids the grid sums are formed inside the per-Gaussian reduction)."""
         g, p = self.grid, self.plan
-        pix = self._empty(p.pix_bytes)
-        partial = self._empty(p.partial_bytes)
+        pix, partial, mode = self._backward_workspaces()
         # host-proven separable grids run the pixel-major grid kernel, which needs no workspace
         separable = (g.mode & 0xff) == _lib.IGS_GRID_SEPARABLE
         gws_bytes = 0 if separable else int(self.lib.igs_gs2d_grid_workspace_bytes(self.B, self.N, g.H, g.W, self.Cp))
@@ -253,7 +276,7 @@ class Splat:
         gx = self._new(self.B, g.H, g.W)
         gy = torch.empty_like(gx)
         _lib.check(self.lib.igs_gs2d_backward_with_grid(
-            _ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), _ptr(out), _ptr(den),
+            _ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, mode, _ptr(g.flag), _ptr(out), _ptr(den),
             _ptr(grad_out_p), self.B, self.N, g.H, g.W, self.Cp, self.eps, _ptr(pix), int(p.pix_bytes), _ptr(partial),
             int(p.partial_bytes), _ptr(gws), gws_bytes, _ptr(gx), _ptr(gy), self.stream), "igs_gs2d_backward_with_grid")
         return partial, self._fit_grid(gx, x_like), self._fit_grid(gy, y_like)
@@ -349,10 +372,12 @@ def require_same_device(dev, tensors: Sequence[Optional[Tensor]], what: str):
                                f"{t.device} while the Gaussian parameters are on {dev}")
 
 
-def run_forward(kind: int, params: Sequence[Tensor], x: Tensor, y: Tensor, eps: float):
+def run_forward(kind: int, params: Sequence[Tensor], x: Tensor, y: Tensor, eps: float, train: bool = False):
     """pack + splat.  Returns (op, keep, packed, col, out, den): `keep` are the fp32 contiguous
     copies of the parameters that the finalize kernel of this kind reads again, `col` the colours
-    padded to the compiled channel count Cp, `out` [B,Cp,H,W] and `den` [B,H,W] in fp32."""
+    padded to the compiled channel count Cp, `out` [B,Cp,H,W] and `den` [B,H,W] in fp32.
+    `train`: a backward through `op` will follow; where the plan allows, the tile lists are then
+    built once for both passes (and `op` holds the backward's workspaces until it is released)."""
     require_gpu(params[0])
     B, N, C = problem_dims(kind, params)
     dev = params[0].device
@@ -375,7 +400,7 @@ def run_forward(kind: int, params: Sequence[Tensor], x: Tensor, y: Tensor, eps: 
             off = _f32c(params[1]) if len(params) == 2 else None
             packed, col = op.pack_feature(feat, off)
             keep = (feat,)
-        out, den = op.forward(packed)
+        out, den = op.forward_shared_lists(packed) if (train and op.plan.lists_shared) else op.forward(packed)
     return op, keep, packed, col, out, den
 
 

@@ -18,6 +18,7 @@ struct FwdArgs {
     float* part;  // [S][B][C+1][HW] when S > 1
     const int* counts;  // separable: Gaussians listed per tile [B][tiles], or per wave rectangle, row after row over the tiles' extent [B][4 tiles]
     const int* lists;   // separable: their indices [B][lists][Np]
+    int list_img, list_row;  // lists per image and per row of rectangles (tiles) in that numbering
     const int* flag;  // AUTO grid mode: run only if *flag == want (nullptr: always run)
     int want;
 };
@@ -369,8 +370,7 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     const int s = blockIdx.y;
     // (wave lists are numbered by rectangle, row after row; rectangles outside the image have none)
     const int rrow = ty * (4 / kHalves) + wyi, rcol = tx * kHalves + wxi;
-    const size_t li = kWave ? ((size_t)b * (4 / kHalves) * a.tiles_y + rrow) * (kHalves * a.tiles_x) + rcol
-                            : (size_t)b * per_img + tl;
+    const size_t li = (size_t)b * a.list_img + (size_t)(kWave ? rrow : ty) * a.list_row + (kWave ? rcol : tx);
     const int count = (!kWave || (rrow * kHalves * P < a.H && rcol * kWaveCols < a.W)) ? a.counts[li] : 0;
     // parts of decreasing length: part i has weight 1 + ramp - 2 ramp i / (S - 1), the sum is S
     auto cut = [&](int i) {  // first entry of part i, a multiple of 4

@@ -222,6 +222,13 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     }
     T = (long)ceil_div(sep ? H : p->hw_padded, p->bwd_per_tile) * p->bwd_tiles_x;
     p->bwd_tiles = (int)T;
+    {   // do the backward's tiles coincide with the forward's wave rectangles (tiles, with one list per tile)?
+        const int frows = fwd_wave_lists(C) ? (64 / kWaveCols) * fwd_sep_p(C)
+                                            : fwd_sep_p(C) * (64 / fg.wcols) * (4 / fg.wx);
+        const int fcols = fwd_wave_lists(C) ? kWaveCols : fg.wcols * fg.wx;
+        p->lists_shared = sep && fcols == kBwdTileW && frows == p->bwd_per_tile &&
+                          ceil_div(W, fcols) == p->bwd_tiles_x;
+    }
     p->fwd_tiles = sep ? fg.tiles_x * fg.tiles_y * (fwd_wave_lists(C) ? 4 : 1) : 0;
     p->pix_stride = sep ? pix_stride_sep(C) : pix_stride_gen(C);
     // records, then one bin record (8 floats) per record, then the call's skip settings (4 floats)
@@ -515,7 +522,7 @@ int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* col
 
 int mode_ok(int grid_mode, const int32_t* grid_flag) {
     const int opts = opts_of(grid_mode);
-    if (opts & ~(IGS_OPT_NO_CULL | IGS_OPT_BIN_LEVELS_1 | IGS_OPT_BIN_LEVELS_2)) return IGS_ERR_BAD_MODE;
+    if (opts & ~(IGS_OPT_NO_CULL | IGS_OPT_BIN_LEVELS_1 | IGS_OPT_BIN_LEVELS_2 | IGS_OPT_LISTS_BUILT)) return IGS_ERR_BAD_MODE;
     if ((opts & IGS_OPT_BIN_LEVELS_1) && (opts & IGS_OPT_BIN_LEVELS_2)) return IGS_ERR_BAD_MODE;
     grid_mode = mode_of(grid_mode);
     if (grid_mode != IGS_GRID_GENERAL && grid_mode != IGS_GRID_SEPARABLE && grid_mode != IGS_GRID_AUTO)
@@ -611,10 +618,41 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
 }  // extern "C"
 
 namespace {
+// The tile lists and slot tables of the separable backward (a = bwd_args of the separable variant);
+// column coordinates x[b * sxb + w * sxw].
+int bin_backward(const BwdArgs& a, const float* x, long sxb, long sxw, const float* packed, int B, int C, int opts,
+                 float* pix_ws, float* partial, hipStream_t st) {
+    BinArgs ba;
+    ba.bins = bins_of(packed, B, a.Np, rec_stride_of(C));
+    ba.limit = limit_of(packed, B, a.Np, rec_stride_of(C));
+    ba.x = x; ba.y = a.y;
+    ba.sxb = sxb; ba.sxw = sxw; ba.syb = a.syb; ba.syh = a.syh;
+    ba.N = a.N; ba.Np = a.Np; ba.H = a.H; ba.W = a.W;
+    ba.tile_w = kBwdTileW; ba.tile_h = a.per_tile;
+    ba.tiles_x = a.tiles_x; ba.tiles_y = a.T / a.tiles_x;
+    ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists);
+    ba.slots = slots_at(partial, B, a.T, 6 + C, a.N);
+    ba.flag = a.flag; ba.want = a.want;
+    ba.no_cull = (opts & IGS_OPT_NO_CULL) != 0;
+    ba.sub_nx = 0; ba.sub_w = 0; ba.sub_h = 0; ba.img_lists = 0; ba.row_lists = 0;
+    const bool levels2 = two_level(a.N, ba.tiles_x, ba.tiles_y, opts);
+    BinPlace cp{nullptr, nullptr};
+    int* cslots = nullptr;
+    if (levels2) {
+        const size_t scratch = ((size_t)B * a.H * a.Wp * pix_stride_sep(C) + (size_t)B * a.Wp) * sizeof(float);
+        cp = super_bins_at(pix_ws, scratch, B, a.T, a.Np, super_tiles(ba.tiles_x, ba.tiles_y, B, a.N).count);
+        cslots = super_slots_at(partial, B, a.T, 6 + C, a.N, a.Np);
+    }
+    return launch_bins(ba, B, levels2, cp, cslots, st);
+}
+
+// pix_ws / partial: the backward's workspaces, when the forward is to run over the backward's tile
+// lists (built here; plan.lists_shared) instead of lists of its own; else nullptr.
 int forward_impl(const float* packed, const float* x, const float* y,
                  const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag, int B,
                  int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
-                 size_t ws_bytes, igs_stream_t stream) {
+                 size_t ws_bytes, float* pix_ws, size_t pix_bytes, float* partial, size_t partial_bytes,
+                 igs_stream_t stream) {
     if (!packed || !x || !y || !grid_strides || !out || !den) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
@@ -624,6 +662,13 @@ int forward_impl(const float* packed, const float* x, const float* y,
     if (rc) return rc;
     if (total.fwd_ws_bytes > 0 && (!ws || ws_bytes < total.fwd_ws_bytes)) return IGS_ERR_WORKSPACE;
     if (((uintptr_t)packed | (uintptr_t)ws) & 15) return IGS_ERR_ALIGNMENT;  // float4 / int lists inside
+    const bool shared = pix_ws != nullptr;
+    if (shared) {
+        if (!partial) return IGS_ERR_NULL_POINTER;
+        if (!total.lists_shared) return IGS_ERR_BAD_SHAPE;
+        if (pix_bytes < total.pix_bytes || partial_bytes < total.partial_bytes) return IGS_ERR_WORKSPACE;
+        if ((uintptr_t)pix_ws & 15) return IGS_ERR_ALIGNMENT;
+    }
     hipStream_t st = (hipStream_t)stream;
     Variant vs[2];
     const int nv = variants_of(grid_mode, grid_flag, vs);
@@ -645,7 +690,20 @@ int forward_impl(const float* packed, const float* x, const float* y,
         a.eps = eps; a.out = out; a.den = den; a.part = (float*)ws;
         a.counts = nullptr; a.lists = nullptr;
         a.flag = vs[i].flag; a.want = vs[i].want;
-        if (sep) {
+        // numbering of the lists: by wave rectangle (or by tile, with one list per tile), row after row
+        constexpr int kHalvesL = 64 / kWaveCols;
+        a.list_row = fwd_wave_lists(C) ? kHalvesL * fg.tiles_x : fg.tiles_x;
+        a.list_img = fwd_wave_lists(C) ? 4 * fg.tiles_x * fg.tiles_y : fg.tiles_x * fg.tiles_y;
+        if (sep && shared) {
+            // the backward's tiles are the forward's wave rectangles (or tiles): its lists serve both
+            BwdArgs bw;
+            rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, partial);
+            if (rc) return rc;
+            rc = bin_backward(bw, x, grid_strides[0], grid_strides[2], packed, B, C, opts_of(grid_mode), pix_ws, partial, st);
+            if (rc) return rc;
+            a.counts = bw.counts; a.lists = bw.lists;
+            a.list_row = bw.tiles_x; a.list_img = bw.T;
+        } else if (sep) {
             const size_t split_bytes = a.S > 1 ? (size_t)a.S * B * (C + 1) * H * W * sizeof(float) : 0;
             const BinPlace bp = bins_at(ws, split_bytes, B, plan.fwd_tiles);
             BinArgs ba;
@@ -735,7 +793,17 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
                      int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
                      size_t ws_bytes, igs_stream_t stream) {
     return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
-                        ws_bytes, stream);
+                        ws_bytes, nullptr, 0, nullptr, 0, stream);
+}
+
+int igs_gs2d_forward_shared_lists(const float* packed, const float* x, const float* y,
+                                  const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                                  int B, int N, int H, int W, int C, float eps, float* out, float* den,
+                                  void* ws, size_t ws_bytes, float* pix_ws, size_t pix_bytes, float* partial,
+                                  size_t partial_bytes, igs_stream_t stream) {
+    if (!pix_ws || !partial) return IGS_ERR_NULL_POINTER;
+    return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
+                        ws_bytes, pix_ws, pix_bytes, partial, partial_bytes, stream);
 }
 
 int igs_gs2d_forward_static_ws(const float* packed, const float* x, const float* y,
@@ -752,7 +820,7 @@ int igs_gs2d_forward_static_ws(const float* packed, const float* x, const float*
     rc = static_scratch(&ws);
     if (rc) return rc;
     return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
-                        IGS_STATIC_SCRATCH_BYTES, stream);
+                        IGS_STATIC_SCRATCH_BYTES, nullptr, 0, nullptr, 0, stream);
 }
 
 }  // extern "C"
@@ -907,29 +975,9 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
         rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C, pix_ws, partial);
         if (rc) return rc;
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
-        if (sep) {
-            BinArgs ba;
-            ba.bins = bins_of(packed, B, a.Np, rec_stride_of(C));
-            ba.limit = limit_of(packed, B, a.Np, rec_stride_of(C));
-            ba.x = a.xs; ba.y = y;               // the prologue's compact column coordinates
-            ba.sxb = a.Wp; ba.sxw = 1; ba.syb = a.syb; ba.syh = a.syh;
-            ba.N = N; ba.Np = a.Np; ba.H = H; ba.W = W;
-            ba.tile_w = kBwdTileW; ba.tile_h = a.per_tile;
-            ba.tiles_x = a.tiles_x; ba.tiles_y = a.T / a.tiles_x;
-            ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists);
-            ba.slots = slots_at(partial, B, a.T, 6 + C, N);
-            ba.flag = a.flag; ba.want = a.want;
-            ba.no_cull = (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0;
-            ba.sub_nx = 0; ba.sub_w = 0; ba.sub_h = 0; ba.img_lists = 0; ba.row_lists = 0;
-            const bool levels2 = two_level(N, ba.tiles_x, ba.tiles_y, opts_of(grid_mode));
-            BinPlace cp{nullptr, nullptr};
-            int* cslots = nullptr;
-            if (levels2) {
-                const size_t scratch = ((size_t)B * H * a.Wp * pix_stride_sep(C) + (size_t)B * a.Wp) * sizeof(float);
-                cp = super_bins_at(pix_ws, scratch, B, a.T, a.Np, super_tiles(ba.tiles_x, ba.tiles_y, B, N).count);
-                cslots = super_slots_at(partial, B, a.T, 6 + C, N, a.Np);
-            }
-            rc = launch_bins(ba, B, levels2, cp, cslots, st);
+        if (sep && !(opts_of(grid_mode) & IGS_OPT_LISTS_BUILT)) {
+            // (the prologue's compact column coordinates: the same values as the grid's)
+            rc = bin_backward(a, a.xs, a.Wp, 1, packed, B, C, opts_of(grid_mode), pix_ws, partial, st);
             if (rc) return rc;
         }
         if (gg.g_x != nullptr && !sep) a.grid_part = reinterpret_cast<float2*>(gg.ws);

@@ -148,11 +148,19 @@ class GaussianImageFit:
         return ws
 
     # ------------------------------------------------------------------ the step
-    def _enqueue_render(self, n: int, ws: dict, st):
+    def _enqueue_render(self, n: int, ws: dict, st, train: bool = False):
+        """pack + forward.  `train`: the backward follows; where the plan allows (`lists_shared`) the
+        tile lists are then built once, in the backward's workspaces, for both passes."""
         lib, g, p = self.lib, self.grid, ws["plan"]
         B, C, Cp, H, W = self.B, self.C, self.Cp, g.H, g.W
         _lib.check(lib.igs_gs2d_pack_feature(_ptr(self.params), None, B, n, C, Cp, self.eps, *ws["skip_weight"],
                                              _ptr(ws["packed"]), _ptr(ws["col"]), st), "igs_gs2d_pack_feature")
+        if train and p.lists_shared:
+            _lib.check(lib.igs_gs2d_forward_shared_lists(
+                _ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n, H, W, Cp, self.eps,
+                _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]), int(p.fwd_ws_bytes), _ptr(ws["pix"]),
+                int(p.pix_bytes), _ptr(ws["partial"]), int(p.partial_bytes), st), "igs_gs2d_forward_shared_lists")
+            return
         _lib.check(lib.igs_gs2d_forward(_ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n,
                                         H, W, Cp, self.eps, _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]),
                                         int(p.fwd_ws_bytes), st), "igs_gs2d_forward")
@@ -174,7 +182,8 @@ class GaussianImageFit:
                                                       _ptr(ws["out"]), _ptr(ws["den"]), _ptr(grad_out), B, n, H, W, Cp,
                                                       self.eps, _ptr(ws["pix"]), int(p.pix_bytes), st),
                        "igs_gs2d_backward_prologue")
-        _lib.check(lib.igs_gs2d_backward_reduce(_ptr(ws["packed"]), _ptr(ws["col"]), _ptr(g.y), g.strides, g.mode,
+        mode = g.mode | (_lib.IGS_OPT_LISTS_BUILT if p.lists_shared else 0)  # (the render of a step built them)
+        _lib.check(lib.igs_gs2d_backward_reduce(_ptr(ws["packed"]), _ptr(ws["col"]), _ptr(g.y), g.strides, mode,
                                                 _ptr(g.flag), B, n, H, W, Cp, _ptr(ws["pix"]), int(p.pix_bytes),
                                                 _ptr(ws["partial"]), int(p.partial_bytes), st),
                    "igs_gs2d_backward_reduce")
@@ -193,13 +202,13 @@ class GaussianImageFit:
     def _enqueue_step(self, n: int):
         ws = self._workspace(n)
         st = _stream(self.device)
-        self._enqueue_render(n, ws, st)
+        self._enqueue_render(n, ws, st, train=True)
         self._enqueue_backward(n, ws, st, None)
 
     def _step_with_loss_fn(self, n: int, loss_fn):
         ws = self._workspace(n)
         st = _stream(self.device)
-        self._enqueue_render(n, ws, st)
+        self._enqueue_render(n, ws, st, train=True)
         image = ws["out"][:, :self.C].detach().requires_grad_(True)       # a view: no copy
         with torch.enable_grad():
             loss = loss_fn(image)

@@ -74,7 +74,7 @@ class _Operator(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, y, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors, eps=1e-6):
         params = (position, cov_inv_00, cov_inv_01, cov_inv_11, alphas, colors)
-        op, keep, packed, col, out, den = run_forward(KIND_COVINV, params, x, y, eps)
+        op, keep, packed, col, out, den = run_forward(KIND_COVINV, params, x, y, eps, train=any(ctx.needs_input_grad))
         ctx.op = op
         ctx.grid_like = ((x.shape, x.dtype), (y.shape, y.dtype))
         ctx.n_keep = len(keep)
@@ -154,7 +154,7 @@ class _RenderFused(torch.autograd.Function):
     @staticmethod
     def forward(ctx, positions, colors, scales, rotations, alphas, x_grid, y_grid, eps):
         params = (positions, colors, scales, rotations, alphas)
-        op, keep, packed, col, out, den = run_forward(KIND_SCALE_ROT, params, x_grid, y_grid, eps)
+        op, keep, packed, col, out, den = run_forward(KIND_SCALE_ROT, params, x_grid, y_grid, eps, train=any(ctx.needs_input_grad))
         ctx.op = op
         ctx.grid_like = ((x_grid.shape, x_grid.dtype), (y_grid.shape, y_grid.dtype))
         ctx.n_keep = len(keep)
@@ -184,7 +184,7 @@ class _RenderFromFeature(torch.autograd.Function):
     @staticmethod
     def forward(ctx, gs_feature, pos_offset, x_grid, y_grid, eps):
         params = (gs_feature,) if pos_offset is None else (gs_feature, pos_offset)
-        op, keep, packed, col, out, den = run_forward(KIND_FEATURE, params, x_grid, y_grid, eps)
+        op, keep, packed, col, out, den = run_forward(KIND_FEATURE, params, x_grid, y_grid, eps, train=any(ctx.needs_input_grad))
         ctx.op = op
         ctx.grid_like = ((x_grid.shape, x_grid.dtype), (y_grid.shape, y_grid.dtype))
         ctx.n_keep = len(keep)

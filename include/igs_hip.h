@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define IGS_ABI_VERSION 6
+#define IGS_ABI_VERSION 7
 #define IGS_MAX_CHANNELS 16
 /* Size of the per-device static scratch array behind igs_gs2d_forward_static_ws. */
 #define IGS_STATIC_SCRATCH_BYTES (64u << 20)
@@ -80,8 +80,13 @@ typedef enum igs_option {
                                      (nothing is skipped): the reference point for checking what
                                      skipping changes */
     IGS_OPT_BIN_LEVELS_1 = 0x200, /* build the per-tile Gaussian lists in one level ...           */
-    IGS_OPT_BIN_LEVELS_2 = 0x400  /* ... or through super-tiles of 4 x 4 tiles, whatever the size;
+    IGS_OPT_BIN_LEVELS_2 = 0x400, /* ... or through super-tiles of 4 x 4 tiles, whatever the size;
                                      without either bit the library chooses by tiles x N          */
+    IGS_OPT_LISTS_BUILT = 0x800   /* igs_gs2d_backward_reduce / igs_gs2d_backward /
+                                     igs_gs2d_backward_with_grid only: the tile lists and slot
+                                     tables are in these workspaces already
+                                     (igs_gs2d_forward_shared_lists built them for this packed
+                                     buffer and these grids); do not build them again            */
 } igs_option;
 
 /* Launch plan and workspace sizes for one problem shape (filled by igs_gs2d_plan).  In AUTO
@@ -112,6 +117,9 @@ typedef struct igs_gs2d_plan_t {
     int32_t fwd_tiles;       /* separable: pixel tiles per image of the forward            */
     int32_t bwd_tiles_x;     /* separable: column bands of the backward tiles              */
     int32_t bwd_tile_w;      /* separable: columns per band                                */
+    int32_t lists_shared;    /* separable: the backward's tiles are the forward's wave
+                                rectangles, so igs_gs2d_forward_shared_lists can build one
+                                set of tile lists for both passes                           */
 } igs_gs2d_plan_t;
 
 int igs_abi_version(void);
@@ -207,6 +215,24 @@ int igs_gs2d_forward_static_ws(const float *packed, const float *x, const float 
                                const int64_t grid_strides[6], int grid_mode,
                                const int32_t *grid_flag, int B, int N, int H, int W, int C,
                                float eps, float *out, float *den, igs_stream_t stream);
+
+/* The forward of a training step on separable grids, where plan.lists_shared says that the
+ * backward's pixel tiles are the forward's wave rectangles: builds the backward's per-tile Gaussian
+ * lists and slot tables in pix_ws / partial (plan.pix_bytes / plan.partial_bytes; the lists depend
+ * on the packed buffer and the grids only) and runs the forward over them instead of binning once
+ * for each pass.  The backward calls on the same workspaces then get IGS_OPT_LISTS_BUILT in their
+ * grid_mode (the prologue writes other parts of pix_ws).  IGS_ERR_BAD_SHAPE where
+ * plan.lists_shared is 0.  Otherwise as igs_gs2d_forward, whose output it matches up to what the
+ * skip tolerance allows (a tile settles what it leaves out by itself, and the tiles of the two
+ * binnings need not be the same); bit for bit with skip_weight = skip_fraction = 0 and one
+ * Gaussian split.  No counterpart in the reference, which evaluates every pair
+ * (src/igs/gs_triton_chunked.py:100-200). */
+int igs_gs2d_forward_shared_lists(const float *packed, const float *x, const float *y,
+                                  const int64_t grid_strides[6], int grid_mode,
+                                  const int32_t *grid_flag, int B, int N, int H, int W, int C,
+                                  float eps, float *out, float *den, void *ws, size_t ws_bytes,
+                                  float *pix_ws, size_t pix_bytes, float *partial,
+                                  size_t partial_bytes, igs_stream_t stream);
 
 /* Backward, stage 1: per-pixel prologue, g^ = grad_out/(den+eps), s = <g^, out>, written
  * as one record per pixel into pix_ws (plan.pix_bytes).  Replaces the per-image pre-pass of

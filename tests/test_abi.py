@@ -133,7 +133,7 @@ def test_argument_errors_are_status_codes_not_crashes(lib):
     assert lib.igs_gs2d_backward_with_grid(fake, fake, fake, fake, st, 0, None, fake, fake, fake, 2, 3000, 10, 13, 3,
                                            1e-6, fake, 1 << 30, fake, 1 << 30, None, 0, fake, fake, None) == -1
     # option bits ride in the grid_mode word; unknown or contradictory ones are rejected
-    assert lib.igs_gs2d_forward(fake, fake, fake, st, 1 | 0x800, None, 1, 8, 4, 4, 3, 1e-6, fake, fake, fake, 1 << 30,
+    assert lib.igs_gs2d_forward(fake, fake, fake, st, 1 | 0x1000, None, 1, 8, 4, 4, 3, 1e-6, fake, fake, fake, 1 << 30,
                                 None) == -5
     assert lib.igs_gs2d_forward(fake, fake, fake, st, 1 | 0x200 | 0x400, None, 1, 8, 4, 4, 3, 1e-6, fake, fake, fake,
                                 1 << 30, None) == -5

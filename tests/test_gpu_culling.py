@@ -612,6 +612,66 @@ def test_more_candidates_than_the_class_store_holds(igs, dev, no_cull, shape):
         assert float((gradse[k] - grads0[k]).double().norm()) <= 1e-5 * n0, k
 
 
+@pytest.mark.parametrize("shape,scales", [((8, 4096, 256, 256, 3), (0.01, 0.2)), ((8, 16384, 128, 160, 3), (0.005, 0.1)),
+                                          ((4, 32768, 96, 128, 16), (0.005, 0.08)), ((2, 200000, 192, 256, 3), (0.002, 0.02))],
+                         ids=lambda v: "x".join(map(str, v)))
+def test_one_set_of_tile_lists_for_both_passes(igs, dev, shape, scales):
+    """Where the backward's tiles are the forward's wave rectangles (`plan.lists_shared`) a step that
+    needs gradients builds the tile lists once, in the backward's workspaces
+    (`igs_gs2d_forward_shared_lists`, then IGS_OPT_LISTS_BUILT), instead of once per pass.  Against
+    the path that bins twice: every gradient bit for bit (the backward's lists are the same lists);
+    the image within what the tolerance allows (the forward's own binning settles a 64 x 64 tile's
+    allowance with one floor for its four rectangles), and bit for bit when only exact zeros are
+    skipped.  The last shape bins in two levels."""
+    from igs_amd import _lib, _splat
+
+    B, N, H, W, C = shape
+    plan = _lib.plan(B, N, H, W, _kernel_channels(C), 1)
+    assert plan.lists_shared == 1
+    _, g = sparse_case(dev, B, N, H, W, C, seed=sum(shape), smin=scales[0], smax=scales[1])
+    params = [g[k] for k in NAMES]
+    need = [True] * 5
+
+    def both(train):
+        op, keep, packed, col, out, den = _splat.run_forward(_splat.KIND_SCALE_ROT, params, g["x_grid"], g["y_grid"],
+                                                             1e-6, train=train)
+        assert (op.shared is not None) == train
+        grads, _, _ = _splat.run_backward(_splat.KIND_SCALE_ROT, op, keep, packed, col, out, den, g["grad_out"], need,
+                                          False, False, None)
+        return out[:, :C], grads
+
+    out_a, grads_a = both(False)
+    out_b, grads_b = both(True)
+    cmax = float(g["colors"].abs().max())
+    assert float((out_a - out_b).abs().max()) <= 2e-7 * cmax + 1e-6
+    for k, ga, gb in zip(NAMES, grads_a, grads_b):
+        assert float(ga.abs().max()) > 0 and torch.equal(ga, gb), k
+    with exact():
+        out_a, grads_a = both(False)
+        out_b, grads_b = both(True)
+    assert torch.equal(out_a, out_b)
+    for k, ga, gb in zip(NAMES, grads_a, grads_b):
+        assert torch.equal(ga, gb), k
+
+
+def test_shared_lists_are_refused_where_the_tilings_differ(igs, dev):
+    """A small problem's backward tiles have fewer rows than the forward's wave rectangles: the plan
+    says so and the combined entry point returns a status instead of running."""
+    from igs_amd import _lib
+    from igs_amd._splat import Grid, Splat, _f32c, _ptr
+
+    B, N, H, W, C = 1, 300, 96, 160, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=2)
+    op = Splat(B, N, C, Grid(g["x_grid"], g["y_grid"], B), 1e-6, dev)
+    assert op.plan.lists_shared == 0
+    packed = op.pack_scale_rot(_f32c(g["positions"]), _f32c(g["scales"]), _f32c(g["rotations"]), _f32c(g["alphas"]),
+                               _f32c(g["colors"]))
+    with pytest.raises(RuntimeError, match="status -2"):
+        op.forward_shared_lists(packed)
+    out, _ = op.forward(packed)
+    assert bool(torch.isfinite(out).all())
+
+
 def no_cull_ctx():
     from igs_amd._splat import library_options
 
