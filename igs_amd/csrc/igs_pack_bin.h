@@ -499,9 +499,9 @@ __global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin
     const float limit = a.limit[0];
     const float fraction = a.limit[1];
     // The image's lists are numbered by tile; with four lists per tile by rectangle, row after row of
-    // rectangles (rectangle l of the tile lies in row 4 ty + l): the numbering that a binning with one
-    // workgroup per rectangle gives (which then sets img_lists, rows of rectangles past the image's
-    // last having no workgroup).
+    // rectangles (rectangle l of the tile lies in row (4 / sub_nx) ty + l / sub_nx and column
+    // sub_nx tx + l % sub_nx): the numbering that a binning with one workgroup per rectangle gives
+    // (which then sets img_lists and row_lists, rectangles outside the image having no workgroup).
     const size_t img_first = (size_t)b * (a.img_lists > 0 ? a.img_lists : tiles * (masks ? 4 : 1));
     const int row_lists = a.row_lists > 0 ? a.row_lists : a.tiles_x * (masks ? a.sub_nx : 1);
     auto list_no = [&](int l) {
