@@ -84,8 +84,10 @@ def test_headline_all_sixteen_images_at_the_benchmarked_plan(dev):
     props = torch.cuda.get_device_properties(dev)
     if props.multi_processor_count == 256:
         # the plan bench.py's step runs on a full MI355X: Gaussians split 8 ways in the forward
-        # (combine kernel on), 4 column bands x 8 row bands in the backward
+        # (combine kernel on), 8 column bands x 8 row bands in the backward, whose tiles are the
+        # forward's wave rectangles: a step with gradients bins once for both passes
         assert (p.fwd_split, p.bwd_tiles, p.bwd_tiles_x, p.bwd_tile_w, p.bwd_per_tile) == (8, 64, 8, 32, 32)
+        assert p.lists_shared == 1
     assert p.fwd_split > 1
     _check_against_oracle("c1", dev, rows=8)
 
