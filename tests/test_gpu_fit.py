@@ -144,6 +144,30 @@ def test_graph_replay_equals_eager_fused_steps(igs, dev):
     assert graphed.step_count == 8
 
 
+def test_graph_capture_with_many_gaussians(igs, dev):
+    """With more than 49152 Gaussians the binning kernel asks for more dynamic LDS than a launch gets
+    by default and raises its limit at the first such launch on the device; here that launch is the
+    one being captured.  The replayed steps equal eager ones bit for bit."""
+    from igs_amd.fit import GaussianImageFit
+
+    B, N, H, W, C = 1, 60000, 64, 64, 3
+    g = torch.Generator().manual_seed(4)
+    block = torch.cat([torch.rand(B, N, 2, generator=g) * 2 - 1, torch.log(torch.rand(B, N, 2, generator=g) * 0.05 + 0.01),
+                       torch.rand(B, N, 1, generator=g), torch.zeros(B, N, 1), torch.rand(B, N, C, generator=g)], -1).to(dev)
+    xg, yg = grids(igs, B, H, W, dev)
+    target = O.smooth_noise_target(H, W, seed=3, C=C).to(dev)
+    eager = GaussianImageFit(block.clone(), target, xg, yg, lr=1e-3)
+    graphed = GaussianImageFit(block.clone(), target, xg, yg, lr=1e-3)
+    graphed.capture()
+    for k in range(3):
+        le = eager.step().clone()
+        lg = graphed.step().clone()
+        torch.cuda.synchronize()
+        assert torch.equal(le, lg), k
+        assert torch.equal(eager.params, graphed.params), k
+    assert float(le) > 0
+
+
 def test_prefix_of_gaussians_and_new_resolution(igs, dev):
     """num_active (scripts/2dgs_img_comp.py:107-111) and a change of target size (:208-217)."""
     from igs_amd.fit import GaussianImageFit
