@@ -216,7 +216,9 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     if (T > maxT) T = maxT;
     if (T < 1) T = 1;
     if (sep) {
-        p->bwd_per_tile = ceil_div(H, T);
+        // With as few bands as the row limit allows, whole bands of kBwdMaxRows rows and a shorter last
+        // one instead of equal ones: the tiles then are the forward's wave rectangles (lists_shared).
+        p->bwd_per_tile = T == ceil_div(H, kBwdMaxRows) ? (H < kBwdMaxRows ? H : kBwdMaxRows) : ceil_div(H, T);
     } else {
         p->bwd_per_tile = (ceil_div(p->hw_padded, T) + 255) & ~255;
     }
