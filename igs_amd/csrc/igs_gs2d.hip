@@ -481,11 +481,26 @@ int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, con
 inline int bwd_gen_groups(int N, int C) { return ceil_div(N, kThreads * bwd_gen_g(C)); }
 
 template <int C>
+// Most workgroups (with full lists) of a separable backward that runs one Gaussian per lane.
+#ifndef IGS_BWD_NARROW_WORKGROUPS
+#define IGS_BWD_NARROW_WORKGROUPS 8192
+#endif
 int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     if (sep) {
         // every list position up to Np is visited: listed Gaussians compute, the others store zeros
-        const dim3 grid(a.T, ceil_div(a.Np, kThreads * bwd_sep_g(C)), B);
-        hipLaunchKernelGGL((k_bwd_sep<C, bwd_sep_g(C)>), grid, dim3(kThreads), 0, st, a);
+        // Two Gaussians per lane where the launch is large; one where even full lists would give each
+        // compute unit only a few workgroups (the lists are usually far shorter than N, so such a launch
+        // runs in one wave of workgroups and its length is that of one workgroup: B=8 N=4096 256x256
+        // 0.406 -> 0.38 ms forward+backward, B=1 N=16384 512x512 0.473 -> 0.464; B=16 N=8192 2.88 -> 2.91 the other way).
+        constexpr int kG = bwd_sep_g(C);
+        const bool narrow = kG > 1 && (long)B * a.T * ceil_div(a.Np, kThreads * kG) <= IGS_BWD_NARROW_WORKGROUPS;
+        if (narrow) {
+            const dim3 grid(a.T, ceil_div(a.Np, kThreads), B);
+            hipLaunchKernelGGL((k_bwd_sep<C, 1>), grid, dim3(kThreads), 0, st, a);
+        } else {
+            const dim3 grid(a.T, ceil_div(a.Np, kThreads * kG), B);
+            hipLaunchKernelGGL((k_bwd_sep<C, kG>), grid, dim3(kThreads), 0, st, a);
+        }
     } else {
         const dim3 grid(bwd_gen_groups(a.N, C), a.T, B);
         if (a.grid_part != nullptr)
