@@ -337,7 +337,8 @@ def all_configs(steps: int, warmup: int) -> int:
     """Forward and forward+backward wall time of the five configurations through the public API
     (allocation included), pairs/s counting all B N H W pairs as scripts/profiling.py:199-211 does,
     and the fraction of the fp32 vector peak by the 42 + 6 C FLOP/pair model (above 1 is possible
-    where culling skips pairs).  The "fit step" rows are the graph-replayed fused iteration of
+    where culling skips pairs).  "c0 1 thread" is the c0 step under
+    torch.autograd.set_multithreading_enabled(False).  The "fit step" rows are the graph-replayed fused iteration of
     igs_amd.fit on the same problem: at c0 the public call is bound by the host's per-call cost
     (Python, torch allocation, autograd: 0.13-0.25 ms depending on the box), the replay is not."""
     import torch
@@ -404,6 +405,10 @@ def all_configs(steps: int, warmup: int) -> int:
                     v.grad = None
         n = max(3, steps // 3) if cfg == "c4" else steps
         rows.append((cfg, B, N, H, W, C, timeit(fwd, n), timeit(step, n)))
+        if cfg == "c0":   # the same public call with autograd's backward run on the calling thread: the hand-over to
+            # the engine's device thread and back is 60-130 us of the host's time per step on the boxes seen
+            with torch.autograd.set_multithreading_enabled(False):
+                rows.append((cfg + " 1 thread", B, N, H, W, C, float("nan"), timeit(step, n)))
         if cfg in ("c0", "c2"):   # the fused fit iteration (render, MSE, backward, AdamW) on the same problem,
             # replayed from a HIP graph: the step without the host's per-call cost
             block = torch.cat([d["positions"], d["scales"].log(), d["rotations"][..., None],

@@ -17,7 +17,7 @@ stream; every FLOP happens in libigs_hip.so.
 from __future__ import annotations
 
 import contextlib
-import ctypes
+import functools
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -71,18 +71,41 @@ def library_options(no_cull: bool = False, bin_levels: Optional[int] = None,
         _option_bits, _skip_tolerance = saved
 
 
+@functools.lru_cache(maxsize=256)
+def _skip_weight(N: int, eps: float, tolerance: float) -> Tuple[float, float]:
+    f = _lib.load().igs_gs2d_skip_weight
+    return float(f(N, eps, tolerance)), float(f(N, 1.0, tolerance))
+
+
 def skip_weight(N: int, eps: float) -> Tuple[float, float]:
     """(skip_weight, skip_fraction) the pack calls of a problem get under the current skip tolerance."""
-    f = _lib.load().igs_gs2d_skip_weight
-    return float(f(int(N), float(eps), float(_skip_tolerance))), float(f(int(N), 1.0, float(_skip_tolerance)))
+    return _skip_weight(int(N), float(eps), float(_skip_tolerance))
 
 
+# The host side of a call is what bounds small problems (a 512-Gaussian 256x256 forward+backward
+# is ~0.1 ms of kernels), so the per-call helpers below take the short routes: addresses and
+# streams travel as plain integers (the signatures convert them), the current stream comes from
+# torch's raw accessor, and the device is switched only when it is not the current one already.
 def _ptr(t: Optional[Tensor]):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    return None if t is None else t.data_ptr()
 
 
-def _stream(dev) -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+_no_guard = contextlib.nullcontext()
+
+
+def _stream(dev) -> int:
+    if _raw_stream is not None and dev.index is not None:
+        return _raw_stream(dev.index)
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _on(dev):
+    """Context in which `dev` is the current device."""
+    if _current_device is not None and dev.index is not None and _current_device() == dev.index:
+        return _no_guard
+    return torch.cuda.device(dev)
 
 
 def _f32c(t: Tensor) -> Tensor:
@@ -382,7 +405,7 @@ def run_forward(kind: int, params: Sequence[Tensor], x: Tensor, y: Tensor, eps: 
     B, N, C = problem_dims(kind, params)
     dev = params[0].device
     require_same_device(dev, list(params) + [x, y], "the forward")
-    with torch.cuda.device(dev):
+    with _on(dev):
         grid = Grid(x, y, B)
         op = Splat(B, N, C, grid, eps, dev)
         if kind == KIND_COVINV:
@@ -414,7 +437,7 @@ def run_backward(kind: int, op: Splat, keep, packed, col, out, den, grad_result:
     require_same_device(dev, [grad_result, packed, col, out, den, *keep], "the backward")
     g_x = g_y = None
     grads: List[Optional[Tensor]] = [None] * len(need)
-    with torch.cuda.device(dev):
+    with _on(dev):
         op.use_current_stream()
         go = op.pad_grad_out(grad_result)
         if (need_x or need_y) and any(need):
