@@ -1143,11 +1143,18 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     SuperSlots sup;
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
     if (rc) return rc;
-    IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<false, kFT>),
-                       (hipStream_t)stream, partial, T, mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), sup, (N + 3) & ~3, cov_inv_00,
-                       cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
-                       g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
+    const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
+    const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C, N);
+    if (sup.cslots != nullptr)
+        launch_finalize_listed<0>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C, cov_inv_00,
+                                               cov_inv_01, cov_inv_11, alphas, 0.0f, g_position, g_cov_inv_00,
+                                               g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors},
+                                  B, (hipStream_t)stream);
+    else
+        IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<false, kFT>),
+                           (hipStream_t)stream, partial, T, flag, T_alt, slots, (N + 3) & ~3, cov_inv_00,
+                           cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
+                           g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
     return launch_status();
 }
 
@@ -1163,11 +1170,18 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     SuperSlots sup;
     rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
     if (rc) return rc;
-    IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<true, kFT>),
-                       (hipStream_t)stream, partial, T, mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C, N), sup, (N + 3) & ~3, scales, rotations,
-                       (const float*)nullptr, alphas, N, C, eps, g_positions,
-                       g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
+    const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
+    const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C, N);
+    if (sup.cslots != nullptr)
+        launch_finalize_listed<1>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C, scales,
+                                               rotations, nullptr, alphas, eps, g_positions, g_scales, g_rotations,
+                                               nullptr, g_alphas, g_colors},
+                                  B, (hipStream_t)stream);
+    else
+        IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<true, kFT>),
+                           (hipStream_t)stream, partial, T, flag, T_alt, slots, (N + 3) & ~3, scales, rotations,
+                           (const float*)nullptr, alphas, N, C, eps, g_positions,
+                           g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
     return launch_status();
 }
 
@@ -1199,10 +1213,17 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
     SuperSlots sup;
     rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt, partial, &sup);
     if (rc) return rc;
-    IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize_feature<kFT>),
-                       (hipStream_t)stream, partial, T, mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr,
-                       T_alt, finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N), sup, (N + 3) & ~3, gs_feature,
-                       N, C, C_kernel, eps, g_feature);
+    const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
+    const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N);
+    if (sup.cslots != nullptr)
+        launch_finalize_listed<2>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C_kernel,
+                                               gs_feature, nullptr, nullptr, nullptr, eps, g_feature, nullptr, nullptr,
+                                               nullptr, nullptr, nullptr},
+                                  B, (hipStream_t)stream);
+    else
+        IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize_feature<kFT>),
+                           (hipStream_t)stream, partial, T, flag, T_alt, slots, (N + 3) & ~3, gs_feature,
+                           N, C, C_kernel, eps, g_feature);
     return launch_status();
 }
 

@@ -170,6 +170,35 @@ def test_two_level_binning_on_materialised_grids(igs, dev):
         assert torch.equal(grads_e[k], grads_m[k]), k
 
 
+def test_two_level_setting_on_a_general_grid(igs, dev):
+    """A stored grid that is not separable runs the general backward (dense partials, no slot
+    tables) whatever the binning setting; the finalize kernel of the two-level setting must then
+    read them as such.  Function level, operator level and the module head."""
+    B, N, H, W, C = 2, 900, 128, 256, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=19, smin=0.01, smax=0.1)
+    xg = (g["x_grid"] + 0.01 * torch.sin(7 * g["y_grid"])).contiguous()
+    yg = g["y_grid"].contiguous()
+    res = []
+    for lv in ("1", "2"):
+        with _Env("IGS_BIN_LEVELS", lv):
+            out, grads = run(igs, g, xg, yg)
+            pos = g["positions"].clone().requires_grad_(True)
+            torch.manual_seed(3)
+            cov = [torch.rand(B, N, 1, 1, device=dev).mul_(m).add_(a).requires_grad_(True)
+                   for m, a in ((300, 100), (40, -20), (300, 100))]   # positive definite forms
+            al, col = g["alphas"].clone().requires_grad_(True), g["colors"].clone().requires_grad_(True)
+            igs.GaussianSplatting2DKernel.apply(xg, yg, pos, *cov, al, col).backward(g["grad_out"])
+            torch.manual_seed(5)
+            m = igs.GaussianSplatting2D(8, 64).to(dev)
+            x = torch.randn(B, 100, 64, device=dev, requires_grad=True)
+            grid = torch.cat([yg, xg], dim=1)
+            m(x, grid=grid)[0].backward(g["grad_out"])
+            res.append((out, *grads.values(), pos.grad, *(c.grad for c in cov), al.grad, col.grad, x.grad))
+    for a, b in zip(*res):
+        assert float(a.abs().max()) > 0
+        assert float((a - b).double().norm()) <= 1e-5 * float(a.double().norm())
+
+
 def test_two_level_binning_against_oracle(igs, dev):
     """Long thin Gaussians (aspect ratios up to 40) under two levels against the fp64 oracle."""
     B, N, H, W, C = 1, 300, 256, 512, 3
