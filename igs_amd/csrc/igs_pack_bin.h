@@ -121,25 +121,44 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
     constexpr double k = -0.72134752044448170368;  // -0.5 * log2(e)
     const float al = alphas[i];
     const float px = position[2 * i], py = position[2 * i + 1];
-    r[0] = px;
-    r[1] = py;
-    r[2] = (float)(k * A);
-    r[3] = (float)(2.0 * k * Bc);
-    r[4] = (float)(k * D);
-    r[5] = al;
-    bool fin = isfinite(al) && isfinite(r[2]) && isfinite(r[3]) && isfinite(r[4]);
-    for (int c = 0; c < C; ++c) {
-        const float v = al * colors[i * C + c];
-        r[6 + c] = v;
-        fin = fin && isfinite(v) && isfinite(colors[i * C + c]);
+    // The record is put together in registers (every index below is a compile-time constant after
+    // unrolling) and stored as float4s: the colour loads are then in flight together and a lane
+    // writes RS / 4 times instead of RS times (C = 16, 131072 records: 39 -> 9 us).
+    float rec[kZeroRecFloats];
+#pragma unroll
+    for (int c = 0; c < kZeroRecFloats; ++c) rec[c] = 0.0f;
+    rec[0] = px;
+    rec[1] = py;
+    rec[2] = (float)(k * A);
+    rec[3] = (float)(2.0 * k * Bc);
+    rec[4] = (float)(k * D);
+    rec[5] = al;
+    bool fin = isfinite(al) && isfinite(rec[2]) && isfinite(rec[3]) && isfinite(rec[4]);
+    float col[IGS_MAX_CHANNELS];
+#pragma unroll
+    for (int c = 0; c < IGS_MAX_CHANNELS; ++c) col[c] = c < C ? colors[i * C + c] : 0.0f;
+#pragma unroll
+    for (int c = 0; c < IGS_MAX_CHANNELS; ++c) {
+        const float v = al * col[c];
+        if (c < C) {
+            rec[6 + c] = v;
+            fin = fin && isfinite(v) && isfinite(col[c]);
+        }
     }
-    for (int c = 6 + C; c < RS; ++c) r[c] = 0.0f;
     const float2 ext = reach_extent(px, py, sxx, syy, bounded && fin, skip_limit(limit, al));
-    write_bin_record(boxes, (size_t)b * Np + n, px, py, ext, r[2], r[3], r[4], al);
+    write_bin_record(boxes, (size_t)b * Np + n, px, py, ext, rec[2], rec[3], rec[4], al);
     if (RS >= 8 + C) {  // room in the record: the y range of the box travels with it
-        r[6 + C] = py - ext.y;
-        r[7 + C] = py + ext.y;
+#pragma unroll
+        for (int c = 6; c < kZeroRecFloats - 1; ++c)
+            if (c == 6 + C) {
+                rec[c] = py - ext.y;
+                rec[c + 1] = py + ext.y;
+            }
     }
+    float4* r4 = reinterpret_cast<float4*>(r);  // records are RS = 4 k floats apart behind a 16-byte aligned base
+#pragma unroll
+    for (int q = 0; q < kZeroRecFloats / 4; ++q)
+        if (4 * q < RS) r4[q] = make_float4(rec[4 * q], rec[4 * q + 1], rec[4 * q + 2], rec[4 * q + 3]);
 }
 
 // Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
