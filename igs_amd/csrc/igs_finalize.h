@@ -285,8 +285,40 @@ __device__ __forceinline__ unsigned int group_ballot(bool p) {
     return kFinGroup == 32 ? (unsigned int)m : (unsigned int)m & ((1u << (kFinGroup % 32)) - 1u);
 }
 
-// Lane `lane` of a group: the sums of fields lane, lane + kFinGroup, .. over the records of
-// Gaussian n.  Group-uniform control flow; the other groups of the wave may be elsewhere.
+// Lane `lane` of a group adds, to its sums of fields lane, lane + kFinGroup, .., the records of
+// Gaussian n in up to kFinGroup tiles: this lane's tile is `t` (`in`: it exists), in ascending lane
+// order.  Group-uniform control flow; the other groups of the wave may be elsewhere.
+__device__ __forceinline__ void group_add_tiles(const float* __restrict__ part, const int* __restrict__ slots,
+                                                int Np, int N, int NF, int n, int lane, int t, bool in,
+                                                float (&acc)[kFinGroupFields]) {
+    const int col = in ? slots[(size_t)t * Np + n] : -1;
+    unsigned int tm = group_ballot(col >= 0);
+    // where this lane's tile keeps the Gaussian's record (in floats; the lanes that read it fetch the two halves)
+    const unsigned long long at = ((unsigned long long)t * N + max(col, 0)) * NF;
+    const int at_lo = (int)(unsigned int)at, at_hi = (int)(at >> 32);
+    while (tm) {
+        float val[kFinGroupAhead][kFinGroupFields];
+#pragma unroll
+        for (int u = 0; u < kFinGroupAhead; ++u) {
+            const bool have = tm != 0u;
+            const int src = have ? __builtin_ctz(tm) : 0;
+            tm &= tm - 1u;  // (0 stays 0)
+            const unsigned int lo = (unsigned int)__shfl(at_lo, src, kFinGroup);
+            const unsigned int hi = (unsigned int)__shfl(at_hi, src, kFinGroup);
+            const float* rec = part + (((unsigned long long)hi << 32) | lo);
+#pragma unroll
+            for (int v = 0; v < kFinGroupFields; ++v)
+                val[u][v] = (have && lane + v * kFinGroup < NF) ? rec[lane + v * kFinGroup] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kFinGroupAhead; ++u)
+#pragma unroll
+            for (int v = 0; v < kFinGroupFields; ++v) acc[v] += val[u][v];
+    }
+}
+
+// All records of Gaussian n after a two-level binning: the listed super-tiles in ascending order,
+// the tiles of each row-major.
 __device__ __forceinline__ void group_sum_listed(const float* __restrict__ part, const int* __restrict__ slots,
                                                  const SuperSlots sup, int Np, int N, int NF, int n, int lane,
                                                  float (&acc)[kFinGroupFields]) {
@@ -297,38 +329,22 @@ __device__ __forceinline__ void group_sum_listed(const float* __restrict__ part,
             const int st = s0 + __builtin_ctz(sm);
             sm &= sm - 1;
             const int sy = st / sup.stiles_x, sx = st - sy * sup.stiles_x;
-            for (int j0 = 0; j0 < kSuperX * kSuperY; j0 += kFinGroup) {  // the super-tile's tiles, row-major
+            for (int j0 = 0; j0 < kSuperX * kSuperY; j0 += kFinGroup) {
                 const int j = j0 + lane;
                 const int ty = sy * kSuperY + j / kSuperX, tx = sx * kSuperX + j % kSuperX;
-                const bool in = j < kSuperX * kSuperY && ty < sup.tiles_y && tx < sup.tiles_x;
-                const int t = ty * sup.tiles_x + tx;
-                const int col = in ? slots[(size_t)t * Np + n] : -1;
-                unsigned int tm = group_ballot(col >= 0);
-                // where this lane's tile keeps the Gaussian's record (in floats; the lanes that read it fetch the two halves)
-                const unsigned long long at = ((unsigned long long)t * N + max(col, 0)) * NF;
-                const int at_lo = (int)(unsigned int)at, at_hi = (int)(at >> 32);
-                while (tm) {
-                    float val[kFinGroupAhead][kFinGroupFields];
-#pragma unroll
-                    for (int u = 0; u < kFinGroupAhead; ++u) {
-                        const bool have = tm != 0u;
-                        const int src = have ? __builtin_ctz(tm) : 0;
-                        tm &= tm - 1u;  // (0 stays 0)
-                        const unsigned int lo = (unsigned int)__shfl(at_lo, src, kFinGroup);
-                        const unsigned int hi = (unsigned int)__shfl(at_hi, src, kFinGroup);
-                        const float* rec = part + (((unsigned long long)hi << 32) | lo);
-#pragma unroll
-                        for (int v = 0; v < kFinGroupFields; ++v)
-                            val[u][v] = (have && lane + v * kFinGroup < NF) ? rec[lane + v * kFinGroup] : 0.0f;
-                    }
-#pragma unroll
-                    for (int u = 0; u < kFinGroupAhead; ++u)
-#pragma unroll
-                        for (int v = 0; v < kFinGroupFields; ++v) acc[v] += val[u][v];
-                }
+                group_add_tiles(part, slots, Np, N, NF, n, lane, ty * sup.tiles_x + tx,
+                                j < kSuperX * kSuperY && ty < sup.tiles_y && tx < sup.tiles_x, acc);
             }
         }
     }
+}
+
+// After a one-level binning: the T tiles in ascending order.
+__device__ __forceinline__ void group_sum_tiles(const float* __restrict__ part, const int* __restrict__ slots,
+                                                int T, int Np, int N, int NF, int n, int lane,
+                                                float (&acc)[kFinGroupFields]) {
+    for (int t0 = 0; t0 < T; t0 += kFinGroup)
+        group_add_tiles(part, slots, Np, N, NF, n, lane, t0 + lane, t0 + lane < T, acc);
 }
 
 // The same over the dense partials of the general backward (every tile holds column n).
@@ -357,13 +373,13 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_listed(const Finalize
     static_assert(kFinGroupBatch % kGroups == 0, "every group takes the same number of Gaussians");
     const int lane = threadIdx.x % kFinGroup, group = threadIdx.x / kFinGroup;
     const int b = blockIdx.y, n0 = blockIdx.x * kFinGroupBatch;
-    const bool general = a.flag != nullptr && *a.flag == 0;
+    const bool general = a.slots == nullptr || (a.flag != nullptr && *a.flag == 0);
     const int T = general ? a.T_alt : a.T;
     const int NF = 6 + a.Cp;
     const float* part = a.partial + (size_t)b * T * NF * a.N;
-    const int* slots = a.slots + (size_t)b * a.T * a.Np;
+    const int* slots = a.slots != nullptr ? a.slots + (size_t)b * a.T * a.Np : nullptr;
     SuperSlots sup = a.sup;
-    sup.cslots += (size_t)b * sup.stiles * a.Np;
+    if (sup.cslots != nullptr) sup.cslots += (size_t)b * sup.stiles * a.Np;
     for (int k = 0; k < kFinGroupBatch / kGroups; ++k) {
         const int ln = k * kGroups + group;  // the groups work on neighbouring Gaussians at any time
         const int n = n0 + ln;
@@ -373,8 +389,10 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_listed(const Finalize
         for (int v = 0; v < kFinGroupFields; ++v) acc[v] = 0.0f;
         if (general)
             group_sum_dense(part, T, a.N, NF, n, lane, acc);
-        else
+        else if (a.sup.cslots != nullptr)
             group_sum_listed(part, slots, sup, a.Np, a.N, NF, n, lane, acc);
+        else
+            group_sum_tiles(part, slots, T, a.Np, a.N, NF, n, lane, acc);
         const size_t i = (size_t)b * a.N + n;
 #pragma unroll
         for (int v = 0; v < kFinGroupFields; ++v) {

@@ -1093,6 +1093,20 @@ int igs_gs2d_backward_grid(const float* packed, const float* x, const float* y,
         }                                                                                           \
     } while (0)
 
+// Which finalize kernel: a group of lanes per Gaussian (k_bwd_finalize_listed) after a two-level
+// binning and wherever the Gaussians alone fill the device; else t-lanes x Gaussians
+// (k_bwd_finalize*), which also spreads the tiles of a Gaussian over lanes.
+#ifndef IGS_FIN_GROUPS_FROM
+#define IGS_FIN_GROUPS_FROM 65536L
+#endif
+#ifndef IGS_FIN_GROUPS_MAX_TILES
+#define IGS_FIN_GROUPS_MAX_TILES 128
+#endif
+static bool finalize_by_groups(const SuperSlots& sup, int B, int N, int T) {
+    if (sup.cslots != nullptr) return true;
+    return (long)B * N >= IGS_FIN_GROUPS_FROM && T <= IGS_FIN_GROUPS_MAX_TILES;
+}
+
 // The slot tables that the separable backward left behind the partial sums (none on general grids).
 static const int* finalize_slots(const float* partial, int grid_mode, int B, int T, int NF, int N) {
     if (mode_of(grid_mode) == IGS_GRID_GENERAL) return nullptr;
@@ -1145,7 +1159,7 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
     const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C, N);
-    if (sup.cslots != nullptr)
+    if (finalize_by_groups(sup, B, N, T))
         launch_finalize_listed<0>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C, cov_inv_00,
                                                cov_inv_01, cov_inv_11, alphas, 0.0f, g_position, g_cov_inv_00,
                                                g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors},
@@ -1172,7 +1186,7 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
     const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C, N);
-    if (sup.cslots != nullptr)
+    if (finalize_by_groups(sup, B, N, T))
         launch_finalize_listed<1>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C, scales,
                                                rotations, nullptr, alphas, eps, g_positions, g_scales, g_rotations,
                                                nullptr, g_alphas, g_colors},
@@ -1215,7 +1229,7 @@ int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
     const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N);
-    if (sup.cslots != nullptr)
+    if (finalize_by_groups(sup, B, N, T))
         launch_finalize_listed<2>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C_kernel,
                                                gs_feature, nullptr, nullptr, nullptr, eps, g_feature, nullptr, nullptr,
                                                nullptr, nullptr, nullptr},
