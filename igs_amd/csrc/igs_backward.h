@@ -204,6 +204,9 @@ constexpr int kBwdTileW = IGS_BWD_TILE_W;
 // totals once per row.  A lane's sums are stored at its list position (coalesced); the finalize
 // kernel finds them through the tile's slot table and takes 0 for unlisted Gaussians, so tiles
 // that a Gaussian does not reach cost neither compute nor memory traffic.
+#ifndef IGS_BWD_TILE_SHIFT
+#define IGS_BWD_TILE_SHIFT 1
+#endif
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     constexpr int CP = pix_stride_sep(C), CP4 = CP / 4;
@@ -217,12 +220,18 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     __shared__ float4 xsh[kBwdTileW / 4];
     __shared__ float ysh[2][RPC + 1];  // row coordinates of the chunk (+1: read-ahead slot)
     IGS_GATE(a);
-    // tiles are the fastest grid dimension: consecutive workgroups (dealt round-robin to the
-    // XCDs) then belong to different tiles, and the list-position groups that have work (the
-    // low ones) are spread over all XCDs
-    const int b = blockIdx.z, t = blockIdx.x, grp = blockIdx.y;
+    // Tiles are the fastest grid dimension: consecutive workgroups (dealt round-robin to the
+    // XCDs, which do not share work afterwards) then belong to different tiles, and the
+    // list-position groups that have work (the low ones) are spread over all XCDs.  The tile of a
+    // workgroup is shifted along its row by the row number and the image: with 8 tiles per row an
+    // XCD would otherwise own one tile column of every image, and the columns differ in work (at
+    // the image's border the lists are shorter; a module at its initialisation puts all Gaussians
+    // near the centre).  An XCD now gets one tile of every row and column of an image.
+    const int b = blockIdx.z, grp = blockIdx.y;
     const int tid = threadIdx.x;
-    const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
+    const int ty = blockIdx.x / a.tiles_x;
+    const int tx = (blockIdx.x - ty * a.tiles_x + ty * IGS_BWD_TILE_SHIFT + b * IGS_BWD_TILE_SHIFT) % a.tiles_x;
+    const int t = ty * a.tiles_x + tx;
     const int count = a.counts[(size_t)b * a.T + t];
     if (grp * G * kThreads >= count) return;  // workgroup-uniform: no listed Gaussian left
     const int* list = a.lists + ((size_t)b * a.T + t) * a.Np;
