@@ -316,17 +316,27 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 // kWave = true (fwd_wave_lists): every wave has a list of its own and streams it independently of
 // the others (no barrier in the kernel); the four waves of a workgroup are the rectangles of one
 // 64 x 4P tile of the binning.
+#ifndef IGS_FWD_ONE_WAVE
+#define IGS_FWD_ONE_WAVE 1
+#endif
+constexpr bool kFwdOneWave = IGS_FWD_ONE_WAVE != 0;
 template <int C, int P, bool kWave>
 __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     constexpr int RS = rec_stride_of(C), R4 = RS / 4;
     IGS_GATE(a);
-    const int tile = xcd_contiguous(blockIdx.x, a.total_tiles);
+    // Waves with lists of their own are launched as workgroups of one wave (kFwdOneWave): the
+    // four waves of a tile share nothing, and a wave slot then frees as soon as its wave ends
+    // instead of when the longest list of the four does.  Workgroup q: XCD q % 8, there tile
+    // (q / 8) / 4 of the XCD's range and wave rectangle (q / 8) % 4 of that tile.
+    constexpr bool kOne = kWave && kFwdOneWave;
+    const int q = kOne ? (int)(blockIdx.x & 7) + 8 * (int)(blockIdx.x >> 5) : (int)blockIdx.x;
+    const int tile = xcd_contiguous(q, a.total_tiles);
     if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int per_img = a.tiles_x * a.tiles_y;
     const int b = tile / per_img;
     const int tl = tile - b * per_img;
     const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
-    const int wave = threadIdx.x >> 6;
+    const int wave = kOne ? (int)((blockIdx.x >> 3) & 3) : (int)(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     // A wave with a list of its own covers kWaveCols columns x (64 / kWaveCols) P rows: lane l has
     // column l % kWaveCols and the P rows of row block l / kWaveCols; the tile of four waves is 64
@@ -413,10 +423,10 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     // for tiles that fewer than 7/8 of the Gaussians reach (workgroup-uniform choice of the loop):
     // there some boxes are small against the image, and those are often small against the tile too.
     if constexpr (kWave) {
-        __shared__ float4 sh0[4][kGaussChunk * R4];  // per wave: the two chunk buffers
-        __shared__ float4 sh1[4][kGaussChunk * R4];
+        __shared__ float4 sh0[kOne ? 1 : 4][kGaussChunk * R4];  // per wave: the two chunk buffers
+        __shared__ float4 sh1[kOne ? 1 : 4][kGaussChunk * R4];
         stream_records_dma<R4, kGaussChunk>(
-            src, reinterpret_cast<const float4*>(a.zero_rec), n1 - n0, sh0[wave], sh1[wave],
+            src, reinterpret_cast<const float4*>(a.zero_rec), n1 - n0, sh0[kOne ? 0 : wave], sh1[kOne ? 0 : wave],
             [&](const float4* r) { body(std::false_type{}, r); }, list);
     } else {
         __shared__ float4 sh[2 * kGaussChunk * R4];

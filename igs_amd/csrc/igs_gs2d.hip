@@ -446,7 +446,10 @@ struct MseArgs {
 template <int C>
 int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
     const dim3 grid(((a.total_tiles + 7) / 8) * 8, a.S, 1);
-    if (sep)
+    if (sep && fwd_wave_lists(C) && kFwdOneWave)  // one wave per workgroup: four workgroups per tile
+        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), fwd_wave_lists(C)>), dim3(grid.x * 4, grid.y, 1), dim3(64), 0,
+                           st, a);
+    else if (sep)
         hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), fwd_wave_lists(C)>), grid, dim3(kThreads), 0, st, a);
     else
         hipLaunchKernelGGL((k_fwd_gen<C, fwd_gen_p(C)>), grid, dim3(kThreads), 0, st, a);
