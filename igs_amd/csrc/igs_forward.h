@@ -316,19 +316,16 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 // kWave = true (fwd_wave_lists): every wave has a list of its own and streams it independently of
 // the others (no barrier in the kernel); the four waves of a workgroup are the rectangles of one
 // 64 x 4P tile of the binning.
-#ifndef IGS_FWD_ONE_WAVE
-#define IGS_FWD_ONE_WAVE 1
-#endif
-constexpr bool kFwdOneWave = IGS_FWD_ONE_WAVE != 0;
-template <int C, int P, bool kWave>
+// (kOne: launched as workgroups of one wave; only with kWave)
+template <int C, int P, bool kWave, bool kOne = false>
 __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
+    static_assert(kWave || !kOne, "one-wave workgroups need a list per wave");
     constexpr int RS = rec_stride_of(C), R4 = RS / 4;
     IGS_GATE(a);
-    // Waves with lists of their own are launched as workgroups of one wave (kFwdOneWave): the
-    // four waves of a tile share nothing, and a wave slot then frees as soon as its wave ends
-    // instead of when the longest list of the four does.  Workgroup q: XCD q % 8, there tile
-    // (q / 8) / 4 of the XCD's range and wave rectangle (q / 8) % 4 of that tile.
-    constexpr bool kOne = kWave && kFwdOneWave;
+    // Waves with lists of their own can be launched as workgroups of one wave (kOne): the four
+    // waves of a tile share nothing, and a wave slot then frees as soon as its wave ends instead
+    // of when the longest list of the four does.  Workgroup q: XCD q % 8, there tile (q / 8) / 4
+    // of the XCD's range and wave rectangle (q / 8) % 4 of that tile.
     const int q = kOne ? (int)(blockIdx.x & 7) + 8 * (int)(blockIdx.x >> 5) : (int)blockIdx.x;
     const int tile = xcd_contiguous(q, a.total_tiles);
     if (tile >= a.total_tiles) return;  // workgroup-uniform

@@ -443,12 +443,19 @@ struct MseArgs {
     float* loss = nullptr;          // 1 float
 };
 
+#ifndef IGS_FWD_ONE_WAVE_FROM
+#define IGS_FWD_ONE_WAVE_FROM 512
+#endif
 template <int C>
 int launch_forward(const FwdArgs& a, bool sep, hipStream_t st) {
     const dim3 grid(((a.total_tiles + 7) / 8) * 8, a.S, 1);
-    if (sep && fwd_wave_lists(C) && kFwdOneWave)  // one wave per workgroup: four workgroups per tile
-        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), fwd_wave_lists(C)>), dim3(grid.x * 4, grid.y, 1), dim3(64), 0,
-                           st, a);
+    // Long list parts (c1: 1024 Gaussians per part and list) run as workgroups of one wave, four per
+    // tile: c1 forward 1.10 -> 1.00 ms.  With short parts the four times as many workgroups cost
+    // more than the earlier release of the wave slots gives (c3, 256 per part: +1.4 % of the step;
+    // c0, 64: +3.5 %); at 512 (c2) it is even.
+    if (sep && fwd_wave_lists(C) && a.Np / a.S >= IGS_FWD_ONE_WAVE_FROM)
+        hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), fwd_wave_lists(C), fwd_wave_lists(C)>),
+                           dim3(grid.x * 4, grid.y, 1), dim3(64), 0, st, a);
     else if (sep)
         hipLaunchKernelGGL((k_fwd_sep<C, fwd_sep_p(C), fwd_wave_lists(C)>), grid, dim3(kThreads), 0, st, a);
     else
