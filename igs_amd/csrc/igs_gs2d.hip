@@ -490,20 +490,18 @@ int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, con
 // grid gradients).
 inline int bwd_gen_groups(int N, int C) { return ceil_div(N, kThreads * bwd_gen_g(C)); }
 
+// Separable backward: every list position up to Np is visited; listed Gaussians compute, the others
+// store zeros.  One Gaussian per lane (k_bwd_sep<C,1>) unless the lists are full by construction
+// (`dense`: IGS_OPT_NO_CULL): a tile's last list-position group is half empty on average, which costs
+// half as many idle lanes with groups of 256 as of 512 entries (c1, lists of ~4200: 3.5 % against 8.9 %),
+// more than the second Gaussian per lane saves by sharing the pixel records' LDS reads (16.3 against
+// 16.0 instructions per pair).  Step times with one / two per lane: c1 2.62 / 2.66 ms, c2 and c3 -2 to
+// -6 % with one; with only exact zeros skipped (lists 86 % full) equal; everything listed 4.67 / 4.62 ms.
 template <int C>
-// Most workgroups (with full lists) of a separable backward that runs one Gaussian per lane.
-#ifndef IGS_BWD_NARROW_WORKGROUPS
-#define IGS_BWD_NARROW_WORKGROUPS 8192
-#endif
-int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
+int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, bool dense, hipStream_t st) {
     if (sep) {
-        // every list position up to Np is visited: listed Gaussians compute, the others store zeros
-        // Two Gaussians per lane where the launch is large; one where even full lists would give each
-        // compute unit only a few workgroups (the lists are usually far shorter than N, so such a launch
-        // runs in one wave of workgroups and its length is that of one workgroup: B=8 N=4096 256x256
-        // 0.406 -> 0.38 ms forward+backward, B=1 N=16384 512x512 0.473 -> 0.464; B=16 N=8192 2.88 -> 2.91 the other way).
         constexpr int kG = bwd_sep_g(C);
-        const bool narrow = kG > 1 && (long)B * a.T * ceil_div(a.Np, kThreads * kG) <= IGS_BWD_NARROW_WORKGROUPS;
+        const bool narrow = kG == 1 || !dense;
         if (narrow) {
             const dim3 grid(a.T, ceil_div(a.Np, kThreads), B);
             hipLaunchKernelGGL((k_bwd_sep<C, 1>), grid, dim3(kThreads), 0, st, a);
@@ -1008,7 +1006,7 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
             if (rc) return rc;
         }
         if (gg.g_x != nullptr && !sep) a.grid_part = reinterpret_cast<float2*>(gg.ws);
-        IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, st));
+        IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0, st));
         if (rc) return rc;
         if (gg.g_x == nullptr) continue;
         if (sep) {  // the pixel-major kernel of its own
