@@ -33,7 +33,7 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 # (factors from the plain-copy calibration of the same profile run).
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
-    "bwd": {"fma": 7.927e8, "mul": 1.519e8, "add": 8.709e7, "trans": 7.152e7, "fetch_kib": 49830, "write_kib": 173100},
+    "bwd": {"fma": 7.643e8, "mul": 1.465e8, "add": 8.396e7, "trans": 6.902e7, "fetch_kib": 54010, "write_kib": 201500},
     "fwd": {"fma": 4.182e8, "mul": 1.316e7, "add": 7.403e7, "trans": 6.971e7, "fetch_kib": 11920, "write_kib": 131100},
 }
 
@@ -292,7 +292,7 @@ def run(args) -> int:
                                               / FP32_VECTOR_PEAK_TFLOPS,
         "roofline": {
             "bound": "valu",
-            "kernel": f"k_bwd_sep<{C},2> (backward per-Gaussian reduction)",
+            "kernel": f"k_bwd_sep<{C},1> (backward per-Gaussian reduction)",
             "achieved": achieved,
             "peak": FP32_VECTOR_PEAK_TFLOPS,
             "unit": "TFLOP/s",
