@@ -205,7 +205,7 @@ constexpr int kBwdTileW = IGS_BWD_TILE_W;
 // kernel finds them through the tile's slot table and takes 0 for unlisted Gaussians, so tiles
 // that a Gaussian does not reach cost neither compute nor memory traffic.
 #ifndef IGS_BWD_TILE_SHIFT
-#define IGS_BWD_TILE_SHIFT 1
+#define IGS_BWD_TILE_SHIFT 5   // tiles per row and per image; odd, so that 8 or 16 tiles per row cycle through all columns (1 / 3 / 5 timed: c2 0.456 / 0.448 / 0.449 ms, c1 and c3 equal)
 #endif
 template <int C, int G>
 __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     // Tiles are the fastest grid dimension: consecutive workgroups (dealt round-robin to the
     // XCDs, which do not share work afterwards) then belong to different tiles, and the
     // list-position groups that have work (the low ones) are spread over all XCDs.  The tile of a
-    // workgroup is shifted along its row by the row number and the image: with 8 tiles per row an
+    // workgroup is shifted along its row by a few tiles per row and image: with 8 tiles per row an
     // XCD would otherwise own one tile column of every image, and the columns differ in work (at
     // the image's border the lists are shorter; a module at its initialisation puts all Gaussians
     // near the centre).  An XCD now gets one tile of every row and column of an image.
