@@ -85,23 +85,12 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
-    ap.add_argument("--issue-rates", action="store_true",
-                    help="instead of the JSON line, run the stand-alone microbenchmark of a SIMD's instruction issue "
-                         "rates (igs_amd/csrc/ubench/issue_rates.hip, built by __graft_entry__.build()) and print "
-                         "its table")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over the batch with no "
               "exchange; no multi-GPU run is part of it). Use --gpus 1.", file=sys.stderr)
         return 2
 
-    if args.issue_rates:
-        import subprocess
-        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "igs_amd", "igs_issue_rates")
-        if not os.path.exists(exe):
-            print("bench.py: %s is not built (python -m igs_amd.build)" % exe, file=sys.stderr)
-            return 1
-        return subprocess.run([exe]).returncode
     # what the separable kernels may skip, for every mode below (explicit arguments of each library call)
     from igs_amd._splat import library_options
     with library_options(no_cull=args.no_cull, skip_tolerance=args.skip_tolerance):

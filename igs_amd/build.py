@@ -13,9 +13,6 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
 SOURCES = [os.path.join(PKG, "csrc", "igs_gs2d.hip")]
 LIB = os.path.join(PKG, "libigs_hip.so")
-# stand-alone microbenchmark of a SIMD's instruction issue rates (run by `bench.py --issue-rates`)
-UBENCH_SOURCE = os.path.join(PKG, "csrc", "ubench", "issue_rates.hip")
-UBENCH = os.path.join(PKG, "igs_issue_rates")
 
 # Packed-fp32 instruction selection is switched off for all device code.
 HIPCC_FLAGS = [
@@ -35,11 +32,6 @@ HIPCC_FLAGS = [
 def build(verbose: bool = True, extra=()) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc, *HIPCC_FLAGS, *extra, "-o", LIB, *SOURCES]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
-    cmd = [hipcc, "-O3", "-std=c++17", "--offload-arch=gfx950",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", UBENCH, UBENCH_SOURCE]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
