@@ -141,9 +141,12 @@ def round_up(v, m):
 
 def packed_numel(B, N, Cp):
     """float32 elements of the packed buffer: per image roundup4(N) records of roundup4(6+Cp)
-    floats plus an 8-float bin record each, then 4 floats for the skip settings and a zero record of 28 (the `packed_bytes`
-    of igs_gs2d_plan, restated so that shape inference under torch.compile needs no library call)."""
-    return B * round_up(N, 4) * (round_up(6 + Cp, 4) + 8) + 32
+    floats plus an 8-float bin record each, the separable kernels' forward records (roundup4(10+Cp); none for
+    more than 8 channels) and backward records (4), then 4 floats for the skip settings and a zero record of
+    28 (the `packed_bytes` of igs_gs2d_plan, restated so that shape inference under torch.compile needs no
+    library call)."""
+    sep = (round_up(10 + Cp, 4) if Cp <= 8 else 0) + 4
+    return B * round_up(N, 4) * (round_up(6 + Cp, 4) + 8 + sep) + 32
 
 
 class Grid:

@@ -130,6 +130,7 @@ struct BwdArgs {
     int tiles_x;   // separable: column bands of kBwdTileW columns
     const int* counts;  // separable: Gaussians listed per tile [B][T]
     const int* lists;   // separable: list + complement [B][T][Np]
+    const float4* brecs;  // separable: the backward records of the packed buffer [B][Np] (sA, skA, D'', tag)
     float* partial;  // [B][T][N][6+C]
     float2* grid_part;  // general grids with grid gradients: [B][groups][HWp] sums of G w (t1, t2)
     const int* flag;
@@ -195,29 +196,40 @@ constexpr int kBwdMinRows = IGS_BWD_MIN_ROWS;
 #endif
 constexpr int kBwdTileW = IGS_BWD_TILE_W;
 
-// Separable grid: lane = G Gaussians taken from the tile's list (those whose reach box meets
+// Separable grid: lane = one Gaussian taken from the tile's list (those whose reach box meets
 // the tile; the others are known to get exactly zero from it); the tile is kBwdTileW columns x
 // per_tile rows.  Its pixel records stream through LDS in chunks of whole tile rows
 // (double-buffered) and are read with broadcast ds_read_b128; the tile's column coordinates sit
-// in LDS for the whole kernel.  Per row the dy part of q is hoisted, and row sums
-// R0 = sum G e, R1 = sum G e dx, R2 = sum G e dx^2 (and the colour sums) are folded into the
-// totals once per row.  A lane's sums are stored at its list position (coalesced); the finalize
-// kernel finds them through the tile's slot table and takes 0 for unlisted Gaussians, so tiles
-// that a Gaussian does not reach cost neither compute nor memory traffic.
+// in LDS for the whole kernel.  A lane's sums are stored at its list position (coalesced); the
+// finalize kernel finds them through the tile's slot table and takes 0 for unlisted Gaussians, so
+// tiles that a Gaussian does not reach cost neither compute nor memory traffic.
+//
+// Exponent with the square completed along the row (write_sep_records):
+//   q' = -(sA dx + skA dy)^2 + D'' dy^2 = -u^2 + cyy,   u = sA x' + (skA dy - sA px')
+// with x', px' relative to the tile's middle column, so that the hoisted row term carries no more
+// rounding than u itself.  Per pair: u (fma), u^2, cyy - u^2, exp2, G = <g^, c> - s (C fma), G e, and
+// the sums of G e {1, u, u^2} and e g^_c: 9 + 2 C instructions and one exponential.  Per row the
+// sums of G e {1, u} are folded with dy into the totals of G e {1, u, dy, u dy, dy^2}; at the end the
+// moments in (u, dy) become those in (dx, dy) (dx = (u - skA dy) / sA).  Lanes whose Gaussian has no
+// completed square (tag of the backward record: a form that is not positive definite, non-finite
+// values) evaluate q' = (A' dx + B2' dy) dx + D' dy^2 term by term instead; what a Gaussian's sums are
+// depends on the Gaussian only, not on which lanes share its wave.
 #ifndef IGS_BWD_TILE_SHIFT
 #define IGS_BWD_TILE_SHIFT 5   // tiles per row and per image; odd, so that 8 or 16 tiles per row cycle through all columns (1 / 3 / 5 timed: c2 0.456 / 0.448 / 0.449 ms, c1 and c3 equal)
 #endif
-template <int C, int G>
-__global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
+template <int C>
+__global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdArgs a) {  // (C = 16: four waves per SIMD, i.e. at most 128 registers)
     constexpr int CP = pix_stride_sep(C), CP4 = CP / 4;
     constexpr int PX = pix_chunk(C) > kBwdTileW ? pix_chunk(C) : kBwdTileW;
     constexpr int RPC = PX / kBwdTileW;          // tile rows per chunk
     constexpr int ROW4 = kBwdTileW * CP4;        // float4 per tile row
     constexpr int E = RPC * ROW4;                // float4 per chunk
     constexpr int PRE = (E + kThreads - 1) / kThreads;
+    constexpr int RS = rec_stride_of(C);
     static_assert(PX % kBwdTileW == 0 && RPC >= 1, "chunk must hold whole tile rows");
     __shared__ float4 sh[2 * E];
-    __shared__ float4 xsh[kBwdTileW / 4];
+    __shared__ float4 xsh[kBwdTileW / 4];   // column coordinates of the tile
+    __shared__ float4 xloc[kBwdTileW / 4];  // the same relative to the tile's middle column
     __shared__ float ysh[2][RPC + 1];  // row coordinates of the chunk (+1: read-ahead slot)
     IGS_GATE(a);
     // Tiles are the fastest grid dimension: consecutive workgroups (dealt round-robin to the
@@ -233,33 +245,36 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     const int tx = (blockIdx.x - ty * a.tiles_x + ty * IGS_BWD_TILE_SHIFT + b * IGS_BWD_TILE_SHIFT) % a.tiles_x;
     const int t = ty * a.tiles_x + tx;
     const int count = a.counts[(size_t)b * a.T + t];
-    if (grp * G * kThreads >= count) return;  // workgroup-uniform: no listed Gaussian left
+    if (grp * kThreads >= count) return;  // workgroup-uniform: no listed Gaussian left
     const int* list = a.lists + ((size_t)b * a.T + t) * a.Np;
-    int n[G], slot[G];
+    const int pos = grp * kThreads + tid;
+    const int n = pos < count ? list[pos] : a.N;  // >= N: an unused lane (nothing is stored for it)
+    const int nc = min(n, a.N - 1);
+    const float* rec = a.packed + ((size_t)b * a.Np + nc) * RS;
+    const float4 br = a.brecs[(size_t)b * a.Np + nc];
+    const float px = rec[0], py = rec[1];
+    const float rA = rec[2], rB2 = rec[3], rD = rec[4];
+    float col[C];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const int pos = (grp * G + g) * kThreads + tid;
-        n[g] = pos < count ? list[pos] : a.N;
-        slot[g] = pos < count ? pos : a.N;
-    }
-    float M[G][6], CG[G][C];
+    for (int c = 0; c < C; ++c) col[c] = a.colors[((size_t)b * a.N + nc) * C + c];
+    // regular lanes: sums of G e {1, u, dy, u^2, u dy, dy^2}; the others: of G e {1, dx, dy, dx^2, dx dy, dy^2}
+    float M[6], CG[C];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
+    for (int f = 0; f < 6; ++f) M[f] = 0.0f;
 #pragma unroll
-        for (int f = 0; f < 6; ++f) M[g][f] = 0.0f;
-#pragma unroll
-        for (int c = 0; c < C; ++c) CG[g][c] = 0.0f;
-    }
-    float px[G], py[G], A[G], B2[G], D[G], col[G][C];
-    bwd_load_gaussians<C, G>(a, b, n, px, py, A, B2, D, col);
+    for (int c = 0; c < C; ++c) CG[c] = 0.0f;
 
     const int c0 = tx * kBwdTileW;
     const int cw = min(a.Wp, c0 + kBwdTileW) - c0;  // columns of this tile, a multiple of 8
     const int r0 = ty * a.per_tile, r1 = min(a.H, r0 + a.per_tile);
     const int chunks = (r1 - r0 + RPC - 1) / RPC;
     const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    if (tid < kBwdTileW / 4)
-        xsh[tid] = 4 * tid < cw ? reinterpret_cast<const float4*>(a.xs + (size_t)b * a.Wp + c0)[tid] : zero;
+    const float xc = a.xs[(size_t)b * a.Wp + c0 + (cw >> 1)];
+    if (tid < kBwdTileW / 4) {
+        const float4 v = 4 * tid < cw ? reinterpret_cast<const float4*>(a.xs + (size_t)b * a.Wp + c0)[tid] : zero;
+        xsh[tid] = v;
+        xloc[tid] = 4 * tid < cw ? make_float4(v.x - xc, v.y - xc, v.z - xc, v.w - xc) : zero;
+    }
 
     // element e of chunk k: float4 (e % ROW4) of tile row (e / ROW4)
     auto fetch = [&](int k, int e) -> float4 {
@@ -283,6 +298,32 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
     if (tid <= RPC) ysh[0][tid] = fetch_y(0, min(tid, RPC - 1));
     __syncthreads();
 
+    // Which evaluation this lane's Gaussian gets on this tile: the completed square where the record has
+    // one and sA times the tile's largest |x'| stays within kSepSpanLimitBwd (NaN coordinates: term by term).
+    float span = 0.0f;
+    bool xbad = false;
+#pragma unroll
+    for (int i = 0; i < kBwdTileW / 4; ++i) {
+        const float4 v = xloc[i];
+        span = fmaxf(span, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        xbad = xbad || !(v.x == v.x && v.y == v.y && v.z == v.z && v.w == v.w);
+    }
+    const bool regular = br.w == 0.0f && !xbad && br.x * span <= kSepSpanLimitBwd;
+    // regular lanes: sA, skA, D''; the others: A', B2', D'
+    const float A = regular ? br.x : rA, B2 = regular ? br.y : rB2, D = regular ? br.z : rD;
+    const float mpx = -A * (px - xc);  // regular lanes: -sA px'
+
+    // the pixel record of column j of a tile row, from LDS (wave-uniform address)
+    auto pixel = [&](const float4* rowrec, int j, float (&pv)[CP]) {
+#pragma unroll
+        for (int q4 = 0; q4 < CP4; ++q4) {
+            const float4 tq = rowrec[j * CP4 + q4];
+            pv[4 * q4] = tq.x;
+            pv[4 * q4 + 1] = tq.y;
+            pv[4 * q4 + 2] = tq.z;
+            pv[4 * q4 + 3] = tq.w;
+        }
+    };
     for (int k = 0; k < chunks; ++k) {
         if (k + 1 < chunks) {
 #pragma unroll
@@ -295,84 +336,101 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
         const float4* cur = sh + (k & 1) * E;
         const float* ycur = ysh[k & 1];
         const int rows = min(RPC, r1 - r0 - k * RPC);
-        float ynext = ycur[0];
+        if (regular) {
+            float ynext = ycur[0];
 #pragma unroll 1
-        for (int rr = 0; rr < rows; ++rr) {
-            // the row coordinate comes from LDS, read one row ahead: a scalar load here would
-            // drain the LDS/scalar counter once per tile row
-            const float yv = ynext;
-            ynext = ycur[rr + 1];
-            float dy[G], cyy[G], bdy[G], R0[G], R1[G], R2[G], RC[G][C];
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                dy[g] = yv - py[g];
-                const float ddy = D[g] * dy[g];
-                cyy[g] = ddy * dy[g];
-                bdy[g] = B2[g] * dy[g];
-                R0[g] = R1[g] = R2[g] = 0.0f;
-#pragma unroll
-                for (int c = 0; c < C; ++c) RC[g][c] = 0.0f;
-            }
-            const float4* rowrec = cur + rr * ROW4;
+            for (int rr = 0; rr < rows; ++rr) {
+                // the row coordinate comes from LDS, read one row ahead: a scalar load here would
+                // drain the LDS/scalar counter once per tile row
+                const float yv = ynext;
+                ynext = ycur[rr + 1];
+                const float dy = yv - py;
+                const float rowoff = fmaf(B2, dy, mpx);
+                const float cyy = (D * dy) * dy;
+                float R0 = 0.0f, R1 = 0.0f;
+                const float4* rowrec = cur + rr * ROW4;
 #pragma unroll 1
-            for (int i = 0; i < cw; i += 4) {
-                const float4 xq = xsh[i >> 2];
-                const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
-                // phase 1: exponents of the 4 x G pairs (independent chains)
-                float dxs[4][G], ee[4][G];
+                for (int i = 0; i < cw; i += 4) {
+                    const float4 xq = xloc[i >> 2];
+                    const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
+                    // phase 1: exponents of the 4 pairs (independent chains)
+                    float us[4], vs[4], ee[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int g = 0; g < G; ++g) {
-                        const float dx = xs4[j] - px[g];
-                        const float tt = fmaf(A[g], dx, bdy[g]);
-                        ee[j][g] = fmaf(tt, dx, cyy[g]);
-                        dxs[j][g] = dx;
+                    for (int j = 0; j < 4; ++j) {
+                        us[j] = fmaf(A, xs4[j], rowoff);
+                        vs[j] = us[j] * us[j];
+                        ee[j] = cyy - vs[j];
                     }
-                // phase 2: transcendentals back to back
+                    // phase 2: transcendentals back to back
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                    for (int j = 0; j < 4; ++j) ee[j] = hw_exp2(ee[j]);
+                    // phase 3: G = <g^, c> - s and the sums
 #pragma unroll
-                    for (int g = 0; g < G; ++g) ee[j][g] = hw_exp2(ee[j][g]);
-                // phase 3: G = <g^, c> - s and the row sums
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float pv[CP];
-#pragma unroll
-                    for (int q4 = 0; q4 < CP4; ++q4) {
-                        const float4 tq = rowrec[(i + j) * CP4 + q4];
-                        pv[4 * q4] = tq.x;
-                        pv[4 * q4 + 1] = tq.y;
-                        pv[4 * q4 + 2] = tq.z;
-                        pv[4 * q4 + 3] = tq.w;
-                    }
-#pragma unroll
-                    for (int g = 0; g < G; ++g) {
-                        const float e = ee[j][g], dx = dxs[j][g];
+                    for (int j = 0; j < 4; ++j) {
+                        float pv[CP];
+                        pixel(rowrec, i + j, pv);
                         float Gv = pv[C];  // -s
 #pragma unroll
-                        for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[g][c], Gv);
-                        const float ge = Gv * e;
-                        R0[g] += ge;
-                        const float t1 = ge * dx;
-                        R1[g] += t1;
-                        R2[g] = fmaf(t1, dx, R2[g]);
+                        for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[c], Gv);
+                        const float ge = Gv * ee[j];
+                        R0 += ge;
+                        R1 = fmaf(ge, us[j], R1);
+                        M[3] = fmaf(ge, vs[j], M[3]);
 #pragma unroll
-                        for (int c = 0; c < C; ++c) RC[g][c] = fmaf(e, pv[c], RC[g][c]);
+                        for (int c = 0; c < C; ++c) CG[c] = fmaf(ee[j], pv[c], CG[c]);
                     }
                 }
+                // the tile row is complete
+                M[0] += R0;
+                M[1] += R1;
+                M[2] = fmaf(dy, R0, M[2]);
+                M[4] = fmaf(dy, R1, M[4]);
+                M[5] = fmaf(dy * dy, R0, M[5]);
             }
-            // the tile row is complete
+        } else {
+            float ynext = ycur[0];
+#pragma unroll 1
+            for (int rr = 0; rr < rows; ++rr) {
+                const float yv = ynext;
+                ynext = ycur[rr + 1];
+                const float dy = yv - py;
+                const float cyy = (D * dy) * dy;
+                const float bdy = B2 * dy;
+                float R0 = 0.0f, R1 = 0.0f, R2 = 0.0f, RC[C];
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                M[g][0] += R0[g];
-                M[g][1] += R1[g];
-                M[g][3] += R2[g];
-                M[g][2] = fmaf(dy[g], R0[g], M[g][2]);
-                M[g][4] = fmaf(dy[g], R1[g], M[g][4]);
-                M[g][5] = fmaf(dy[g] * dy[g], R0[g], M[g][5]);
+                for (int c = 0; c < C; ++c) RC[c] = 0.0f;
+                const float4* rowrec = cur + rr * ROW4;
+#pragma unroll 1
+                for (int i = 0; i < cw; i += 4) {
+                    const float4 xq = xsh[i >> 2];
+                    const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
 #pragma unroll
-                for (int c = 0; c < C; ++c) CG[g][c] += RC[g][c];
+                    for (int j = 0; j < 4; ++j) {
+                        const float dx = xs4[j] - px;
+                        const float tt = fmaf(A, dx, bdy);
+                        const float e = hw_exp2(fmaf(tt, dx, cyy));
+                        float pv[CP];
+                        pixel(rowrec, i + j, pv);
+                        float Gv = pv[C];
+#pragma unroll
+                        for (int c = 0; c < C; ++c) Gv = fmaf(pv[c], col[c], Gv);
+                        const float ge = Gv * e;
+                        R0 += ge;
+                        const float t1 = ge * dx;
+                        R1 += t1;
+                        R2 = fmaf(t1, dx, R2);
+#pragma unroll
+                        for (int c = 0; c < C; ++c) RC[c] = fmaf(e, pv[c], RC[c]);
+                    }
+                }
+                M[0] += R0;
+                M[1] += R1;
+                M[3] += R2;
+                M[2] = fmaf(dy, R0, M[2]);
+                M[4] = fmaf(dy, R1, M[4]);
+                M[5] = fmaf(dy * dy, R0, M[5]);
+#pragma unroll
+                for (int c = 0; c < C; ++c) CG[c] += RC[c];
             }
         }
         if (k + 1 < chunks) {
@@ -386,7 +444,22 @@ __global__ __launch_bounds__(kThreads) void k_bwd_sep(const BwdArgs a) {
         }
         __syncthreads();
     }
-    bwd_store<C, G>(a, b, t, slot, M, CG);
+    if (regular) {
+        // moments in (u, dy) -> moments in (dx, dy), dx = (u - skA dy) / sA; in fp64: once per lane and tile
+        const double iA = 1.0 / (double)A, sk = (double)B2;
+        const double mu = M[1], my = M[2], muu = M[3], muy = M[4], myy = M[5];
+        M[1] = (float)((mu - sk * my) * iA);
+        M[3] = (float)((muu - 2.0 * sk * muy + sk * sk * myy) * (iA * iA));
+        M[4] = (float)((muy - sk * myy) * iA);
+    }
+    if (pos < count) {
+        constexpr int NF = 6 + C;
+        float* out = a.partial + ((size_t)b * a.T + t) * NF * a.N + (size_t)pos * NF;  // one record of NF floats per list position
+#pragma unroll
+        for (int f = 0; f < 6; ++f) out[f] = M[f];
+#pragma unroll
+        for (int c = 0; c < C; ++c) out[6 + c] = CG[c];
+    }
 }
 
 // General grid: the tile is a flat pixel range (multiple of 256); x and y come with the
@@ -414,7 +487,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_gen(const BwdArgs a) {
     const int p0 = t * a.per_tile, p1 = min(a.HWp, p0 + a.per_tile);
     const float4* src = reinterpret_cast<const float4*>(a.pixrec + ((size_t)b * a.HWp + p0) * CP);
     int seen = 0;
-    stream_records_lds<CP4, kPixChunk>(src, p1 - p0, sh, [&](const float4* r) {
+    stream_records_lds<CP4, kPixChunk>(src, p1 - p0, sh, [&](const float4* r, const float4*) {
         float pv[CP];
 #pragma unroll
         for (int q4 = 0; q4 < CP4; ++q4) {

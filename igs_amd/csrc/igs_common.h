@@ -37,6 +37,36 @@ __host__ __device__ constexpr int bwd_gen_g(int C) { return C <= 4 ? IGS_BWD_GEN
 __host__ __device__ constexpr int bwd_sep_g(int C) { return C <= 4 ? IGS_BWD_G : 1; }
 
 __host__ __device__ constexpr int rec_stride_of(int C) { return (6 + C + 3) & ~3; }
+// Records of the separable kernels (see sep_terms): the forward's px, py, sD, skD, A'', alpha,
+// alpha*c_0.., tag, A', B2', D' (none for C > 8: with four rows per lane the hoisted part of the completed square
+// costs what it saves, and that forward reads the plain records); the backward's sA, skA, D'', tag.
+#ifndef IGS_FWD_SQUARE
+#define IGS_FWD_SQUARE 1
+#endif
+__host__ __device__ constexpr bool fwd_square(int C) { return IGS_FWD_SQUARE && fwd_sep_p(C) >= 8; }
+__host__ __device__ constexpr int frec_stride_of(int C) { return fwd_square(C) ? (10 + C + 3) & ~3 : 0; }
+constexpr int kBrecStride = 4;
+// The completed square is evaluated in coordinates relative to the middle of a lane's rows (forward) or
+// of a tile's columns (backward); its rounding grows with s times the largest such coordinate (s = sD, sA:
+// the square's scale; an error of about 1e-7 s |y'| |u| in the exponent), so where that product exceeds a
+// limit (Gaussians sharper than the pixel spacing, grids whose coordinates jump within a tile) the pair is
+// evaluated term by term instead.  The forward, whose result is held to 1e-6, chooses per wave and record
+// (wave-uniform, so the other evaluation costs one instruction per pair more and nothing else) with a
+// tight limit; the backward chooses per lane, where a wave with lanes of both kinds runs both loops, and
+// its sums are held to 1e-4 of the largest: its limit only catches what would be inaccurate beyond that.
+#ifndef IGS_SEP_LIMIT_FWD
+#define IGS_SEP_LIMIT_FWD 8.0f
+#endif
+#ifndef IGS_SEP_LIMIT_BWD
+#define IGS_SEP_LIMIT_BWD 64.0f
+#endif
+constexpr float kSepSpanLimitFwd = IGS_SEP_LIMIT_FWD;
+constexpr float kSepSpanLimitBwd = IGS_SEP_LIMIT_BWD;
+// floats of the packed buffer per (padded) Gaussian: record, bin record, forward and backward records
+// of the separable kernels
+__host__ __device__ constexpr int packed_floats_per_gaussian(int C) {
+    return rec_stride_of(C) + 8 + frec_stride_of(C) + kBrecStride;
+}
 __host__ __device__ constexpr int pix_stride_sep(int C) { return (C + 1 + 3) & ~3; }
 __host__ __device__ constexpr int pix_stride_gen(int C) { return (C + 3 + 3) & ~3; }
 

@@ -5,6 +5,7 @@
 // ----------------------------------------------------------------------------- forward
 struct FwdArgs {
     const float* packed;  // [B][Np][RS]
+    const float* frecs;   // separable kernels: their forward records [B][Np][frec_stride_of(C)]
     const float* zero_rec;  // an all-zero record behind the packed buffer's skip settings
     const float* x;
     const float* y;
@@ -102,6 +103,48 @@ __device__ __forceinline__ GRec<C> lds_grec(const float4* r) {
     return g;
 }
 
+// A forward record of the separable kernels (sep_terms): px, py, sD, skD, A'' (q' = -(sD dy + skD dx)^2 +
+// A'' dx^2), alpha, alpha*c_0.., the tag (sD again, or NaN where the form has no completed square) and
+// A', B2', D' for the evaluation term by term.  The completed square needs the first 7 + C floats only.
+template <int C>
+struct FRec {
+    float px, py, sD, skD, A2, al;
+    float ac[C];
+    float tag;
+};
+template <int C>
+__device__ __forceinline__ FRec<C> lds_frec(const float4* r) {
+    constexpr int R4 = (7 + C + 3) / 4;
+    float v[4 * R4];
+#pragma unroll
+    for (int i = 0; i < R4; ++i) {
+        const float4 t = r[i];
+        v[4 * i] = t.x;
+        v[4 * i + 1] = t.y;
+        v[4 * i + 2] = t.z;
+        v[4 * i + 3] = t.w;
+    }
+    FRec<C> g;
+    g.px = v[0];
+    g.py = v[1];
+    g.sD = v[2];
+    g.skD = v[3];
+    g.A2 = v[4];
+    g.al = v[5];
+#pragma unroll
+    for (int c = 0; c < C; ++c) g.ac[c] = v[6 + c];
+    g.tag = v[6 + C];
+    return g;
+}
+// A', B2', D' of a forward record (floats 7 + C .. 9 + C)
+template <int C>
+__device__ __forceinline__ void lds_frec_terms(const float4* r, float& A, float& B2, float& D) {
+    const float* f = reinterpret_cast<const float*>(r);
+    A = f[7 + C];
+    B2 = f[8 + C];
+    D = f[9 + C];
+}
+
 // Keeps a wave-uniform value in a VGPR (an empty asm the compiler cannot see through), so that
 // instructions using it stay VGPR-only.
 __device__ __forceinline__ float in_vgpr(float v) {
@@ -122,12 +165,13 @@ constexpr int kStreamUnroll = IGS_STREAM_UNROLL;  // records whose LDS reads are
 constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
 
 // Streams `count` records of R4 float4 each from global memory to every wave of the
-// workgroup through the double-buffered LDS window sh[2][CH*R4]; body(const float4* rec) runs
-// once per record with a wave-uniform LDS pointer.  Records past `count` in the last chunk
+// workgroup through the double-buffered LDS window sh[2][CH*R4]; body(rec, lds) runs once per record
+// with its first RD float4 in registers (read from a wave-uniform LDS address) and the wave-uniform
+// LDS pointer to the whole record.  Records past `count` in the last chunk
 // read as all-zero (for a Gaussian record: alpha = 0, adds exactly 0).  Must be called by all
 // NT threads of the workgroup (it contains barriers; with NT = 64, one wave, they cost nothing).
 // With kGather, record i of the stream is src record index[i] (a tile's Gaussian list).
-template <int R4, int CH, bool kGather = false, int NT = kThreads, class Body>
+template <int R4, int CH, bool kGather = false, int NT = kThreads, int RD = R4, class Body>
 __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
                                                    float4* sh, Body&& body,
                                                    const int* __restrict__ index = nullptr) {
@@ -182,15 +226,15 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
         const int lim = min(CH, (count - k * CH + kStreamUnroll - 1) / kStreamUnroll * kStreamUnroll);
 #pragma unroll 1
         for (int n = 0; n < lim; n += kStreamUnroll) {
-            float4 rr[kStreamUnroll][R4];
+            float4 rr[kStreamUnroll][RD];
 #pragma unroll
             for (int u = 0; u < kStreamUnroll; ++u)
 #pragma unroll
-                for (int i = 0; i < R4; ++i) rr[u][i] = cur[(n + u) * R4 + i];
+                for (int i = 0; i < RD; ++i) rr[u][i] = cur[(n + u) * R4 + i];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < kStreamUnroll; ++u) {
-                body(rr[u]);
+                body(rr[u], cur + (n + u) * R4);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -213,7 +257,7 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
 // vmcnt wait per chunk separates the two.  Slots past `count` load the all-zero record `zero_rec`.
 // The two buffers are separate arrays and the chunk loop is unrolled by two, so that every LDS read
 // names the buffer it reads.
-template <int R4, int CH, class Body>
+template <int R4, int CH, int RD = R4, class Body>
 __device__ __forceinline__ void stream_records_dma(const float4* __restrict__ src,
                                                    const float4* __restrict__ zero_rec, int count,
                                                    float4* sh0, float4* sh1, Body&& body,
@@ -257,15 +301,15 @@ __device__ __forceinline__ void stream_records_dma(const float4* __restrict__ sr
         const int lim = min(CH, (count - k * CH + kStreamUnroll - 1) / kStreamUnroll * kStreamUnroll);
 #pragma unroll 1
         for (int n = 0; n < lim; n += kStreamUnroll) {
-            float4 rr[kStreamUnroll][R4];
+            float4 rr[kStreamUnroll][RD];
 #pragma unroll
             for (int u = 0; u < kStreamUnroll; ++u)
 #pragma unroll
-                for (int i = 0; i < R4; ++i) rr[u][i] = cur[(n + u) * R4 + i];
+                for (int i = 0; i < RD; ++i) rr[u][i] = cur[(n + u) * R4 + i];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < kStreamUnroll; ++u) {
-                body(rr[u]);
+                body(rr[u], cur + (n + u) * R4);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -310,17 +354,28 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 }
 
 // Separable grid: lane = one column, P consecutive rows; wave = 64 columns x P rows (kWave = false) or
-// kWaveCols columns x 64 / kWaveCols blocks of P rows (kWave = true).  Per Gaussian
-// and lane: dx, A'dx^2, B2'dx once, then per pixel dy, 2 fma, exp2, 1 + C fma.
+// kWaveCols columns x 64 / kWaveCols blocks of P rows (kWave = true).  The square is completed along
+// the column (sep_terms): q' = -(sD dy + skD dx)^2 + A'' dx^2 = -u^2 + c0 with
+// u = sD y' + (skD dx - sD py'), y' and py' relative to the lane's middle row so that the hoisted term
+// carries no more rounding than u itself.  Per Gaussian and lane: dx, A''dx^2, py', the hoisted term of u
+// once (6 instructions), then per pixel 2 fma, exp2, 1 + C fma.  Records without a completed square, or
+// with sD times the largest |y'| of the wave above kSepSpanLimitFwd (one wave-uniform comparison of the tag
+// with the wave's limit), are evaluated term by term: q' = (D' dy + B2' dx) dy + A' dx^2.
 // kWave = false: workgroup = wx x (4/wx) waves, all four streaming the tile's Gaussian list.
 // kWave = true (fwd_wave_lists): every wave has a list of its own and streams it independently of
 // the others (no barrier in the kernel); the four waves of a workgroup are the rectangles of one
 // 64 x 4P tile of the binning.
 // (kOne: launched as workgroups of one wave; only with kWave)
 template <int C, int P, bool kWave, bool kOne = false>
-__global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
+__global__ __launch_bounds__(kThreads, P >= 16 ? 3 : 1) void k_fwd_sep(const FwdArgs a) {  // (16 rows per lane: three waves per SIMD, i.e. at most 168 registers)
     static_assert(kWave || !kOne, "one-wave workgroups need a list per wave");
-    constexpr int RS = rec_stride_of(C), R4 = RS / 4;
+    constexpr bool kSq = fwd_square(C);  // completed square (its own records) or term by term (the plain ones)
+    static_assert(kSq == (P >= 8) || !IGS_FWD_SQUARE, "the completed square goes with 8 or more rows per lane");
+    constexpr int RS = kSq ? frec_stride_of(C) : rec_stride_of(C), R4 = RS / 4;
+#ifndef IGS_FWD_READ_ALL
+#define IGS_FWD_READ_ALL 0
+#endif
+    constexpr int RD = kSq && !IGS_FWD_READ_ALL ? (7 + C + 3) / 4 : R4;  // float4 of a record that every evaluation reads
     IGS_GATE(a);
     // Waves with lists of their own can be launched as workgroups of one wave (kOne): the four
     // waves of a tile share nothing, and a wave slot then frees as soon as its wave ends instead
@@ -373,6 +428,29 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
         wylo = -__builtin_inff();
         wyhi = __builtin_inff();
     }
+    // With the completed square the rows are, from here on, relative to the lane's middle row yc, if that
+    // loses nothing (yv - yc is exact for the neighbouring rows of an ordinary grid; where coordinates
+    // jump within a wave's rows it is not, and the wave keeps them as they are, yc = 0).
+    float yc = 0.0f, span = 0.0f;
+    if (kSq) {
+        const float mid = yv[P / 2];
+        bool exact = true;
+#pragma unroll
+        for (int p = 0; p < P; ++p) exact = exact && ((yv[p] - mid) + mid == yv[p]);
+        yc = __ballot(!exact) == 0ull ? mid : 0.0f;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            yv[p] = in_vgpr(yv[p] - yc);
+            span = fmaxf(span, fabsf(yv[p]));
+        }
+        if (ybad) span = __builtin_nanf("");
+        if (wcols == 32) {  // two row blocks per wave: the larger of the two (NaN if either is)
+            const float o = __shfl_xor(span, 32);
+            span = (span != span || o != o) ? __builtin_nanf("") : fmaxf(span, o);
+        }
+    }
+    // records with tag = sD <= sd_limit take the completed square (a NaN on either side: term by term)
+    const float sd_limit = in_vgpr(fminf(kSepSpanLimitFwd / span, 3.0e38f));
     // this unit's Gaussians (those whose ellipse reaches it), split S ways by list position
     const int s = blockIdx.y;
     // (wave lists are numbered by rectangle, row after row; rectangles outside the image have none)
@@ -388,32 +466,76 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     const int n0 = cut(s);
     const int n1 = s + 1 == a.S ? count : cut(s + 1);
     const int* list = a.lists + li * a.Np + n0;
-    const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
-    auto body = [&](auto wave_skip, const float4* r) {
-        const GRec<C> g = lds_grec<C>(r);
-        // A list shared by four waves of P rows each: a wave whose own rows the reach box misses
-        // skips the record (wave-uniform: the record is the same in all lanes).
-        if (decltype(wave_skip)::value && __ballot(!(g.yhi < wylo || g.ylo > wyhi)) == 0ull) return;
-        const float dx = xv - g.px;
-        const float adx = g.A * dx;
-        const float c0 = adx * dx;
-        const float c1 = g.B2 * dx;
+    const float4* src = reinterpret_cast<const float4*>((kSq ? a.frecs : a.packed) + (size_t)b * a.Np * RS);
+    // the exponents of the lane's P pixels for one record, and its alpha and alpha*c
+    auto exponents = [&](auto wave_skip, const float4* r, const float4* lds, float (&e)[P], float& al, float (&ac)[C]) -> bool {
+        if constexpr (kSq) {
+            const FRec<C> g = lds_frec<C>(r);
+            al = g.al;
+#pragma unroll
+            for (int c = 0; c < C; ++c) ac[c] = g.ac[c];
+            const float dx = xv - g.px;
+            const float pyl = g.py - yc;
+            if (__ballot(g.tag <= sd_limit) != 0ull) {  // wave-uniform: both sides are
+                const float c0 = (g.A2 * dx) * dx;
+                const float off = fmaf(g.skD, dx, -(g.sD * pyl));
+#pragma unroll
+                for (int p = 0; p < P; ++p) {
+                    const float u = fmaf(g.sD, yv[p], off);
+                    e[p] = fmaf(-u, u, c0);
+                }
+            } else {  // no completed square, or its scale is too large for this wave's rows
+                float Ap, B2p, Dp;
+                lds_frec_terms<C>(RD == R4 ? r : lds, Ap, B2p, Dp);
+                // py - yc = pyl + lo exactly (two-sum), so that dy = y - py carries one rounding, as without
+                // the shift (the sharp Gaussians that come here need it); lo, half an ulp of pyl at most,
+                // goes into the constant and the linear coefficient of the form in dy0 = y' - pyl:
+                // q' = (D' dy0 + c1 - 2 D' lo) dy0 + (c0 - c1 lo), up to D' lo^2 < 1e-9
+                const float bb = pyl - g.py;
+                const float lo = (g.py - (pyl - bb)) + (-yc - bb);
+                const float c1p = B2p * dx;
+                const float c0 = fmaf(-c1p, lo, (Ap * dx) * dx);
+                const float c1 = fmaf(-2.0f * Dp, lo, c1p);
+#pragma unroll
+                for (int p = 0; p < P; ++p) {
+                    const float dy = yv[p] - pyl;
+                    const float t = fmaf(Dp, dy, c1);
+                    e[p] = fmaf(t, dy, c0);
+                }
+            }
+        } else {
+            const GRec<C> g = lds_grec<C>(r);
+            // A list shared by four waves of P rows each: a wave whose own rows the reach box misses
+            // skips the record (wave-uniform: the record is the same in all lanes).
+            if (decltype(wave_skip)::value && __ballot(!(g.yhi < wylo || g.ylo > wyhi)) == 0ull) return false;
+            al = g.al;
+#pragma unroll
+            for (int c = 0; c < C; ++c) ac[c] = g.ac[c];
+            const float dx = xv - g.px;
+            const float adx = g.A * dx;
+            const float c0 = adx * dx;
+            const float c1 = g.B2 * dx;
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                const float dy = yv[p] - g.py;
+                const float t = fmaf(g.D, dy, c1);
+                e[p] = fmaf(t, dy, c0);
+            }
+        }
+        return true;
+    };
+    auto body = [&](auto wave_skip, const float4* r, const float4* lds) {
         // three phases, so that the P independent chains overlap their latencies and the
         // transcendental ops issue back to back
-        float e[P];
-#pragma unroll
-        for (int p = 0; p < P; ++p) {
-            const float dy = yv[p] - g.py;
-            const float t = fmaf(g.D, dy, c1);
-            e[p] = fmaf(t, dy, c0);
-        }
+        float e[P], al, ac[C];
+        if (!exponents(wave_skip, r, lds, e, al, ac)) return;
 #pragma unroll
         for (int p = 0; p < P; ++p) e[p] = hw_exp2(e[p]);
 #pragma unroll
         for (int p = 0; p < P; ++p) {
-            dsum[p] = fmaf(e[p], g.al, dsum[p]);
+            dsum[p] = fmaf(e[p], al, dsum[p]);
 #pragma unroll
-            for (int c = 0; c < C; ++c) num[p][c] = fmaf(e[p], g.ac[c], num[p][c]);
+            for (int c = 0; c < C; ++c) num[p][c] = fmaf(e[p], ac[c], num[p][c]);
         }
     };
     // The per-wave test of a shared list costs a few percent when it never fires, so it is used only
@@ -422,17 +544,17 @@ __global__ __launch_bounds__(kThreads) void k_fwd_sep(const FwdArgs a) {
     if constexpr (kWave) {
         __shared__ float4 sh0[kOne ? 1 : 4][kGaussChunk * R4];  // per wave: the two chunk buffers
         __shared__ float4 sh1[kOne ? 1 : 4][kGaussChunk * R4];
-        stream_records_dma<R4, kGaussChunk>(
+        stream_records_dma<R4, kGaussChunk, RD>(
             src, reinterpret_cast<const float4*>(a.zero_rec), n1 - n0, sh0[kOne ? 0 : wave], sh1[kOne ? 0 : wave],
-            [&](const float4* r) { body(std::false_type{}, r); }, list);
+            [&](const float4* r, const float4* lds) { body(std::false_type{}, r, lds); }, list);
     } else {
         __shared__ float4 sh[2 * kGaussChunk * R4];
-        if (rec_has_yrange(C) && 8L * count < 7L * a.Np)
-            stream_records_lds<R4, kGaussChunk, true>(
-                src, n1 - n0, sh, [&](const float4* r) { body(std::true_type{}, r); }, list);
+        if (!kSq && rec_has_yrange(C) && 8L * count < 7L * a.Np)
+            stream_records_lds<R4, kGaussChunk, true, kThreads, RD>(
+                src, n1 - n0, sh, [&](const float4* r, const float4* lds) { body(std::true_type{}, r, lds); }, list);
         else
-            stream_records_lds<R4, kGaussChunk, true>(
-                src, n1 - n0, sh, [&](const float4* r) { body(std::false_type{}, r); }, list);
+            stream_records_lds<R4, kGaussChunk, true, kThreads, RD>(
+                src, n1 - n0, sh, [&](const float4* r, const float4* lds) { body(std::false_type{}, r, lds); }, list);
     }
     if (col < a.W) {
 #pragma unroll
@@ -474,7 +596,7 @@ __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
     const int n0 = s * a.n_per_split;
     const int n1 = min(a.Np, n0 + a.n_per_split);
     const float4* src = reinterpret_cast<const float4*>(a.packed + ((size_t)b * a.Np + n0) * RS);
-    stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r) {
+    stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r, const float4*) {
         const GRec<C> g = lds_grec<C>(r);
         float e[P];
 #pragma unroll

@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_grid(const GridGradArgs a) {
         sx[j] = sy[j] = 0.0f;
     }
     const float4* src = reinterpret_cast<const float4*>(a.packed + (size_t)b * a.Np * RS);
-    stream_records_lds<R4, kGaussChunk>(src, a.Np, sh, [&](const float4* r) {
+    stream_records_lds<R4, kGaussChunk>(src, a.Np, sh, [&](const float4* r, const float4*) {
         const GRec<C> g = lds_grec<C>(r);
         const float hb = 0.5f * g.B2;
         // phases: exponents, transcendentals back to back, accumulation

@@ -234,8 +234,8 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
     p->fwd_tiles = sep ? fg.tiles_x * fg.tiles_y * (fwd_wave_lists(C) ? 4 : 1) : 0;
     p->pix_stride = sep ? pix_stride_sep(C) : pix_stride_gen(C);
     // records, then one bin record (8 floats) per record, then the call's skip settings (4 floats)
-    // and an all-zero record
-    p->packed_bytes = ((uint64_t)B * p->n_padded * (p->rec_stride + 8) + 4 + kZeroRecFloats) * sizeof(float);
+    // and an all-zero record, then the separable kernels' forward and backward records
+    p->packed_bytes = ((uint64_t)B * p->n_padded * packed_floats_per_gaussian(C) + 4 + kZeroRecFloats) * sizeof(float);
     p->fwd_ws_bytes = S > 1 ? (uint64_t)S * B * (C + 1) * H * W * sizeof(float) : 0;
     p->pix_bytes = sep ? ((uint64_t)B * H * p->w_padded * p->pix_stride + (uint64_t)B * p->w_padded) * sizeof(float)
                        : (uint64_t)B * p->hw_padded * p->pix_stride * sizeof(float);
@@ -300,6 +300,14 @@ inline const float4* bins_of(const float* packed, int B, int Np, int RS) {
 // The skip limit the pack kernel left behind the boxes.
 inline const float* limit_of(const float* packed, int B, int Np, int RS) {
     return packed + (size_t)B * Np * (RS + 8);
+}
+// The separable kernels' records behind the zero record: the forward's [B][Np][frec_stride_of(C)], then
+// the backward's [B][Np] float4.
+inline const float* frecs_of(const float* packed, int B, int Np, int C) {
+    return packed + (size_t)B * Np * (rec_stride_of(C) + 8) + 4 + kZeroRecFloats;
+}
+inline const float4* brecs_of(const float* packed, int B, int Np, int C) {
+    return reinterpret_cast<const float4*>(frecs_of(packed, B, Np, C) + (size_t)B * Np * frec_stride_of(C));
 }
 // Skip weight of a pack call -> limit in units of the kernels' exponent (see reach_box); a weight of
 // 0 (or one too small to matter) is the exact limit.
@@ -490,25 +498,14 @@ int launch_bwd_prologue(const BwdArgs& a, int B, bool sep, const float* out, con
 // grid gradients).
 inline int bwd_gen_groups(int N, int C) { return ceil_div(N, kThreads * bwd_gen_g(C)); }
 
-// Separable backward: every list position up to Np is visited; listed Gaussians compute, the others
-// store zeros.  One Gaussian per lane (k_bwd_sep<C,1>) unless the lists are full by construction
-// (`dense`: IGS_OPT_NO_CULL): a tile's last list-position group is half empty on average, which costs
-// half as many idle lanes with groups of 256 as of 512 entries (c1, lists of ~4200: 3.5 % against 8.9 %),
-// more than the second Gaussian per lane saves by sharing the pixel records' LDS reads (16.3 against
-// 16.0 instructions per pair).  Step times with one / two per lane: c1 2.62 / 2.66 ms, c2 and c3 -2 to
-// -6 % with one; with only exact zeros skipped (lists 86 % full) equal; everything listed 4.67 / 4.62 ms.
+// Separable backward: every list position up to Np is visited by a lane (one Gaussian per lane: a tile's
+// last list-position group is half empty on average, which costs half as many idle lanes with groups of
+// 256 as of 512 entries); workgroups past a tile's count return at once.
 template <int C>
-int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, bool dense, hipStream_t st) {
+int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     if (sep) {
-        constexpr int kG = bwd_sep_g(C);
-        const bool narrow = kG == 1 || !dense;
-        if (narrow) {
-            const dim3 grid(a.T, ceil_div(a.Np, kThreads), B);
-            hipLaunchKernelGGL((k_bwd_sep<C, 1>), grid, dim3(kThreads), 0, st, a);
-        } else {
-            const dim3 grid(a.T, ceil_div(a.Np, kThreads * kG), B);
-            hipLaunchKernelGGL((k_bwd_sep<C, kG>), grid, dim3(kThreads), 0, st, a);
-        }
+        const dim3 grid(a.T, ceil_div(a.Np, kThreads), B);
+        hipLaunchKernelGGL((k_bwd_sep<C>), grid, dim3(kThreads), 0, st, a);
     } else {
         const dim3 grid(bwd_gen_groups(a.N, C), a.T, B);
         if (a.grid_part != nullptr)
@@ -534,6 +531,7 @@ int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* col
     a.tiles_x = plan.bwd_tiles_x;
     a.per_tile = plan.bwd_per_tile;
     a.counts = nullptr; a.lists = nullptr;
+    a.brecs = packed ? brecs_of(packed, B, plan.n_padded, C) : nullptr;
     if (sep && pix_ws) {
         const size_t scratch = ((size_t)B * H * plan.w_padded * plan.pix_stride + (size_t)B * plan.w_padded) * sizeof(float);
         const BinPlace bp = bins_at(pix_ws, scratch, B, plan.bwd_tiles);
@@ -619,7 +617,9 @@ int igs_gs2d_pack_covinv(const float* position, const float* cov_inv_00, const f
     hipLaunchKernelGGL((k_pack<false>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, position, cov_inv_00, cov_inv_01, cov_inv_11, alphas,
                        colors, N, Np, C, rec_stride_of(C), 0.0f, limit, skip_fraction, packed,
-                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C))));
+                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C))),
+                       const_cast<float*>(frecs_of(packed, B, Np, C)), frec_stride_of(C),
+                       const_cast<float4*>(brecs_of(packed, B, Np, C)));
     return launch_status();
 }
 
@@ -636,7 +636,9 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
     hipLaunchKernelGGL((k_pack<true>), dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, positions, scales, rotations, (const float*)nullptr,
                        alphas, colors, N, Np, C, rec_stride_of(C), eps, limit, skip_fraction, packed,
-                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C))));
+                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C))),
+                       const_cast<float*>(frecs_of(packed, B, Np, C)), frec_stride_of(C),
+                       const_cast<float4*>(brecs_of(packed, B, Np, C)));
     return launch_status();
 }
 
@@ -705,6 +707,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
         const FwdGeometry fg = fwd_geometry(B, H, W, C, sep);
         FwdArgs a;
         a.packed = packed; a.x = x; a.y = y;
+        a.frecs = frecs_of(packed, B, plan.n_padded, C);
         a.zero_rec = limit_of(packed, B, plan.n_padded, plan.rec_stride) + 4;
         a.sxb = grid_strides[0]; a.sxh = grid_strides[1]; a.sxw = grid_strides[2];
         a.syb = grid_strides[3]; a.syh = grid_strides[4]; a.syw = grid_strides[5];
@@ -1006,7 +1009,7 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
             if (rc) return rc;
         }
         if (gg.g_x != nullptr && !sep) a.grid_part = reinterpret_cast<float2*>(gg.ws);
-        IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, (opts_of(grid_mode) & IGS_OPT_NO_CULL) != 0, st));
+        IGS_DISPATCH_C(C, rc = launch_bwd_reduce<kC>(a, B, sep, st));
         if (rc) return rc;
         if (gg.g_x == nullptr) continue;
         if (sep) {  // the pixel-major kernel of its own
@@ -1220,7 +1223,9 @@ int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int 
     hipLaunchKernelGGL(k_pack_feature, dim3(ceil_div(Np, kThreads), B), dim3(kThreads), 0,
                        (hipStream_t)stream, gs_feature, pos_offset, N, Np, C, C_kernel,
                        rec_stride_of(C_kernel), eps, limit, skip_fraction, packed,
-                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C_kernel))), colors_out);
+                       const_cast<float4*>(bins_of(packed, B, Np, rec_stride_of(C_kernel))),
+                       const_cast<float*>(frecs_of(packed, B, Np, C_kernel)), frec_stride_of(C_kernel),
+                       const_cast<float4*>(brecs_of(packed, B, Np, C_kernel)), colors_out);
     return launch_status();
 }
 

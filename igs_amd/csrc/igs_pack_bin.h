@@ -69,6 +69,40 @@ __device__ __forceinline__ void write_skip_limit(float4* bins, int B, int Np, fl
     for (int i = 0; i < kZeroRecFloats / 4; ++i) tail[1 + i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 }
 
+// Records of the separable kernels.  With a positive definite form the square can be completed,
+//   q' = A'dx^2 + B2'dx dy + D'dy^2 = -(sD dy + skD dx)^2 + A''dx^2      (forward: rows inside a column)
+//                                    = -(sA dx + skA dy)^2 + D''dy^2      (backward: columns inside a row)
+// with sD = sqrt(-D'), skD = -B2' / (2 sD), A'' = A' - B2'^2 / (4 D') = k det / D (k = -0.5 log2 e) and
+// the same with A and D exchanged: one term per pair instead of two, the other hoisted, and both terms
+// are non-positive, so nothing cancels however long and tilted the ellipse is.  The six values are
+// formed in fp64 from the unrounded A, B, D (A'' and D'' from the determinant: the difference
+// A' - B2'^2 / (4 D') of the rounded values would lose the digits that a thin ellipse needs).
+// A record whose form is not positive definite, or has a non-finite value anywhere, is tagged (forward
+// record: NaN in place of a copy of sD, which a single comparison with the wave's limit on sD turns into
+// the choice of the evaluation; backward record: 1 in place of 0): the kernels evaluate it term by term
+// as on general grids, from A', B2', D', which the forward record carries as well.
+struct SepTerms {
+    float sD, skD, A2, sA, skA, D2;
+    bool regular;
+};
+__device__ __forceinline__ SepTerms sep_terms(double A, double Bc, double D, double det, bool finite_record) {
+    constexpr double k = -0.72134752044448170368;
+    SepTerms t;
+    const double sD = sqrt(-k * D), sA = sqrt(-k * A);
+    t.sD = (float)sD;
+    t.skD = (float)(-k * Bc / sD);
+    t.A2 = (float)(k * det / D);
+    t.sA = (float)sA;
+    t.skA = (float)(-k * Bc / sA);
+    t.D2 = (float)(k * det / A);
+    t.regular = finite_record && A > 0.0 && D > 0.0 && det > 0.0 && isfinite(t.sD) && isfinite(t.skD) &&
+                isfinite(t.A2) && isfinite(t.sA) && isfinite(t.skA) && isfinite(t.D2) && t.sD > 0.0f && t.sA > 0.0f;
+    return t;
+}
+__device__ __forceinline__ void write_brec(float4* brec, size_t i, const SepTerms& t) {
+    brec[i] = t.regular ? make_float4(t.sA, t.skA, t.D2, 0.0f) : make_float4(0.0f, 0.0f, 0.0f, 1.0f);
+}
+
 // One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
 // with A' = k A, B2' = 2 k B, D' = k D, k = -0.5 log2 e.  Records N..Np-1 are zero.
 template <bool kScaleRot>
@@ -81,21 +115,26 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
                                                    int Np, int C, int RS, float eps,
                                                    float limit, float fraction,
                                                    float* __restrict__ packed,
-                                                   float4* __restrict__ boxes) {
+                                                   float4* __restrict__ boxes,
+                                                   float* __restrict__ frecs, int RSF,
+                                                   float4* __restrict__ brecs) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit, fraction);
     if (n >= Np) return;
     float* r = packed + ((size_t)b * Np + n) * RS;
+    float* fr = frecs + ((size_t)b * Np + n) * RSF;
     if (n >= N) {  // padding: alpha = 0 and e = exp2(0) = 1, so it contributes exactly 0
         for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        for (int c = 0; c < RSF; ++c) fr[c] = 0.0f;
+        brecs[(size_t)b * Np + n] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         write_empty_bin_record(boxes, (size_t)b * Np + n);
         return;
     }
     const size_t i = (size_t)b * N + n;
     // The closed form runs in fp64 and is rounded once: an error of a few fp32 ulp in A', B2', D'
     // would be multiplied by |q| (tens, for sharp Gaussians) in the exponent.  O(BN) work.
-    double A, Bc, D, sxx, syy;
+    double A, Bc, D, sxx, syy, det;
     bool bounded;
     if (kScaleRot) {
         const double s0 = p0[2 * i], s1 = p0[2 * i + 1];
@@ -108,12 +147,13 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
         D = sn * sn * i0 + cs * cs * i1;
         sxx = cs * cs * v0 + sn * sn * v1;
         syy = sn * sn * v0 + cs * cs * v1;
+        det = i0 * i1;
         bounded = v0 > 0.0 && v1 > 0.0;
     } else {
         A = p0[i];
         Bc = p1[i];
         D = p2[i];
-        const double det = A * D - Bc * Bc;
+        det = A * D - Bc * Bc;
         bounded = A > 0.0 && det > 0.0;
         sxx = D / det;
         syy = A / det;
@@ -159,6 +199,29 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
 #pragma unroll
     for (int q = 0; q < kZeroRecFloats / 4; ++q)
         if (4 * q < RS) r4[q] = make_float4(rec[4 * q], rec[4 * q + 1], rec[4 * q + 2], rec[4 * q + 3]);
+    // the separable kernels' records: the same with the completed square in place of A', B2', D' and a
+    // tag behind the colours
+    const SepTerms t = sep_terms(A, Bc, D, det, bounded && fin && isfinite(px) && isfinite(py));
+    write_brec(brecs, (size_t)b * Np + n, t);
+    if (RSF == 0) return;
+    const float Ap = rec[2], B2p = rec[3], Dp = rec[4];
+    rec[2] = t.sD;
+    rec[3] = t.skD;
+    rec[4] = t.A2;
+#pragma unroll
+    for (int c = 6; c < kZeroRecFloats - 5; ++c)
+        if (c == 6 + C) {
+            rec[c] = t.regular ? t.sD : __builtin_nanf("");
+            rec[c + 1] = Ap;
+            rec[c + 2] = B2p;
+            rec[c + 3] = Dp;
+            rec[c + 4] = 0.0f;
+            rec[c + 5] = 0.0f;
+        }
+    float4* f4 = reinterpret_cast<float4*>(fr);
+#pragma unroll
+    for (int q = 0; q < kZeroRecFloats / 4; ++q)
+        if (4 * q < RSF) f4[q] = make_float4(rec[4 * q], rec[4 * q + 1], rec[4 * q + 2], rec[4 * q + 3]);
 }
 
 // Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
@@ -172,14 +235,19 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
                                                            float limit, float fraction,
                                                            float* __restrict__ packed,
                                                            float4* __restrict__ boxes,
+                                                           float* __restrict__ frecs, int RSF,
+                                                           float4* __restrict__ brecs,
                                                            float* __restrict__ colors_out) {
     const int n = blockIdx.x * kThreads + threadIdx.x;
     const int b = blockIdx.y;
     if (n == 0 && b == 0) write_skip_limit(boxes, gridDim.y, Np, limit, fraction);
     if (n >= Np) return;
     float* r = packed + ((size_t)b * Np + n) * RS;
+    float* fr = frecs + ((size_t)b * Np + n) * RSF;
     if (n >= N) {
         for (int c = 0; c < RS; ++c) r[c] = 0.0f;
+        for (int c = 0; c < RSF; ++c) fr[c] = 0.0f;
+        brecs[(size_t)b * Np + n] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         write_empty_bin_record(boxes, (size_t)b * Np + n);
         return;
     }
@@ -220,6 +288,22 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
         r[6 + Cp] = py - ext.y;
         r[7 + Cp] = py + ext.y;
     }
+    // the separable kernels' records (see sep_terms)
+    const SepTerms t = sep_terms(A, Bc, D, i0 * i1, fin && v0 > 0.0 && v1 > 0.0 && isfinite(px) && isfinite(py));
+    write_brec(brecs, (size_t)b * Np + n, t);
+    if (RSF == 0) return;
+    fr[0] = px;
+    fr[1] = py;
+    fr[2] = t.sD;
+    fr[3] = t.skD;
+    fr[4] = t.A2;
+    fr[5] = 1.0f;
+    for (int c = 0; c < Cp; ++c) fr[6 + c] = c < C ? f[6 + c] : 0.0f;
+    for (int c = 6 + Cp; c < RSF; ++c) fr[c] = 0.0f;
+    fr[6 + Cp] = t.regular ? t.sD : __builtin_nanf("");
+    fr[7 + Cp] = r[2];
+    fr[8 + Cp] = r[3];
+    fr[9 + Cp] = r[4];
 }
 
 // ----------------------------------------------------------------------------- binning

@@ -105,8 +105,10 @@ typedef struct igs_gs2d_plan_t {
     uint64_t packed_bytes;   /* packed Gaussian buffer: records, then one bin record (8
                                 floats: reach box and quadratic form, what the tile lists
                                 are built from) per record, then the call's skip settings
-                                (4 floats) and an all-zero record (28 floats):
-                                (B*n_padded*(rec_stride+8) + 32)*4                         */
+                                (4 floats) and an all-zero record (28 floats), then the
+                                separable kernels' own records (forward: roundup4(10+C)
+                                floats, none for C > 8; backward: 4 floats):
+                                (B*n_padded*(rec_stride+8+sep) + 32)*4                     */
     uint64_t fwd_ws_bytes;   /* forward scratch: split partials (fwd_split > 1) and, on
                                 separable grids, the per-tile Gaussian lists (plus those
                                 of the super-tiles when there are 32 tiles or more)         */

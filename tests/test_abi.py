@@ -60,6 +60,12 @@ def test_plan_struct_matches_header_layout(lib):
         assert ct is {"int32_t": ctypes.c_int32, "uint64_t": ctypes.c_uint64}[typ], name
 
 
+def _sep_record_floats(C):
+    """Floats per Gaussian of the separable kernels' own records: the forward's (px, py, three terms, alpha,
+    C colours, a tag, the three plain terms; rounded up to 4; none for more than 8 channels) and the backward's 4."""
+    return ((10 + C + 3) // 4 * 4 if C <= 8 else 0) + 4
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2])
 def test_plan_arithmetic(lib, mode):
     from igs_amd import _lib
@@ -69,7 +75,8 @@ def test_plan_arithmetic(lib, mode):
         assert p.n_padded % 4 == 0 and p.n_padded >= N
         assert p.fwd_n_per_split % 4 == 0 and p.fwd_split * p.fwd_n_per_split >= p.n_padded
         assert (p.fwd_split - 1) * p.fwd_n_per_split < p.n_padded          # no empty split
-        assert p.packed_bytes == (B * p.n_padded * (p.rec_stride + 8) + 32) * 4    # records + bin records + skip settings + zero record
+        # records + bin records + the separable kernels' forward and backward records, skip settings + zero record
+        assert p.packed_bytes == (B * p.n_padded * (p.rec_stride + 8 + _sep_record_floats(C)) + 32) * 4
         assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
         assert p.bwd_tiles >= 1 and p.partial_bytes >= B * p.bwd_tiles * (6 + C) * N * 4
         if mode != 0:
@@ -266,7 +273,7 @@ def test_plan_invariants_over_random_shapes(lib):
             Np = p.n_padded
             assert Np % 4 == 0 and N <= Np < N + 4
             assert p.rec_stride % 4 == 0 and p.rec_stride >= 6 + C
-            assert p.packed_bytes == (B * Np * (p.rec_stride + 8) + 32) * 4
+            assert p.packed_bytes == (B * Np * (p.rec_stride + 8 + _sep_record_floats(C)) + 32) * 4
             assert 1 <= p.fwd_split <= 64 and p.fwd_n_per_split % 4 == 0
             assert p.fwd_split * p.fwd_n_per_split >= Np > (p.fwd_split - 1) * p.fwd_n_per_split
             assert p.bwd_tiles >= 1 and p.bwd_per_tile >= 1
