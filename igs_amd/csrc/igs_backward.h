@@ -214,6 +214,9 @@ constexpr int kBwdTileW = IGS_BWD_TILE_W;
 // completed square (tag of the backward record: a form that is not positive definite, non-finite
 // values) evaluate q' = (A' dx + B2' dy) dx + D' dy^2 term by term instead; what a Gaussian's sums are
 // depends on the Gaussian only, not on which lanes share its wave.
+#ifndef IGS_BWD_COLS_IN_REGS
+#define IGS_BWD_COLS_IN_REGS 1
+#endif
 #ifndef IGS_BWD_TILE_SHIFT
 #define IGS_BWD_TILE_SHIFT 5   // tiles per row and per image; odd, so that 8 or 16 tiles per row cycle through all columns (1 / 3 / 5 timed: c2 0.456 / 0.448 / 0.449 ms, c1 and c3 equal)
 #endif
@@ -302,9 +305,14 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
     // one and sA times the tile's largest |x'| stays within kSepSpanLimitBwd (NaN coordinates: term by term).
     float span = 0.0f;
     bool xbad = false;
+    float xl[kBwdTileW];
 #pragma unroll
     for (int i = 0; i < kBwdTileW / 4; ++i) {
         const float4 v = xloc[i];
+        xl[4 * i] = v.x;
+        xl[4 * i + 1] = v.y;
+        xl[4 * i + 2] = v.z;
+        xl[4 * i + 3] = v.w;
         span = fmaxf(span, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
         xbad = xbad || !(v.x == v.x && v.y == v.y && v.z == v.z && v.w == v.w);
     }
@@ -312,6 +320,13 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
     // regular lanes: sA, skA, D''; the others: A', B2', D'
     const float A = regular ? br.x : rA, B2 = regular ? br.y : rB2, D = regular ? br.z : rD;
     const float mpx = -A * (px - xc);  // regular lanes: -sA px'
+    // with few channels there are registers for sA x' of the tile's columns (regular lanes)
+    constexpr bool kColsInRegs = IGS_BWD_COLS_IN_REGS && C <= 4;
+    float sx[kColsInRegs ? kBwdTileW : 1];
+    if (kColsInRegs) {
+#pragma unroll
+        for (int j = 0; j < kBwdTileW; ++j) sx[j] = A * xl[j];
+    }
 
     // the pixel record of column j of a tile row, from LDS (wave-uniform address)
     auto pixel = [&](const float4* rowrec, int j, float (&pv)[CP]) {
@@ -349,15 +364,12 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
                 const float cyy = (D * dy) * dy;
                 float R0 = 0.0f, R1 = 0.0f;
                 const float4* rowrec = cur + rr * ROW4;
-#pragma unroll 1
-                for (int i = 0; i < cw; i += 4) {
-                    const float4 xq = xloc[i >> 2];
-                    const float xs4[4] = {xq.x, xq.y, xq.z, xq.w};
+                // four pairs (columns i..i+3) from their u
+                auto four_pairs = [&](int i, const float (&us)[4]) {
                     // phase 1: exponents of the 4 pairs (independent chains)
-                    float us[4], vs[4], ee[4];
+                    float vs[4], ee[4];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        us[j] = fmaf(A, xs4[j], rowoff);
                         vs[j] = us[j] * us[j];
                         ee[j] = cyy - vs[j];
                     }
@@ -378,6 +390,29 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
                         M[3] = fmaf(ge, vs[j], M[3]);
 #pragma unroll
                         for (int c = 0; c < C; ++c) CG[c] = fmaf(ee[j], pv[c], CG[c]);
+                    }
+                };
+                if constexpr (kColsInRegs) {
+                    // The columns' sA x' sit in registers: no coordinate reads and no loop in a row (the
+                    // compiler then starts the LDS reads of a group of pixel records inside the arithmetic of
+                    // the group before; reading them one group ahead by hand was no faster).  Columns beyond the
+                    // tile's width (a multiple of 8, workgroup-uniform) are skipped per 8 columns.
+#pragma unroll
+                    for (int i = 0; i < kBwdTileW; i += 8) {
+                        if (i >= cw) break;
+#pragma unroll
+                        for (int h = 0; h < 8; h += 4) {
+                            const float us[4] = {sx[i + h] + rowoff, sx[i + h + 1] + rowoff, sx[i + h + 2] + rowoff,
+                                                 sx[i + h + 3] + rowoff};
+                            four_pairs(i + h, us);
+                        }
+                    }
+                } else {
+#pragma unroll 1
+                    for (int i = 0; i < cw; i += 4) {
+                        const float4 xq = xloc[i >> 2];
+                        const float us[4] = {fmaf(A, xq.x, rowoff), fmaf(A, xq.y, rowoff), fmaf(A, xq.z, rowoff), fmaf(A, xq.w, rowoff)};
+                        four_pairs(i, us);
                     }
                 }
                 // the tile row is complete

@@ -366,8 +366,11 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 // the others (no barrier in the kernel); the four waves of a workgroup are the rectangles of one
 // 64 x 4P tile of the binning.
 // (kOne: launched as workgroups of one wave; only with kWave)
+#ifndef IGS_FWD_MIN_WAVES
+#define IGS_FWD_MIN_WAVES 3
+#endif
 template <int C, int P, bool kWave, bool kOne = false>
-__global__ __launch_bounds__(kThreads, P >= 16 ? 3 : 1) void k_fwd_sep(const FwdArgs a) {  // (16 rows per lane: three waves per SIMD, i.e. at most 168 registers)
+__global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_fwd_sep(const FwdArgs a) {  // (16 rows per lane: three waves per SIMD, i.e. at most 168 registers)
     static_assert(kWave || !kOne, "one-wave workgroups need a list per wave");
     constexpr bool kSq = fwd_square(C);  // completed square (its own records) or term by term (the plain ones)
     static_assert(kSq == (P >= 8) || !IGS_FWD_SQUARE, "the completed square goes with 8 or more rows per lane");
