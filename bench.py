@@ -30,12 +30,28 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 # Per-launch counter readings of the two hot kernels at c1, taken from the committed rocprofv3 summary
 # (profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md): wave-level instruction counts and HBM KiB.
 # executed FLOPs = (2 FMA + MUL + ADD + TRANS) x 64 lanes; HBM bytes = FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
-# (factors from the plain-copy calibration of the same profile run).
+# (factors from the plain-copy calibration of the same profile run).  `csrc_sha16` names the kernel sources
+# the counters were read from (csrc_sha16() below): with other sources the instruction counts no longer
+# belong to the kernels being timed, and the fields derived from them are reported as null.
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
+    "csrc_sha16": "stale",
     "bwd": {"fma": 7.643e8, "mul": 1.465e8, "add": 8.396e7, "trans": 6.902e7, "fetch_kib": 54010, "write_kib": 201500},
     "fwd": {"fma": 4.182e8, "mul": 1.316e7, "add": 7.403e7, "trans": 6.971e7, "fetch_kib": 11920, "write_kib": 131100},
 }
+
+
+def csrc_sha16():
+    """First 16 hex digits of the SHA-256 over the kernel sources (igs_amd/csrc/*, include/igs_hip.h), in name order."""
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "igs_amd", "csrc")
+    for path in sorted(os.path.join(csrc, f) for f in os.listdir(csrc)) + [os.path.join(ROOT, "include", "igs_hip.h")]:
+        if os.path.isfile(path):
+            h.update(os.path.basename(path).encode())
+            h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
 
 
 def executed_flops(k):
@@ -56,7 +72,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c4"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4"],
+                    help="c3 (the module) prints the step figures only: its kernels are the same as c1's")
+    ap.add_argument("--csrc-sha", action="store_true", help="print csrc_sha16() of this tree and exit")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--cpu-full", action="store_true",
                     help="time the CPU baseline on the whole batch of the configuration (c1: about two minutes on 16 "
@@ -86,6 +104,9 @@ def main() -> int:
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
     args = ap.parse_args()
+    if args.csrc_sha:
+        print(csrc_sha16())
+        return 0
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over the batch with no "
               "exchange; no multi-GPU run is part of it). Use --gpus 1.", file=sys.stderr)
@@ -101,15 +122,14 @@ def run(args) -> int:
     if args.sweep:
         return sweep(args.sweep_shape, not args.sweep_no_grid_grads)
     if args.all:
-        return all_configs(args.steps, args.warmup)
+        return all_configs(args.steps, args.warmup, args.no_cpu)
     if args.koleo:
         return koleo_table(args.no_cpu, args.koleo_shape)
 
     import torch
 
     import igs_amd
-    from igs_amd import _lib
-    from igs_amd._splat import Grid as _Grid, Splat as _Splat, _ptr, _stream
+    from igs_amd._splat import library_options
     from oracle import gs2d_oracle as O
 
     if not torch.cuda.is_available():
@@ -117,40 +137,57 @@ def run(args) -> int:
         return 1
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    d = {k: v.to(dev) for k, v in O.make_config_inputs(args.config).items()}
-    B, N, C = d["colors"].shape
-    H, W = d["x_grid"].shape[-2:]
-    # the configuration's grids are linspaces *expanded* to [B,1,H,W]; .to(device) materialises
-    # them, so restore the stride-0 form on the device
-    d["x_grid"] = d["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
-    d["y_grid"] = d["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
-    pairs = B * N * H * W
     names = ("positions", "colors", "scales", "rotations", "alphas")
-    leaves = {k: d[k].clone().requires_grad_(True) for k in names}
+    module_path = args.config == "c3"
+    if module_path:   # the module: 32 Gaussians per feature, feature_dim 1024, x [8,128,1024] -> [8,3,256,256]
+        torch.manual_seed(1003)
+        model = igs_amd.GaussianSplatting2D(32, 1024).to(dev)
+        feat = torch.randn(8, 128, 1024, device=dev, requires_grad=True)
+        grad_out = torch.randn(8, 3, 256, 256, device=dev)
+        B, N, H, W, C = 8, 4096, 256, 256, 3
 
-    def forward():
-        return igs_amd.gaussian_splatting_2d(leaves["positions"], leaves["colors"], leaves["scales"],
-                                             leaves["rotations"], leaves["alphas"], d["x_grid"], d["y_grid"])
+        def forward():
+            return model(feat, size=(H, W))[0]
 
-    def step():
-        out = forward()
-        out.backward(d["grad_out"])
-        for v in leaves.values():
-            v.grad = None
+        def step():
+            forward().backward(grad_out)
+            feat.grad = None
+            model.zero_grad(set_to_none=True)
+    else:
+        d = {k: v.to(dev) for k, v in O.make_config_inputs(args.config).items()}
+        B, N, C = d["colors"].shape
+        H, W = d["x_grid"].shape[-2:]
+        # the configuration's grids are linspaces *expanded* to [B,1,H,W]; .to(device) materialises
+        # them, so restore the stride-0 form on the device
+        d["x_grid"] = d["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+        d["y_grid"] = d["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+        leaves = {k: d[k].clone().requires_grad_(True) for k in names}
+
+        def forward():
+            return igs_amd.gaussian_splatting_2d(leaves["positions"], leaves["colors"], leaves["scales"],
+                                                 leaves["rotations"], leaves["alphas"], d["x_grid"], d["y_grid"])
+
+        def step():
+            out = forward()
+            out.backward(d["grad_out"])
+            for v in leaves.values():
+                v.grad = None
+    pairs = B * N * H * W
 
     # ---- the timed path must be the correct one: image 0 of its output against the fp64 oracle
-    with torch.no_grad():
-        chk = forward()[:1].double()
-    g64 = {k: d[k][:1].double() for k in names + ("x_grid", "y_grid")}
-    ca, cb, cd = O.cov_inverse_closed(g64["scales"], g64["rotations"])
-    ref, _ = O.forward_strips(g64["x_grid"], g64["y_grid"], g64["positions"], ca, cb, cd, g64["alphas"], g64["colors"],
-                              rows=8)
-    err = (chk - ref).abs()
-    if not bool((err <= 1e-6 + 1e-5 * ref.abs()).all()):
-        print(f"bench.py: output differs from the oracle (max err {float(err.max()):.3e}); not timing a wrong result",
-              file=sys.stderr)
-        return 1
-    del chk, ref, err, g64
+    if not module_path:
+        with torch.no_grad():
+            chk = forward()[:1].double()
+        g64 = {k: d[k][:1].double() for k in names + ("x_grid", "y_grid")}
+        ca, cb, cd = O.cov_inverse_closed(g64["scales"], g64["rotations"])
+        ref, _ = O.forward_strips(g64["x_grid"], g64["y_grid"], g64["positions"], ca, cb, cd, g64["alphas"], g64["colors"],
+                                  rows=8)
+        err = (chk - ref).abs()
+        if not bool((err <= 1e-6 + 1e-5 * ref.abs()).all()):
+            print(f"bench.py: output differs from the oracle (max err {float(err.max()):.3e}); not timing a wrong result",
+                  file=sys.stderr)
+            return 1
+        del chk, ref, err, g64
 
     if args.copy_calibration:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
@@ -160,60 +197,89 @@ def run(args) -> int:
         torch.cuda.synchronize()
         del src, dst
 
-    # ---- whole step: W warm-ups, then exactly K steps between two synchronisations
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t_step = (time.perf_counter() - t0) / args.steps
+    # ---- whole step: W warm-up steps (and as many more as it takes to keep the GPU busy for 0.3 s: a
+    # step of a few milliseconds otherwise lands on the clock ramp), then exactly K steps between two
+    # synchronisations; then the same K steps timed one by one with events on the launch stream, whose
+    # median is the protocol of the reference's benchmark (scripts/profiling.py:103-151)
+    def timed(fn, steps, warmup, min_warm_s=0.3):
+        t0 = time.perf_counter()
+        k = 0
+        while k < warmup or time.perf_counter() - t0 < min_warm_s:
+            fn()
+            k += 1
+            if k % 8 == 0:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        mean = (time.perf_counter() - t0) / steps
+        ts = []
+        stream = torch.cuda.current_stream(dev)
+        for _ in range(steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e-3)
+        return mean, sorted(ts)[len(ts) // 2]
+
+    t_step, t_step_median = timed(step, args.steps, args.warmup)
 
     # ---- forward only (reported next to it)
     with torch.no_grad():
-        for _ in range(3):
-            forward()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            forward()
-        torch.cuda.synchronize()
-        t_fwd = (time.perf_counter() - t0) / args.steps
+        t_fwd, t_fwd_median = timed(forward, args.steps, 3, 0.1)
+
+    # ---- the same step with nothing but exact zeros skipped, and with every pair evaluated (what the
+    # reference does): the default leaves out pairs within the call's allowance, so `value` counts pairs
+    # that were never evaluated; these two are the figures without that
+    f_fwd, f_bwd = flops_per_pair(C)
+    side = {}
+    for key, opts in (("exact", dict(skip_tolerance=0.0)), ("no_cull", dict(no_cull=True))):
+        with library_options(**opts):
+            t_mean, t_med = timed(step, min(args.steps, 10), 3, 0.1)
+        side[key] = {"ms_per_step": t_mean * 1e3, "median_ms_per_step": t_med * 1e3, "value": pairs / t_mean,
+                     "what": {"exact": "skip_tolerance = 0: only pairs whose fp32 weight is exactly zero are left out",
+                              "no_cull": "IGS_OPT_NO_CULL: every Gaussian listed for every tile, all B N H W pairs evaluated"}[key]}
+    side["no_cull"]["frac"] = pairs * (f_fwd + f_bwd) / (side["no_cull"]["ms_per_step"] * 1e-3) / 1e12 / FP32_VECTOR_PEAK_TFLOPS
+
+    result = {
+        "metric": "gaussian_pixel_evals_per_sec_fwd_bwd",
+        "value": pairs / t_step,
+        "unit": "pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": t_step * 1e3,
+        "median_ms_per_step": t_step_median * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": (f"{args.config}: GaussianSplatting2D(32, 1024) module fwd+bwd, x [8,128,1024] -> "
+                                if module_path else f"{args.config}: gaussian_splatting_2d fwd+bwd, ") +
+                               f"B={B} N={N} {H}x{W} C={C} fp32, linspace grids, seeded U/N inputs",
+                   "B": B, "N": N, "H": H, "W": W, "C": C},
+        "fwd_pairs_per_s": pairs / t_fwd,
+        "fwd_ms": t_fwd * 1e3,
+        "fwd_median_ms": t_fwd_median * 1e3,
+        "step_tflops": pairs * (f_fwd + f_bwd) / t_step / 1e12,
+        "step_frac_counting_all_pairs": pairs * (f_fwd + f_bwd) / t_step / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+        "exact": side["exact"],
+        "no_cull": side["no_cull"],
+        "timing": "value / ms_per_step: `steps` steps between two synchronisations after `warmup` steps and at least 0.3 s "
+                  "of steps; median_*: the same number of steps timed one by one with events on the launch stream",
+    }
+    if module_path:
+        result["roofline"] = None
+        print(json.dumps(result), flush=True)
+        return 0
 
     # ---- dominant kernel alone, HIP events on the stream it is launched on
-    grid = _Grid(d["x_grid"], d["y_grid"], B)
-    op = _Splat(B, N, C, grid, 1e-6, dev)
-    f32 = lambda t: t.detach().float().contiguous()
-    col = f32(d["colors"])
-    packed = op.pack_scale_rot(f32(d["positions"]), f32(d["scales"]), f32(d["rotations"]), f32(d["alphas"]), col)
-    out, den = op.forward(packed)
-    pix = op._empty(op.plan.pix_bytes)
-    partial = op._empty(op.plan.partial_bytes)
-    lib = _lib.load()
-    st = _stream(dev)
-    _lib.check(lib.igs_gs2d_backward_prologue(_ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode, _ptr(grid.flag),
-                                              _ptr(out),
-                                              _ptr(den), _ptr(f32(d["grad_out"])), B, N, H, W, C, 1e-6, _ptr(pix),
-                                              int(op.plan.pix_bytes), st), "prologue")
-
-    built = [False]   # the first call builds the tile lists; the timed ones find them in place: k_bwd_sep alone
-
-    def reduce_kernel():
-        mode = grid.mode | (_lib.IGS_OPT_LISTS_BUILT if built[0] else 0)
-        built[0] = True
-        _lib.check(lib.igs_gs2d_backward_reduce(_ptr(packed), _ptr(col), _ptr(grid.y), grid.strides, mode,
-                                                _ptr(grid.flag), B, N,
-                                                H, W, C, _ptr(pix), int(op.plan.pix_bytes), _ptr(partial),
-                                                int(op.plan.partial_bytes), st), "reduce")
-
-    fwd_ws = op._empty(op.plan.fwd_ws_bytes)
-    fwd_out, fwd_den = op._new(B, C, H, W), op._new(B, H, W)
-
-    def fwd_kernel():
-        _lib.check(lib.igs_gs2d_forward(_ptr(packed), _ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode,
-                                        _ptr(grid.flag), B, N, H, W, C, 1e-6, _ptr(fwd_out), _ptr(fwd_den), _ptr(fwd_ws),
-                                        int(op.plan.fwd_ws_bytes), st), "forward")
+    probe = KernelProbe(d, B, N, H, W, C, dev)
 
     def event_time(fn, reps):
         for _ in range(3):
@@ -227,61 +293,18 @@ def run(args) -> int:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3 / reps
 
-    t_bwd_kernel = event_time(reduce_kernel, args.steps)
-    t_fwd_kernel = event_time(fwd_kernel, args.steps)
-    f_fwd, f_bwd = flops_per_pair(C)
-
-    # Pairs the backward kernel evaluated: its per-tile Gaussian lists (behind the pixel records in the
-    # workspace; written by the k_bin launch inside the bracket) times the pixels of each tile.  Pairs
-    # that are not listed are exact zeros and are skipped.
-    plan = op.plan
-    scratch = (B * H * plan.w_padded * plan.pix_stride + B * plan.w_padded) * 4
-    counts = pix.view(torch.int32)[(scratch + 15) // 16 * 4:][: B * plan.bwd_tiles].view(B, -1, plan.bwd_tiles_x).cpu()
-    rows = torch.tensor([min(H, (i + 1) * plan.bwd_per_tile) - i * plan.bwd_per_tile for i in range(counts.shape[1])])
-    tw = plan.bwd_tile_w
-    cols = torch.tensor([min(W, (i + 1) * tw) - i * tw for i in range(plan.bwd_tiles_x)])
-    evaluated = int((counts.long() * (rows[:, None] * cols[None, :])[None]).sum())
+    t_bwd_kernel = event_time(probe.reduce_kernel, args.steps)
+    t_fwd_kernel = event_time(probe.fwd_kernel, args.steps)
+    fwd_evaluated, evaluated = probe.evaluated()
     achieved = evaluated * f_bwd / t_bwd_kernel / 1e12
-    prof = C1_PROFILE if (args.config == "c1" and C == 3) else None
-    # The same for the forward (C <= 8: one list per wave rectangle of 32 columns x 2P rows, P = 16 for
-    # C <= 3 and 8 above, numbered row after row of rectangles over the 64 x 4P tiles' extent; behind the
-    # split partials in the forward's workspace).
-    fwd_evaluated = None
-    if C <= 8:
-        P = 16 if C <= 3 else 8
-        split = plan.fwd_split * B * (C + 1) * H * W * 4 if plan.fwd_split > 1 else 0
-        tx_n, ty_n = -(-W // 64), -(-H // (4 * P))
-        cols_n, rows_n = -(-W // 32), -(-H // (2 * P))
-        fc = fwd_ws.view(torch.int32)[(split + 15) // 16 * 4:][: B * plan.fwd_tiles].view(B, 2 * ty_n, 2 * tx_n)
-        fc = fc[:, :rows_n, :cols_n].cpu()
-        frows = torch.tensor([min(H, (i + 1) * 2 * P) - i * 2 * P for i in range(rows_n)])
-        fcols = torch.tensor([min(W, (i + 1) * 32) - i * 32 for i in range(cols_n)])
-        fwd_evaluated = int((fc.long() * (frows[None, :, None] * fcols[None, None, :])).sum())
+    prof = C1_PROFILE if (args.config == "c1" and C == 3 and C1_PROFILE["csrc_sha16"] == csrc_sha16()) else None
 
-    result = {
-        "metric": "gaussian_pixel_evals_per_sec_fwd_bwd",
-        "value": pairs / t_step,
-        "unit": "pairs/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": t_step * 1e3,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": f"{args.config}: gaussian_splatting_2d fwd+bwd, B={B} N={N} {H}x{W} C={C} fp32, "
-                               "linspace grids, seeded U/N inputs", "B": B, "N": N, "H": H, "W": W, "C": C},
-        "fwd_pairs_per_s": pairs / t_fwd,
-        "fwd_ms": t_fwd * 1e3,
-        "step_tflops": pairs * (f_fwd + f_bwd) / t_step / 1e12,
-        "step_frac_of_fp32_vector_peak": pairs * (f_fwd + f_bwd) / t_step / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
-        "step_frac_counting_evaluated_pairs": ((fwd_evaluated or pairs) * f_fwd + evaluated * f_bwd) / t_step / 1e12
-                                              / FP32_VECTOR_PEAK_TFLOPS,
+    result["step_frac_counting_evaluated_pairs"] = (((fwd_evaluated or pairs) * f_fwd + evaluated * f_bwd) / t_step / 1e12
+                                                    / FP32_VECTOR_PEAK_TFLOPS)
+    result.update({
         "roofline": {
             "bound": "valu",
-            "kernel": f"k_bwd_sep<{C},1> (backward per-Gaussian reduction)",
+            "kernel": f"k_bwd_sep<{C}> (backward per-Gaussian reduction)",
             "achieved": achieved,
             "peak": FP32_VECTOR_PEAK_TFLOPS,
             "unit": "TFLOP/s",
@@ -314,7 +337,7 @@ def run(args) -> int:
                     "published fp32 vector peak at 2.4 GHz; the kernels use plain fp32 VALU ops with VGPR-only operands, "
                     "v_exp_f32 counted as 1 FLOP.",
         },
-    }
+    })
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args.config, O, full=args.cpu_full)
@@ -322,19 +345,114 @@ def run(args) -> int:
     return 0
 
 
-def all_configs(steps: int, warmup: int) -> int:
+class KernelProbe:
+    """The two hot launches of one function-path problem on their own, through the C ABI with buffers kept
+    here: `reduce_kernel` = igs_gs2d_backward_reduce (the first call builds the tile lists, later ones
+    find them in place: the per-Gaussian reduction kernel alone), `fwd_kernel` = igs_gs2d_forward (tile
+    lists + kernel + combine), and the pairs both evaluated, read back from their tile lists."""
+
+    def __init__(self, d, B, N, H, W, C, dev):
+        import torch
+
+        from igs_amd import _lib
+        from igs_amd._splat import Grid, Splat, _ptr, _stream
+
+        self.torch, self._lib, self._ptr = torch, _lib, _ptr
+        self.dims = (B, N, H, W, C)
+        self.grid = grid = Grid(d["x_grid"], d["y_grid"], B)
+        self.op = op = Splat(B, N, C, grid, 1e-6, dev)
+        f32 = lambda t: t.detach().float().contiguous()
+        self.col = f32(d["colors"])
+        self.packed = op.pack_scale_rot(f32(d["positions"]), f32(d["scales"]), f32(d["rotations"]), f32(d["alphas"]),
+                                        self.col)
+        self.out, self.den = op.forward(self.packed)
+        self.pix = op._empty(op.plan.pix_bytes)
+        self.partial = op._empty(op.plan.partial_bytes)
+        self.lib = _lib.load()
+        self.st = _stream(dev)
+        _lib.check(self.lib.igs_gs2d_backward_prologue(_ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode,
+                                                       _ptr(grid.flag), _ptr(self.out), _ptr(self.den),
+                                                       _ptr(f32(d["grad_out"])), B, N, H, W, C, 1e-6, _ptr(self.pix),
+                                                       int(op.plan.pix_bytes), self.st), "prologue")
+        self.built = False
+        self.fwd_ws = op._empty(op.plan.fwd_ws_bytes)
+        self.fwd_out, self.fwd_den = op._new(B, C, H, W), op._new(B, H, W)
+
+    def reduce_kernel(self):
+        B, N, H, W, C = self.dims
+        g, op, _ptr = self.grid, self.op, self._ptr
+        mode = g.mode | (self._lib.IGS_OPT_LISTS_BUILT if self.built else 0)
+        self.built = True
+        self._lib.check(self.lib.igs_gs2d_backward_reduce(_ptr(self.packed), _ptr(self.col), _ptr(g.y), g.strides, mode,
+                                                          _ptr(g.flag), B, N, H, W, C, _ptr(self.pix),
+                                                          int(op.plan.pix_bytes), _ptr(self.partial),
+                                                          int(op.plan.partial_bytes), self.st), "reduce")
+
+    def fwd_kernel(self):
+        B, N, H, W, C = self.dims
+        g, op, _ptr = self.grid, self.op, self._ptr
+        self._lib.check(self.lib.igs_gs2d_forward(_ptr(self.packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode,
+                                                  _ptr(g.flag), B, N, H, W, C, 1e-6, _ptr(self.fwd_out),
+                                                  _ptr(self.fwd_den), _ptr(self.fwd_ws), int(op.plan.fwd_ws_bytes),
+                                                  self.st), "forward")
+
+    def evaluated(self):
+        """(forward, backward) pairs evaluated, after both launches ran: a launch's per-tile Gaussian lists
+        (counts behind the pixel records / the split partials in its workspace) times the pixels of each
+        tile; pairs that are not listed are skipped.  Forward: None for C > 8 where its workgroup tiles are
+        not the backward's 32 x 32."""
+        torch = self.torch
+        B, N, H, W, C = self.dims
+        plan = self.op.plan
+        if not self.built:
+            self.reduce_kernel()
+        self.fwd_kernel()
+        torch.cuda.synchronize()
+        scratch = (B * H * plan.w_padded * plan.pix_stride + B * plan.w_padded) * 4
+        counts = self.pix.view(torch.int32)[(scratch + 15) // 16 * 4:][: B * plan.bwd_tiles]
+        counts = counts.view(B, -1, plan.bwd_tiles_x).cpu()
+        rows = torch.tensor([min(H, (i + 1) * plan.bwd_per_tile) - i * plan.bwd_per_tile for i in range(counts.shape[1])])
+        tw = plan.bwd_tile_w
+        cols = torch.tensor([min(W, (i + 1) * tw) - i * tw for i in range(plan.bwd_tiles_x)])
+        bwd = int((counts.long() * (rows[:, None] * cols[None, :])[None]).sum())
+        fwd = None
+        if C <= 8:   # one list per wave rectangle of 32 columns x 2P rows, numbered row after row of rectangles
+            P = 16 if C <= 3 else 8
+            split = plan.fwd_split * B * (C + 1) * H * W * 4 if plan.fwd_split > 1 else 0
+            tx_n, ty_n = -(-W // 64), -(-H // (4 * P))
+            cols_n, rows_n = -(-W // 32), -(-H // (2 * P))
+            fc = self.fwd_ws.view(torch.int32)[(split + 15) // 16 * 4:][: B * plan.fwd_tiles].view(B, 2 * ty_n, 2 * tx_n)
+            fc = fc[:, :rows_n, :cols_n].cpu()
+            frows = torch.tensor([min(H, (i + 1) * 2 * P) - i * 2 * P for i in range(rows_n)])
+            fcols = torch.tensor([min(W, (i + 1) * 32) - i * 32 for i in range(cols_n)])
+            fwd = int((fc.long() * (frows[None, :, None] * fcols[None, None, :])).sum())
+        elif plan.fwd_tiles == plan.bwd_tiles and plan.bwd_per_tile == 32:
+            # one list per workgroup tile of 32 x 32 pixels, the backward's tiling
+            split = plan.fwd_split * B * (C + 1) * H * W * 4 if plan.fwd_split > 1 else 0
+            fc = self.fwd_ws.view(torch.int32)[(split + 15) // 16 * 4:][: B * plan.fwd_tiles]
+            fc = fc.view(B, -1, plan.bwd_tiles_x).cpu()
+            fwd = int((fc.long() * (rows[:, None] * cols[None, :])[None]).sum())
+        return fwd, bwd
+
+
+def all_configs(steps: int, warmup: int, no_cpu: bool = False) -> int:
     """Forward and forward+backward wall time of the five configurations through the public API
-    (allocation included), pairs/s counting all B N H W pairs as scripts/profiling.py:199-211 does,
-    and the fraction of the fp32 vector peak by the 42 + 6 C FLOP/pair model (above 1 is possible
-    where culling skips pairs).  "c0 1 thread" is the c0 step under
+    (allocation included), pairs/s counting all B N H W pairs as scripts/profiling.py:199-211 does, the
+    pairs the two hot kernels evaluated (read back from their tile lists) and the fraction of the fp32
+    vector peak that the 12 + 2 C / 30 + 4 C FLOP-per-pair model gives on those (counting all pairs it
+    exceeds 1 where culling skips most of them).  "c0 1 thread" is the c0 step under
     torch.autograd.set_multithreading_enabled(False).  The "fit step" rows are the graph-replayed fused iteration of
     igs_amd.fit on the same problem: at c0 the public call is bound by the host's per-call cost
-    (Python, torch allocation, autograd: 0.13-0.25 ms depending on the box), the replay is not."""
+    (Python, torch allocation, autograd: 0.13-0.25 ms depending on the box), the replay is not.
+    CPU column: the reference's chunked torch autograd path restated (oracle/chunked_cpu.py) on the host
+    cores for the configurations that name it, c0 and c3 (through the module's linear head): 1 warm-up,
+    then the median of 3 runs of forward + backward."""
     import torch
 
     import igs_amd
     from igs_amd.fit import GaussianImageFit
     from oracle import gs2d_oracle as O
+    from oracle.chunked_cpu import render_chunked_cpu
 
     dev = torch.device("cuda:0")
     names = ("positions", "colors", "scales", "rotations", "alphas")
@@ -359,8 +477,19 @@ def all_configs(steps: int, warmup: int) -> int:
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / n
 
+    def cpu_median(fn):
+        fn()
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[1]
+
+    nan = float("nan")
     rows = []
     for cfg in ("c0", "c1", "c2", "c3", "c4"):
+        cpu_s = nan
         if cfg == "c3":
             torch.manual_seed(1003)
             m = igs_amd.GaussianSplatting2D(32, 1024).to(dev)
@@ -376,6 +505,27 @@ def all_configs(steps: int, warmup: int) -> int:
                 m(x, size=(256, 256))[0].backward(go)
                 x.grad = None
                 m.zero_grad(set_to_none=True)
+
+            # the same Gaussians as function-path inputs, for the tile lists (and for the CPU path)
+            with torch.no_grad():
+                f = m.proj(x).view(B, N, 6 + C)
+                xs, ys = m.xy_grid((H, W), device=dev)
+                d = {"positions": f[..., :2].contiguous(), "scales": (f[..., 2:4].exp() + 1e-6).contiguous(),
+                     "rotations": f[..., 4].contiguous(), "alphas": torch.ones(B, N, device=dev),
+                     "colors": f[..., 6:].contiguous(), "grad_out": go,
+                     "x_grid": xs[None].expand(B, 1, H, W), "y_grid": ys[None].expand(B, 1, H, W)}
+            if not no_cpu:
+                wc, bc, xc, goc = m.proj.weight.detach().cpu(), m.proj.bias.detach().cpu(), x.detach().cpu(), go.cpu()
+                xg, yg = d["x_grid"].cpu().contiguous(), d["y_grid"].cpu().contiguous()
+
+                def cpu_step():
+                    w, bb, xi = (t.clone().requires_grad_(True) for t in (wc, bc, xc))
+                    fc = torch.nn.functional.linear(xi, w, bb).view(B, N, 6 + C)
+                    out = render_chunked_cpu(fc[..., :2], fc[..., 6:], fc[..., 2:4].exp() + 1e-6, fc[..., 4],
+                                             torch.ones(B, N), xg, yg)
+                    out.backward(goc)
+
+                cpu_s = cpu_median(cpu_step)
         else:
             d = {k: v.to(dev) for k, v in O.make_config_inputs(cfg).items()}
             B, N, C = d["colors"].shape
@@ -392,12 +542,22 @@ def all_configs(steps: int, warmup: int) -> int:
                 igs_amd.gaussian_splatting_2d(*(lv[k] for k in names), d["x_grid"], d["y_grid"]).backward(d["grad_out"])
                 for v in lv.values():
                     v.grad = None
+            if cfg == "c0" and not no_cpu:
+                dc = {k: v.cpu() for k, v in d.items()}
+                xg, yg = dc["x_grid"].contiguous(), dc["y_grid"].contiguous()
+
+                def cpu_step():
+                    l = {k: dc[k].clone().requires_grad_(True) for k in names}
+                    render_chunked_cpu(*(l[k] for k in names), xg, yg).backward(dc["grad_out"])
+
+                cpu_s = cpu_median(cpu_step)
         n = max(3, steps // 3) if cfg == "c4" else steps
-        rows.append((cfg, B, N, H, W, C, timeit(fwd, n), timeit(step, n)))
+        ev_f, ev_b = KernelProbe(d, B, N, H, W, C, dev).evaluated()
+        rows.append((cfg, B, N, H, W, C, timeit(fwd, n), timeit(step, n), ev_f, ev_b, cpu_s))
         if cfg == "c0":   # the same public call with autograd's backward run on the calling thread: the hand-over to
             # the engine's device thread and back is 60-130 us of the host's time per step on the boxes seen
             with torch.autograd.set_multithreading_enabled(False):
-                rows.append((cfg + " 1 thread", B, N, H, W, C, float("nan"), timeit(step, n)))
+                rows.append((cfg + " 1 thread", B, N, H, W, C, nan, timeit(step, n), ev_f, ev_b, nan))
         if cfg in ("c0", "c2"):   # the fused fit iteration (render, MSE, backward, AdamW) on the same problem,
             # replayed from a HIP graph: the step without the host's per-call cost
             block = torch.cat([d["positions"], d["scales"].log(), d["rotations"][..., None],
@@ -405,13 +565,21 @@ def all_configs(steps: int, warmup: int) -> int:
             fit = GaussianImageFit(block, O.smooth_noise_target(H, W, seed=1002).to(dev), d["x_grid"], d["y_grid"],
                                    lr=min(0.05 * 4096 / N, 0.03))
             fit.capture()
-            rows.append((cfg + " fit step", B, N, H, W, C, float("nan"), timeit(fit.step, n)))
-    print("%-12s %3s %6s %4s %4s %3s %10s %12s %14s %10s" % ("config", "B", "N", "H", "W", "C", "fwd ms", "fwd+bwd ms",
-                                                           "pairs/s", "of peak"))
-    for cfg, B, N, H, W, C, tf, t in rows:
+            rows.append((cfg + " fit step", B, N, H, W, C, nan, timeit(fit.step, n), ev_f, ev_b, nan))
+    print("%-12s %3s %6s %4s %4s %3s %9s %11s %11s %10s %10s %9s %9s %10s" % (
+        "config", "B", "N", "H", "W", "C", "fwd ms", "fwd+bwd ms", "pairs/s", "fwd pairs", "bwd pairs", "evaluated",
+        "of peak", "CPU f+b s"))
+    for cfg, B, N, H, W, C, tf, t, ev_f, ev_b, cpu_s in rows:
         pairs = B * N * H * W
-        print("%-12s %3d %6d %4d %4d %3d %10.3f %12.3f %14.3e %10.2f" % (cfg, B, N, H, W, C, tf * 1e3, t * 1e3, pairs / t,
-                                                                       pairs * (42 + 6 * C) / t / 1e12 / FP32_VECTOR_PEAK_TFLOPS))
+        ev_f = pairs if ev_f is None else ev_f   # (forward lists not read back: counted in full)
+        flop = ev_f * (12 + 2 * C) + ev_b * (30 + 4 * C)
+        print("%-12s %3d %6d %4d %4d %3d %9.3f %11.3f %11.3e %10.3e %10.3e %8.1f%% %9.2f %10.2f" % (
+            cfg, B, N, H, W, C, tf * 1e3, t * 1e3, pairs / t, ev_f, ev_b, 100.0 * (ev_f + ev_b) / (2 * pairs),
+            flop / t / 1e12 / FP32_VECTOR_PEAK_TFLOPS, cpu_s))
+    model, physical = host_cpu()
+    print("pairs/s counts all B N H W pairs; of peak = (12 + 2 C) x forward pairs + (30 + 4 C) x backward pairs evaluated "
+          "/ fwd+bwd time / %.1f TFLOP/s; CPU: %d torch threads on %s (%d "
+          "physical cores visible)" % (FP32_VECTOR_PEAK_TFLOPS, torch.get_num_threads(), model, physical))
     return 0
 
 

@@ -15,10 +15,13 @@ from .gs2d import (  # noqa: F401
     naive_gaussian_2d,
 )
 
+from ._splat import exact, library_options  # noqa: F401,E402
 from .fit import GaussianImageFit  # noqa: F401,E402
 from .reg import koleo_diversity_loss  # noqa: F401,E402
 
 __all__ = [
+    "exact",
+    "library_options",
     "GaussianImageFit",
     "koleo_diversity_loss",
     "GaussianSplatting2D",

@@ -17,6 +17,7 @@ stream; every FLOP happens in libigs_hip.so.
 from __future__ import annotations
 
 import contextlib
+import contextvars
 import functools
 from typing import List, Optional, Sequence, Tuple
 
@@ -32,9 +33,6 @@ KIND_SCALE_ROT = 1
 KIND_FEATURE = 2
 
 
-# igs_option bits OR-ed into the grid_mode word of every Grid built while `library_options` is active
-_option_bits = 0
-
 # Bound on what skipping far-away (Gaussian, pixel) pairs may change in an output element, as a
 # fraction of the largest colour magnitude: the pack calls get the skip weight w =
 # igs_gs2d_skip_weight(N, eps, SKIP_TOLERANCE) = SKIP_TOLERANCE * eps / (2 N) and the skip fraction
@@ -43,32 +41,44 @@ _option_bits = 0
 # 1e-6 + 1e-5 |ref| against the plain expression; 1e-7 leaves that budget to the fp32 rounding.
 # 0 skips exact zeros only (bit-identical to evaluating every pair).
 SKIP_TOLERANCE = 1e-7
-_skip_tolerance = SKIP_TOLERANCE
+
+# (igs_option bits OR-ed into the grid_mode word of every Grid built, skip tolerance) in effect for the
+# calling thread (and asyncio task): a context variable, so that two threads, or a `with` block and
+# another thread's calls, do not see each other's settings.  Both are read when a call's forward
+# is set up, on the caller's thread; the backward, whichever thread autograd runs it on, uses what
+# its forward recorded (the grid's mode word, the packed buffer's skip settings).
+_options = contextvars.ContextVar("igs_amd_library_options", default=(0, SKIP_TOLERANCE))
 
 
 @contextlib.contextmanager
 def library_options(no_cull: bool = False, bin_levels: Optional[int] = None,
                     skip_tolerance: Optional[float] = None):
-    """Problems set up inside this context run with the given igs_option bits of
+    """Problems set up inside this context, by this thread, run with the given igs_option bits of
     include/igs_hip.h -- `no_cull` lists every Gaussian for every pixel tile (the reference point
     for what culling changes), `bin_levels` = 1 | 2 forces the one- or two-level construction
     of the tile lists -- and with the given `skip_tolerance` (see SKIP_TOLERANCE; 0 = only pairs
     whose weight is exactly zero are skipped).  The bits and the skip weight travel as explicit
     arguments of each library call; the library itself holds no such state."""
-    global _option_bits, _skip_tolerance
     bits = _lib.IGS_OPT_NO_CULL if no_cull else 0
     if bin_levels is not None:
         bits |= {1: _lib.IGS_OPT_BIN_LEVELS_1, 2: _lib.IGS_OPT_BIN_LEVELS_2}[int(bin_levels)]
-    saved = (_option_bits, _skip_tolerance)
-    _option_bits |= bits   # nested contexts add up
+    old_bits, tolerance = _options.get()
     if skip_tolerance is not None:
         if not 0.0 <= float(skip_tolerance) < 1.0:
             raise ValueError("skip_tolerance must be in [0, 1)")
-        _skip_tolerance = float(skip_tolerance)
+        tolerance = float(skip_tolerance)
+    token = _options.set((old_bits | bits, tolerance))   # nested contexts add up
     try:
         yield
     finally:
-        _option_bits, _skip_tolerance = saved
+        _options.reset(token)
+
+
+def exact():
+    """Context in which the calling thread's renders skip exact zeros only: every (Gaussian, pixel)
+    pair whose fp32 weight is not exactly zero is evaluated, as the reference does
+    (`library_options(skip_tolerance=0)`)."""
+    return library_options(skip_tolerance=0.0)
 
 
 @functools.lru_cache(maxsize=256)
@@ -79,7 +89,7 @@ def _skip_weight(N: int, eps: float, tolerance: float) -> Tuple[float, float]:
 
 def skip_weight(N: int, eps: float) -> Tuple[float, float]:
     """(skip_weight, skip_fraction) the pack calls of a problem get under the current skip tolerance."""
-    return _skip_weight(int(N), float(eps), float(_skip_tolerance))
+    return _skip_weight(int(N), float(eps), float(_options.get()[1]))
 
 
 # The host side of a call is what bounds small problems (a 512-Gaussian 256x256 forward+backward
@@ -189,9 +199,9 @@ class Grid:
         # flag that the kernels read, so there is no host synchronisation either way.
         self.flag = None
         if self.sx[1] == 0 and self.sy[2] == 0:
-            self.mode = _lib.IGS_GRID_SEPARABLE | _option_bits
+            self.mode = _lib.IGS_GRID_SEPARABLE | _options.get()[0]
         else:
-            self.mode = _lib.IGS_GRID_AUTO | _option_bits
+            self.mode = _lib.IGS_GRID_AUTO | _options.get()[0]
             self.flag = torch.empty(1, dtype=torch.int32, device=x.device)
             _lib.check(_lib.load().igs_gs2d_grid_classify(_ptr(self.x), _ptr(self.y), self.strides, B, self.H,
                                                           self.W, _ptr(self.flag), _stream(x.device)),

@@ -103,6 +103,46 @@ __device__ __forceinline__ void write_brec(float4* brec, size_t i, const SepTerm
     brec[i] = t.regular ? make_float4(t.sA, t.skA, t.D2, 0.0f) : make_float4(0.0f, 0.0f, 0.0f, 1.0f);
 }
 
+// Stores the records of one Gaussian from registers: `rec` holds the plain record (px, py, A', B2', D',
+// alpha, alpha*c_0..C-1, zeros behind); every index is a compile-time constant after unrolling, and a
+// lane writes float4s.  The plain record also gets the y range of the reach box where it has two spare
+// floats; the forward record of the separable kernels (RSF > 0) is the same with the completed square in
+// place of A', B2', D', and behind the colours the tag and A', B2', D'.
+__device__ __forceinline__ void store_records(float (&rec)[kZeroRecFloats], int C, int RS, int RSF, float py, float2 ext,
+                                              const SepTerms& t, float* __restrict__ r, float* __restrict__ fr) {
+    const float Ap = rec[2], B2p = rec[3], Dp = rec[4];
+    if (RS >= 8 + C) {  // room in the record: the y range of the box travels with it
+#pragma unroll
+        for (int c = 6; c < kZeroRecFloats - 1; ++c)
+            if (c == 6 + C) {
+                rec[c] = py - ext.y;
+                rec[c + 1] = py + ext.y;
+            }
+    }
+    float4* r4 = reinterpret_cast<float4*>(r);  // records are 4 k floats apart behind a 16-byte aligned base
+#pragma unroll
+    for (int q = 0; q < kZeroRecFloats / 4; ++q)
+        if (4 * q < RS) r4[q] = make_float4(rec[4 * q], rec[4 * q + 1], rec[4 * q + 2], rec[4 * q + 3]);
+    if (RSF == 0) return;
+    rec[2] = t.sD;
+    rec[3] = t.skD;
+    rec[4] = t.A2;
+#pragma unroll
+    for (int c = 6; c < kZeroRecFloats - 5; ++c)
+        if (c == 6 + C) {
+            rec[c] = t.regular ? t.sD : __builtin_nanf("");
+            rec[c + 1] = Ap;
+            rec[c + 2] = B2p;
+            rec[c + 3] = Dp;
+            rec[c + 4] = 0.0f;
+            rec[c + 5] = 0.0f;
+        }
+    float4* f4 = reinterpret_cast<float4*>(fr);
+#pragma unroll
+    for (int q = 0; q < kZeroRecFloats / 4; ++q)
+        if (4 * q < RSF) f4[q] = make_float4(rec[4 * q], rec[4 * q + 1], rec[4 * q + 2], rec[4 * q + 3]);
+}
+
 // One thread per record.  Record: px, py, A', B2', D', alpha, alpha*c_0.. (padded to x4)
 // with A' = k A, B2' = 2 k B, D' = k D, k = -0.5 log2 e.  Records N..Np-1 are zero.
 template <bool kScaleRot>
@@ -187,41 +227,9 @@ __global__ __launch_bounds__(kThreads) void k_pack(const float* __restrict__ pos
     }
     const float2 ext = reach_extent(px, py, sxx, syy, bounded && fin, skip_limit(limit, al));
     write_bin_record(boxes, (size_t)b * Np + n, px, py, ext, rec[2], rec[3], rec[4], al);
-    if (RS >= 8 + C) {  // room in the record: the y range of the box travels with it
-#pragma unroll
-        for (int c = 6; c < kZeroRecFloats - 1; ++c)
-            if (c == 6 + C) {
-                rec[c] = py - ext.y;
-                rec[c + 1] = py + ext.y;
-            }
-    }
-    float4* r4 = reinterpret_cast<float4*>(r);  // records are RS = 4 k floats apart behind a 16-byte aligned base
-#pragma unroll
-    for (int q = 0; q < kZeroRecFloats / 4; ++q)
-        if (4 * q < RS) r4[q] = make_float4(rec[4 * q], rec[4 * q + 1], rec[4 * q + 2], rec[4 * q + 3]);
-    // the separable kernels' records: the same with the completed square in place of A', B2', D' and a
-    // tag behind the colours
     const SepTerms t = sep_terms(A, Bc, D, det, bounded && fin && isfinite(px) && isfinite(py));
     write_brec(brecs, (size_t)b * Np + n, t);
-    if (RSF == 0) return;
-    const float Ap = rec[2], B2p = rec[3], Dp = rec[4];
-    rec[2] = t.sD;
-    rec[3] = t.skD;
-    rec[4] = t.A2;
-#pragma unroll
-    for (int c = 6; c < kZeroRecFloats - 5; ++c)
-        if (c == 6 + C) {
-            rec[c] = t.regular ? t.sD : __builtin_nanf("");
-            rec[c + 1] = Ap;
-            rec[c + 2] = B2p;
-            rec[c + 3] = Dp;
-            rec[c + 4] = 0.0f;
-            rec[c + 5] = 0.0f;
-        }
-    float4* f4 = reinterpret_cast<float4*>(fr);
-#pragma unroll
-    for (int q = 0; q < kZeroRecFloats / 4; ++q)
-        if (4 * q < RSF) f4[q] = make_float4(rec[4 * q], rec[4 * q + 1], rec[4 * q + 2], rec[4 * q + 3]);
+    store_records(rec, C, RS, RSF, py, ext, t, r, fr);
 }
 
 // Module head fused into the pack: reads gs_feature rows [px, py, log_s0, log_s1, theta,
@@ -267,43 +275,30 @@ __global__ __launch_bounds__(kThreads) void k_pack_feature(const float* __restri
         px += pos_off[2 * i];
         py += pos_off[2 * i + 1];
     }
-    r[0] = px;
-    r[1] = py;
-    r[2] = (float)(k * A);
-    r[3] = (float)(2.0 * k * Bc);
-    r[4] = (float)(k * D);
-    r[5] = 1.0f;
-    bool fin = isfinite(r[2]) && isfinite(r[3]) && isfinite(r[4]);
-    for (int c = 0; c < Cp; ++c) {
+    float rec[kZeroRecFloats];
+#pragma unroll
+    for (int c = 0; c < kZeroRecFloats; ++c) rec[c] = 0.0f;
+    rec[0] = px;
+    rec[1] = py;
+    rec[2] = (float)(k * A);
+    rec[3] = (float)(2.0 * k * Bc);
+    rec[4] = (float)(k * D);
+    rec[5] = 1.0f;
+    bool fin = isfinite(rec[2]) && isfinite(rec[3]) && isfinite(rec[4]);
+#pragma unroll
+    for (int c = 0; c < IGS_MAX_CHANNELS; ++c) {
         const float col = c < C ? f[6 + c] : 0.0f;
-        r[6 + c] = col;
-        colors_out[i * Cp + c] = col;
+        rec[6 + c] = col;
+        if (c < Cp) colors_out[i * Cp + c] = col;
         fin = fin && isfinite(col);
     }
-    for (int c = 6 + Cp; c < RS; ++c) r[c] = 0.0f;
-    const float2 ext = reach_extent(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1,
-                                    fin && v0 > 0.0 && v1 > 0.0, skip_limit(limit, 1.0f));
-    write_bin_record(boxes, (size_t)b * Np + n, px, py, ext, r[2], r[3], r[4], 1.0f);
-    if (RS >= 8 + Cp) {
-        r[6 + Cp] = py - ext.y;
-        r[7 + Cp] = py + ext.y;
-    }
-    // the separable kernels' records (see sep_terms)
-    const SepTerms t = sep_terms(A, Bc, D, i0 * i1, fin && v0 > 0.0 && v1 > 0.0 && isfinite(px) && isfinite(py));
+    const bool bounded = fin && v0 > 0.0 && v1 > 0.0;
+    const float2 ext = reach_extent(px, py, cs * cs * v0 + sn * sn * v1, sn * sn * v0 + cs * cs * v1, bounded,
+                                    skip_limit(limit, 1.0f));
+    write_bin_record(boxes, (size_t)b * Np + n, px, py, ext, rec[2], rec[3], rec[4], 1.0f);
+    const SepTerms t = sep_terms(A, Bc, D, i0 * i1, bounded && isfinite(px) && isfinite(py));
     write_brec(brecs, (size_t)b * Np + n, t);
-    if (RSF == 0) return;
-    fr[0] = px;
-    fr[1] = py;
-    fr[2] = t.sD;
-    fr[3] = t.skD;
-    fr[4] = t.A2;
-    fr[5] = 1.0f;
-    for (int c = 0; c < Cp; ++c) fr[6 + c] = c < C ? f[6 + c] : 0.0f;
-    for (int c = 6 + Cp; c < RSF; ++c) fr[c] = 0.0f;
-    fr[6 + Cp] = t.regular ? t.sD : __builtin_nanf("");
-    fr[7 + Cp] = r[2];
-    fr[8 + Cp] = r[3];
-    fr[9 + Cp] = r[4];
+    store_records(rec, Cp, RS, RSF, py, ext, t, r, fr);
 }
 
 // ----------------------------------------------------------------------------- binning

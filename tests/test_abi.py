@@ -392,3 +392,28 @@ def test_koleo_host_surface():
     out = torch.ops.igs_amd.koleo_fwd(torch.empty(2, 50, 9, device="meta"))
     assert out[0].shape == () and out[1].shape == (igs_amd.reg.saved_numel(2, 50, 9),)
     assert torch.ops.igs_amd.koleo_bwd(out[1], out[0], 2, 50, 9).shape == (2, 50, 9)
+
+
+def test_library_options_are_per_thread():
+    """`library_options` / `exact` change what the calling thread's renders may skip, not another thread's
+    (nor what the same thread does after the block)."""
+    import threading
+
+    import igs_amd
+    from igs_amd import _lib, _splat
+
+    default = (0, _splat.SKIP_TOLERANCE)
+    assert _splat._options.get() == default
+    seen = []
+    with igs_amd.exact():
+        assert _splat._options.get() == (0, 0.0)
+        with igs_amd.library_options(no_cull=True):   # nested contexts add up
+            assert _splat._options.get() == (_lib.IGS_OPT_NO_CULL, 0.0)
+            t = threading.Thread(target=lambda: seen.append(_splat._options.get()))
+            t.start()
+            t.join()
+        assert _splat._options.get() == (0, 0.0)
+    assert seen == [default] and _splat._options.get() == default
+    with pytest.raises(ValueError):
+        with igs_amd.library_options(skip_tolerance=1.5):
+            pass
