@@ -218,7 +218,7 @@ class Splat:
         self.grid, self.eps, self.device = grid, float(eps), device
         self.plan = _lib.plan(B, N, grid.H, grid.W, self.Cp, grid.mode)
         self.skip_weight = skip_weight(N, self.eps)
-        self.shared = None   # (pix, partial) with the tile lists in place, after forward_shared_lists
+        self.shared = None   # (pix, partial) with the tile lists in place, after forward_train
         self.stream = None
         self.use_current_stream()
 
@@ -267,20 +267,21 @@ class Splat:
                                              int(p.fwd_ws_bytes), self.stream), "igs_gs2d_forward")
         return out, den
 
-    def forward_shared_lists(self, packed: Tensor) -> Tuple[Tensor, Tensor]:
-        """The forward of a step whose backward will follow, where the plan says that both passes can
-        run over one set of tile lists (`plan.lists_shared`): the lists are built once, in the
-        backward's workspaces, which this object keeps for `backward_partials*`."""
+    def forward_train(self, packed: Tensor) -> Tuple[Tensor, Tensor]:
+        """The forward of a step whose backward will follow: the backward's tile lists are built now,
+        in the backward's workspaces, which this object keeps for `backward_partials*` -- one set of
+        lists for both passes where the plan says their tilings coincide (`plan.lists_shared`), else
+        beside the forward's own, in the same launch."""
         g, p = self.grid, self.plan
         out = self._new(self.B, self.Cp, g.H, g.W)
         den = self._new(self.B, g.H, g.W)
         ws = self._empty(p.fwd_ws_bytes) if p.fwd_ws_bytes else None
         pix = self._empty(p.pix_bytes)
         partial = self._empty(p.partial_bytes)
-        _lib.check(self.lib.igs_gs2d_forward_shared_lists(
+        _lib.check(self.lib.igs_gs2d_forward_train(
             _ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), self.B, self.N, g.H, g.W, self.Cp,
             self.eps, _ptr(out), _ptr(den), _ptr(ws), int(p.fwd_ws_bytes), _ptr(pix), int(p.pix_bytes), _ptr(partial),
-            int(p.partial_bytes), self.stream), "igs_gs2d_forward_shared_lists")
+            int(p.partial_bytes), self.stream), "igs_gs2d_forward_train")
         self.shared = (pix, partial)
         return out, den
 
@@ -436,7 +437,8 @@ def run_forward(kind: int, params: Sequence[Tensor], x: Tensor, y: Tensor, eps: 
             off = _f32c(params[1]) if len(params) == 2 else None
             packed, col = op.pack_feature(feat, off)
             keep = (feat,)
-        out, den = op.forward_shared_lists(packed) if (train and op.plan.lists_shared) else op.forward(packed)
+        general = (grid.mode & 0xff) == _lib.IGS_GRID_GENERAL   # (no tile lists on general grids)
+        out, den = op.forward_train(packed) if (train and not general) else op.forward(packed)
     return op, keep, packed, col, out, den
 
 

@@ -12,7 +12,7 @@ constexpr int kThreads = 256;
 #define IGS_FWD_SEP_P 16
 #endif
 #ifndef IGS_BWD_G
-#define IGS_BWD_G 2
+#define IGS_BWD_G 1
 #endif
 #ifndef IGS_FWD_WAVES
 #define IGS_FWD_WAVES 8
@@ -20,8 +20,10 @@ constexpr int kThreads = 256;
 #ifndef IGS_FWD_MAX_SPLIT
 #define IGS_FWD_MAX_SPLIT 64
 #endif
+// (backward: four waves per SIMD wanted; only small problems are split further than the 32-row tiles that
+// keep the lists short: B=1 N=2048 256x256 fit step 159 / 145 / 141 / 145 us with 16 / 8 / 4 / 2)
 #ifndef IGS_BWD_WAVES
-#define IGS_BWD_WAVES 16
+#define IGS_BWD_WAVES 4
 #endif
 // rows per lane in the separable forward: as many as the accumulator VGPRs (P x (C+1)) allow
 __host__ __device__ constexpr int fwd_sep_p(int C) { return C <= 3 ? IGS_FWD_SEP_P : (C <= 8 ? 8 : 4); }
@@ -32,9 +34,9 @@ __host__ __device__ constexpr int fwd_gen_p(int C) { return C <= 4 ? 8 : 4; }
 #define IGS_BWD_GEN_G 4
 #endif
 __host__ __device__ constexpr int bwd_gen_g(int C) { return C <= 4 ? IGS_BWD_GEN_G : 2; }
-// Gaussians per lane, separable backward: two independent chains per pixel record where the sums of two
-// fit in registers (C <= 4); with wide colour vectors one (B=4, N=32768, 384x640, C=16: 3.38 -> 3.08 ms)
-__host__ __device__ constexpr int bwd_sep_g(int C) { return C <= 4 ? IGS_BWD_G : 1; }
+// Gaussians per lane, separable backward: one (a tile's last group of list positions is half empty on
+// average, and its idle lanes cost more with two per lane than sharing the pixel records' reads saves)
+__host__ __device__ constexpr int bwd_sep_g(int) { return IGS_BWD_G; }
 
 __host__ __device__ constexpr int rec_stride_of(int C) { return (6 + C + 3) & ~3; }
 // Records of the separable kernels (see sep_terms): the forward's px, py, sD, skD, A'', alpha,

@@ -6,35 +6,49 @@
 // Decoupled-weight-decay Adam over one flat parameter block, the update of torch.optim.AdamW
 // (amsgrad off) as the fit script configures it (scripts/2dgs_img_comp.py:186-193).  The
 // step counter and learning rate live in device memory so that a captured graph advances:
-//   state = {lr, t, 1 - beta1^t, sqrt(1 - beta2^t)}; lr is written by the host, the rest by
-// k_adamw_tick (one thread, powers in double).
-__global__ void k_adamw_tick(float* __restrict__ state, float beta1, float beta2) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    const float t = state[1] + 1.0f;
-    state[1] = t;
-    state[2] = (float)(1.0 - pow((double)beta1, (double)t));
-    state[3] = (float)sqrt(1.0 - pow((double)beta2, (double)t));
-}
-
+//   state = {lr, t, 1 - beta1^t, sqrt(1 - beta2^t), ticket, -, -, -}; lr is written by the host.
+// Every workgroup reads t, forms the bias corrections of step t + 1 (one thread, powers in double)
+// and updates its elements; the workgroup that finishes last (integer ticket, zero before and after
+// the launch) writes t + 1 and the corrections back, when no workgroup needs the old t any more.
+constexpr int kAdamStateFloats = 8;
 __global__ __launch_bounds__(kThreads) void k_adamw(float* __restrict__ param,
                                                     const float* __restrict__ grad,
                                                     float* __restrict__ exp_avg,
                                                     float* __restrict__ exp_avg_sq, long n,
-                                                    const float* __restrict__ state, float beta1,
+                                                    float* __restrict__ state, float beta1,
                                                     float beta2, float eps, float weight_decay) {
+    __shared__ float corr[3];  // t + 1, 1 - beta1^(t+1), sqrt(1 - beta2^(t+1))
+    if (threadIdx.x == 0) {
+        const float t = state[1] + 1.0f;
+        corr[0] = t;
+        corr[1] = (float)(1.0 - pow((double)beta1, (double)t));
+        corr[2] = (float)sqrt(1.0 - pow((double)beta2, (double)t));
+    }
+    __syncthreads();
     const long i = (long)blockIdx.x * kThreads + threadIdx.x;
-    if (i >= n) return;
-    const float lr = state[0], bc1 = state[2], bc2_sqrt = state[3];
-    const float g = grad[i];
-    float p = param[i] * (1.0f - lr * weight_decay);
-    float m = exp_avg[i];
-    m = fmaf(g - m, 1.0f - beta1, m);
-    const float v = fmaf(g * g, 1.0f - beta2, exp_avg_sq[i] * beta2);
-    const float denom = sqrtf(v) / bc2_sqrt + eps;
-    p -= (lr / bc1) * (m / denom);
-    param[i] = p;
-    exp_avg[i] = m;
-    exp_avg_sq[i] = v;
+    if (i < n) {
+        const float lr = state[0], bc1 = corr[1], bc2_sqrt = corr[2];
+        const float g = grad[i];
+        float p = param[i] * (1.0f - lr * weight_decay);
+        float m = exp_avg[i];
+        m = fmaf(g - m, 1.0f - beta1, m);
+        const float v = fmaf(g * g, 1.0f - beta2, exp_avg_sq[i] * beta2);
+        const float denom = sqrtf(v) / bc2_sqrt + eps;
+        p -= (lr / bc1) * (m / denom);
+        param[i] = p;
+        exp_avg[i] = m;
+        exp_avg_sq[i] = v;
+    }
+    __syncthreads();  // every thread of the workgroup has read what it needs of `state`
+    if (threadIdx.x == 0) {
+        unsigned int* ticket = reinterpret_cast<unsigned int*>(state + 4);
+        if (atomicAdd(ticket, 1u) == gridDim.x - 1u) {  // every workgroup has read t
+            state[1] = corr[0];
+            state[2] = corr[1];
+            state[3] = corr[2];
+            *ticket = 0u;
+        }
+    }
 }
 
 // ----------------------------------------------------------------------------- position penalty

@@ -404,6 +404,27 @@ int launch_bins(BinArgs fine, int B, bool levels2, const BinPlace& coarse, int* 
     return launch_bin(fine, 1, B, st);
 }
 
+// One launch for two single-level, one-list-per-tile binnings over the same Gaussians (k_bin_pair).
+// Returns -1 (and launches nothing) where the two do not fit one launch: the class store of either beyond
+// the default LDS, or four lists per tile.
+int launch_bin_pair(BinArgs first, BinArgs second, int B, hipStream_t st) {
+    if (first.sub_nx > 0 || second.sub_nx > 0 || first.N != second.N || first.Np != second.Np) return -1;
+    const size_t class_bytes = (size_t)first.Np;
+    if (class_bytes > kBinClassBytesDefault) return -1;
+    for (BinArgs* a : {&first, &second}) {
+        a->chunk = 0;
+        a->cand_counts = nullptr; a->cand_lists = nullptr;
+        a->cand_K = 0; a->cand_chunk = 0; a->stiles_x = 0; a->stiles = 0;
+        a->store_classes = 1;
+    }
+    const int threads = bin_threads(first.N, false);
+    const int n_first = first.tiles_x * first.tiles_y;
+    hipLaunchKernelGGL(k_bin_pair, dim3(n_first + second.tiles_x * second.tiles_y, 1, B), dim3(threads), class_bytes, st,
+                       first, second, n_first);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? IGS_OK : (int)e;
+}
+
 inline int launch_status() {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? IGS_OK : (int)e;
@@ -647,8 +668,8 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
 namespace {
 // The tile lists and slot tables of the separable backward (a = bwd_args of the separable variant);
 // column coordinates x[b * sxb + w * sxw].
-int bin_backward(const BwdArgs& a, const float* x, long sxb, long sxw, const float* packed, int B, int C, int opts,
-                 float* pix_ws, float* partial, hipStream_t st) {
+BinArgs backward_bin_args(const BwdArgs& a, const float* x, long sxb, long sxw, const float* packed, int B, int C,
+                          int opts, float* partial) {
     BinArgs ba;
     ba.bins = bins_of(packed, B, a.Np, rec_stride_of(C));
     ba.limit = limit_of(packed, B, a.Np, rec_stride_of(C));
@@ -662,6 +683,16 @@ int bin_backward(const BwdArgs& a, const float* x, long sxb, long sxw, const flo
     ba.flag = a.flag; ba.want = a.want;
     ba.no_cull = (opts & IGS_OPT_NO_CULL) != 0;
     ba.sub_nx = 0; ba.sub_w = 0; ba.sub_h = 0; ba.img_lists = 0; ba.row_lists = 0;
+    ba.chunk = 0;
+    ba.cand_counts = nullptr; ba.cand_lists = nullptr;
+    ba.cand_K = 0; ba.cand_chunk = 0; ba.stiles_x = 0; ba.stiles = 0;
+    ba.store_classes = 0;
+    return ba;
+}
+
+int bin_backward(const BwdArgs& a, const float* x, long sxb, long sxw, const float* packed, int B, int C, int opts,
+                 float* pix_ws, float* partial, hipStream_t st) {
+    const BinArgs ba = backward_bin_args(a, x, sxb, sxw, packed, B, C, opts, partial);
     const bool levels2 = two_level(a.N, ba.tiles_x, ba.tiles_y, opts);
     BinPlace cp{nullptr, nullptr};
     int* cslots = nullptr;
@@ -673,8 +704,10 @@ int bin_backward(const BwdArgs& a, const float* x, long sxb, long sxw, const flo
     return launch_bins(ba, B, levels2, cp, cslots, st);
 }
 
-// pix_ws / partial: the backward's workspaces, when the forward is to run over the backward's tile
-// lists (built here; plan.lists_shared) instead of lists of its own; else nullptr.
+// pix_ws / partial: the backward's workspaces, when this is the forward of a training step: the
+// backward's tile lists are then built here as well (they depend on the packed Gaussians and the grid
+// only) -- one set for both passes where the tilings coincide (plan.lists_shared), else the
+// backward's beside the forward's own, in one launch where that is possible; else nullptr.
 int forward_impl(const float* packed, const float* x, const float* y,
                  const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag, int B,
                  int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
@@ -689,10 +722,9 @@ int forward_impl(const float* packed, const float* x, const float* y,
     if (rc) return rc;
     if (total.fwd_ws_bytes > 0 && (!ws || ws_bytes < total.fwd_ws_bytes)) return IGS_ERR_WORKSPACE;
     if (((uintptr_t)packed | (uintptr_t)ws) & 15) return IGS_ERR_ALIGNMENT;  // float4 / int lists inside
-    const bool shared = pix_ws != nullptr;
-    if (shared) {
+    const bool train = pix_ws != nullptr;  // the backward's tile lists are built here as well
+    if (train) {
         if (!partial) return IGS_ERR_NULL_POINTER;
-        if (!total.lists_shared) return IGS_ERR_BAD_SHAPE;
         if (pix_bytes < total.pix_bytes || partial_bytes < total.partial_bytes) return IGS_ERR_WORKSPACE;
         if ((uintptr_t)pix_ws & 15) return IGS_ERR_ALIGNMENT;
     }
@@ -722,6 +754,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
         constexpr int kHalvesL = 64 / kWaveCols;
         a.list_row = fwd_wave_lists(C) ? kHalvesL * fg.tiles_x : fg.tiles_x;
         a.list_img = fwd_wave_lists(C) ? 4 * fg.tiles_x * fg.tiles_y : fg.tiles_x * fg.tiles_y;
+        const bool shared = train && plan.lists_shared;
         if (sep && shared) {
             // the backward's tiles are the forward's wave rectangles (or tiles): its lists serve both
             BwdArgs bw;
@@ -768,7 +801,26 @@ int forward_impl(const float* packed, const float* x, const float* y,
             const BinPlace cp = levels2 ? super_bins_at(ws, split_bytes, B, plan.fwd_tiles, plan.n_padded,
                                                         super_tiles(fg.tiles_x, fg.tiles_y, B, N).count)
                                         : BinPlace{nullptr, nullptr};
-            rc = launch_bins(ba, B, levels2, cp, nullptr, st);
+            rc = -1;
+            if (train) {
+                // The tilings differ (small problems: the backward's tiles have fewer rows so that there
+                // are enough of them): the backward's lists are built now as well, in its workspaces, in
+                // the same launch where both binnings are of the plain kind, else in a second one.
+                BwdArgs bw;
+                rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, partial);
+                if (rc) return rc;
+                rc = -1;
+                if (!levels2 && !two_level(N, bw.tiles_x, bw.T / bw.tiles_x, opts_of(grid_mode)))
+                    rc = launch_bin_pair(ba, backward_bin_args(bw, x, grid_strides[0], grid_strides[2], packed, B, C,
+                                                               opts_of(grid_mode), partial), B, st);
+                if (rc < 0) {
+                    rc = bin_backward(bw, x, grid_strides[0], grid_strides[2], packed, B, C, opts_of(grid_mode), pix_ws,
+                                      partial, st);
+                    if (rc) return rc;
+                    rc = -1;
+                }
+            }
+            if (rc < 0) rc = launch_bins(ba, B, levels2, cp, nullptr, st);
             if (rc) return rc;
             a.counts = bp.counts; a.lists = bp.lists;
         }
@@ -824,7 +876,7 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
                         ws_bytes, nullptr, 0, nullptr, 0, stream);
 }
 
-int igs_gs2d_forward_shared_lists(const float* packed, const float* x, const float* y,
+int igs_gs2d_forward_train(const float* packed, const float* x, const float* y,
                                   const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
                                   int B, int N, int H, int W, int C, float eps, float* out, float* den,
                                   void* ws, size_t ws_bytes, float* pix_ws, size_t pix_bytes, float* partial,
@@ -937,9 +989,6 @@ int igs_adamw_step(float* param, const float* grad, float* exp_avg, float* exp_a
     if (!param || !grad || !exp_avg || !exp_avg_sq || !state) return IGS_ERR_NULL_POINTER;
     if (count < 1 || count > (int64_t)kThreads * 0x7fffffff) return IGS_ERR_BAD_SHAPE;
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(k_adamw_tick, dim3(1), dim3(64), 0, st, state, beta1, beta2);
-    int rc = launch_status();
-    if (rc) return rc;
     hipLaunchKernelGGL(k_adamw, dim3((unsigned)((count + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
                        param, grad, exp_avg, exp_avg_sq, (long)count, state, beta1, beta2, eps, weight_decay);
     return launch_status();

@@ -444,8 +444,9 @@ __device__ __forceinline__ float least_weight(float4 q0, float4 q1, float txlo, 
     return w > 0.0f ? w : 0.0f;  // NaN, inf - inf and the like count as nothing
 }
 
+// (the body of k_bin for tile `t` of a's launch: also called by k_bin_pair, one launch for two sets of lists)
 template <bool kMasks>
-__global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin(const BinArgs a) {
+__device__ __forceinline__ void bin_tile(const BinArgs& a, const int t) {
     if (a.flag != nullptr && *a.flag != a.want) return;
     __shared__ float red[4][kBinWaves];
     __shared__ int wsum[kMasks ? 4 : 1][kBinWaves];
@@ -465,7 +466,7 @@ __global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin
         for (int l = 0; l < (kMasks ? 4 : 1); ++l) wsum[l][tid] = 0;
     }
     const int tiles = a.tiles_x * a.tiles_y;
-    const int t = blockIdx.x, kc = blockIdx.y, K = gridDim.y, b = blockIdx.z;
+    const int kc = blockIdx.y, K = gridDim.y, b = blockIdx.z;
     const int ty = t / a.tiles_x, tx = t - ty * a.tiles_x;
     const int c0 = tx * a.tile_w, c1 = min(a.W, c0 + a.tile_w);
     const int r0 = ty * a.tile_h, r1 = min(a.H, r0 + a.tile_h);
@@ -824,4 +825,17 @@ __global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin
     if (tid == 0)
 #pragma unroll
         for (int l = 0; l < kL; ++l) a.counts[masks ? list_no(l) : list_no(0) * K + kc] = total[l];
+}
+
+template <bool kMasks>
+__global__ __launch_bounds__(kMasks ? kBinThreadsMasks : kBinThreads) void k_bin(const BinArgs a) {
+    bin_tile<kMasks>(a, blockIdx.x);
+}
+
+// Two sets of one-list-per-tile lists from one launch (the forward's and the backward's of a training
+// step where their tilings differ): workgroups [0, first_tiles) take the tiles of `a`, the others those of
+// `b`.  Both are single-level binnings over the same Gaussians (gridDim.y = 1).
+__global__ __launch_bounds__(kBinThreads) void k_bin_pair(const BinArgs a, const BinArgs b, const int first_tiles) {
+    const bool second = (int)blockIdx.x >= first_tiles;   // workgroup-uniform
+    bin_tile<false>(second ? b : a, (int)blockIdx.x - (second ? first_tiles : 0));
 }

@@ -78,7 +78,7 @@ class GaussianImageFit:
             self.exp_avg = torch.zeros_like(self.params)
             self.exp_avg_sq = torch.zeros_like(self.params)
             # {lr, t, 1 - beta1^t, sqrt(1 - beta2^t)}
-            self.state = torch.zeros(4, dtype=torch.float32, device=self.device)
+            self.state = torch.zeros(8, dtype=torch.float32, device=self.device)   # lr, t, bias corrections, ticket
             self.loss = torch.zeros((), dtype=torch.float32, device=self.device)
         self._ws: Dict[int, dict] = {}
         self._graphs: Dict[int, torch.cuda.CUDAGraph] = {}
@@ -149,17 +149,18 @@ class GaussianImageFit:
 
     # ------------------------------------------------------------------ the step
     def _enqueue_render(self, n: int, ws: dict, st, train: bool = False):
-        """pack + forward.  `train`: the backward follows; where the plan allows (`lists_shared`) the
-        tile lists are then built once, in the backward's workspaces, for both passes."""
+        """pack + forward.  `train`: the backward follows; its tile lists are then built by the forward's
+        binning launch, in the backward's workspaces (one set for both passes where the plan's tilings
+        coincide, `lists_shared`)."""
         lib, g, p = self.lib, self.grid, ws["plan"]
         B, C, Cp, H, W = self.B, self.C, self.Cp, g.H, g.W
         _lib.check(lib.igs_gs2d_pack_feature(_ptr(self.params), None, B, n, C, Cp, self.eps, *ws["skip_weight"],
                                              _ptr(ws["packed"]), _ptr(ws["col"]), st), "igs_gs2d_pack_feature")
-        if train and p.lists_shared:
-            _lib.check(lib.igs_gs2d_forward_shared_lists(
+        if train:
+            _lib.check(lib.igs_gs2d_forward_train(
                 _ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n, H, W, Cp, self.eps,
                 _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]), int(p.fwd_ws_bytes), _ptr(ws["pix"]),
-                int(p.pix_bytes), _ptr(ws["partial"]), int(p.partial_bytes), st), "igs_gs2d_forward_shared_lists")
+                int(p.pix_bytes), _ptr(ws["partial"]), int(p.partial_bytes), st), "igs_gs2d_forward_train")
             return
         _lib.check(lib.igs_gs2d_forward(_ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n,
                                         H, W, Cp, self.eps, _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]),
@@ -182,7 +183,7 @@ class GaussianImageFit:
                                                       _ptr(ws["out"]), _ptr(ws["den"]), _ptr(grad_out), B, n, H, W, Cp,
                                                       self.eps, _ptr(ws["pix"]), int(p.pix_bytes), st),
                        "igs_gs2d_backward_prologue")
-        mode = g.mode | (_lib.IGS_OPT_LISTS_BUILT if p.lists_shared else 0)  # (the render of a step built them)
+        mode = g.mode | _lib.IGS_OPT_LISTS_BUILT  # (the render of a step built them)
         _lib.check(lib.igs_gs2d_backward_reduce(_ptr(ws["packed"]), _ptr(ws["col"]), _ptr(g.y), g.strides, mode,
                                                 _ptr(g.flag), B, n, H, W, Cp, _ptr(ws["pix"]), int(p.pix_bytes),
                                                 _ptr(ws["partial"]), int(p.partial_bytes), st),

@@ -85,7 +85,7 @@ typedef enum igs_option {
     IGS_OPT_LISTS_BUILT = 0x800   /* igs_gs2d_backward_reduce / igs_gs2d_backward /
                                      igs_gs2d_backward_with_grid only: the tile lists and slot
                                      tables are in these workspaces already
-                                     (igs_gs2d_forward_shared_lists built them for this packed
+                                     (igs_gs2d_forward_train built them for this packed
                                      buffer and these grids); do not build them again            */
 } igs_option;
 
@@ -120,7 +120,7 @@ typedef struct igs_gs2d_plan_t {
     int32_t bwd_tiles_x;     /* separable: column bands of the backward tiles              */
     int32_t bwd_tile_w;      /* separable: columns per band                                */
     int32_t lists_shared;    /* separable: the backward's tiles are the forward's wave
-                                rectangles, so igs_gs2d_forward_shared_lists can build one
+                                rectangles, so igs_gs2d_forward_train can build one
                                 set of tile lists for both passes                           */
 } igs_gs2d_plan_t;
 
@@ -218,18 +218,19 @@ int igs_gs2d_forward_static_ws(const float *packed, const float *x, const float 
                                const int32_t *grid_flag, int B, int N, int H, int W, int C,
                                float eps, float *out, float *den, igs_stream_t stream);
 
-/* The forward of a training step on separable grids, where plan.lists_shared says that the
- * backward's pixel tiles are the forward's wave rectangles: builds the backward's per-tile Gaussian
- * lists and slot tables in pix_ws / partial (plan.pix_bytes / plan.partial_bytes; the lists depend
- * on the packed buffer and the grids only) and runs the forward over them instead of binning once
- * for each pass.  The backward calls on the same workspaces then get IGS_OPT_LISTS_BUILT in their
- * grid_mode (the prologue writes other parts of pix_ws).  IGS_ERR_BAD_SHAPE where
- * plan.lists_shared is 0.  Otherwise as igs_gs2d_forward, whose output it matches up to what the
- * skip tolerance allows (a tile settles what it leaves out by itself, and the tiles of the two
- * binnings need not be the same); bit for bit with skip_weight = skip_fraction = 0 and one
- * Gaussian split.  No counterpart in the reference, which evaluates every pair
- * (src/igs/gs_triton_chunked.py:100-200). */
-int igs_gs2d_forward_shared_lists(const float *packed, const float *x, const float *y,
+/* The forward of a training step (a backward on the same packed buffer and grids follows): as
+ * igs_gs2d_forward, and on separable grids the backward's per-tile Gaussian lists and slot tables are
+ * built as well, in pix_ws / partial (plan.pix_bytes / plan.partial_bytes; the lists depend on the
+ * packed buffer and the grids only).  Where plan.lists_shared says that the backward's pixel tiles
+ * are the forward's wave rectangles, that one set of lists serves both passes (one binning per
+ * step instead of two); elsewhere (small problems, whose backward tiles have fewer rows) the
+ * backward's lists are made beside the forward's own by the same launch.  The backward calls on
+ * the same workspaces then get IGS_OPT_LISTS_BUILT in their grid_mode (the prologue writes other
+ * parts of pix_ws).  The output matches igs_gs2d_forward's up to what the skip tolerance allows
+ * (a tile settles what it leaves out by itself, and the tiles of the two binnings need not be the
+ * same); bit for bit with skip_weight = skip_fraction = 0 and one Gaussian split.  No counterpart
+ * in the reference, which evaluates every pair (src/igs/gs_triton_chunked.py:100-200). */
+int igs_gs2d_forward_train(const float *packed, const float *x, const float *y,
                                   const int64_t grid_strides[6], int grid_mode,
                                   const int32_t *grid_flag, int B, int N, int H, int W, int C,
                                   float eps, float *out, float *den, void *ws, size_t ws_bytes,
@@ -358,9 +359,10 @@ int igs_gs2d_position_penalty(const float *gs_feature, int64_t rows, int row_flo
  * over a flat block of `count` floats, in place:
  *   p *= 1 - lr wd;  m += (g - m)(1 - beta1);  v = beta2 v + (1 - beta2) g^2;
  *   p -= lr / (1 - beta1^t) * m / (sqrt(v) / sqrt(1 - beta2^t) + eps).
- * state is 4 floats of device memory {lr, t, 1 - beta1^t, sqrt(1 - beta2^t)}: the caller
- * writes lr (and t = 0 before the first step); every call increments t on the device, so a
- * captured graph of the call advances on each replay. */
+ * state is 8 floats of device memory {lr, t, 1 - beta1^t, sqrt(1 - beta2^t), ticket, 0, 0, 0}: the
+ * caller zeroes it before the first step and writes lr; every call increments t on the device (the
+ * last workgroup to finish does, through the integer ticket, which is zero again when the call is
+ * done), so a captured graph of the call advances on each replay.  One launch. */
 int igs_adamw_step(float *param, const float *grad, float *exp_avg, float *exp_avg_sq,
                    int64_t count, float *state, float beta1, float beta2, float eps,
                    float weight_decay, igs_stream_t stream);

@@ -659,7 +659,7 @@ def test_more_candidates_than_the_class_store_holds(igs, dev, no_cull, shape):
 def test_one_set_of_tile_lists_for_both_passes(igs, dev, shape, scales):
     """Where the backward's tiles are the forward's wave rectangles (`plan.lists_shared`) a step that
     needs gradients builds the tile lists once, in the backward's workspaces
-    (`igs_gs2d_forward_shared_lists`, then IGS_OPT_LISTS_BUILT), instead of once per pass.  Against
+    (`igs_gs2d_forward_train`, then IGS_OPT_LISTS_BUILT), instead of once per pass.  Against
     the path that bins twice: every gradient bit for bit (the backward's lists are the same lists);
     the image within what the tolerance allows (the forward's own binning settles a 64 x 64 tile's
     allowance with one floor for its four rectangles), and bit for bit when only exact zeros are
@@ -695,22 +695,26 @@ def test_one_set_of_tile_lists_for_both_passes(igs, dev, shape, scales):
         assert torch.equal(ga, gb), k
 
 
-def test_shared_lists_are_refused_where_the_tilings_differ(igs, dev):
-    """A small problem's backward tiles have fewer rows than the forward's wave rectangles: the plan
-    says so and the combined entry point returns a status instead of running."""
-    from igs_amd import _lib
-    from igs_amd._splat import Grid, Splat, _f32c, _ptr
+def test_training_forward_where_the_tilings_differ(igs, dev, monkeypatch):
+    """A small problem's backward tiles have fewer rows than the forward's wave rectangles (the plan
+    says so): the training forward then builds the backward's lists beside its own, in one launch,
+    and image and gradients are those of a forward and a backward that each bin for themselves, bit
+    for bit."""
+    from igs_amd._splat import Grid, Splat
 
     B, N, H, W, C = 1, 300, 96, 160, 3
     _, g = sparse_case(dev, B, N, H, W, C, seed=2)
-    op = Splat(B, N, C, Grid(g["x_grid"], g["y_grid"], B), 1e-6, dev)
-    assert op.plan.lists_shared == 0
-    packed = op.pack_scale_rot(_f32c(g["positions"]), _f32c(g["scales"]), _f32c(g["rotations"]), _f32c(g["alphas"]),
-                               _f32c(g["colors"]))
-    with pytest.raises(RuntimeError, match="status -2"):
-        op.forward_shared_lists(packed)
-    out, _ = op.forward(packed)
-    assert bool(torch.isfinite(out).all())
+    assert Splat(B, N, C, Grid(g["x_grid"], g["y_grid"], B), 1e-6, dev).plan.lists_shared == 0
+    used = []
+    real = Splat.forward_train
+    monkeypatch.setattr(Splat, "forward_train", lambda self, packed: (used.append(1), real(self, packed))[1])
+    out, grads = run(igs, g)
+    assert used, "the training forward was not taken"
+    monkeypatch.setattr(Splat, "forward_train", lambda self, packed: self.forward(packed))   # (leaves `shared` unset)
+    out0, grads0 = run(igs, g)
+    assert float(out.abs().max()) > 0 and torch.equal(out, out0)
+    for k in NAMES:
+        assert torch.equal(grads[k], grads0[k]), k
 
 
 def no_cull_ctx():

@@ -101,7 +101,7 @@ def test_adamw_kernel_against_torch_optimizer(igs, dev):
     p0 = torch.randn(n, generator=g).to(dev)
     p = p0.clone()
     m, v = torch.zeros_like(p), torch.zeros_like(p)
-    state = torch.tensor([0.01, 0, 0, 0], dtype=torch.float32, device=dev)
+    state = torch.tensor([0.01, 0, 0, 0, 0, 0, 0, 0], dtype=torch.float32, device=dev)   # lr, t, corrections, ticket
     q = p0.clone().requires_grad_(True)
     opt = torch.optim.AdamW([q], lr=0.01, **HYPER)
     for k in range(20):
