@@ -14,7 +14,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 LIB_PATH = os.environ.get("IGS_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "libigs_hip.so")
 
-ABI_VERSION = 7  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
+ABI_VERSION = 8  # IGS_ABI_VERSION of include/igs_hip.h this binding was written against
 IGS_GRID_GENERAL = 0
 IGS_GRID_SEPARABLE = 1
 IGS_GRID_AUTO = 2
@@ -86,8 +86,7 @@ SIGNATURES = {
     "igs_gs2d_forward": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
                                  c_float, _FP, _FP, c_void_p, c_size_t, c_void_p]),
     "igs_gs2d_forward_train": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
-                                              c_float, _FP, _FP, c_void_p, c_size_t, _FP, c_size_t, _FP, c_size_t,
-                                              c_void_p]),
+                                       c_float, _FP, _FP, c_void_p, c_size_t, _FP, c_size_t, _FP, c_void_p]),
     "igs_gs2d_forward_static_ws": (c_int, [_FP, _FP, _FP, _STRIDES, c_int, _FP, c_int, c_int, c_int, c_int, c_int,
                                            c_float, _FP, _FP, c_void_p]),
     "igs_gs2d_backward_prologue": (c_int, [_FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int,
@@ -102,13 +101,13 @@ SIGNATURES = {
                                             c_size_t, _FP, _FP, c_void_p]),
     "igs_gs2d_backward_grid": (c_int, [_FP, _FP, _FP, _STRIDES, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                        c_float, _FP, _FP, c_void_p]),
-    "igs_gs2d_finalize_covinv": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
+    "igs_gs2d_finalize_covinv": (c_int, [_FP, _FP, c_int, _FP, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                          _FP, _FP, _FP, _FP, _FP, _FP, c_void_p]),
-    "igs_gs2d_finalize_scale_rot": (c_int, [_FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
+    "igs_gs2d_finalize_scale_rot": (c_int, [_FP, _FP, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int, c_int, c_int,
                                             c_float, _FP, _FP, _FP, _FP, _FP, c_void_p]),
     "igs_gs2d_pack_feature": (c_int, [_FP, _FP, c_int, c_int, c_int, c_int, c_float, c_float, c_float, _FP, _FP,
                                       c_void_p]),
-    "igs_gs2d_finalize_feature": (c_int, [_FP, c_int, _FP, _FP, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+    "igs_gs2d_finalize_feature": (c_int, [_FP, _FP, c_int, _FP, _FP, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                           _FP, c_void_p]),
     "igs_gs2d_mse_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "igs_gs2d_backward_prologue_mse": (c_int, [_FP, _FP, _STRIDES, c_int, _FP, _FP, _FP, _FP, c_int, c_int, c_int,

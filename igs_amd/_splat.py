@@ -42,6 +42,15 @@ KIND_FEATURE = 2
 # 0 skips exact zeros only (bit-identical to evaluating every pair).
 SKIP_TOLERANCE = 1e-7
 
+# Partial sums of the separable backward: one record per listed (Gaussian, tile) pair.  Above this many
+# bytes for *every* pair (plan.partial_bytes: B=4, N=32768, 384x640, C=16 is 2.8 GB, of which 4 % are
+# listed), a training forward leaves the number of listed pairs in pinned host memory and the backward
+# allocates by it, which makes the host wait until the device has passed the forward's binning (2 % of
+# that step; a step of a fraction of a millisecond would lose a third, its host no longer running ahead);
+# below, the array is allocated in full (B=16, N=8192, 256x256: 0.3 GB for the duration of the backward)
+# and nothing waits for the device.
+COMPACT_PARTIALS_FROM = 512 << 20
+
 # (igs_option bits OR-ed into the grid_mode word of every Grid built, skip tolerance) in effect for the
 # calling thread (and asyncio task): a context variable, so that two threads, or a `with` block and
 # another thread's calls, do not see each other's settings.  Both are read when a call's forward
@@ -268,38 +277,53 @@ class Splat:
         return out, den
 
     def forward_train(self, packed: Tensor) -> Tuple[Tensor, Tensor]:
-        """The forward of a step whose backward will follow: the backward's tile lists are built now,
-        in the backward's workspaces, which this object keeps for `backward_partials*` -- one set of
-        lists for both passes where the plan says their tilings coincide (`plan.lists_shared`), else
-        beside the forward's own, in the same launch."""
+        """The forward of a step whose backward will follow: the backward's tile lists and tables are
+        built now, in the backward's pixel workspace, which this object keeps for `backward_partials*`
+        -- one set of lists for both passes where the plan says their tilings coincide
+        (`plan.lists_shared`), else beside the forward's own, in the same launch.  Where the partial
+        sums of every (Gaussian, tile) pair would be large, the number of listed pairs is written to
+        pinned host memory, and the backward sizes its partial-sum array by it."""
         g, p = self.grid, self.plan
         out = self._new(self.B, self.Cp, g.H, g.W)
         den = self._new(self.B, g.H, g.W)
         ws = self._empty(p.fwd_ws_bytes) if p.fwd_ws_bytes else None
         pix = self._empty(p.pix_bytes)
-        partial = self._empty(p.partial_bytes)
+        total = done = None
+        if p.partial_bytes > COMPACT_PARTIALS_FROM:
+            total = torch.empty(1, dtype=torch.int64, pin_memory=True)
         _lib.check(self.lib.igs_gs2d_forward_train(
             _ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), self.B, self.N, g.H, g.W, self.Cp,
-            self.eps, _ptr(out), _ptr(den), _ptr(ws), int(p.fwd_ws_bytes), _ptr(pix), int(p.pix_bytes), _ptr(partial),
-            int(p.partial_bytes), self.stream), "igs_gs2d_forward_train")
-        self.shared = (pix, partial)
+            self.eps, _ptr(out), _ptr(den), _ptr(ws), int(p.fwd_ws_bytes), _ptr(pix), int(p.pix_bytes), _ptr(total),
+            self.stream), "igs_gs2d_forward_train")
+        if total is not None:
+            done = torch.cuda.Event()
+            done.record(torch.cuda.current_stream(self.device))
+        self.shared = (pix, total, done)
         return out, den
 
     def _backward_workspaces(self):
-        """(pix, partial, grid_mode): the workspaces that hold the tile lists already, if the forward
-        built them, else fresh ones."""
+        """(pix, partial, grid_mode): the pixel workspace that holds the tile lists already, if the
+        forward built them, else a fresh one; the partial-sum array, sized by the number of listed
+        (Gaussian, tile) pairs where the forward left it (the wait is for a point of the stream that
+        lies before the forward's own kernels), else for every pair."""
+        nbytes = int(self.plan.partial_bytes)
         if self.shared is not None:
-            return (*self.shared, self.grid.mode | _lib.IGS_OPT_LISTS_BUILT)
-        return self._empty(self.plan.pix_bytes), self._empty(self.plan.partial_bytes), self.grid.mode
+            pix, total, done = self.shared
+            if total is not None and (self.grid.mode & 0xff) == _lib.IGS_GRID_SEPARABLE:
+                done.synchronize()
+                nbytes = max(int(total.item()), 1) * (6 + self.Cp) * 4
+            return pix, self._empty(nbytes), self.grid.mode | _lib.IGS_OPT_LISTS_BUILT
+        return self._empty(self.plan.pix_bytes), self._empty(nbytes), self.grid.mode
 
-    def backward_partials(self, packed, colors_p, out, den, grad_out_p) -> Tensor:
+    def backward_partials(self, packed, colors_p, out, den, grad_out_p) -> Tuple[Tensor, Tensor]:
+        """(partial, pix): the partial sums and the pixel workspace whose tables the finalize call reads."""
         g, p = self.grid, self.plan
         pix, partial, mode = self._backward_workspaces()
         _lib.check(self.lib.igs_gs2d_backward(_ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, mode,
                                               _ptr(g.flag), _ptr(out), _ptr(den), _ptr(grad_out_p), self.B, self.N, g.H, g.W,
                                               self.Cp, self.eps, _ptr(pix), int(p.pix_bytes), _ptr(partial),
-                                              int(p.partial_bytes), self.stream), "igs_gs2d_backward")
-        return partial
+                                              partial.numel() * 4, self.stream), "igs_gs2d_backward")
+        return partial, pix
 
     def backward_partials_with_grid(self, packed, colors_p, out, den, grad_out_p, x_like, y_like):
         """The per-Gaussian partial sums and d L / d x_grid, d L / d y_grid from one call (on general
@@ -315,8 +339,8 @@ class Splat:
         _lib.check(self.lib.igs_gs2d_backward_with_grid(
             _ptr(packed), _ptr(colors_p), _ptr(g.x), _ptr(g.y), g.strides, mode, _ptr(g.flag), _ptr(out), _ptr(den),
             _ptr(grad_out_p), self.B, self.N, g.H, g.W, self.Cp, self.eps, _ptr(pix), int(p.pix_bytes), _ptr(partial),
-            int(p.partial_bytes), _ptr(gws), gws_bytes, _ptr(gx), _ptr(gy), self.stream), "igs_gs2d_backward_with_grid")
-        return partial, self._fit_grid(gx, x_like), self._fit_grid(gy, y_like)
+            partial.numel() * 4, _ptr(gws), gws_bytes, _ptr(gx), _ptr(gy), self.stream), "igs_gs2d_backward_with_grid")
+        return partial, pix, self._fit_grid(gx, x_like), self._fit_grid(gy, y_like)
 
     def _fit_grid(self, gr, like):
         shape, dtype = like
@@ -456,7 +480,7 @@ def run_backward(kind: int, op: Splat, keep, packed, col, out, den, grad_result:
         op.use_current_stream()
         go = op.pad_grad_out(grad_result)
         if (need_x or need_y) and any(need):
-            partial, g_x, g_y = op.backward_partials_with_grid(packed, col, out, den, go, *grid_like)
+            partial, pix, g_x, g_y = op.backward_partials_with_grid(packed, col, out, den, go, *grid_like)
             g_x, g_y = (g_x if need_x else None), (g_y if need_y else None)
         else:
             if need_x or need_y:
@@ -464,14 +488,14 @@ def run_backward(kind: int, op: Splat, keep, packed, col, out, den, grad_result:
                 g_x, g_y = (g_x if need_x else None), (g_y if need_y else None)
             if not any(need):
                 return grads, g_x, g_y
-            partial = op.backward_partials(packed, col, out, den, go)
+            partial, pix = op.backward_partials(packed, col, out, den, go)
         mode, flag, H, W = op.grid.mode, _ptr(op.grid.flag), op.grid.H, op.grid.W
         if kind == KIND_COVINV:
             a, b, d, al = keep
             g_pos = op._new(B, N, 2) if need[0] else None
             g_a, g_b, g_d, g_al = (op._new(B, N) if need[k] else None for k in (1, 2, 3, 4))
             g_col = op._new(B, N, Cp) if need[5] else None
-            _lib.check(op.lib.igs_gs2d_finalize_covinv(_ptr(partial), mode, flag, _ptr(a), _ptr(b), _ptr(d), _ptr(al),
+            _lib.check(op.lib.igs_gs2d_finalize_covinv(_ptr(partial), _ptr(pix), mode, flag, _ptr(a), _ptr(b), _ptr(d), _ptr(al),
                                                        B, N, H, W, Cp, _ptr(g_pos), _ptr(g_a), _ptr(g_b), _ptr(g_d),
                                                        _ptr(g_al), _ptr(g_col), op.stream),
                        "igs_gs2d_finalize_covinv")
@@ -485,7 +509,7 @@ def run_backward(kind: int, op: Splat, keep, packed, col, out, den, grad_result:
             g_sc = op._new(B, N, 2) if need[2] else None
             g_rot = op._new(B, N) if need[3] else None
             g_al = op._new(B, N) if need[4] else None
-            _lib.check(op.lib.igs_gs2d_finalize_scale_rot(_ptr(partial), mode, flag, _ptr(sc), _ptr(rot), _ptr(al),
+            _lib.check(op.lib.igs_gs2d_finalize_scale_rot(_ptr(partial), _ptr(pix), mode, flag, _ptr(sc), _ptr(rot), _ptr(al),
                                                           B, N, H, W, Cp, op.eps, _ptr(g_pos), _ptr(g_sc), _ptr(g_rot),
                                                           _ptr(g_al), _ptr(g_col), op.stream),
                        "igs_gs2d_finalize_scale_rot")
@@ -495,7 +519,7 @@ def run_backward(kind: int, op: Splat, keep, packed, col, out, den, grad_result:
         else:
             (feat,) = keep
             g_feat = op._new(B, N, 6 + C)
-            _lib.check(op.lib.igs_gs2d_finalize_feature(_ptr(partial), mode, flag, _ptr(feat), B, N, H, W, C, Cp,
+            _lib.check(op.lib.igs_gs2d_finalize_feature(_ptr(partial), _ptr(pix), mode, flag, _ptr(feat), B, N, H, W, C, Cp,
                                                         op.eps, _ptr(g_feat), op.stream),
                        "igs_gs2d_finalize_feature")
             grads = [g_feat if need[0] else None]

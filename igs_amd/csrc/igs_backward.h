@@ -131,7 +131,10 @@ struct BwdArgs {
     const int* counts;  // separable: Gaussians listed per tile [B][T]
     const int* lists;   // separable: list + complement [B][T][Np]
     const float4* brecs;  // separable: the backward records of the packed buffer [B][Np] (sA, skA, D'', tag)
-    float* partial;  // [B][T][N][6+C]
+    const long long* offsets;  // separable: first record of each tile in `partial` [B T + 1], the last = total
+    long long capacity;        // separable: records that `partial` holds
+    int* overflow;             // separable: set where the total exceeds the capacity (nothing is stored then for the tiles that do not fit)
+    float* partial;  // general grids: [B][T][N][6+C]; separable: the listed entries' records, tile after tile
     float2* grid_part;  // general grids with grid gradients: [B][groups][HWp] sums of G w (t1, t2)
     const int* flag;
     int want;
@@ -248,7 +251,10 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
     const int tx = (blockIdx.x - ty * a.tiles_x + ty * IGS_BWD_TILE_SHIFT + b * IGS_BWD_TILE_SHIFT) % a.tiles_x;
     const int t = ty * a.tiles_x + tx;
     const int count = a.counts[(size_t)b * a.T + t];
+    if (blockIdx.x == 0 && grp == 0 && b == 0 && tid == 0) *a.overflow = a.offsets[(size_t)gridDim.z * a.T] > a.capacity;
     if (grp * kThreads >= count) return;  // workgroup-uniform: no listed Gaussian left
+    const long long first = a.offsets[(size_t)b * a.T + t];
+    if (first + count > a.capacity) return;  // workgroup-uniform: the caller's array does not hold this tile's records
     const int* list = a.lists + ((size_t)b * a.T + t) * a.Np;
     const int pos = grp * kThreads + tid;
     const int n = pos < count ? list[pos] : a.N;  // >= N: an unused lane (nothing is stored for it)
@@ -489,7 +495,7 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
     }
     if (pos < count) {
         constexpr int NF = 6 + C;
-        float* out = a.partial + ((size_t)b * a.T + t) * NF * a.N + (size_t)pos * NF;  // one record of NF floats per list position
+        float* out = a.partial + (size_t)(first + pos) * NF;  // one record of NF floats per list position
 #pragma unroll
         for (int f = 0; f < 6; ++f) out[f] = M[f];
 #pragma unroll

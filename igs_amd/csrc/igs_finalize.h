@@ -18,11 +18,13 @@ constexpr int kFinAhead = 4;    // tiles whose loads are issued together by a t-
 constexpr int kFinColours = 8;  // colour channels summed per further pass
 constexpr int kFinFirst = 9;    // fields of the first pass: the six moments and up to three colours (C <= 3: one pass)
 
-// `part` is the image's partial array [T][N][NF]; the Gaussian's column in tile t is
-// slots[t * Np + n] when a slot table is given (negative: the tile holds nothing for it), else n.
-// Only the first `nv` (<= NV) of the fields are read.
+// General grids: `part` is the image's partial array [T][N][NF] and the Gaussian's column in every tile
+// is n (slots, toff: nullptr).  Separable grids: `part` is the compact array of all images, tile t of
+// this image starts at record toff[t], and the Gaussian's record in it is number slots[t * Np + n]
+// (negative: the tile holds nothing for it).  Only the first `nv` (<= NV) of the fields are read.
 template <int NV, int FT>
 __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const int* __restrict__ slots,
+                                         const long long* __restrict__ toff,
                                          int Np, int n, int T, int NF, int N, int f0, bool valid,
                                          float (&out)[NV], float* red, int nv = NV) {
     constexpr int FN = 256 / FT;
@@ -32,7 +34,7 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const i
     for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
     if (valid) {
         // kFinAhead tiles at a time: their slot entries first, then all their partials (loads of
-        // absent entries go to column 0 and are replaced by 0), then the sums in tile order, so that
+        // absent entries go to the array's first record and are replaced by 0), then the sums in tile order, so that
         // the loads of a group are in flight together instead of one dependent pair after the other
         for (int t0 = tl; t0 < T; t0 += FT * kFinAhead) {
             int col[kFinAhead];
@@ -45,7 +47,9 @@ __device__ __forceinline__ void tile_sum(const float* __restrict__ part, const i
 #pragma unroll
             for (int u = 0; u < kFinAhead; ++u) {
                 const int t = min(t0 + u * FT, T - 1);
-                const float* src = part + ((size_t)t * N + max(col[u], 0)) * NF + f0;
+                const size_t record = slots ? (col[u] >= 0 ? (size_t)(toff[t] + col[u]) : (size_t)0)
+                                            : (size_t)t * N + max(col[u], 0);
+                const float* src = part + record * NF + f0;
 #pragma unroll
                 for (int v = 0; v < NV; ++v) val[u][v] = v < nv ? src[v] : 0.0f;
             }
@@ -155,7 +159,8 @@ __device__ __forceinline__ void finalize_feature_geometry(const float* M, const 
 template <bool kScaleRot, int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
-    const int* __restrict__ slots_in, int Np, const float* __restrict__ p0,
+    const int* __restrict__ slots_in, const long long* __restrict__ offsets, const int* __restrict__ overflow,
+    int Np, const float* __restrict__ p0,
     const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ alphas,
     int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
@@ -170,16 +175,21 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + C;
     const size_t i = (size_t)b * N + min(n, N - 1);
-    const float* part = partial + (size_t)b * T * NF * N;
-    // the slot table belongs to the separable variant
-    const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
-                           ? slots_in + (size_t)b * T * Np : nullptr;
+    // the slot table and the compact array belong to the separable variant
+    const bool listed = slots_in != nullptr && !(flag != nullptr && *flag == 0);
+    const int* slots = listed ? slots_in + (size_t)b * T * Np : nullptr;
+    const long long* toff = listed ? offsets + (size_t)b * T : nullptr;
+    const float* part = listed ? partial : partial + (size_t)b * T * NF * N;
+    const bool lost = listed && *overflow != 0;  // the partial sums did not fit the caller's array: no gradient is known
     const int nn = min(n, N - 1);
     // first pass: the moments and, when wanted, the first colours (they follow the moments)
     constexpr int kC0 = kFinFirst - 6;
     float M[kFinFirst];
     const int nfirst = g_col ? min(kFinFirst, NF) : 6;
-    tile_sum<kFinFirst, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red, nfirst);
+    tile_sum<kFinFirst, FT>(part, slots, toff, Np, nn, T, NF, N, 0, valid && !lost, M, red, nfirst);
+    if (lost)
+#pragma unroll
+        for (int v = 0; v < kFinFirst; ++v) M[v] = __builtin_nanf("");
     if (writer) finalize_geometry<kScaleRot>(M, i, p0, p1, p2, alphas, eps, g_pos, g0, g1, g2, g_alpha);
     if (g_col) {  // kernel-argument uniform, so the barriers inside tile_sum are safe
         const float al = alphas[i];
@@ -190,11 +200,11 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
         for (int c0 = kC0; c0 < C; c0 += kFinColours) {  // further colour sums, kFinColours channels per pass
             float sc[kFinColours];
             const int nc = min(kFinColours, C - c0);
-            tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+            tile_sum<kFinColours, FT>(part, slots, toff, Np, nn, T, NF, N, 6 + c0, valid && !lost, sc, red, nc);
             if (writer)
 #pragma unroll
                 for (int c = 0; c < kFinColours; ++c)
-                    if (c < nc) g_col[i * C + c0 + c] = al * sc[c];
+                    if (c < nc) g_col[i * C + c0 + c] = lost ? __builtin_nanf("") : al * sc[c];
         }
     }
 }
@@ -204,7 +214,8 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
 template <int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
-    const int* __restrict__ slots_in, int Np, const float* __restrict__ feat, int N,
+    const int* __restrict__ slots_in, const long long* __restrict__ offsets, const int* __restrict__ overflow,
+    int Np, const float* __restrict__ feat, int N,
     int C, int Cp,
     float eps, float* __restrict__ g_feat) {
     constexpr int FN = 256 / FT;
@@ -216,13 +227,18 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const int T = (flag != nullptr && *flag == 0) ? T_alt : T_in;
     const int NF = 6 + Cp;
     const size_t i = (size_t)b * N + min(n, N - 1);
-    const float* part = partial + (size_t)b * T * NF * N;
-    const int* slots = (slots_in != nullptr && !(flag != nullptr && *flag == 0))
-                           ? slots_in + (size_t)b * T * Np : nullptr;
+    const bool listed = slots_in != nullptr && !(flag != nullptr && *flag == 0);
+    const int* slots = listed ? slots_in + (size_t)b * T * Np : nullptr;
+    const long long* toff = listed ? offsets + (size_t)b * T : nullptr;
+    const float* part = listed ? partial : partial + (size_t)b * T * NF * N;
+    const bool lost = listed && *overflow != 0;
     const int nn = min(n, N - 1);
     constexpr int kC0 = kFinFirst - 6;
     float M[kFinFirst];
-    tile_sum<kFinFirst, FT>(part, slots, Np, nn, T, NF, N, 0, valid, M, red, min(kFinFirst, NF));
+    tile_sum<kFinFirst, FT>(part, slots, toff, Np, nn, T, NF, N, 0, valid && !lost, M, red, min(kFinFirst, NF));
+    if (lost)
+#pragma unroll
+        for (int v = 0; v < kFinFirst; ++v) M[v] = __builtin_nanf("");
     float* g = g_feat + i * (6 + C);
     if (writer) {
         finalize_feature_geometry(M, feat + i * (6 + C), eps, g);
@@ -233,11 +249,11 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     for (int c0 = kC0; c0 < C; c0 += kFinColours) {
         float sc[kFinColours];
         const int nc = min(kFinColours, C - c0);
-        tile_sum<kFinColours, FT>(part, slots, Np, nn, T, NF, N, 6 + c0, valid, sc, red, nc);
+        tile_sum<kFinColours, FT>(part, slots, toff, Np, nn, T, NF, N, 6 + c0, valid && !lost, sc, red, nc);
         if (writer)
 #pragma unroll
             for (int c = 0; c < kFinColours; ++c)
-                if (c < nc) g[6 + c0 + c] = sc[c];
+                if (c < nc) g[6 + c0 + c] = lost ? __builtin_nanf("") : sc[c];
     }
 }
 
@@ -272,6 +288,8 @@ struct FinalizeArgs {
     int T, T_alt;
     const int* flag;    // AUTO grid mode: *flag == 0 -> the general backward ran (T_alt dense tiles, no tables)
     const int* slots;   // [B][T][Np] of the separable backward
+    const long long* offsets;  // [B T + 1]: the tiles' first records in its compact partial array
+    const int* overflow;       // set where that array was too small
     SuperSlots sup;
     int Np, N, C, Cp;   // C: channels of the caller's rows (feature kind), Cp: of the records
     const float *p0, *p1, *p2, *alphas;  // cov_inv_* | scales, rotations | gs_feature
@@ -289,12 +307,13 @@ __device__ __forceinline__ unsigned int group_ballot(bool p) {
 // Gaussian n in up to kFinGroup tiles: this lane's tile is `t` (`in`: it exists), in ascending lane
 // order.  Group-uniform control flow; the other groups of the wave may be elsewhere.
 __device__ __forceinline__ void group_add_tiles(const float* __restrict__ part, const int* __restrict__ slots,
+                                                const long long* __restrict__ toff,
                                                 int Np, int N, int NF, int n, int lane, int t, bool in,
                                                 float (&acc)[kFinGroupFields]) {
     const int col = in ? slots[(size_t)t * Np + n] : -1;
     unsigned int tm = group_ballot(col >= 0);
     // where this lane's tile keeps the Gaussian's record (in floats; the lanes that read it fetch the two halves)
-    const unsigned long long at = ((unsigned long long)t * N + max(col, 0)) * NF;
+    const unsigned long long at = col >= 0 ? (unsigned long long)(toff[t] + col) * NF : 0ull;
     const int at_lo = (int)(unsigned int)at, at_hi = (int)(at >> 32);
     while (tm) {
         float val[kFinGroupAhead][kFinGroupFields];
@@ -320,6 +339,7 @@ __device__ __forceinline__ void group_add_tiles(const float* __restrict__ part, 
 // All records of Gaussian n after a two-level binning: the listed super-tiles in ascending order,
 // the tiles of each row-major.
 __device__ __forceinline__ void group_sum_listed(const float* __restrict__ part, const int* __restrict__ slots,
+                                                 const long long* __restrict__ toff,
                                                  const SuperSlots sup, int Np, int N, int NF, int n, int lane,
                                                  float (&acc)[kFinGroupFields]) {
     for (int s0 = 0; s0 < sup.stiles; s0 += kFinGroup) {
@@ -332,7 +352,7 @@ __device__ __forceinline__ void group_sum_listed(const float* __restrict__ part,
             for (int j0 = 0; j0 < kSuperX * kSuperY; j0 += kFinGroup) {
                 const int j = j0 + lane;
                 const int ty = sy * kSuperY + j / kSuperX, tx = sx * kSuperX + j % kSuperX;
-                group_add_tiles(part, slots, Np, N, NF, n, lane, ty * sup.tiles_x + tx,
+                group_add_tiles(part, slots, toff, Np, N, NF, n, lane, ty * sup.tiles_x + tx,
                                 j < kSuperX * kSuperY && ty < sup.tiles_y && tx < sup.tiles_x, acc);
             }
         }
@@ -341,10 +361,11 @@ __device__ __forceinline__ void group_sum_listed(const float* __restrict__ part,
 
 // After a one-level binning: the T tiles in ascending order.
 __device__ __forceinline__ void group_sum_tiles(const float* __restrict__ part, const int* __restrict__ slots,
+                                                const long long* __restrict__ toff,
                                                 int T, int Np, int N, int NF, int n, int lane,
                                                 float (&acc)[kFinGroupFields]) {
     for (int t0 = 0; t0 < T; t0 += kFinGroup)
-        group_add_tiles(part, slots, Np, N, NF, n, lane, t0 + lane, t0 + lane < T, acc);
+        group_add_tiles(part, slots, toff, Np, N, NF, n, lane, t0 + lane, t0 + lane < T, acc);
 }
 
 // The same over the dense partials of the general backward (every tile holds column n).
@@ -376,8 +397,10 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_listed(const Finalize
     const bool general = a.slots == nullptr || (a.flag != nullptr && *a.flag == 0);
     const int T = general ? a.T_alt : a.T;
     const int NF = 6 + a.Cp;
-    const float* part = a.partial + (size_t)b * T * NF * a.N;
+    const float* part = general ? a.partial + (size_t)b * T * NF * a.N : a.partial;
     const int* slots = a.slots != nullptr ? a.slots + (size_t)b * a.T * a.Np : nullptr;
+    const long long* toff = general ? nullptr : a.offsets + (size_t)b * a.T;
+    const bool lost = !general && *a.overflow != 0;  // the partial sums did not fit the caller's array
     SuperSlots sup = a.sup;
     if (sup.cslots != nullptr) sup.cslots += (size_t)b * sup.stiles * a.Np;
     for (int k = 0; k < kFinGroupBatch / kGroups; ++k) {
@@ -387,12 +410,15 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_listed(const Finalize
         float acc[kFinGroupFields];
 #pragma unroll
         for (int v = 0; v < kFinGroupFields; ++v) acc[v] = 0.0f;
-        if (general)
+        if (lost) {
+#pragma unroll
+            for (int v = 0; v < kFinGroupFields; ++v) acc[v] = __builtin_nanf("");
+        } else if (general)
             group_sum_dense(part, T, a.N, NF, n, lane, acc);
         else if (a.sup.cslots != nullptr)
-            group_sum_listed(part, slots, sup, a.Np, a.N, NF, n, lane, acc);
+            group_sum_listed(part, slots, toff, sup, a.Np, a.N, NF, n, lane, acc);
         else
-            group_sum_tiles(part, slots, T, a.Np, a.N, NF, n, lane, acc);
+            group_sum_tiles(part, slots, toff, T, a.Np, a.N, NF, n, lane, acc);
         const size_t i = (size_t)b * a.N + n;
 #pragma unroll
         for (int v = 0; v < kFinGroupFields; ++v) {

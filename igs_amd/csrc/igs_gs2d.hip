@@ -170,6 +170,65 @@ inline size_t super_bins_bytes(int B, int stiles, int Np) {
     return ((size_t)B * stiles * kBinMaxChunks + (size_t)B * stiles * Np) * sizeof(int);
 }
 
+// Where the tile lists of a separable launch live inside its workspace.
+struct BinPlace {
+    int* counts;
+    int* lists;
+};
+inline BinPlace bins_at(void* ws, size_t scratch_bytes, int B, int tiles) {
+    char* base = static_cast<char*>(ws) + align16(scratch_bytes);
+    BinPlace bp;
+    bp.counts = reinterpret_cast<int*>(base);
+    bp.lists = bp.counts + (((size_t)B * tiles + 3) & ~(size_t)3);
+    return bp;
+}
+
+// The super-tile lists that follow the tile lists of a launch.
+inline BinPlace super_bins_at(void* ws, size_t scratch_bytes, int B, int tiles, int Np, int stiles) {
+    char* base = static_cast<char*>(ws) + align16(align16(scratch_bytes) + bins_bytes(B, tiles, Np));
+    BinPlace bp;
+    bp.counts = reinterpret_cast<int*>(base);
+    bp.lists = bp.counts + (size_t)B * stiles * kBinMaxChunks;
+    return bp;
+}
+
+// The tables of the separable backward behind the pixel records in its workspace (`scratch_bytes`:
+// records + column coordinates): the tile lists (counts [B][T], lists [B][T][Np]), the super-tile lists
+// where the tile grid reserves them (stiles > 0), the slot tables [B][T][Np] (Gaussian -> position in
+// the tile's list, or -1) and those of the super-tiles, the tiles' first records in the compact
+// partial-sum array (B T + 1 64-bit offsets, the last being the total) and a flag that the backward
+// raises when that array is too small for them.
+struct BwdTables {
+    BinPlace bins, super;
+    int* slots;
+    int* super_slots;
+    long long* offsets;
+    int* overflow;
+    size_t bytes;  // of the workspace up to the end of the tables
+};
+inline BwdTables bwd_tables_at(void* ws, size_t scratch_bytes, int B, int T, int Np, int stiles) {
+    BwdTables t;
+    char* base = static_cast<char*>(ws);
+    size_t at = align16(scratch_bytes);
+    t.bins = bins_at(ws, scratch_bytes, B, T);
+    at += bins_bytes(B, T, Np);
+    t.super = BinPlace{nullptr, nullptr};
+    if (stiles > 0) {
+        t.super = super_bins_at(ws, scratch_bytes, B, T, Np, stiles);
+        at = align16(at) + super_bins_bytes(B, stiles, Np);
+    }
+    at = align16(at);
+    t.slots = reinterpret_cast<int*>(base + at);
+    at = align16(at + (size_t)B * T * Np * sizeof(int));
+    t.super_slots = stiles > 0 ? reinterpret_cast<int*>(base + at) : nullptr;
+    if (stiles > 0) at = align16(at + (size_t)B * stiles * Np * sizeof(int));
+    t.offsets = reinterpret_cast<long long*>(base + at);
+    at = align16(at + ((size_t)B * T + 1) * sizeof(long long));
+    t.overflow = reinterpret_cast<int*>(base + at);
+    t.bytes = at + 16;
+    return t;
+}
+
 // A grid_mode argument of the ABI: the igs_grid_mode in the low byte, IGS_OPT_* bits above it.
 inline int mode_of(int word) { return word & 0xff; }
 inline int opts_of(int word) { return word & ~0xff; }
@@ -245,53 +304,15 @@ int plan_one(int B, int N, int H, int W, int C, int grid_mode, igs_gs2d_plan_t* 
         if (super_reserved(fg.tiles_x, fg.tiles_y))
             p->fwd_ws_bytes = align16(p->fwd_ws_bytes) +
                               super_bins_bytes(B, super_tiles(fg.tiles_x, fg.tiles_y, B, N).count, p->n_padded);
-        p->pix_bytes = align16(p->pix_bytes) + bins_bytes(B, p->bwd_tiles, p->n_padded);
-        if (super_reserved(p->bwd_tiles_x, bwd_tiles_y))
-            p->pix_bytes = align16(p->pix_bytes) +
-                           super_bins_bytes(B, super_tiles(p->bwd_tiles_x, bwd_tiles_y, B, N).count, p->n_padded);
+        // the backward's tables behind its pixel records: see bwd_tables_at
+        p->pix_bytes = bwd_tables_at(nullptr, p->pix_bytes, B, (int)T, p->n_padded,
+                                     super_reserved(p->bwd_tiles_x, bwd_tiles_y)
+                                         ? super_tiles(p->bwd_tiles_x, bwd_tiles_y, B, N).count : 0).bytes;
     }
+    // the partial sums when every Gaussian is listed for every tile (general grids: always); the separable
+    // backward needs (listed entries) x (6 + C) floats, see igs_gs2d_forward_train
     p->partial_bytes = (uint64_t)B * T * (6 + C) * N * sizeof(float);
-    if (sep) {  // the slot tables [B][T][Np] (Gaussian -> position in the tile's list) follow,
-                // then those of the super-tiles
-        p->partial_bytes = align16(p->partial_bytes) + (uint64_t)B * T * p->n_padded * sizeof(int);
-        if (super_reserved(p->bwd_tiles_x, bwd_tiles_y))
-            p->partial_bytes = align16(p->partial_bytes) +
-                               (uint64_t)B * super_tiles(p->bwd_tiles_x, bwd_tiles_y, B, N).count * p->n_padded * sizeof(int);
-    }
     return IGS_OK;
-}
-
-// The slot tables of the separable backward inside the partial buffer.
-inline int* slots_at(float* partial, int B, int T, int NF, int N) {
-    return reinterpret_cast<int*>(reinterpret_cast<char*>(partial) +
-                                  align16((size_t)B * T * NF * N * sizeof(float)));
-}
-
-// Where the tile lists of a separable launch live inside its workspace.
-struct BinPlace {
-    int* counts;
-    int* lists;
-};
-inline BinPlace bins_at(void* ws, size_t scratch_bytes, int B, int tiles) {
-    char* base = static_cast<char*>(ws) + align16(scratch_bytes);
-    BinPlace bp;
-    bp.counts = reinterpret_cast<int*>(base);
-    bp.lists = bp.counts + (((size_t)B * tiles + 3) & ~(size_t)3);
-    return bp;
-}
-
-// The super-tile lists that follow the tile lists of a launch.
-inline BinPlace super_bins_at(void* ws, size_t scratch_bytes, int B, int tiles, int Np, int stiles) {
-    char* base = static_cast<char*>(ws) + align16(align16(scratch_bytes) + bins_bytes(B, tiles, Np));
-    BinPlace bp;
-    bp.counts = reinterpret_cast<int*>(base);
-    bp.lists = bp.counts + (size_t)B * stiles * kBinMaxChunks;
-    return bp;
-}
-// The super-tile slot tables that follow the slot tables in the partial buffer.
-inline int* super_slots_at(float* partial, int B, int T, int NF, int N, int Np) {
-    char* slots = reinterpret_cast<char*>(slots_at(partial, B, T, NF, N));
-    return reinterpret_cast<int*>(slots + align16((size_t)B * T * Np * sizeof(int)));
 }
 
 inline const float4* bins_of(const float* packed, int B, int Np, int RS) {
@@ -537,8 +558,19 @@ int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     return launch_status();
 }
 
+// The separable backward's tables inside its pixel workspace (plan: the separable variant's).
+inline BwdTables tables_of(const igs_gs2d_plan_t& plan, void* pix_ws) {
+    const int B = plan.B, T = plan.bwd_tiles, tiles_y = T / plan.bwd_tiles_x;
+    const size_t scratch = ((size_t)B * plan.H * plan.w_padded * plan.pix_stride + (size_t)B * plan.w_padded) * sizeof(float);
+    return bwd_tables_at(pix_ws, scratch, B, T, plan.n_padded,
+                         super_reserved(plan.bwd_tiles_x, tiles_y) ? super_tiles(plan.bwd_tiles_x, tiles_y, B, plan.N).count : 0);
+}
+
+// partial_bytes: what the caller's partial-sum array holds (its capacity in records bounds what the
+// separable backward may store).
 int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* colors, const float* y,
-             const int64_t gs[6], int B, int N, int H, int W, int C, float* pix_ws, float* partial) {
+             const int64_t gs[6], int B, int N, int H, int W, int C, float* pix_ws, float* partial,
+             size_t partial_bytes = 0) {
     igs_gs2d_plan_t plan;
     const int rc = plan_one(B, N, H, W, C, v.mode, &plan);
     if (rc) return rc;
@@ -551,12 +583,13 @@ int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* col
     a.T = plan.bwd_tiles;
     a.tiles_x = plan.bwd_tiles_x;
     a.per_tile = plan.bwd_per_tile;
-    a.counts = nullptr; a.lists = nullptr;
+    a.counts = nullptr; a.lists = nullptr; a.offsets = nullptr; a.overflow = nullptr;
+    a.capacity = (long long)(partial_bytes / ((6 + C) * sizeof(float)));
     a.brecs = packed ? brecs_of(packed, B, plan.n_padded, C) : nullptr;
     if (sep && pix_ws) {
-        const size_t scratch = ((size_t)B * H * plan.w_padded * plan.pix_stride + (size_t)B * plan.w_padded) * sizeof(float);
-        const BinPlace bp = bins_at(pix_ws, scratch, B, plan.bwd_tiles);
-        a.counts = bp.counts; a.lists = bp.lists;
+        const BwdTables t = tables_of(plan, pix_ws);
+        a.counts = t.bins.counts; a.lists = t.bins.lists;
+        a.offsets = t.offsets; a.overflow = t.overflow;
     }
     a.partial = partial;
     a.grid_part = nullptr;
@@ -666,10 +699,10 @@ int igs_gs2d_pack_scale_rot(const float* positions, const float* scales, const f
 }  // extern "C"
 
 namespace {
-// The tile lists and slot tables of the separable backward (a = bwd_args of the separable variant);
-// column coordinates x[b * sxb + w * sxw].
-BinArgs backward_bin_args(const BwdArgs& a, const float* x, long sxb, long sxw, const float* packed, int B, int C,
-                          int opts, float* partial) {
+// The tile lists and slot tables of the separable backward (a = bwd_args of the separable variant, t = its
+// tables); column coordinates x[b * sxb + w * sxw].
+BinArgs backward_bin_args(const BwdArgs& a, const BwdTables& t, const float* x, long sxb, long sxw, const float* packed,
+                          int B, int C, int opts) {
     BinArgs ba;
     ba.bins = bins_of(packed, B, a.Np, rec_stride_of(C));
     ba.limit = limit_of(packed, B, a.Np, rec_stride_of(C));
@@ -678,8 +711,8 @@ BinArgs backward_bin_args(const BwdArgs& a, const float* x, long sxb, long sxw, 
     ba.N = a.N; ba.Np = a.Np; ba.H = a.H; ba.W = a.W;
     ba.tile_w = kBwdTileW; ba.tile_h = a.per_tile;
     ba.tiles_x = a.tiles_x; ba.tiles_y = a.T / a.tiles_x;
-    ba.counts = const_cast<int*>(a.counts); ba.lists = const_cast<int*>(a.lists);
-    ba.slots = slots_at(partial, B, a.T, 6 + C, a.N);
+    ba.counts = t.bins.counts; ba.lists = t.bins.lists;
+    ba.slots = t.slots;
     ba.flag = a.flag; ba.want = a.want;
     ba.no_cull = (opts & IGS_OPT_NO_CULL) != 0;
     ba.sub_nx = 0; ba.sub_w = 0; ba.sub_h = 0; ba.img_lists = 0; ba.row_lists = 0;
@@ -690,18 +723,20 @@ BinArgs backward_bin_args(const BwdArgs& a, const float* x, long sxb, long sxw, 
     return ba;
 }
 
-int bin_backward(const BwdArgs& a, const float* x, long sxb, long sxw, const float* packed, int B, int C, int opts,
-                 float* pix_ws, float* partial, hipStream_t st) {
-    const BinArgs ba = backward_bin_args(a, x, sxb, sxw, packed, B, C, opts, partial);
+// After the backward's binning: the tiles' first records in the compact partial-sum array (and the
+// total, to `total_out` as well when given: device-accessible memory, e.g. pinned host memory).
+int launch_tile_offsets(const BwdArgs& a, const BwdTables& t, int B, long long* total_out, hipStream_t st) {
+    hipLaunchKernelGGL(k_tile_offsets, dim3(1), dim3(kBinThreads), 0, st, (const int*)t.bins.counts, B * a.T, t.offsets,
+                       t.overflow, total_out, a.flag, a.want);
+    return launch_status();
+}
+
+int bin_backward(const BwdArgs& a, const BwdTables& t, const float* x, long sxb, long sxw, const float* packed, int B,
+                 int C, int opts, long long* total_out, hipStream_t st) {
+    const BinArgs ba = backward_bin_args(a, t, x, sxb, sxw, packed, B, C, opts);
     const bool levels2 = two_level(a.N, ba.tiles_x, ba.tiles_y, opts);
-    BinPlace cp{nullptr, nullptr};
-    int* cslots = nullptr;
-    if (levels2) {
-        const size_t scratch = ((size_t)B * a.H * a.Wp * pix_stride_sep(C) + (size_t)B * a.Wp) * sizeof(float);
-        cp = super_bins_at(pix_ws, scratch, B, a.T, a.Np, super_tiles(ba.tiles_x, ba.tiles_y, B, a.N).count);
-        cslots = super_slots_at(partial, B, a.T, 6 + C, a.N, a.Np);
-    }
-    return launch_bins(ba, B, levels2, cp, cslots, st);
+    const int rc = launch_bins(ba, B, levels2, t.super, levels2 ? t.super_slots : nullptr, st);
+    return rc ? rc : launch_tile_offsets(a, t, B, total_out, st);
 }
 
 // pix_ws / partial: the backward's workspaces, when this is the forward of a training step: the
@@ -711,7 +746,7 @@ int bin_backward(const BwdArgs& a, const float* x, long sxb, long sxw, const flo
 int forward_impl(const float* packed, const float* x, const float* y,
                  const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag, int B,
                  int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
-                 size_t ws_bytes, float* pix_ws, size_t pix_bytes, float* partial, size_t partial_bytes,
+                 size_t ws_bytes, float* pix_ws, size_t pix_bytes, long long* total_out,
                  igs_stream_t stream) {
     if (!packed || !x || !y || !grid_strides || !out || !den) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
@@ -724,8 +759,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
     if (((uintptr_t)packed | (uintptr_t)ws) & 15) return IGS_ERR_ALIGNMENT;  // float4 / int lists inside
     const bool train = pix_ws != nullptr;  // the backward's tile lists are built here as well
     if (train) {
-        if (!partial) return IGS_ERR_NULL_POINTER;
-        if (pix_bytes < total.pix_bytes || partial_bytes < total.partial_bytes) return IGS_ERR_WORKSPACE;
+        if (pix_bytes < total.pix_bytes) return IGS_ERR_WORKSPACE;
         if ((uintptr_t)pix_ws & 15) return IGS_ERR_ALIGNMENT;
     }
     hipStream_t st = (hipStream_t)stream;
@@ -758,9 +792,10 @@ int forward_impl(const float* packed, const float* x, const float* y,
         if (sep && shared) {
             // the backward's tiles are the forward's wave rectangles (or tiles): its lists serve both
             BwdArgs bw;
-            rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, partial);
+            rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr);
             if (rc) return rc;
-            rc = bin_backward(bw, x, grid_strides[0], grid_strides[2], packed, B, C, opts_of(grid_mode), pix_ws, partial, st);
+            rc = bin_backward(bw, tables_of(plan, pix_ws), x, grid_strides[0], grid_strides[2], packed, B, C,
+                              opts_of(grid_mode), total_out, st);
             if (rc) return rc;
             a.counts = bw.counts; a.lists = bw.lists;
             a.list_row = bw.tiles_x; a.list_img = bw.T;
@@ -807,15 +842,21 @@ int forward_impl(const float* packed, const float* x, const float* y,
                 // are enough of them): the backward's lists are built now as well, in its workspaces, in
                 // the same launch where both binnings are of the plain kind, else in a second one.
                 BwdArgs bw;
-                rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, partial);
+                rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr);
                 if (rc) return rc;
+                const BwdTables bt = tables_of(plan, pix_ws);
                 rc = -1;
-                if (!levels2 && !two_level(N, bw.tiles_x, bw.T / bw.tiles_x, opts_of(grid_mode)))
-                    rc = launch_bin_pair(ba, backward_bin_args(bw, x, grid_strides[0], grid_strides[2], packed, B, C,
-                                                               opts_of(grid_mode), partial), B, st);
+                if (!levels2 && !two_level(N, bw.tiles_x, bw.T / bw.tiles_x, opts_of(grid_mode))) {
+                    rc = launch_bin_pair(ba, backward_bin_args(bw, bt, x, grid_strides[0], grid_strides[2], packed, B, C,
+                                                               opts_of(grid_mode)), B, st);
+                    if (rc == 0) {
+                        rc = launch_tile_offsets(bw, bt, B, total_out, st);
+                        if (rc) return rc;
+                    }
+                }
                 if (rc < 0) {
-                    rc = bin_backward(bw, x, grid_strides[0], grid_strides[2], packed, B, C, opts_of(grid_mode), pix_ws,
-                                      partial, st);
+                    rc = bin_backward(bw, bt, x, grid_strides[0], grid_strides[2], packed, B, C, opts_of(grid_mode),
+                                      total_out, st);
                     if (rc) return rc;
                     rc = -1;
                 }
@@ -873,17 +914,17 @@ int igs_gs2d_forward(const float* packed, const float* x, const float* y,
                      int N, int H, int W, int C, float eps, float* out, float* den, void* ws,
                      size_t ws_bytes, igs_stream_t stream) {
     return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
-                        ws_bytes, nullptr, 0, nullptr, 0, stream);
+                        ws_bytes, nullptr, 0, nullptr, stream);
 }
 
 int igs_gs2d_forward_train(const float* packed, const float* x, const float* y,
-                                  const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
-                                  int B, int N, int H, int W, int C, float eps, float* out, float* den,
-                                  void* ws, size_t ws_bytes, float* pix_ws, size_t pix_bytes, float* partial,
-                                  size_t partial_bytes, igs_stream_t stream) {
-    if (!pix_ws || !partial) return IGS_ERR_NULL_POINTER;
+                           const int64_t grid_strides[6], int grid_mode, const int32_t* grid_flag,
+                           int B, int N, int H, int W, int C, float eps, float* out, float* den,
+                           void* ws, size_t ws_bytes, float* pix_ws, size_t pix_bytes, int64_t* listed_total,
+                           igs_stream_t stream) {
+    if (!pix_ws) return IGS_ERR_NULL_POINTER;
     return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
-                        ws_bytes, pix_ws, pix_bytes, partial, partial_bytes, stream);
+                        ws_bytes, pix_ws, pix_bytes, reinterpret_cast<long long*>(listed_total), stream);
 }
 
 int igs_gs2d_forward_static_ws(const float* packed, const float* x, const float* y,
@@ -900,7 +941,7 @@ int igs_gs2d_forward_static_ws(const float* packed, const float* x, const float*
     rc = static_scratch(&ws);
     if (rc) return rc;
     return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
-                        IGS_STATIC_SCRATCH_BYTES, nullptr, 0, nullptr, 0, stream);
+                        IGS_STATIC_SCRATCH_BYTES, nullptr, 0, nullptr, stream);
 }
 
 }  // extern "C"
@@ -1042,19 +1083,28 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
     igs_gs2d_plan_t total;
     rc = make_plan(B, N, H, W, C, grid_mode, &total);
     if (rc) return rc;
-    if (pix_bytes < total.pix_bytes || partial_bytes < total.partial_bytes) return IGS_ERR_WORKSPACE;
+    if (pix_bytes < total.pix_bytes) return IGS_ERR_WORKSPACE;
+    // The partial sums: general grids store every Gaussian for every tile (plan.partial_bytes); the
+    // separable backward stores the listed entries only, packed tile after tile, and raises the
+    // workspace's overflow flag where `partial_bytes` does not hold them (the finalize calls then
+    // return NaN gradients): plan.partial_bytes always does.
+    if (mode_of(grid_mode) != IGS_GRID_SEPARABLE && partial_bytes < total.partial_bytes) return IGS_ERR_WORKSPACE;
+    if (partial_bytes < (size_t)(6 + C) * sizeof(float)) return IGS_ERR_WORKSPACE;
     if (((uintptr_t)packed | (uintptr_t)pix_ws) & 15) return IGS_ERR_ALIGNMENT;  // float4 / int lists inside
     hipStream_t st = (hipStream_t)stream;
     Variant vs[2];
     const int nv = variants_of(grid_mode, grid_flag, vs);
     for (int i = 0; i < nv; ++i) {
         BwdArgs a;
-        rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C, pix_ws, partial);
+        rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C, pix_ws, partial, partial_bytes);
         if (rc) return rc;
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
         if (sep && !(opts_of(grid_mode) & IGS_OPT_LISTS_BUILT)) {
             // (the prologue's compact column coordinates: the same values as the grid's)
-            rc = bin_backward(a, a.xs, a.Wp, 1, packed, B, C, opts_of(grid_mode), pix_ws, partial, st);
+            igs_gs2d_plan_t plan;
+            rc = plan_one(B, N, H, W, C, IGS_GRID_SEPARABLE, &plan);
+            if (rc) return rc;
+            rc = bin_backward(a, tables_of(plan, pix_ws), a.xs, a.Wp, 1, packed, B, C, opts_of(grid_mode), nullptr, st);
             if (rc) return rc;
         }
         if (gg.g_x != nullptr && !sep) a.grid_part = reinterpret_cast<float2*>(gg.ws);
@@ -1167,44 +1217,50 @@ static bool finalize_by_groups(const SuperSlots& sup, int B, int N, int T) {
     return (long)B * N >= IGS_FIN_GROUPS_FROM && T <= IGS_FIN_GROUPS_MAX_TILES;
 }
 
-// The slot tables that the separable backward left behind the partial sums (none on general grids).
-static const int* finalize_slots(const float* partial, int grid_mode, int B, int T, int NF, int N) {
-    if (mode_of(grid_mode) == IGS_GRID_GENERAL) return nullptr;
-    return slots_at(const_cast<float*>(partial), B, T, NF, N);
-}
-
-// T of the separable (or only) variant and of the general variant under AUTO; the super-tile slot
-// tables of the separable backward when it binned in two levels.
-static int finalize_tiles(int grid_mode, int B, int N, int H, int W, int C, int* T, int* T_alt,
-                          const float* partial, SuperSlots* sup) {
+// What the finalize kernels need of the backward that ran: T of the separable (or only) variant and of
+// the general variant under AUTO; the separable backward's tables in its pixel workspace (slot tables,
+// the tiles' first records in the compact partial array, the overflow flag; none on general grids) and
+// the super-tile slot tables when it binned in two levels.
+struct FinalizeTables {
+    int T, T_alt;
+    const int* slots;
+    const long long* offsets;
+    const int* overflow;
+    SuperSlots sup;
+};
+static int finalize_tables(int grid_mode, int B, int N, int H, int W, int C, const float* pix_ws, FinalizeTables* ft) {
     const int opts = opts_of(grid_mode);
     grid_mode = mode_of(grid_mode);
     igs_gs2d_plan_t plan;
     int rc = plan_one(B, N, H, W, C, grid_mode == IGS_GRID_AUTO ? IGS_GRID_SEPARABLE : grid_mode, &plan);
     if (rc) return rc;
-    *T = plan.bwd_tiles;
-    *T_alt = plan.bwd_tiles;
-    *sup = SuperSlots{nullptr, 1, 1, 1, 1};
+    ft->T = plan.bwd_tiles;
+    ft->T_alt = plan.bwd_tiles;
+    ft->slots = nullptr; ft->offsets = nullptr; ft->overflow = nullptr;
+    ft->sup = SuperSlots{nullptr, 1, 1, 1, 1};
     if (grid_mode != IGS_GRID_GENERAL) {
+        if (!pix_ws) return IGS_ERR_NULL_POINTER;
+        const BwdTables t = tables_of(plan, const_cast<float*>(pix_ws));
+        ft->slots = t.slots; ft->offsets = t.offsets; ft->overflow = t.overflow;
         const int tiles_y = plan.bwd_tiles / plan.bwd_tiles_x;
         if (two_level(N, plan.bwd_tiles_x, tiles_y, opts)) {
             const SuperGeometry sg = super_tiles(plan.bwd_tiles_x, tiles_y, B, N);
-            sup->cslots = super_slots_at(const_cast<float*>(partial), B, plan.bwd_tiles, 6 + C, N, plan.n_padded);
-            sup->tiles_x = plan.bwd_tiles_x;
-            sup->tiles_y = tiles_y;
-            sup->stiles_x = sg.x;
-            sup->stiles = sg.count;
+            ft->sup.cslots = t.super_slots;
+            ft->sup.tiles_x = plan.bwd_tiles_x;
+            ft->sup.tiles_y = tiles_y;
+            ft->sup.stiles_x = sg.x;
+            ft->sup.stiles = sg.count;
         }
     }
     if (grid_mode == IGS_GRID_AUTO) {
         rc = plan_one(B, N, H, W, C, IGS_GRID_GENERAL, &plan);
         if (rc) return rc;
-        *T_alt = plan.bwd_tiles;
+        ft->T_alt = plan.bwd_tiles;
     }
     return IGS_OK;
 }
 
-int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t* grid_flag,
+int igs_gs2d_finalize_covinv(const float* partial, const float* pix_ws, int grid_mode, const int32_t* grid_flag,
                              const float* cov_inv_00, const float* cov_inv_01,
                              const float* cov_inv_11, const float* alphas, int B, int N, int H, int W,
                              int C, float* g_position, float* g_cov_inv_00, float* g_cov_inv_01,
@@ -1213,26 +1269,26 @@ int igs_gs2d_finalize_covinv(const float* partial, int grid_mode, const int32_t*
     if (!partial || !cov_inv_00 || !cov_inv_01 || !cov_inv_11 || !alphas) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
-    int T, T_alt;
-    SuperSlots sup;
-    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
+    FinalizeTables ft;
+    rc = finalize_tables(grid_mode, B, N, H, W, C, pix_ws, &ft);
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
-    const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C, N);
-    if (finalize_by_groups(sup, B, N, T))
-        launch_finalize_listed<0>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C, cov_inv_00,
+    if (finalize_by_groups(ft.sup, B, N, ft.T))
+        launch_finalize_listed<0>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.sup,
+                                               (N + 3) & ~3, N, C, C, cov_inv_00,
                                                cov_inv_01, cov_inv_11, alphas, 0.0f, g_position, g_cov_inv_00,
                                                g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors},
                                   B, (hipStream_t)stream);
     else
         IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<false, kFT>),
-                           (hipStream_t)stream, partial, T, flag, T_alt, slots, (N + 3) & ~3, cov_inv_00,
+                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow,
+                           (N + 3) & ~3, cov_inv_00,
                            cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
                            g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
     return launch_status();
 }
 
-int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32_t* grid_flag,
+int igs_gs2d_finalize_scale_rot(const float* partial, const float* pix_ws, int grid_mode, const int32_t* grid_flag,
                                 const float* scales, const float* rotations, const float* alphas,
                                 int B, int N, int H, int W, int C, float eps, float* g_positions,
                                 float* g_scales, float* g_rotations, float* g_alphas, float* g_colors,
@@ -1240,20 +1296,20 @@ int igs_gs2d_finalize_scale_rot(const float* partial, int grid_mode, const int32
     if (!partial || !scales || !rotations || !alphas) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
-    int T, T_alt;
-    SuperSlots sup;
-    rc = finalize_tiles(grid_mode, B, N, H, W, C, &T, &T_alt, partial, &sup);
+    FinalizeTables ft;
+    rc = finalize_tables(grid_mode, B, N, H, W, C, pix_ws, &ft);
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
-    const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C, N);
-    if (finalize_by_groups(sup, B, N, T))
-        launch_finalize_listed<1>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C, scales,
+    if (finalize_by_groups(ft.sup, B, N, ft.T))
+        launch_finalize_listed<1>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.sup,
+                                               (N + 3) & ~3, N, C, C, scales,
                                                rotations, nullptr, alphas, eps, g_positions, g_scales, g_rotations,
                                                nullptr, g_alphas, g_colors},
                                   B, (hipStream_t)stream);
     else
         IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<true, kFT>),
-                           (hipStream_t)stream, partial, T, flag, T_alt, slots, (N + 3) & ~3, scales, rotations,
+                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow,
+                           (N + 3) & ~3, scales, rotations,
                            (const float*)nullptr, alphas, N, C, eps, g_positions,
                            g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
     return launch_status();
@@ -1278,27 +1334,27 @@ int igs_gs2d_pack_feature(const float* gs_feature, const float* pos_offset, int 
     return launch_status();
 }
 
-int igs_gs2d_finalize_feature(const float* partial, int grid_mode, const int32_t* grid_flag,
+int igs_gs2d_finalize_feature(const float* partial, const float* pix_ws, int grid_mode, const int32_t* grid_flag,
                               const float* gs_feature, int B, int N, int H, int W, int C,
                               int C_kernel, float eps, float* g_feature, igs_stream_t stream) {
     if (!partial || !gs_feature || !g_feature) return IGS_ERR_NULL_POINTER;
     int rc = mode_ok(grid_mode, grid_flag);
     if (rc) return rc;
     if (C < 1 || C > C_kernel || !channels_compiled(C_kernel)) return IGS_ERR_BAD_CHANNELS;
-    int T, T_alt;
-    SuperSlots sup;
-    rc = finalize_tiles(grid_mode, B, N, H, W, C_kernel, &T, &T_alt, partial, &sup);
+    FinalizeTables ft;
+    rc = finalize_tables(grid_mode, B, N, H, W, C_kernel, pix_ws, &ft);
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
-    const int* slots = finalize_slots(partial, grid_mode, B, T, 6 + C_kernel, N);
-    if (finalize_by_groups(sup, B, N, T))
-        launch_finalize_listed<2>(FinalizeArgs{partial, T, T_alt, flag, slots, sup, (N + 3) & ~3, N, C, C_kernel,
+    if (finalize_by_groups(ft.sup, B, N, ft.T))
+        launch_finalize_listed<2>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.sup,
+                                               (N + 3) & ~3, N, C, C_kernel,
                                                gs_feature, nullptr, nullptr, nullptr, eps, g_feature, nullptr, nullptr,
                                                nullptr, nullptr, nullptr},
                                   B, (hipStream_t)stream);
     else
         IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize_feature<kFT>),
-                           (hipStream_t)stream, partial, T, flag, T_alt, slots, (N + 3) & ~3, gs_feature,
+                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow,
+                           (N + 3) & ~3, gs_feature,
                            N, C, C_kernel, eps, g_feature);
     return launch_status();
 }

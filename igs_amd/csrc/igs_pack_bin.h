@@ -839,3 +839,43 @@ __global__ __launch_bounds__(kBinThreads) void k_bin_pair(const BinArgs a, const
     const bool second = (int)blockIdx.x >= first_tiles;   // workgroup-uniform
     bin_tile<false>(second ? b : a, (int)blockIdx.x - (second ? first_tiles : 0));
 }
+
+// Exclusive prefix of the tile counts [tiles] (all images' tiles in order): offsets[i] = first record of
+// tile i in the compact partial-sum array, offsets[tiles] = total number of listed entries (also stored to
+// `total_out` when given: device-accessible memory of the caller).  One workgroup; fixed order.
+__global__ __launch_bounds__(kBinThreads) void k_tile_offsets(const int* __restrict__ counts, int tiles,
+                                                              long long* __restrict__ offsets, int* __restrict__ overflow,
+                                                              long long* __restrict__ total_out,
+                                                              const int* __restrict__ flag, int want) {
+    if (flag != nullptr && *flag != want) return;
+    __shared__ long long wsum[kBinThreads / 64];
+    __shared__ long long carry;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) {
+        carry = 0;
+        *overflow = 0;
+    }
+    __syncthreads();
+    for (int i0 = 0; i0 < tiles; i0 += kBinThreads) {
+        const int i = i0 + tid;
+        const long long c = i < tiles ? counts[i] : 0;
+        long long incl = c;  // inclusive prefix within the wave
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const long long o = __shfl_up(incl, d);
+            incl += lane >= d ? o : 0;
+        }
+        if (lane == 63) wsum[wave] = incl;
+        __syncthreads();
+        long long before = carry;
+        for (int w = 0; w < wave; ++w) before += wsum[w];
+        if (i < tiles) offsets[i] = before + incl - c;
+        __syncthreads();
+        if (tid == kBinThreads - 1) carry = before + incl;
+        __syncthreads();
+    }
+    if (tid == 0) {
+        offsets[tiles] = carry;
+        if (total_out != nullptr) *total_out = carry;
+    }
+}

@@ -160,7 +160,7 @@ class GaussianImageFit:
             _lib.check(lib.igs_gs2d_forward_train(
                 _ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n, H, W, Cp, self.eps,
                 _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]), int(p.fwd_ws_bytes), _ptr(ws["pix"]),
-                int(p.pix_bytes), _ptr(ws["partial"]), int(p.partial_bytes), st), "igs_gs2d_forward_train")
+                int(p.pix_bytes), None, st), "igs_gs2d_forward_train")
             return
         _lib.check(lib.igs_gs2d_forward(_ptr(ws["packed"]), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), B, n,
                                         H, W, Cp, self.eps, _ptr(ws["out"]), _ptr(ws["den"]), _ptr(ws["fwd_ws"]),
@@ -188,7 +188,7 @@ class GaussianImageFit:
                                                 _ptr(g.flag), B, n, H, W, Cp, _ptr(ws["pix"]), int(p.pix_bytes),
                                                 _ptr(ws["partial"]), int(p.partial_bytes), st),
                    "igs_gs2d_backward_reduce")
-        _lib.check(lib.igs_gs2d_finalize_feature(_ptr(ws["partial"]), g.mode, _ptr(g.flag), _ptr(self.params), B, n, H,
+        _lib.check(lib.igs_gs2d_finalize_feature(_ptr(ws["partial"]), _ptr(ws["pix"]), g.mode, _ptr(g.flag), _ptr(self.params), B, n, H,
                                                  W, C, Cp, self.eps, _ptr(ws["g_feat"]), st),
                    "igs_gs2d_finalize_feature")
         if self.position_penalty != 0.0:

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define IGS_ABI_VERSION 7
+#define IGS_ABI_VERSION 8
 #define IGS_MAX_CHANNELS 16
 /* Size of the per-device static scratch array behind igs_gs2d_forward_static_ws. */
 #define IGS_STATIC_SCRATCH_BYTES (64u << 20)
@@ -113,9 +113,14 @@ typedef struct igs_gs2d_plan_t {
                                 separable grids, the per-tile Gaussian lists (plus those
                                 of the super-tiles when there are 32 tiles or more)         */
     uint64_t pix_bytes;      /* backward scratch: per-pixel records and, on separable
-                                grids, the Gaussian lists as above                          */
-    uint64_t partial_bytes;  /* backward partial sums B*T*(6+C)*N*4 and, on separable
-                                grids, the slot tables of the tiles (and super-tiles)       */
+                                grids, the backward's tables: the Gaussian lists as above,
+                                the slot tables of the tiles (and super-tiles), the tiles'
+                                first records in the partial-sum array, an overflow flag    */
+    uint64_t partial_bytes;  /* backward partial sums when every Gaussian is stored for
+                                every tile, B*T*(6+C)*N*4: what general grids need, and an
+                                upper bound of what the separable backward needs, which is
+                                (6+C)*4 bytes per listed (Gaussian, tile) entry, see
+                                igs_gs2d_forward_train                                     */
     int32_t fwd_tiles;       /* separable: pixel tiles per image of the forward            */
     int32_t bwd_tiles_x;     /* separable: column bands of the backward tiles              */
     int32_t bwd_tile_w;      /* separable: columns per band                                */
@@ -219,23 +224,28 @@ int igs_gs2d_forward_static_ws(const float *packed, const float *x, const float 
                                float eps, float *out, float *den, igs_stream_t stream);
 
 /* The forward of a training step (a backward on the same packed buffer and grids follows): as
- * igs_gs2d_forward, and on separable grids the backward's per-tile Gaussian lists and slot tables are
- * built as well, in pix_ws / partial (plan.pix_bytes / plan.partial_bytes; the lists depend on the
- * packed buffer and the grids only).  Where plan.lists_shared says that the backward's pixel tiles
- * are the forward's wave rectangles, that one set of lists serves both passes (one binning per
- * step instead of two); elsewhere (small problems, whose backward tiles have fewer rows) the
- * backward's lists are made beside the forward's own by the same launch.  The backward calls on
- * the same workspaces then get IGS_OPT_LISTS_BUILT in their grid_mode (the prologue writes other
- * parts of pix_ws).  The output matches igs_gs2d_forward's up to what the skip tolerance allows
- * (a tile settles what it leaves out by itself, and the tiles of the two binnings need not be the
- * same); bit for bit with skip_weight = skip_fraction = 0 and one Gaussian split.  No counterpart
- * in the reference, which evaluates every pair (src/igs/gs_triton_chunked.py:100-200). */
+ * igs_gs2d_forward, and on separable grids the backward's tables (per-tile Gaussian lists, slot
+ * tables, the tiles' first records in the partial-sum array) are built as well, in pix_ws
+ * (plan.pix_bytes; they depend on the packed buffer and the grids only).  Where plan.lists_shared
+ * says that the backward's pixel tiles are the forward's wave rectangles, that one set of lists
+ * serves both passes (one binning per step instead of two); elsewhere (small problems, whose
+ * backward tiles have fewer rows) the backward's lists are made beside the forward's own by the
+ * same launch.  The backward calls on the same pix_ws then get IGS_OPT_LISTS_BUILT in their
+ * grid_mode (the prologue writes other parts of pix_ws).
+ * listed_total, when not NULL, receives the number of listed (Gaussian, tile) entries, i.e. the
+ * records the separable backward will store: its partial-sum array then needs listed_total *
+ * (6+C) * 4 bytes (at least one record) instead of plan.partial_bytes.  The kernel writes it, so it
+ * must be memory the device can write (device memory, or pinned host memory that the caller reads
+ * after the stream reaches this point).
+ * The output matches igs_gs2d_forward's up to what the skip tolerance allows (a tile settles what
+ * it leaves out by itself, and the tiles of the two binnings need not be the same); bit for bit
+ * with skip_weight = skip_fraction = 0 and one Gaussian split.  No counterpart in the reference,
+ * which evaluates every pair (src/igs/gs_triton_chunked.py:100-200). */
 int igs_gs2d_forward_train(const float *packed, const float *x, const float *y,
-                                  const int64_t grid_strides[6], int grid_mode,
-                                  const int32_t *grid_flag, int B, int N, int H, int W, int C,
-                                  float eps, float *out, float *den, void *ws, size_t ws_bytes,
-                                  float *pix_ws, size_t pix_bytes, float *partial,
-                                  size_t partial_bytes, igs_stream_t stream);
+                           const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag,
+                           int B, int N, int H, int W, int C, float eps, float *out, float *den,
+                           void *ws, size_t ws_bytes, float *pix_ws, size_t pix_bytes,
+                           int64_t *listed_total, igs_stream_t stream);
 
 /* Backward, stage 1: per-pixel prologue, g^ = grad_out/(den+eps), s = <g^, out>, written
  * as one record per pixel into pix_ws (plan.pix_bytes).  Replaces the per-image pre-pass of
@@ -247,11 +257,20 @@ int igs_gs2d_backward_prologue(const float *x, const float *y, const int64_t gri
                                int C, float eps, float *pix_ws, size_t pix_bytes,
                                igs_stream_t stream);
 
-/* Backward, stage 2: the recomputing per-Gaussian reduction over pixel tiles into
- * partial [B,T,N,6+C] (plan.partial_bytes).  Replaces the Gaussian loop of the reference
- * backward, src/igs/gs2d.py:180-246 / src/igs/gs_triton.py:159-405.  colors [B,N,C].
- * pix_ws is the buffer stage 1 filled (16-byte aligned); on separable grids this stage also
- * writes its per-tile Gaussian lists behind the pixel records in it. */
+/* Backward, stage 2: the recomputing per-Gaussian reduction over pixel tiles into `partial`.
+ * Replaces the Gaussian loop of the reference backward, src/igs/gs2d.py:180-246 /
+ * src/igs/gs_triton.py:159-405.  colors [B,N,C].  pix_ws is the buffer stage 1 filled (16-byte
+ * aligned); on separable grids this stage also writes its tables (per-tile Gaussian lists, slot
+ * tables, record offsets) behind the pixel records in it, unless IGS_OPT_LISTS_BUILT says that
+ * igs_gs2d_forward_train did.
+ * partial: general grids store one record of 6+C sums for every Gaussian and tile, [B,T,N,6+C]
+ * (plan.partial_bytes, required).  The separable backward stores the records of the listed
+ * (Gaussian, tile) entries only, tile after tile: partial_bytes may be as small as their number
+ * (igs_gs2d_forward_train's listed_total) * (6+C) * 4, at least one record; plan.partial_bytes
+ * always suffices.  Where partial_bytes does not hold them, nothing is stored for the tiles that
+ * do not fit and the flag in pix_ws is raised, upon which the finalize calls return NaN for every
+ * gradient (no status: nothing here waits for the device).  In AUTO mode plan.partial_bytes is
+ * required. */
 int igs_gs2d_backward_reduce(const float *packed, const float *colors, const float *y,
                              const int64_t grid_strides[6], int grid_mode, const int32_t *grid_flag,
                              int B, int N, int H, int W, int C, float *pix_ws,
@@ -294,9 +313,12 @@ int igs_gs2d_backward_grid(const float *packed, const float *x, const float *y,
 /* Backward, stage 3 (operator level): fixed-order sum of the tile partials and the
  * gradients of the operator inputs (the tail of src/igs/gs2d.py:207-246, :252-262).  The
  * shape and grid mode must be those given to igs_gs2d_backward (they fix the tile count).
- * Any output pointer may be NULL (not wanted).
+ * Any output pointer may be NULL (not wanted).  pix_ws: the backward's pixel workspace, whose
+ * tables say where a Gaussian's records are (separable and AUTO modes; may be NULL with
+ * IGS_GRID_GENERAL).
  * g_position [B,N,2]; g_cov_inv_* [B,N]; g_alphas [B,N]; g_colors [B,N,C]. */
-int igs_gs2d_finalize_covinv(const float *partial, int grid_mode, const int32_t *grid_flag,
+int igs_gs2d_finalize_covinv(const float *partial, const float *pix_ws, int grid_mode,
+                             const int32_t *grid_flag,
                              const float *cov_inv_00, const float *cov_inv_01,
                              const float *cov_inv_11, const float *alphas, int B, int N, int H,
                              int W, int C, float *g_position, float *g_cov_inv_00,
@@ -306,7 +328,8 @@ int igs_gs2d_finalize_covinv(const float *partial, int grid_mode, const int32_t 
 /* Backward, stage 3 (function level): as above plus the chain rule through the closed-form
  * covariance inverse to scales [B,N,2] and rotations [B,N] (the autograd of
  * src/igs/gs2d.py:548-580). */
-int igs_gs2d_finalize_scale_rot(const float *partial, int grid_mode, const int32_t *grid_flag,
+int igs_gs2d_finalize_scale_rot(const float *partial, const float *pix_ws, int grid_mode,
+                                const int32_t *grid_flag,
                                 const float *scales, const float *rotations, const float *alphas,
                                 int B, int N, int H, int W, int C, float eps, float *g_positions,
                                 float *g_scales, float *g_rotations, float *g_alphas,
@@ -324,7 +347,8 @@ int igs_gs2d_finalize_scale_rot(const float *partial, int grid_mode, const int32
 int igs_gs2d_pack_feature(const float *gs_feature, const float *pos_offset, int B, int N, int C,
                           int C_kernel, float eps, float skip_weight, float skip_fraction,
                           float *packed, float *colors_out, igs_stream_t stream);
-int igs_gs2d_finalize_feature(const float *partial, int grid_mode, const int32_t *grid_flag,
+int igs_gs2d_finalize_feature(const float *partial, const float *pix_ws, int grid_mode,
+                              const int32_t *grid_flag,
                               const float *gs_feature, int B, int N, int H, int W, int C,
                               int C_kernel, float eps, float *g_feature, igs_stream_t stream);
 

@@ -123,7 +123,7 @@ def test_argument_errors_are_status_codes_not_crashes(lib):
     assert lib.igs_gs2d_skip_weight(8192, 1e-6, 1e-7) == pytest.approx(1e-13 / 16384, rel=1e-6)
     assert lib.igs_gs2d_skip_weight(8192, 0.0, 1e-7) == 0.0 and lib.igs_gs2d_skip_weight(8192, 1e-6, 0.0) == 0.0
     assert lib.igs_gs2d_skip_weight(1, 1.0, 0.9) < 1.0
-    assert lib.igs_gs2d_finalize_covinv(None, 1, None, None, None, None, None, 1, 8, 4, 4, 3,
+    assert lib.igs_gs2d_finalize_covinv(None, None, 1, None, None, None, None, None, 1, 8, 4, 4, 3,
                                         None, None, None, None, None, None, None) == -1
     assert lib.igs_gs2d_backward_with_grid(None, None, None, None, st, 1, None, None, None, None, 1, 8, 4, 4, 3, 1e-6,
                                            None, 0, None, 0, None, 0, None, None, None) == -1
@@ -284,8 +284,11 @@ def test_plan_invariants_over_random_shapes(lib):
                 assert p.bwd_tiles_x * p.bwd_tile_w >= p.w_padded >= W and p.w_padded % 8 == 0
                 assert p.fwd_tiles >= 1
                 assert p.fwd_ws_bytes >= B * p.fwd_tiles * (Np + 1) * 4
-                assert p.pix_bytes >= (B * H * p.w_padded * p.pix_stride + B * p.w_padded) * 4 + B * p.bwd_tiles * (Np + 1) * 4
-                assert p.partial_bytes >= B * p.bwd_tiles * ((6 + C) * N + Np) * 4      # + slot tables
+                # pixel records and column coordinates, tile lists, slot tables, the tiles' record offsets
+                assert p.pix_bytes >= ((B * H * p.w_padded * p.pix_stride + B * p.w_padded) * 4
+                                       + B * p.bwd_tiles * (2 * Np + 1) * 4 + (B * p.bwd_tiles + 1) * 8)
+                if mode == 1:    # a record for every (Gaussian, tile) pair (AUTO: the larger of the two variants')
+                    assert p.partial_bytes == B * p.bwd_tiles * (6 + C) * N * 4
             else:
                 assert p.hw_padded % 4 == 0 and p.bwd_tiles * p.bwd_per_tile >= p.hw_padded >= H * W
 

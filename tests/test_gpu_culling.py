@@ -717,6 +717,54 @@ def test_training_forward_where_the_tilings_differ(igs, dev, monkeypatch):
         assert torch.equal(grads[k], grads0[k]), k
 
 
+def test_partial_sums_sized_by_the_lists_and_too_small(igs, dev):
+    """The separable backward stores one record per listed (Gaussian, tile) pair, tile after tile: an
+    array of `listed_total` records (the count the training forward leaves) gives the gradients of the
+    full-size array bit for bit, and one that is too small is not overrun: the finalize call then
+    returns NaN everywhere."""
+    from igs_amd import _lib
+    from igs_amd._splat import Grid, Splat, _f32c, _ptr
+
+    B, N, H, W, C = 2, 500, 96, 160, 3
+    _, g = sparse_case(dev, B, N, H, W, C, seed=21)
+    op = Splat(B, N, C, Grid(g["x_grid"], g["y_grid"], B), 1e-6, dev)
+    p, grid, lib = op.plan, op.grid, op.lib
+    col = _f32c(g["colors"])
+    sc, rot, al = _f32c(g["scales"]), _f32c(g["rotations"]), _f32c(g["alphas"])
+    packed = op.pack_scale_rot(_f32c(g["positions"]), sc, rot, al, col)
+    out, den = op._new(B, C, H, W), op._new(B, H, W)
+    ws, pix = op._empty(p.fwd_ws_bytes), op._empty(p.pix_bytes)
+    total = torch.zeros(1, dtype=torch.int64, device=dev)
+    _lib.check(lib.igs_gs2d_forward_train(_ptr(packed), _ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode, _ptr(grid.flag),
+                                          B, N, H, W, C, 1e-6, _ptr(out), _ptr(den), _ptr(ws), int(p.fwd_ws_bytes),
+                                          _ptr(pix), int(p.pix_bytes), _ptr(total), op.stream), "forward_train")
+    listed = int(total.item())
+    assert 0 < listed < B * p.bwd_tiles * N                 # a sparse scene: far fewer pairs than all
+    go = _f32c(g["grad_out"])
+
+    def gradients(records):
+        partial = torch.full((max(records, 1) * (6 + C),), float("nan"), device=dev)
+        _lib.check(lib.igs_gs2d_backward(_ptr(packed), _ptr(col), _ptr(grid.x), _ptr(grid.y), grid.strides,
+                                         grid.mode | _lib.IGS_OPT_LISTS_BUILT, _ptr(grid.flag), _ptr(out), _ptr(den),
+                                         _ptr(go), B, N, H, W, C, 1e-6, _ptr(pix), int(p.pix_bytes), _ptr(partial),
+                                         partial.numel() * 4, op.stream), "backward")
+        gp, gs, gr, ga, gc = op._new(B, N, 2), op._new(B, N, 2), op._new(B, N), op._new(B, N), op._new(B, N, C)
+        _lib.check(lib.igs_gs2d_finalize_scale_rot(_ptr(partial), _ptr(pix), grid.mode, _ptr(grid.flag), _ptr(sc), _ptr(rot),
+                                                   _ptr(al), B, N, H, W, C, 1e-6, _ptr(gp), _ptr(gs), _ptr(gr), _ptr(ga),
+                                                   _ptr(gc), op.stream), "finalize")
+        torch.cuda.synchronize()
+        return gp, gs, gr, ga, gc
+
+    full = gradients(B * p.bwd_tiles * N)
+    assert all(bool(torch.isfinite(t).all()) for t in full) and float(full[0].abs().max()) > 0
+    exact_fit = gradients(listed)
+    assert all(torch.equal(a, b) for a, b in zip(full, exact_fit))
+    for records in (listed - 1, listed // 2, 1):
+        assert all(bool(torch.isnan(t).all()) for t in gradients(records)), records
+    again = gradients(listed)                               # the flag follows the array of each call
+    assert all(torch.equal(a, b) for a, b in zip(full, again))
+
+
 def no_cull_ctx():
     from igs_amd._splat import library_options
 
