@@ -133,7 +133,8 @@ struct BwdArgs {
     const float4* brecs;  // separable: the backward records of the packed buffer [B][Np] (sA, skA, D'', tag)
     const long long* offsets;  // separable: first record of each tile in `partial` [B T + 1], the last = total
     long long capacity;        // separable: records that `partial` holds
-    int* overflow;             // separable: set where the total exceeds the capacity (nothing is stored then for the tiles that do not fit)
+    int* overflow;             // separable: [0] set where the total exceeds the capacity (nothing is stored then for the tiles that do not fit), [1] the stamp of the problem the tables were built for
+    int stamp;                 // separable: tables_stamp of this call
     float* partial;  // general grids: [B][T][N][6+C]; separable: the listed entries' records, tile after tile
     float2* grid_part;  // general grids with grid gradients: [B][groups][HWp] sums of G w (t1, t2)
     const int* flag;
@@ -250,14 +251,19 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
     const int ty = blockIdx.x / a.tiles_x;
     const int tx = (blockIdx.x - ty * a.tiles_x + ty * IGS_BWD_TILE_SHIFT + b * IGS_BWD_TILE_SHIFT) % a.tiles_x;
     const int t = ty * a.tiles_x + tx;
-    const int count = a.counts[(size_t)b * a.T + t];
-    if (blockIdx.x == 0 && grp == 0 && b == 0 && tid == 0) *a.overflow = a.offsets[(size_t)gridDim.z * a.T] > a.capacity;
+    // Tables that were not built for this problem (a caller's IGS_OPT_LISTS_BUILT on other workspaces) are
+    // not read: nothing is stored, and the flag makes the finalize kernels return NaN.
+    const bool foreign = a.overflow[1] != a.stamp;
+    if (blockIdx.x == 0 && grp == 0 && b == 0 && tid == 0)
+        a.overflow[0] = foreign || a.offsets[(size_t)gridDim.z * a.T] > a.capacity;
+    if (foreign) return;  // uniform
+    const int count = min(a.counts[(size_t)b * a.T + t], a.Np);
     if (grp * kThreads >= count) return;  // workgroup-uniform: no listed Gaussian left
     const long long first = a.offsets[(size_t)b * a.T + t];
     if (first + count > a.capacity) return;  // workgroup-uniform: the caller's array does not hold this tile's records
     const int* list = a.lists + ((size_t)b * a.T + t) * a.Np;
     const int pos = grp * kThreads + tid;
-    const int n = pos < count ? list[pos] : a.N;  // >= N: an unused lane (nothing is stored for it)
+    const int n = pos < count ? max(list[pos], 0) : a.N;  // >= N: an unused lane (nothing is stored for it)
     const int nc = min(n, a.N - 1);
     const float* rec = a.packed + ((size_t)b * a.Np + nc) * RS;
     const float4 br = a.brecs[(size_t)b * a.Np + nc];

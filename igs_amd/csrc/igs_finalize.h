@@ -160,7 +160,7 @@ template <bool kScaleRot, int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
     const int* __restrict__ slots_in, const long long* __restrict__ offsets, const int* __restrict__ overflow,
-    int Np, const float* __restrict__ p0,
+    int stamp, int Np, const float* __restrict__ p0,
     const float* __restrict__ p1, const float* __restrict__ p2, const float* __restrict__ alphas,
     int N, int C, float eps, float* __restrict__ g_pos, float* __restrict__ g0,
     float* __restrict__ g1, float* __restrict__ g2, float* __restrict__ g_alpha,
@@ -180,7 +180,8 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize(
     const int* slots = listed ? slots_in + (size_t)b * T * Np : nullptr;
     const long long* toff = listed ? offsets + (size_t)b * T : nullptr;
     const float* part = listed ? partial : partial + (size_t)b * T * NF * N;
-    const bool lost = listed && *overflow != 0;  // the partial sums did not fit the caller's array: no gradient is known
+    // the partial sums did not fit the caller's array, or the tables are not this problem's: no gradient is known
+    const bool lost = listed && (overflow[0] != 0 || overflow[1] != stamp);
     const int nn = min(n, N - 1);
     // first pass: the moments and, when wanted, the first colours (they follow the moments)
     constexpr int kC0 = kFinFirst - 6;
@@ -215,7 +216,7 @@ template <int FT>
 __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const float* __restrict__ partial, int T_in, const int* __restrict__ flag, int T_alt,
     const int* __restrict__ slots_in, const long long* __restrict__ offsets, const int* __restrict__ overflow,
-    int Np, const float* __restrict__ feat, int N,
+    int stamp, int Np, const float* __restrict__ feat, int N,
     int C, int Cp,
     float eps, float* __restrict__ g_feat) {
     constexpr int FN = 256 / FT;
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_feature(
     const int* slots = listed ? slots_in + (size_t)b * T * Np : nullptr;
     const long long* toff = listed ? offsets + (size_t)b * T : nullptr;
     const float* part = listed ? partial : partial + (size_t)b * T * NF * N;
-    const bool lost = listed && *overflow != 0;
+    const bool lost = listed && (overflow[0] != 0 || overflow[1] != stamp);
     const int nn = min(n, N - 1);
     constexpr int kC0 = kFinFirst - 6;
     float M[kFinFirst];
@@ -289,7 +290,8 @@ struct FinalizeArgs {
     const int* flag;    // AUTO grid mode: *flag == 0 -> the general backward ran (T_alt dense tiles, no tables)
     const int* slots;   // [B][T][Np] of the separable backward
     const long long* offsets;  // [B T + 1]: the tiles' first records in its compact partial array
-    const int* overflow;       // set where that array was too small
+    const int* overflow;       // [0] set where that array was too small, [1] the stamp of the tables
+    int stamp;                 // tables_stamp of this call
     SuperSlots sup;
     int Np, N, C, Cp;   // C: channels of the caller's rows (feature kind), Cp: of the records
     const float *p0, *p1, *p2, *alphas;  // cov_inv_* | scales, rotations | gs_feature
@@ -400,7 +402,7 @@ __global__ __launch_bounds__(kThreads) void k_bwd_finalize_listed(const Finalize
     const float* part = general ? a.partial + (size_t)b * T * NF * a.N : a.partial;
     const int* slots = a.slots != nullptr ? a.slots + (size_t)b * a.T * a.Np : nullptr;
     const long long* toff = general ? nullptr : a.offsets + (size_t)b * a.T;
-    const bool lost = !general && *a.overflow != 0;  // the partial sums did not fit the caller's array
+    const bool lost = !general && (a.overflow[0] != 0 || a.overflow[1] != a.stamp);  // no gradient is known
     SuperSlots sup = a.sup;
     if (sup.cslots != nullptr) sup.cslots += (size_t)b * sup.stiles * a.Np;
     for (int k = 0; k < kFinGroupBatch / kGroups; ++k) {

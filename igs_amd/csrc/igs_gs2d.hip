@@ -558,6 +558,18 @@ int launch_bwd_reduce(const BwdArgs& a, int B, bool sep, hipStream_t st) {
     return launch_status();
 }
 
+// Names the problem a set of backward tables belongs to (shape, tiling, binning depth): written beside the
+// tables and compared by the kernels that read them.  Never 0.
+inline int tables_stamp(const igs_gs2d_plan_t& plan, int opts) {
+    unsigned long long h = 0x9E3779B97F4A7C15ull;
+    const int tiles_y = plan.bwd_tiles / (plan.bwd_tiles_x > 0 ? plan.bwd_tiles_x : 1);
+    const int v[] = {plan.B, plan.N, plan.H, plan.W, plan.C, plan.bwd_tiles, plan.bwd_tiles_x, plan.bwd_per_tile,
+                     two_level(plan.N, plan.bwd_tiles_x, tiles_y, opts) ? 2 : 1};
+    for (int x : v) h = (h ^ (unsigned long long)(unsigned int)x) * 0x100000001B3ull;
+    const int s = (int)(h ^ (h >> 32));
+    return s != 0 ? s : 1;
+}
+
 // The separable backward's tables inside its pixel workspace (plan: the separable variant's).
 inline BwdTables tables_of(const igs_gs2d_plan_t& plan, void* pix_ws) {
     const int B = plan.B, T = plan.bwd_tiles, tiles_y = T / plan.bwd_tiles_x;
@@ -570,7 +582,7 @@ inline BwdTables tables_of(const igs_gs2d_plan_t& plan, void* pix_ws) {
 // separable backward may store).
 int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* colors, const float* y,
              const int64_t gs[6], int B, int N, int H, int W, int C, float* pix_ws, float* partial,
-             size_t partial_bytes = 0) {
+             size_t partial_bytes = 0, int opts = 0) {
     igs_gs2d_plan_t plan;
     const int rc = plan_one(B, N, H, W, C, v.mode, &plan);
     if (rc) return rc;
@@ -584,6 +596,7 @@ int bwd_args(BwdArgs& a, const Variant& v, const float* packed, const float* col
     a.tiles_x = plan.bwd_tiles_x;
     a.per_tile = plan.bwd_per_tile;
     a.counts = nullptr; a.lists = nullptr; a.offsets = nullptr; a.overflow = nullptr;
+    a.stamp = sep ? tables_stamp(plan, opts) : 0;
     a.capacity = (long long)(partial_bytes / ((6 + C) * sizeof(float)));
     a.brecs = packed ? brecs_of(packed, B, plan.n_padded, C) : nullptr;
     if (sep && pix_ws) {
@@ -627,6 +640,7 @@ const char* igs_status_string(int status) {
         case IGS_ERR_ALIGNMENT: return "buffer not 16-byte aligned";
         case IGS_ERR_BAD_SKIP_WEIGHT: return "skip weight outside [0, 1)";
         case IGS_ERR_STATIC_SCRATCH: return "problem needs more scratch than the static array holds (IGS_STATIC_SCRATCH_BYTES)";
+        case IGS_ERR_STATIC_BUSY: return "the static scratch array is still in use by a call on another stream";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -727,7 +741,7 @@ BinArgs backward_bin_args(const BwdArgs& a, const BwdTables& t, const float* x, 
 // total, to `total_out` as well when given: device-accessible memory, e.g. pinned host memory).
 int launch_tile_offsets(const BwdArgs& a, const BwdTables& t, int B, long long* total_out, hipStream_t st) {
     hipLaunchKernelGGL(k_tile_offsets, dim3(1), dim3(kBinThreads), 0, st, (const int*)t.bins.counts, B * a.T, t.offsets,
-                       t.overflow, total_out, a.flag, a.want);
+                       t.overflow, a.stamp, total_out, a.flag, a.want);
     return launch_status();
 }
 
@@ -792,7 +806,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
         if (sep && shared) {
             // the backward's tiles are the forward's wave rectangles (or tiles): its lists serve both
             BwdArgs bw;
-            rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr);
+            rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr, 0, opts_of(grid_mode));
             if (rc) return rc;
             rc = bin_backward(bw, tables_of(plan, pix_ws), x, grid_strides[0], grid_strides[2], packed, B, C,
                               opts_of(grid_mode), total_out, st);
@@ -842,7 +856,7 @@ int forward_impl(const float* packed, const float* x, const float* y,
                 // are enough of them): the backward's lists are built now as well, in its workspaces, in
                 // the same launch where both binnings are of the plain kind, else in a second one.
                 BwdArgs bw;
-                rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr);
+                rc = bwd_args(bw, vs[i], packed, nullptr, y, grid_strides, B, N, H, W, C, pix_ws, nullptr, 0, opts_of(grid_mode));
                 if (rc) return rc;
                 const BwdTables bt = tables_of(plan, pix_ws);
                 rc = -1;
@@ -886,23 +900,32 @@ static __device__ __align__(256) unsigned char scratch[IGS_STATIC_SCRATCH_BYTES]
 namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
-void* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each device, resolved once
+// Per device: the device address of `scratch` (resolved once) and the guard against overlapping use of it.
+struct StaticScratch {
+    void* ptr = nullptr;
+    hipEvent_t done = nullptr;     // recorded behind every call outside graph capture
+    hipStream_t stream = nullptr;  // of that call
+    bool recorded = false;
+};
+StaticScratch g_scratch[kMaxDevices];
 
-// The current device's copy of the static scratch array (resolved on the first call on that device).
-int static_scratch(void** ptr) {
+// The current device's entry (address and event made on the first call on that device).  Caller holds the mutex.
+int static_scratch(StaticScratch** out) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= kMaxDevices) return IGS_ERR_NO_DEVICE;
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (g_scratch_ptr[dev] == nullptr) {
+    StaticScratch& s = g_scratch[dev];
+    if (s.ptr == nullptr) {
         void* p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return (int)e;
         if (p == nullptr) return IGS_ERR_NO_DEVICE;
-        g_scratch_ptr[dev] = p;
+        e = hipEventCreateWithFlags(&s.done, hipEventDisableTiming);
+        if (e != hipSuccess) return (int)e;
+        s.ptr = p;
     }
-    *ptr = g_scratch_ptr[dev];
+    *out = &s;
     return IGS_OK;
 }
 }  // namespace
@@ -937,11 +960,24 @@ int igs_gs2d_forward_static_ws(const float* packed, const float* x, const float*
     rc = make_plan(B, N, H, W, C, grid_mode, &total);
     if (rc) return rc;
     if (total.fwd_ws_bytes > (uint64_t)IGS_STATIC_SCRATCH_BYTES) return IGS_ERR_STATIC_SCRATCH;
-    void* ws = nullptr;
-    rc = static_scratch(&ws);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);  // (held over the enqueue: calls of two threads do not interleave)
+    StaticScratch* sc = nullptr;
+    rc = static_scratch(&sc);
     if (rc) return rc;
-    return forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, ws,
-                        IGS_STATIC_SCRATCH_BYTES, nullptr, 0, nullptr, stream);
+    hipStream_t st = (hipStream_t)stream;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
+    const bool guarded = capture == hipStreamCaptureStatusNone;
+    // the previous call's work still running on another stream: it is reading and writing the array
+    if (guarded && sc->recorded && sc->stream != st && hipEventQuery(sc->done) == hipErrorNotReady)
+        return IGS_ERR_STATIC_BUSY;
+    rc = forward_impl(packed, x, y, grid_strides, grid_mode, grid_flag, B, N, H, W, C, eps, out, den, sc->ptr,
+                      IGS_STATIC_SCRATCH_BYTES, nullptr, 0, nullptr, stream);
+    if (rc == IGS_OK && guarded && hipEventRecord(sc->done, st) == hipSuccess) {
+        sc->recorded = true;
+        sc->stream = st;
+    }
+    return rc;
 }
 
 }  // extern "C"
@@ -1096,7 +1132,8 @@ int backward_reduce(const float* packed, const float* colors, const float* y,
     const int nv = variants_of(grid_mode, grid_flag, vs);
     for (int i = 0; i < nv; ++i) {
         BwdArgs a;
-        rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C, pix_ws, partial, partial_bytes);
+        rc = bwd_args(a, vs[i], packed, colors, y, grid_strides, B, N, H, W, C, pix_ws, partial, partial_bytes,
+                      opts_of(grid_mode));
         if (rc) return rc;
         const bool sep = vs[i].mode == IGS_GRID_SEPARABLE;
         if (sep && !(opts_of(grid_mode) & IGS_OPT_LISTS_BUILT)) {
@@ -1226,6 +1263,7 @@ struct FinalizeTables {
     const int* slots;
     const long long* offsets;
     const int* overflow;
+    int stamp;
     SuperSlots sup;
 };
 static int finalize_tables(int grid_mode, int B, int N, int H, int W, int C, const float* pix_ws, FinalizeTables* ft) {
@@ -1237,11 +1275,13 @@ static int finalize_tables(int grid_mode, int B, int N, int H, int W, int C, con
     ft->T = plan.bwd_tiles;
     ft->T_alt = plan.bwd_tiles;
     ft->slots = nullptr; ft->offsets = nullptr; ft->overflow = nullptr;
+    ft->stamp = 0;
     ft->sup = SuperSlots{nullptr, 1, 1, 1, 1};
     if (grid_mode != IGS_GRID_GENERAL) {
         if (!pix_ws) return IGS_ERR_NULL_POINTER;
         const BwdTables t = tables_of(plan, const_cast<float*>(pix_ws));
         ft->slots = t.slots; ft->offsets = t.offsets; ft->overflow = t.overflow;
+        ft->stamp = tables_stamp(plan, opts);
         const int tiles_y = plan.bwd_tiles / plan.bwd_tiles_x;
         if (two_level(N, plan.bwd_tiles_x, tiles_y, opts)) {
             const SuperGeometry sg = super_tiles(plan.bwd_tiles_x, tiles_y, B, N);
@@ -1274,14 +1314,14 @@ int igs_gs2d_finalize_covinv(const float* partial, const float* pix_ws, int grid
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
     if (finalize_by_groups(ft.sup, B, N, ft.T))
-        launch_finalize_listed<0>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.sup,
+        launch_finalize_listed<0>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.stamp, ft.sup,
                                                (N + 3) & ~3, N, C, C, cov_inv_00,
                                                cov_inv_01, cov_inv_11, alphas, 0.0f, g_position, g_cov_inv_00,
                                                g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors},
                                   B, (hipStream_t)stream);
     else
         IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<false, kFT>),
-                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow,
+                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow, ft.stamp,
                            (N + 3) & ~3, cov_inv_00,
                            cov_inv_01, cov_inv_11, alphas, N, C, 0.0f, g_position,
                            g_cov_inv_00, g_cov_inv_01, g_cov_inv_11, g_alphas, g_colors);
@@ -1301,14 +1341,14 @@ int igs_gs2d_finalize_scale_rot(const float* partial, const float* pix_ws, int g
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
     if (finalize_by_groups(ft.sup, B, N, ft.T))
-        launch_finalize_listed<1>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.sup,
+        launch_finalize_listed<1>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.stamp, ft.sup,
                                                (N + 3) & ~3, N, C, C, scales,
                                                rotations, nullptr, alphas, eps, g_positions, g_scales, g_rotations,
                                                nullptr, g_alphas, g_colors},
                                   B, (hipStream_t)stream);
     else
         IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize<true, kFT>),
-                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow,
+                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow, ft.stamp,
                            (N + 3) & ~3, scales, rotations,
                            (const float*)nullptr, alphas, N, C, eps, g_positions,
                            g_scales, g_rotations, (float*)nullptr, g_alphas, g_colors);
@@ -1346,14 +1386,14 @@ int igs_gs2d_finalize_feature(const float* partial, const float* pix_ws, int gri
     if (rc) return rc;
     const int32_t* flag = mode_of(grid_mode) == IGS_GRID_AUTO ? grid_flag : nullptr;
     if (finalize_by_groups(ft.sup, B, N, ft.T))
-        launch_finalize_listed<2>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.sup,
+        launch_finalize_listed<2>(FinalizeArgs{partial, ft.T, ft.T_alt, flag, ft.slots, ft.offsets, ft.overflow, ft.stamp, ft.sup,
                                                (N + 3) & ~3, N, C, C_kernel,
                                                gs_feature, nullptr, nullptr, nullptr, eps, g_feature, nullptr, nullptr,
                                                nullptr, nullptr, nullptr},
                                   B, (hipStream_t)stream);
     else
         IGS_FINALIZE_LAUNCH(B, N, (k_bwd_finalize_feature<kFT>),
-                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow,
+                           (hipStream_t)stream, partial, ft.T, flag, ft.T_alt, ft.slots, ft.offsets, ft.overflow, ft.stamp,
                            (N + 3) & ~3, gs_feature,
                            N, C, C_kernel, eps, g_feature);
     return launch_status();

@@ -843,9 +843,11 @@ __global__ __launch_bounds__(kBinThreads) void k_bin_pair(const BinArgs a, const
 // Exclusive prefix of the tile counts [tiles] (all images' tiles in order): offsets[i] = first record of
 // tile i in the compact partial-sum array, offsets[tiles] = total number of listed entries (also stored to
 // `total_out` when given: device-accessible memory of the caller).  One workgroup; fixed order.
+// overflow[1] receives `stamp`, a value that names the problem the tables were built for (tables_stamp): the
+// kernels that trust tables built earlier (IGS_OPT_LISTS_BUILT) compare it with their own.
 __global__ __launch_bounds__(kBinThreads) void k_tile_offsets(const int* __restrict__ counts, int tiles,
                                                               long long* __restrict__ offsets, int* __restrict__ overflow,
-                                                              long long* __restrict__ total_out,
+                                                              int stamp, long long* __restrict__ total_out,
                                                               const int* __restrict__ flag, int want) {
     if (flag != nullptr && *flag != want) return;
     __shared__ long long wsum[kBinThreads / 64];
@@ -853,7 +855,8 @@ __global__ __launch_bounds__(kBinThreads) void k_tile_offsets(const int* __restr
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid == 0) {
         carry = 0;
-        *overflow = 0;
+        overflow[0] = 0;
+        overflow[1] = stamp;
     }
     __syncthreads();
     for (int i0 = 0; i0 < tiles; i0 += kBinThreads) {

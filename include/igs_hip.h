@@ -43,6 +43,8 @@ typedef enum igs_status {
     IGS_ERR_ALIGNMENT = -7,      /* a buffer that must be 16-byte aligned is not */
     IGS_ERR_STATIC_SCRATCH = -8, /* igs_gs2d_forward_static_ws: the plan's fwd_ws_bytes exceeds
                                     IGS_STATIC_SCRATCH_BYTES */
+    IGS_ERR_STATIC_BUSY = -10,   /* igs_gs2d_forward_static_ws: the previous call on this device, made on
+                                    another stream, has not finished with the one scratch array */
     IGS_ERR_BAD_SKIP_WEIGHT = -9 /* a pack call's skip_weight or skip_fraction is negative, NaN
                                     or >= 1 */
 } igs_status;
@@ -215,7 +217,12 @@ int igs_gs2d_forward(const float *packed, const float *x, const float *y,
  * igs_gs2d_forward).  Same kernels, same launch plan and bit-identical results as
  * igs_gs2d_forward.  All calls on one GPU share that GPU's array: calls that overlap in time on
  * one GPU (two streams, two threads) race on it; nothing in it has to start at zero and its
- * contents mean nothing after the call.  The first call on a device resolves the array's device
+ * contents mean nothing after the call.  A cheap guard catches the common case: a call made on
+ * another stream than the previous one while that one's work has not finished (an event recorded
+ * behind each call, queried without waiting) returns IGS_ERR_STATIC_BUSY instead of running; calls
+ * on one stream are ordered by the stream and never refused.  The guard is off while the stream
+ * is being captured into a graph (a replayed graph's overlap with other work stays the caller's
+ * to exclude).  The first call on a device resolves the array's device
  * address (hipGetSymbolAddress, which may load the code object there): make that call outside
  * graph capture, with that device current. */
 int igs_gs2d_forward_static_ws(const float *packed, const float *x, const float *y,

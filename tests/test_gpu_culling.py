@@ -743,6 +743,7 @@ def test_partial_sums_sized_by_the_lists_and_too_small(igs, dev):
     go = _f32c(g["grad_out"])
 
     def gradients(records):
+        nonlocal pix
         partial = torch.full((max(records, 1) * (6 + C),), float("nan"), device=dev)
         _lib.check(lib.igs_gs2d_backward(_ptr(packed), _ptr(col), _ptr(grid.x), _ptr(grid.y), grid.strides,
                                          grid.mode | _lib.IGS_OPT_LISTS_BUILT, _ptr(grid.flag), _ptr(out), _ptr(den),
@@ -763,6 +764,14 @@ def test_partial_sums_sized_by_the_lists_and_too_small(igs, dev):
         assert all(bool(torch.isnan(t).all()) for t in gradients(records)), records
     again = gradients(listed)                               # the flag follows the array of each call
     assert all(torch.equal(a, b) for a, b in zip(full, again))
+    # IGS_OPT_LISTS_BUILT on a workspace whose tables were never built (here: bytes of another problem's
+    # run) is not trusted: the tables carry a stamp of their problem, nothing is read through them and
+    # the gradients come back NaN
+    good = pix
+    for fill in (0.0, 1.0e9, -3.0):
+        pix = torch.full_like(good, fill)
+        assert all(bool(torch.isnan(t).all()) for t in gradients(B * p.bwd_tiles * N)), fill
+    pix = good
 
 
 def no_cull_ctx():

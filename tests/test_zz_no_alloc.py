@@ -85,3 +85,42 @@ def test_static_scratch_forward_rejects_what_does_not_fit(dev):
                                         1e-6, ptr, ptr, None)
     assert rc == -8
     assert b"static" in lib.igs_status_string(rc)
+
+
+def test_static_scratch_forward_refuses_an_overlapping_call_on_another_stream(dev):
+    """One array per GPU: a call on another stream than the previous one, while that one's work is
+    still running, gets a status instead of the array; on the same stream, or once the work is done,
+    calls go through."""
+    from igs_amd import _lib
+    from igs_amd._splat import Grid, Splat, _ptr
+
+    lib = _lib.load()
+    B, N, H, W, C = 1, 512, 64, 64, 3
+    d = {k: v.to(dev, torch.float32) for k, v in O.make_config_inputs("c1", B=B, N=N, H=H, W=W).items()}
+    xg = d["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+    yg = d["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+    with torch.cuda.device(dev):
+        grid = Grid(xg, yg, B)
+        op = Splat(B, N, C, grid, 1e-6, dev)
+        packed = op.pack_scale_rot(d["positions"].contiguous(), d["scales"].contiguous(), d["rotations"].contiguous(),
+                                   d["alphas"].contiguous(), d["colors"].contiguous())
+        ref_out, _ = op.forward(packed)
+        out, den = torch.empty_like(ref_out), op._new(B, H, W)
+        s1, s2 = torch.cuda.Stream(dev), torch.cuda.Stream(dev)
+        torch.cuda.synchronize()
+
+        def call(stream):
+            return lib.igs_gs2d_forward_static_ws(_ptr(packed), _ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode,
+                                                  _ptr(grid.flag), B, N, H, W, op.Cp, 1e-6, _ptr(out), _ptr(den),
+                                                  stream.cuda_stream)
+
+        with torch.cuda.stream(s1):
+            torch.cuda._sleep(200_000_000)      # keeps s1 busy for a fraction of a second: the call behind it cannot have finished
+        assert call(s1) == 0
+        assert call(s1) == 0                    # the same stream: ordered, never refused
+        rc = call(s2)
+        assert rc == -10 and b"still in use" in lib.igs_status_string(rc)
+        torch.cuda.synchronize()
+        assert call(s2) == 0                    # the earlier work is done
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref_out)
