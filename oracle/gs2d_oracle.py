@@ -334,6 +334,128 @@ def tile_first_skipped_class(classes, N: int, w: float, f: float, floor: float):
     return first
 
 
+def backward_with_lists(x, y, position, a, b_, d, alphas, colors, grad_out, eps, keep_fwd, keep_bwd):
+    """What the kernels compute when lists leave pairs out, restated densely (small inputs only):
+    the forward sums the pairs of `keep_fwd` [B,N,H,W] (bool), the backward takes that forward's
+    image and denominator and sums, for every Gaussian, the pairs of `keep_bwd`; the formulas are
+    those of `backward_strips`.  With both masks all true this is `backward_strips` itself.
+    Returns (out, grads).  No counterpart in the reference, which evaluates every pair
+    (src/igs/gs_triton_chunked.py:100-200)."""
+    B, N, C = colors.shape
+    x, y = _as4(x, B), _as4(y, B)
+    A, Bc, D = (t.reshape(B, N, 1, 1) for t in (a, b_, d))
+    dx = x - position[..., 0, None, None]
+    dy = y - position[..., 1, None, None]
+    e = torch.exp(-0.5 * (dx * dx * A + 2 * dx * dy * Bc + dy * dy * D))
+    wgt = e * alphas[..., None, None]
+    wf = wgt * keep_fwd
+    den = wf.sum(1, keepdim=True) + eps                                   # [B,1,H,W]
+    out = torch.einsum("bnhw,bnc->bchw", wf, colors) / den
+    gh = grad_out / den
+    G = torch.einsum("bchw,bnc->bnhw", gh, colors) - (gh * out).sum(1, keepdim=True)
+    G = G * keep_bwd
+    Gw = G * wgt
+    lx, ly = A * dx + Bc * dy, Bc * dx + D * dy
+    grads = dict(
+        position=torch.stack([(Gw * lx).sum((2, 3)), (Gw * ly).sum((2, 3))], dim=-1),
+        cov_inv_00=(-0.5 * Gw * dx * dx).sum((2, 3)),
+        cov_inv_01=(-Gw * dx * dy).sum((2, 3)),
+        cov_inv_11=(-0.5 * Gw * dy * dy).sum((2, 3)),
+        alphas=(G * e).sum((2, 3)),
+        colors=torch.einsum("bchw,bnhw->bnc", gh, wgt * keep_bwd),
+    )
+    return out, grads
+
+
+def culling_gradient_bound(x, y, position, a, b_, d, alphas, colors, grad_out, eps, tolerance):
+    """How far the lists can move a gradient, for alphas >= 0 (so every denominator is >= 0 and
+    |out| <= max|c|).  Write D = den + eps, g1 = sum_c |g_c| of a pixel, K = max|c| + max|out|,
+    m_n = max(1, alpha_n).  Per pixel the largest terms u_n of the Gaussians a tile leaves out add up
+    to at most the allowance A = N (w + f S) <= tolerance D (`tile_first_skipped_class`; both the
+    forward's and the backward's tiling keep to it, each with its own floor S).
+
+    The kernels' gradient of a parameter th of Gaussian n is sum over the backward's kept pixels of
+    G' dw/dth with G' = <g, c_n - out'> / D' taken from the forward's own (culled) image.  Against
+    the sum over all pixels of G dw/dth it differs by
+      (1) the pairs the backward leaves out.  |G| <= g1 K / D and, with e <= u / m, q >= 2 ln(m / u):
+          e q^k <= (u / m) (2 ln(m / u) + 2 k)^k  (e q^k falls beyond q = 2 k, where it is (2 k / e)^k),
+          |dw/dth| <= |w| P_th q^k  with  (P, k) = (1 / m, 0) for alpha (dw/dalpha = e),
+          (sqrt(A), 1/2), (sqrt(D), 1/2) for the position (Cauchy-Schwarz in the metric of q),
+          (Sxx / 2, 1), (sqrt(Sxx Syy), 1), (Syy / 2, 1) for cov_inv_00 / 01 / 11 (S the covariance:
+          dx^2 <= q Sxx, dy^2 <= q Syy), and for a colour |g_c| |w| / D.
+          u (2 ln(m / u) + 2 k)^k grows with u and is concave on u <= m (k <= 1), the u_n of a pixel
+          add up to at most tolerance D and D >= eps, so (Jensen) over ALL Gaussians
+              sum_n |(1)| / P_th,n  <=  tolerance Lam^k sum_px g1 K  =: T Lam^k,
+          Lam = max(2, 2 + 2 ln(N max m / (tolerance eps)));  for the colours sum_n |(1)| <= tolerance sum |g_c|.
+      (2) G' - G on the kept pairs.  With a = A / D <= tolerance: D' >= (1 - a) D,
+          |1/D' - 1/D| <= a / ((1 - a) D), |out' - out| <= a K / (1 - a), hence
+          |G' - G| <= tau g1 K / D with tau = tolerance (2 - tolerance) / (1 - tolerance)^2, and
+              |(2)| <= tau Gam_th,n,   Gam_th,n = sum_px g1 K / D |dw_n/dth|
+          -- the gradient's own sum with every term replaced by the bound of its absolute value; for
+          a colour |(2)| <= tolerance / (1 - tolerance) sum_px |g_c| |w| / D  (<= tau Gam).
+    So  |d th_n| <= T Lam^k P_th,n + tau Gam_th,n  for every element, and over a whole tensor
+    sum_n |d th_n| / P_th,n <= T Lam^k + tau sum_n Gam_th,n / P_th,n.
+
+    Returns (first, gamma, tau): dicts of per-element tensors first = T Lam^k P (the colours:
+    tolerance sum_px |g_c|, the same for every Gaussian) and gamma = Gam, named like the gradients of
+    `backward_strips`; dense evaluation, small inputs only.  No counterpart in the reference, which
+    evaluates every pair (src/igs/gs_triton_chunked.py:100-200)."""
+    B, N, C = colors.shape
+    x, y = _as4(x, B), _as4(y, B)
+    A, Bc, D = (t.reshape(B, N, 1, 1) for t in (a, b_, d))
+    dx = x - position[..., 0, None, None]
+    dy = y - position[..., 1, None, None]
+    q = dx * dx * A + 2 * dx * dy * Bc + dy * dy * D
+    e = torch.exp(-0.5 * q)
+    wgt = (e * alphas[..., None, None]).abs()
+    den = (e * alphas[..., None, None]).sum(1, keepdim=True) + eps
+    out = torch.einsum("bnhw,bnc->bchw", e * alphas[..., None, None], colors) / den
+    K = colors.abs().max() + out.abs().amax(1, keepdim=True)                # [B,1,H,W]
+    g1 = grad_out.abs().sum(1, keepdim=True)
+    s = g1 * K / den.abs()
+    m = torch.clamp(alphas.abs(), min=1.0)
+    lam = max(2.0, 2.0 + 2.0 * math.log(N * float(m.max()) / (tolerance * eps)))
+    T = tolerance * (g1 * K).sum((1, 2, 3))[:, None]                        # [B,1]
+    tau = tolerance * (2 - tolerance) / (1 - tolerance) ** 2
+    An, Bn, Dn = (t.reshape(B, N) for t in (a, b_, d))
+    det = An * Dn - Bn * Bn
+    sxx, syy = Dn / det, An / det
+    first = dict(
+        alphas=T / m,
+        position=T[..., None] * math.sqrt(lam) * torch.stack([An.sqrt(), Dn.sqrt()], dim=-1),
+        cov_inv_00=T * lam * 0.5 * sxx,
+        cov_inv_01=T * lam * (sxx * syy).sqrt(),
+        cov_inv_11=T * lam * 0.5 * syy,
+        colors=(tolerance * grad_out.abs().sum((2, 3)))[:, None, :].expand(B, N, C),
+    )
+    sw = s * wgt
+    gamma = dict(
+        alphas=(s * e).sum((2, 3)),
+        position=torch.stack([(sw * (A * dx + Bc * dy).abs()).sum((2, 3)),
+                              (sw * (Bc * dx + D * dy).abs()).sum((2, 3))], dim=-1),
+        cov_inv_00=(0.5 * sw * dx * dx).sum((2, 3)),
+        cov_inv_01=(sw * (dx * dy).abs()).sum((2, 3)),
+        cov_inv_11=(0.5 * sw * dy * dy).sum((2, 3)),
+        colors=torch.einsum("bchw,bnhw->bnc", grad_out.abs() / den.abs(), wgt),
+    )
+    return first, gamma, tau
+
+
+def chain_bound_to_scale_rotation(scales, rotations, bA, bB, bD, eps=1e-6):
+    """Carries element-wise bounds on the gradients of (cov_inv_00, 01, 11) to bounds on those of
+    (scales [B,N,2], rotations [B,N]): `chain_to_scale_rotation` with every coefficient replaced by
+    its absolute value (the chain is linear per Gaussian)."""
+    c, s = torch.cos(rotations), torch.sin(rotations)
+    i0 = 1.0 / (scales[..., 0] ** 2 + eps)
+    i1 = 1.0 / (scales[..., 1] ** 2 + eps)
+    bi0 = bA * c * c + bB * (c * s).abs() + bD * s * s
+    bi1 = bA * s * s + bB * (c * s).abs() + bD * c * c
+    bs = torch.stack([bi0 * (2 * scales[..., 0].abs() * i0 * i0),
+                      bi1 * (2 * scales[..., 1].abs() * i1 * i1)], dim=-1)
+    bth = (bD + bA) * 2 * (c * s * (i0 - i1)).abs() + bB * ((c * c - s * s) * (i0 - i1)).abs()
+    return bs, bth
+
+
 def reach_q(alphas, w: float):
     """q_max of each Gaussian's reach box under skip weight w: five binades beyond its skip limit
     (the exact-zero case gives REACH_Q)."""

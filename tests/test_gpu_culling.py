@@ -624,6 +624,51 @@ def test_default_skip_tolerance_stays_within_its_bound(igs, dev, alpha_scale):
         assert float(d.norm()) <= 1e-5 * float(grads0[k].double().norm()), k
 
 
+@pytest.mark.parametrize("tolerance,alpha_scale,smax", [(1e-7, 1.0, 0.03), (1e-3, 1.0, 0.03), (1e-3, 25.0, 0.03),
+                                                        (1e-2, 0.05, 0.3)])
+def test_gradients_under_culling_stay_within_their_bound(igs, dev, tolerance, alpha_scale, smax):
+    """The gradients of the default lists (and of far coarser ones) against the run that lists every
+    Gaussian for every tile: every element within the oracle's bound T Lam^k P + tau Gam
+    (`culling_gradient_bound`, chained to scales and rotations with absolute coefficients), plus the
+    rounding of two fp32 evaluations whose sums are grouped differently, priced at 2e-6 Gam (Gam is
+    the gradient's own sum with every term taken by its bound); and over each tensor the summed form."""
+    from igs_amd._splat import library_options
+
+    B, N, H, W, C = 2, 120, 96, 128, 3
+    d64, g = sparse_case(dev, B, N, H, W, C, seed=29, smin=0.003, smax=smax)
+    g["alphas"] = (g["alphas"] * alpha_scale).contiguous()
+    assert bool((g["alphas"] >= 0).all())
+    with library_options(skip_tolerance=tolerance):
+        out, grads = run(igs, g)
+    with library_options(no_cull=True):
+        out0, grads0 = run(igs, g)
+    assert bool((out - out0).abs().max() <= tolerance * g["colors"].abs().max() + 3e-7 * out0.abs().max())
+    c = {k: v.double().cpu() for k, v in g.items()}
+    a, b, dd = (t.reshape(B, N) for t in O.cov_inverse_closed(c["scales"], c["rotations"], 1e-6))
+    first, gamma, tau = O.culling_gradient_bound(c["x_grid"], c["y_grid"], c["positions"], a, b, dd, c["alphas"],
+                                                 c["colors"], c["grad_out"], 1e-6, tolerance)
+
+    def chained(t):
+        bs, bth = O.chain_bound_to_scale_rotation(c["scales"], c["rotations"], t["cov_inv_00"], t["cov_inv_01"],
+                                                  t["cov_inv_11"], 1e-6)
+        return dict(positions=t["position"], colors=t["colors"], alphas=t["alphas"], scales=bs, rotations=bth)
+
+    first, gamma = chained(first), chained(gamma)
+    used = {}
+    for k in NAMES:
+        delta = (grads[k] - grads0[k]).double().cpu().abs()
+        bound = first[k] + (tau + 2e-6) * gamma[k]
+        assert bool((delta <= bound).all()), (k, float((delta / bound).max()))
+        assert bool((gamma[k] * (1 + 1e-5) >= grads0[k].double().cpu().abs()).all()), k
+        if k != "colors":
+            lhs = float((delta / first[k]).sum())
+            rhs = 1.0 + (tau + 2e-6) * float((gamma[k] / first[k]).sum())
+            assert lhs <= rhs, (k, lhs, rhs)
+        used[k] = float(delta.max())
+    if tolerance >= 1e-3:     # coarse lists do leave pairs out that count
+        assert max(used.values()) > 0, used
+
+
 @pytest.mark.parametrize("shape", [(1, 140000, 48, 48, 1), (33, 33000, 64, 256, 3)], ids=lambda v: "x".join(map(str, v)))
 def test_more_candidates_than_the_class_store_holds(igs, dev, no_cull, shape):
     """The binning keeps each candidate's weight class in LDS between the scan that settles what a

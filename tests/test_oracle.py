@@ -482,3 +482,121 @@ def test_skip_weight_bound_by_brute_force():
     # |alpha| = 4 moves the limit by two binades, |alpha| < 1 by nothing
     l = O.skip_limit(torch.tensor([0.25, 1.0, 4.0], dtype=F64), 2.0 ** -50)
     assert l.tolist() == [50.0, 50.0, 52.0]
+
+
+def _tile_keep_mask(pos, a, b, d, al, xs, ys, th, tw, w, f):
+    """[1,N,H,W] mask of the pairs that tiles of th x tw pixels keep under `tile_first_skipped_class`."""
+    N, H, W = al.shape[1], ys.numel(), xs.numel()
+    keep = torch.ones(1, N, H, W, dtype=torch.bool)
+    for r0 in range(0, H, th):
+        for c0 in range(0, W, tw):
+            r1, c1 = min(r0 + th, H) - 1, min(c0 + tw, W) - 1
+            rect = (xs[c0], xs[c1], ys[r0], ys[r1])
+            S = float(O.tile_weight_floor(pos[..., 0], pos[..., 1], a, b, d, al, *rect))
+            cls = O.weight_class(O.min_q_over_rect(pos[..., 0], pos[..., 1], a, b, d, *rect), al)[0]
+            first = O.tile_first_skipped_class(cls, N, w, f, S)
+            keep[0, :, r0:r1 + 1, c0:c1 + 1] = ~(cls >= first)[:, None, None]
+    return keep
+
+
+def test_gradient_bound_under_culling_by_brute_force():
+    """Pins `culling_gradient_bound`, not its formula: fp64 gradients with and without the pairs the
+    per-tile rule leaves out -- the forward's tiling and the backward's differ, as in the kernels, and
+    the backward uses the culled image -- on the worst-case scenes of the forward's bound (sparse,
+    most denominators far below eps, alphas beyond 1) and on a dense one where the floors carry the
+    allowance; every element within its bound, every tensor within the summed bound.  Two constructed
+    pixels come close to the two terms, so neither is slack by more than a small factor; dropping the
+    1/(den+eps), the factor K, or the second term fails them."""
+    g = torch.Generator().manual_seed(11)
+    C, eps = 3, 1e-6
+    names = ("position", "cov_inv_00", "cov_inv_01", "cov_inv_11", "alphas", "colors")
+    worst = {k: 0.0 for k in names}
+    scenes = [(60, 0.004, 0.034, 1e-7, 1.0), (60, 0.004, 0.034, 1e-3, 1.0), (60, 0.004, 0.034, 1e-3, 30.0),
+              (300, 0.02, 0.27, 1e-3, 1.0), (300, 0.02, 0.27, 0.05, 0.02), (120, 0.01, 0.1, 0.2, 5.0)]
+    for N, smin, smax, tol, amax in scenes:
+        H, W = 48, 64
+        pos = torch.rand(1, N, 2, generator=g, dtype=F64) * 2 - 1
+        sc = torch.rand(1, N, 2, generator=g, dtype=F64) * (smax - smin) + smin
+        rot = torch.rand(1, N, generator=g, dtype=F64) * 2 * math.pi
+        al = torch.rand(1, N, generator=g, dtype=F64) * amax
+        col = torch.rand(1, N, C, generator=g, dtype=F64) * 2 - 1
+        go = torch.randn(1, C, H, W, generator=g, dtype=F64)
+        a, b, d = (t.reshape(1, N) for t in O.cov_inverse_closed(sc, rot, eps))
+        xs, ys = torch.linspace(-1, 1, W, dtype=F64), torch.linspace(-1, 1, H, dtype=F64)
+        x, y = xs.view(1, 1, 1, W).expand(1, 1, H, W), ys.view(1, 1, H, 1).expand(1, 1, H, W)
+        w, f = O.skip_weight(N, eps, tol), O.skip_weight(N, 1.0, tol)
+        keep_f = _tile_keep_mask(pos, a, b, d, al, xs, ys, 16, 32, w, f)
+        keep_b = _tile_keep_mask(pos, a, b, d, al, xs, ys, 32, 8, w, f)
+        assert not bool(keep_f.all()) and not bool(keep_b.all()) and not bool((keep_f == keep_b).all())
+        every = torch.ones_like(keep_f)
+        out0, g0 = O.backward_with_lists(x, y, pos, a, b, d, al, col, go, eps, every, every)
+        ref = O.backward_strips(x, y, pos, a, b, d, al, col, go, eps)
+        for k in names:
+            torch.testing.assert_close(g0[k], ref[k], rtol=1e-11, atol=1e-13)
+        out1, g1 = O.backward_with_lists(x, y, pos, a, b, d, al, col, go, eps, keep_f, keep_b)
+        assert float((out1 - out0).abs().max()) <= tol * float(col.abs().max())
+        first, gamma, tau = O.culling_gradient_bound(x, y, pos, a, b, d, al, col, go, eps, tol)
+        assert tau >= 2 * tol
+        for k in names:
+            delta = (g1[k] - g0[k]).abs()
+            bound = first[k] + tau * gamma[k]
+            assert bool((delta <= bound).all()), (k, N, tol, float((delta / bound).max()))
+            if k != "colors":        # the summed form: all Gaussians share one allowance per pixel
+                lhs = float((delta / first[k]).sum())
+                rhs = 1.0 + tau * float((gamma[k] / first[k]).sum())
+                assert lhs <= rhs, (k, N, tol, lhs, rhs)
+                worst[k] = max(worst[k], lhs / rhs)
+            else:
+                worst[k] = max(worst[k], float((delta / bound).max()))
+            assert bool((gamma[k] >= g0[k].abs() * (1 - 1e-12)).all())    # Gam bounds the gradient itself
+    # (random scenes use little of it, as they use little of the forward's tolerance: few of a tile's
+    # Gaussians sit just under the threshold; the constructed pixels below are what comes close)
+    assert max(worst.values()) < 1e-2, worst
+
+    # One pixel that sees a heavy Gaussian of colour -1, a light one of colour +1 (k) and Nd faint
+    # ones of colour +1 whose weights add up to the whole allowance tolerance (den + eps).
+    Nd, tol = 20, 1e-3
+    N = Nd + 2
+    x = y = torch.zeros(1, 1, 1, 1, dtype=F64)
+    pos = torch.zeros(1, N, 2, dtype=F64)
+    a = d = torch.full((1, N), 100.0, dtype=F64)
+    b = torch.zeros(1, N, dtype=F64)
+    col = torch.ones(1, N, 1, dtype=F64)
+    col[0, 0, 0] = -1.0
+    al = torch.ones(1, N, dtype=F64)
+    al[0, 1] = 1e-3
+    Dfull = (1.0 + 1e-3 + eps) / (1 - tol)
+    u = tol * Dfull / Nd
+    r = math.sqrt(-2 * math.log(u) / 100.0)                      # e = u at distance r
+    pos[0, 2:, 0] = r
+    go = torch.ones(1, 1, 1, 1, dtype=F64)
+    every = torch.ones(1, N, 1, 1, dtype=torch.bool)
+    faint = every.clone()
+    faint[0, 2:] = False
+    _, g0 = O.backward_with_lists(x, y, pos, a, b, d, al, col, go, eps, every, every)
+    first, gamma, tau = O.culling_gradient_bound(x, y, pos, a, b, d, al, col, go, eps, tol)
+    # (2): the forward leaves the faint ones out, the backward nothing: d alpha_k moves by nearly tau Gam
+    _, g2 = O.backward_with_lists(x, y, pos, a, b, d, al, col, go, eps, faint, every)
+    moved = float((g2["alphas"] - g0["alphas"]).abs()[0, 1])
+    assert 0.9 * tau * float(gamma["alphas"][0, 1]) <= moved <= tau * float(gamma["alphas"][0, 1])
+    # (1): the backward leaves them out, the forward nothing: their d alpha, summed, lose nearly T
+    _, g3 = O.backward_with_lists(x, y, pos, a, b, d, al, col, go, eps, every, faint)
+    lost = float((g3["alphas"] - g0["alphas"]).abs().sum())
+    T = float(first["alphas"][0, 0])                              # m = 1: T itself
+    assert 0.9 * T <= lost <= T
+    assert bool((g3["alphas"][0, 2:] == 0).all()) and float(g3["alphas"][0, 1]) == float(g0["alphas"][0, 1])
+    # and their moments stay within the log factor's bound while using more than the bare allowance
+    lost_a = float((g3["cov_inv_00"] - g0["cov_inv_00"]).abs().sum())
+    sxx = 1.0 / 100.0
+    assert T * 0.5 * sxx < lost_a <= float(first["cov_inv_00"][0, 2]) 
+
+    # scale / rotation: the chain with absolute coefficients bounds the chained difference
+    sc = torch.rand(1, 7, 2, generator=g, dtype=F64) * 0.2 + 0.01
+    rot = torch.rand(1, 7, generator=g, dtype=F64) * 6
+    dA, dB, dD = (torch.randn(1, 7, generator=g, dtype=F64) for _ in range(3))
+    gs, gth = O.chain_to_scale_rotation(sc, rot, dA, dB, dD, eps)
+    bs, bth = O.chain_bound_to_scale_rotation(sc, rot, dA.abs(), dB.abs(), dD.abs(), eps)
+    assert bool((gs.abs() <= bs * (1 + 1e-12)).all()) and bool((gth.abs() <= bth * (1 + 1e-12)).all())
+    same = O.chain_bound_to_scale_rotation(sc, torch.zeros_like(rot), dA.abs(), dB.abs() * 0, dD.abs(), eps)
+    exact = O.chain_to_scale_rotation(sc, torch.zeros_like(rot), dA.abs(), dB * 0, dD.abs(), eps)
+    torch.testing.assert_close(same[0], exact[0].abs(), rtol=1e-12, atol=0)   # attained where nothing cancels
