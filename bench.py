@@ -100,6 +100,9 @@ def main() -> int:
                     help="bound on what skipped pairs may change in an output element, as a fraction of the largest "
                          "colour (default: the library's 1e-7; 0 = skip exact zeros only)")
     ap.add_argument("--no-cull", action="store_true", help="evaluate every pair (IGS_OPT_NO_CULL)")
+    ap.add_argument("--default-only", action="store_true",
+                    help="leave out the `exact` and `no_cull` legs (for profiling: every launch of the run then belongs "
+                         "to the default path)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (known traffic) so that a rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE run of this command carries its own scale")
@@ -238,12 +241,16 @@ def run(args) -> int:
     f_fwd, f_bwd = flops_per_pair(C)
     side = {}
     for key, opts in (("exact", dict(skip_tolerance=0.0)), ("no_cull", dict(no_cull=True))):
+        if args.default_only:
+            side[key] = None
+            continue
         with library_options(**opts):
             t_mean, t_med = timed(step, min(args.steps, 10), 3, 0.1)
         side[key] = {"ms_per_step": t_mean * 1e3, "median_ms_per_step": t_med * 1e3, "value": pairs / t_mean,
                      "what": {"exact": "skip_tolerance = 0: only pairs whose fp32 weight is exactly zero are left out",
                               "no_cull": "IGS_OPT_NO_CULL: every Gaussian listed for every tile, all B N H W pairs evaluated"}[key]}
-    side["no_cull"]["frac"] = pairs * (f_fwd + f_bwd) / (side["no_cull"]["ms_per_step"] * 1e-3) / 1e12 / FP32_VECTOR_PEAK_TFLOPS
+    if side["no_cull"]:
+        side["no_cull"]["frac"] = pairs * (f_fwd + f_bwd) / (side["no_cull"]["ms_per_step"] * 1e-3) / 1e12 / FP32_VECTOR_PEAK_TFLOPS
 
     result = {
         "metric": "gaussian_pixel_evals_per_sec_fwd_bwd",
