@@ -11,7 +11,7 @@ B=16, N=8192, 256x256, C=3, fp32.  Prints ONE JSON line:
   cpu_baseline : the chunked torch autograd path of the reference restated on the CPU
                  (oracle/chunked_cpu.py), timed on this box's host cores on a bounded sample.
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu] | --all | --sweep
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu] [--default-only] | --fit | --all | --sweep | --koleo
 """
 from __future__ import annotations
 
@@ -100,6 +100,9 @@ def main() -> int:
                     help="bound on what skipped pairs may change in an output element, as a fraction of the largest "
                          "colour (default: the library's 1e-7; 0 = skip exact zeros only)")
     ap.add_argument("--no-cull", action="store_true", help="evaluate every pair (IGS_OPT_NO_CULL)")
+    ap.add_argument("--fit", action="store_true",
+                    help="instead of the JSON line of the operator, time the fused fit iteration (render, MSE, backward, "
+                         "AdamW; igs_amd.fit) of --config c0 or c2, replayed from a HIP graph, and print its own line")
     ap.add_argument("--default-only", action="store_true",
                     help="leave out the `exact` and `no_cull` legs (for profiling: every launch of the run then belongs "
                          "to the default path)")
@@ -128,6 +131,8 @@ def run(args) -> int:
         return all_configs(args.steps, args.warmup, args.no_cpu)
     if args.koleo:
         return koleo_table(args.no_cpu, args.koleo_shape)
+    if args.fit:
+        return fit_step(args.config, args.steps, args.warmup)
 
     import torch
 
@@ -587,6 +592,48 @@ def all_configs(steps: int, warmup: int, no_cpu: bool = False) -> int:
     print("pairs/s counts all B N H W pairs; of peak = (12 + 2 C) x forward pairs + (30 + 4 C) x backward pairs evaluated "
           "/ fwd+bwd time / %.1f TFLOP/s; CPU: %d torch threads on %s (%d "
           "physical cores visible)" % (FP32_VECTOR_PEAK_TFLOPS, torch.get_num_threads(), model, physical))
+    return 0
+
+
+def fit_step(cfg: str, steps: int, warmup: int) -> int:
+    """The fused fit iteration of the reference's image-fitting script (scripts/2dgs_img_comp.py:186-240: render, MSE
+    against the target, backward, AdamW on one parameter block) on the Gaussians of `cfg`, captured once and replayed
+    from a HIP graph: `warmup` replays and at least 0.3 s of them, then `steps` replays between two synchronisations."""
+    import torch
+
+    from igs_amd.fit import GaussianImageFit
+    from oracle import gs2d_oracle as O
+
+    if cfg not in ("c0", "c2"):
+        print("bench.py --fit: one image per fit (c0 or c2)", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    d = {k: v.to(dev) for k, v in O.make_config_inputs(cfg).items()}
+    B, N, C = d["colors"].shape
+    H, W = d["x_grid"].shape[-2:]
+    xg = d["x_grid"][:1, :, :1, :].expand(B, 1, H, W)
+    yg = d["y_grid"][:1, :, :, :1].expand(B, 1, H, W)
+    block = torch.cat([d["positions"], d["scales"].log(), d["rotations"][..., None],
+                       torch.zeros_like(d["rotations"])[..., None], d["colors"]], -1)
+    fit = GaussianImageFit(block, O.smooth_noise_target(H, W, seed=1002).to(dev), xg, yg, lr=min(0.05 * 4096 / N, 0.03))
+    fit.capture()
+    t0 = time.perf_counter()
+    k = 0
+    while k < warmup or time.perf_counter() - t0 < 0.3:
+        fit.step()
+        k += 1
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fit.step()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / steps
+    pairs = B * N * H * W
+    print(json.dumps({"metric": "fit_step_ms", "value": t * 1e3, "unit": "ms", "higher_is_better": False, "n_gpus": 1,
+                      "steps": steps, "warmup": warmup, "pairs_per_s": pairs / t, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": f"{cfg}: fit iteration (render + MSE + backward + AdamW), HIP graph replay, "
+                                             f"B={B} N={N} {H}x{W} C={C}", "B": B, "N": N, "H": H, "W": W, "C": C}}),
+          flush=True)
     return 0
 
 

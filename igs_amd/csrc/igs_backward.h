@@ -328,7 +328,14 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
         span = fmaxf(span, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
         xbad = xbad || !(v.x == v.x && v.y == v.y && v.z == v.z && v.w == v.w);
     }
-    const bool regular = br.w == 0.0f && !xbad && br.x * span <= kSepSpanLimitBwd;
+    bool regular = br.w == 0.0f && !xbad && br.x * span <= kSepSpanLimitBwd;
+    // A tile's last group of list positions is half empty on average (short lists: mostly).  A wave without
+    // a listed Gaussian only helps to load the pixel records; the unused lanes of the other waves take the
+    // evaluation of their wave's listed lanes, so that they do not make it run both loops.
+    const bool live = pos < count;
+    const bool wave_live = __ballot(live) != 0ull;
+    const bool wave_regular = __ballot(live && regular) != 0ull;
+    if (!live) regular = wave_regular;
     // regular lanes: sA, skA, D''; the others: A', B2', D'
     const float A = regular ? br.x : rA, B2 = regular ? br.y : rB2, D = regular ? br.z : rD;
     const float mpx = -A * (px - xc);  // regular lanes: -sA px'
@@ -363,7 +370,9 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
         const float4* cur = sh + (k & 1) * E;
         const float* ycur = ysh[k & 1];
         const int rows = min(RPC, r1 - r0 - k * RPC);
-        if (regular) {
+        if (!wave_live) {
+            // (wave-uniform) nothing to evaluate
+        } else if (regular) {
             float ynext = ycur[0];
 #pragma unroll 1
             for (int rr = 0; rr < rows; ++rr) {
