@@ -22,6 +22,7 @@ struct FwdArgs {
     int list_img, list_row;  // lists per image and per row of rectangles (tiles) in that numbering
     const int* flag;  // AUTO grid mode: run only if *flag == want (nullptr: always run)
     int want;
+    float ramp;  // separable: how far the parts of a list differ in length (kSplitRamp, or 0 when all waves are resident at once)
 };
 
 // AUTO grid mode launches both the separable and the general variant of a kernel; the
@@ -67,6 +68,8 @@ __host__ __device__ constexpr bool fwd_wave_lists(int C) { return fwd_sep_p(C) >
 // A tile's list is cut into S parts for S workgroups (blockIdx.y). The parts shrink linearly from
 // (1 + ramp) to (1 - ramp) times the mean: workgroups start part by part, so the last to start are
 // the shortest (B=16 N=8192 256x256: forward 1.30 ms with equal parts, 1.23 ms with ramp 0.6 to 0.8).
+// Where the whole launch is resident at once (small problems) nothing starts later, the longest part
+// decides, and the parts are equal (B=1 N=2048 256x256: fit step 146 -> 141 us).
 #ifndef IGS_SPLIT_RAMP
 #define IGS_SPLIT_RAMP 0.7f
 #endif
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     const int count = (!kWave || (rrow * kHalves * P < a.H && rcol * kWaveCols < a.W)) ? a.counts[li] : 0;
     // parts of decreasing length: part i has weight 1 + ramp - 2 ramp i / (S - 1), the sum is S
     auto cut = [&](int i) {  // first entry of part i, a multiple of 4
-        const float f = a.S > 1 ? (float)i * (1.0f + kSplitRamp - kSplitRamp * (float)(i - 1) / (float)(a.S - 1)) / (float)a.S
+        const float f = a.S > 1 ? (float)i * (1.0f + a.ramp - a.ramp * (float)(i - 1) / (float)(a.S - 1)) / (float)a.S
                                 : (float)i;
         return min(count, ((int)((float)count * f) + 3) & ~3);
     };

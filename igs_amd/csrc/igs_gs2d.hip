@@ -798,6 +798,11 @@ int forward_impl(const float* packed, const float* x, const float* y,
         a.eps = eps; a.out = out; a.den = den; a.part = (float*)ws;
         a.counts = nullptr; a.lists = nullptr;
         a.flag = vs[i].flag; a.want = vs[i].want;
+        {   // parts of unequal length only where the launch takes several rounds of resident waves (three per SIMD)
+            int cus = device_cus();
+            if (cus <= 0) cus = 256;
+            a.ramp = 4L * fg.total_tiles * a.S > 12L * cus ? kSplitRamp : 0.0f;
+        }
         // numbering of the lists: by wave rectangle (or by tile, with one list per tile), row after row
         constexpr int kHalvesL = 64 / kWaveCols;
         a.list_row = fwd_wave_lists(C) ? kHalvesL * fg.tiles_x : fg.tiles_x;
