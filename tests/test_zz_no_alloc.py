@@ -20,6 +20,9 @@ def dev():
     return torch.device("cuda:0")
 
 
+_set_up = False
+
+
 def _both_forwards(dev, B, N, H, W, C, seed, general=False):
     from igs_amd import _lib
     from igs_amd._splat import Grid, Splat, _ptr, _stream
@@ -44,11 +47,18 @@ def _both_forwards(dev, B, N, H, W, C, seed, general=False):
         den = torch.full_like(ref_den, float("nan"))
         torch.cuda.synchronize()
         before = torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info(dev)[0]     # the device's own count: sees allocations made past torch
         rc = lib.igs_gs2d_forward_static_ws(_ptr(packed), _ptr(grid.x), _ptr(grid.y), grid.strides, grid.mode,
                                             _ptr(grid.flag), B, N, H, W, op.Cp, 1e-6, _ptr(out), _ptr(den),
                                             _stream(dev))
         torch.cuda.synchronize()
         assert torch.cuda.memory_stats(dev)["allocation.all.allocated"] == before
+        # (the first call on a device resolves the array's address and creates the guard's event: set-up, not
+        # checked; every later call must leave the device's free memory where it was)
+        global _set_up
+        if _set_up:
+            assert torch.cuda.mem_get_info(dev)[0] >= free_before
+        _set_up = True
     return rc, op.plan, (out, den), (ref_out, ref_den)
 
 
