@@ -289,7 +289,9 @@ class Splat:
         ws = self._empty(p.fwd_ws_bytes) if p.fwd_ws_bytes else None
         pix = self._empty(p.pix_bytes)
         total = done = None
-        if p.partial_bytes > COMPACT_PARTIALS_FROM:
+        # (not while the stream is being captured into a graph: a replay cannot wait for a host read;
+        # the backward then takes the array for every pair)
+        if p.partial_bytes > COMPACT_PARTIALS_FROM and not torch.cuda.is_current_stream_capturing():
             total = torch.empty(1, dtype=torch.int64, pin_memory=True)
         _lib.check(self.lib.igs_gs2d_forward_train(
             _ptr(packed), _ptr(g.x), _ptr(g.y), g.strides, g.mode, _ptr(g.flag), self.B, self.N, g.H, g.W, self.Cp,

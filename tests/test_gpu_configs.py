@@ -202,11 +202,16 @@ def test_module_fused_head_equals_unfused_render(igs, dev):
             assert rel(u, v) < 1e-4
 
 
-def test_step_is_hip_graph_capturable(igs, dev):
+@pytest.mark.parametrize("sized_by_lists", [False, True], ids=["dense", "compact"])
+def test_step_is_hip_graph_capturable(igs, dev, monkeypatch, sized_by_lists):
     """A forward+backward step recorded into a HIP graph (the library only launches kernels on the
     stream it is given: no allocation, no synchronisation, no memset).  The graph is replayed
     several times with new inputs, with eager work and synchronisations in between, and every
-    replay is checked against the eager result."""
+    replay is checked against the eager result.  `compact`: the problem counts as one whose partial
+    sums are sized by the lists (a host read of the forward's count before the backward); under
+    capture that read is left out and the eager steps in between still take it."""
+    if sized_by_lists:
+        monkeypatch.setattr("igs_amd._splat.COMPACT_PARTIALS_FROM", 0)
     B, N, H, W = 2, 300, 40, 56
     names = ("positions", "colors", "scales", "rotations", "alphas")
     cases = [O.make_inputs(B, N, H, W, 3, 0.05, 0.4, seed=600 + i) for i in range(4)]
