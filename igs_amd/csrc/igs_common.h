@@ -82,3 +82,8 @@ __device__ __forceinline__ int xcd_contiguous(int linear, int total) {
     const int per = (total + 7) >> 3;
     return (linear & 7) * per + (linear >> 3);
 }
+// The same with the XCD's range walked from another starting tile (`rot` tiles further on, cyclically).
+__device__ __forceinline__ int xcd_contiguous_from(int linear, int total, int rot) {
+    const int per = (total + 7) >> 3;
+    return (linear & 7) * per + ((linear >> 3) + rot) % per;
+}

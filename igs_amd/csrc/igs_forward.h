@@ -388,7 +388,11 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     // of when the longest list of the four does.  Workgroup q: XCD q % 8, there tile (q / 8) / 4
     // of the XCD's range and wave rectangle (q / 8) % 4 of that tile.
     const int q = kOne ? (int)(blockIdx.x & 7) + 8 * (int)(blockIdx.x >> 5) : (int)blockIdx.x;
-    const int tile = xcd_contiguous(q, a.total_tiles);
+    // (each part of the lists starts one tile further on in the XCD's range: the workgroups of consecutive parts
+    // otherwise reach the compute units in the same tile order, and where a few tiles hold most of the work --
+    // Gaussians crowded around the image centre -- the same units get the long lists every time: B=8 N=4096
+    // 256x256 at a module's initialisation, forward kernel 89 -> 82 us; 3, 5 or 7 tiles: 84-88)
+    const int tile = xcd_contiguous_from(q, a.total_tiles, (int)blockIdx.y);
     if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int per_img = a.tiles_x * a.tiles_y;
     const int b = tile / per_img;
