@@ -11,9 +11,6 @@ constexpr int kThreads = 256;
 #ifndef IGS_FWD_SEP_P
 #define IGS_FWD_SEP_P 16
 #endif
-#ifndef IGS_BWD_G
-#define IGS_BWD_G 1
-#endif
 #ifndef IGS_FWD_WAVES
 #define IGS_FWD_WAVES 8
 #endif
@@ -36,7 +33,7 @@ __host__ __device__ constexpr int fwd_gen_p(int C) { return C <= 4 ? 8 : 4; }
 __host__ __device__ constexpr int bwd_gen_g(int C) { return C <= 4 ? IGS_BWD_GEN_G : 2; }
 // Gaussians per lane, separable backward: one (a tile's last group of list positions is half empty on
 // average, and its idle lanes cost more with two per lane than sharing the pixel records' reads saves)
-__host__ __device__ constexpr int bwd_sep_g(int) { return IGS_BWD_G; }
+__host__ __device__ constexpr int bwd_sep_g(int) { return 1; }
 
 __host__ __device__ constexpr int rec_stride_of(int C) { return (6 + C + 3) & ~3; }
 // Records of the separable kernels (see sep_terms): the forward's px, py, sD, skD, A'', alpha,

@@ -378,10 +378,7 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     constexpr bool kSq = fwd_square(C);  // completed square (its own records) or term by term (the plain ones)
     static_assert(kSq == (P >= 8) || !IGS_FWD_SQUARE, "the completed square goes with 8 or more rows per lane");
     constexpr int RS = kSq ? frec_stride_of(C) : rec_stride_of(C), R4 = RS / 4;
-#ifndef IGS_FWD_READ_ALL
-#define IGS_FWD_READ_ALL 0
-#endif
-    constexpr int RD = kSq && !IGS_FWD_READ_ALL ? (7 + C + 3) / 4 : R4;  // float4 of a record that every evaluation reads
+    constexpr int RD = kSq ? (7 + C + 3) / 4 : R4;  // float4 of a record that every evaluation reads
     IGS_GATE(a);
     // Waves with lists of their own can be launched as workgroups of one wave (kOne): the four
     // waves of a tile share nothing, and a wave slot then frees as soon as its wave ends instead
