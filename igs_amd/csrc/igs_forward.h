@@ -389,12 +389,18 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     // otherwise reach the compute units in the same tile order, and where a few tiles hold most of the work --
     // Gaussians crowded around the image centre -- the same units get the long lists every time: B=8 N=4096
     // 256x256 at a module's initialisation, forward kernel 89 -> 82 us; 3, 5 or 7 tiles: 84-88)
-    const int tile = xcd_contiguous_from(q, a.total_tiles, (int)blockIdx.y);
+    // A single image: every XCD reads all of its Gaussians anyway, and a contiguous range of tiles would give
+    // the XCDs that hold the top and the bottom rows the short lists (B=1 N=16384 512x512: 43 000-67 000 list
+    // entries per XCD).  The tiles are dealt round-robin instead, each tile row shifted against the one above so
+    // that an XCD does not end up with one tile column: forward call 0.207 -> 0.199 ms.
+    const bool dealt = a.B == 1;
+    const int tile = dealt ? q : xcd_contiguous_from(q, a.total_tiles, (int)blockIdx.y);
     if (tile >= a.total_tiles) return;  // workgroup-uniform
     const int per_img = a.tiles_x * a.tiles_y;
     const int b = tile / per_img;
     const int tl = tile - b * per_img;
-    const int ty = tl / a.tiles_x, tx = tl - ty * a.tiles_x;
+    const int ty = tl / a.tiles_x;
+    const int tx = dealt ? (tl - ty * a.tiles_x + 3 * ty + (int)blockIdx.y) % a.tiles_x : tl - ty * a.tiles_x;
     const int wave = kOne ? (int)((blockIdx.x >> 3) & 3) : (int)(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     // A wave with a list of its own covers kWaveCols columns x (64 / kWaveCols) P rows: lane l has
