@@ -35,7 +35,7 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 # belong to the kernels being timed, and the fields derived from them are reported as null.
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
-    "csrc_sha16": "65590d178833fde2",
+    "csrc_sha16": "9fb8a21f2d84902d",
     "bwd": {"fma": 6.841e8, "mul": 1.439e8, "add": 7.404e7, "trans": 6.770e7, "fetch_kib": 55720, "write_kib": 147400},
     "fwd": {"fma": 4.069e8, "mul": 1.268e7, "add": 8.904e6, "trans": 6.713e7, "fetch_kib": 12740, "write_kib": 131100},
 }
