@@ -174,10 +174,13 @@ constexpr int kGaussChunk = IGS_GCHUNK;  // Gaussian records per LDS buffer
 // read as all-zero (for a Gaussian record: alpha = 0, adds exactly 0).  Must be called by all
 // NT threads of the workgroup (it contains barriers; with NT = 64, one wave, they cost nothing).
 // With kGather, record i of the stream is src record index[i] (a tile's Gaussian list).
-template <int R4, int CH, bool kGather = false, int NT = kThreads, int RD = R4, class Body>
-__device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
-                                                   float4* sh, Body&& body,
-                                                   const int* __restrict__ index = nullptr) {
+// The general form: fetch(lds record) returns the registers one evaluation reads, body(those, lds record) is
+// the evaluation; kGrouped: body(the registers of the kStreamUnroll records of a group, lds record of the
+// first) runs once per group.
+template <int R4, int CH, bool kGather, int NT, bool kGrouped, class Fetch, class Body>
+__device__ __forceinline__ void stream_records_lds_f(const float4* __restrict__ src, int count,
+                                                     float4* sh, Fetch&& fetch, Body&& body,
+                                                     const int* __restrict__ index) {
     constexpr int E = CH * R4;                          // float4 per chunk
     constexpr int PRE = (E + NT - 1) / NT;              // float4 per thread per chunk
     const int total = count * R4;
@@ -229,16 +232,19 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
         const int lim = min(CH, (count - k * CH + kStreamUnroll - 1) / kStreamUnroll * kStreamUnroll);
 #pragma unroll 1
         for (int n = 0; n < lim; n += kStreamUnroll) {
-            float4 rr[kStreamUnroll][RD];
+            decltype(fetch(cur)) rr[kStreamUnroll];
 #pragma unroll
-            for (int u = 0; u < kStreamUnroll; ++u)
-#pragma unroll
-                for (int i = 0; i < RD; ++i) rr[u][i] = cur[(n + u) * R4 + i];
+            for (int u = 0; u < kStreamUnroll; ++u) rr[u] = fetch(cur + (n + u) * R4);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int u = 0; u < kStreamUnroll; ++u) {
-                body(rr[u], cur + (n + u) * R4);
+            if constexpr (kGrouped) {
+                body(rr, cur + n * R4);
                 __builtin_amdgcn_sched_barrier(0);
+            } else {
+#pragma unroll
+                for (int u = 0; u < kStreamUnroll; ++u) {
+                    body(rr[u], cur + (n + u) * R4);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
         if (k + 1 < chunks) {
@@ -253,6 +259,27 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
     }
 }
 
+// The first RD float4 of a record as the registers of an evaluation.
+template <int RD>
+struct RecHead {
+    float4 v[RD];
+};
+template <int RD>
+__device__ __forceinline__ RecHead<RD> rec_head(const float4* rec) {
+    RecHead<RD> h;
+#pragma unroll
+    for (int i = 0; i < RD; ++i) h.v[i] = rec[i];
+    return h;
+}
+template <int R4, int CH, bool kGather = false, int NT = kThreads, int RD = R4, class Body>
+__device__ __forceinline__ void stream_records_lds(const float4* __restrict__ src, int count,
+                                                   float4* sh, Body&& body,
+                                                   const int* __restrict__ index = nullptr) {
+    stream_records_lds_f<R4, CH, kGather, NT, false>(
+        src, count, sh, [](const float4* rec) { return rec_head<RD>(rec); },
+        [&](const RecHead<RD>& h, const float4* lds) { body(h.v, lds); }, index);
+}
+
 // The same stream for one wave on its own (wave-uniform `count`, `index` and buffers; no barrier, so
 // the waves of a workgroup may run it with different lists), without staging registers: the records of the next
 // chunk go from global memory straight into the other LDS buffer (global_load_lds_dwordx4: lane l
@@ -260,11 +287,12 @@ __device__ __forceinline__ void stream_records_lds(const float4* __restrict__ sr
 // vmcnt wait per chunk separates the two.  Slots past `count` load the all-zero record `zero_rec`.
 // The two buffers are separate arrays and the chunk loop is unrolled by two, so that every LDS read
 // names the buffer it reads.
-template <int R4, int CH, int RD = R4, class Body>
-__device__ __forceinline__ void stream_records_dma(const float4* __restrict__ src,
-                                                   const float4* __restrict__ zero_rec, int count,
-                                                   float4* sh0, float4* sh1, Body&& body,
-                                                   const int* __restrict__ index) {
+// (fetch, body and kGrouped as in stream_records_lds_f)
+template <int R4, int CH, bool kGrouped, class Fetch, class Body>
+__device__ __forceinline__ void stream_records_dma_f(const float4* __restrict__ src,
+                                                     const float4* __restrict__ zero_rec, int count,
+                                                     float4* sh0, float4* sh1, Fetch&& fetch, Body&& body,
+                                                     const int* __restrict__ index) {
     constexpr int E = CH * R4;  // float4 per chunk
     static_assert(E % 64 == 0 && CH % kStreamUnroll == 0, "a chunk is a whole number of wave loads");
     constexpr int PRE = E / 64;
@@ -304,16 +332,19 @@ __device__ __forceinline__ void stream_records_dma(const float4* __restrict__ sr
         const int lim = min(CH, (count - k * CH + kStreamUnroll - 1) / kStreamUnroll * kStreamUnroll);
 #pragma unroll 1
         for (int n = 0; n < lim; n += kStreamUnroll) {
-            float4 rr[kStreamUnroll][RD];
+            decltype(fetch(cur)) rr[kStreamUnroll];
 #pragma unroll
-            for (int u = 0; u < kStreamUnroll; ++u)
-#pragma unroll
-                for (int i = 0; i < RD; ++i) rr[u][i] = cur[(n + u) * R4 + i];
+            for (int u = 0; u < kStreamUnroll; ++u) rr[u] = fetch(cur + (n + u) * R4);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int u = 0; u < kStreamUnroll; ++u) {
-                body(rr[u], cur + (n + u) * R4);
+            if constexpr (kGrouped) {
+                body(rr, cur + n * R4);
                 __builtin_amdgcn_sched_barrier(0);
+            } else {
+#pragma unroll
+                for (int u = 0; u < kStreamUnroll; ++u) {
+                    body(rr[u], cur + (n + u) * R4);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
     };
@@ -337,6 +368,16 @@ __device__ __forceinline__ void stream_records_dma(const float4* __restrict__ sr
         compute(sh1, k + 1);
         landed();
     }
+}
+
+template <int R4, int CH, int RD = R4, class Body>
+__device__ __forceinline__ void stream_records_dma(const float4* __restrict__ src,
+                                                   const float4* __restrict__ zero_rec, int count,
+                                                   float4* sh0, float4* sh1, Body&& body,
+                                                   const int* __restrict__ index) {
+    stream_records_dma_f<R4, CH, false>(
+        src, zero_rec, count, sh0, sh1, [](const float4* rec) { return rec_head<RD>(rec); },
+        [&](const RecHead<RD>& h, const float4* lds) { body(h.v, lds); }, index);
 }
 
 template <int C>
@@ -372,6 +413,23 @@ __device__ __forceinline__ void fwd_store(const FwdArgs& a, int b, int s, int p,
 #ifndef IGS_FWD_MIN_WAVES
 #define IGS_FWD_MIN_WAVES 3
 #endif
+// The accumulation out[pixel][channel] += w[pixel] (alpha, alpha c_0, ..)[channel] over the Gaussians is a
+// rank-1 update of a 64 x (1 + C) matrix per row of pixels.  v_mfma_f32_4x4x1_16b_f32 (16 blocks of 4 x 4,
+// K = 1) with A = four channel values (lane 4 b + i holds channel i, the same in all blocks) and B = the row's
+// weights (lane = pixel) leaves channel i of pixel `lane` in register i of the lane: the layout of the vector
+// form, full fp32, the same order of summation, one matrix instruction of two passes for four vector FMAs.
+// The matrix instructions of a group of records are issued back to back behind the group's vector
+// arithmetic: a vector instruction behind a matrix one waits for it to drain, and alternating the two was
+// slower than no matrix instructions at all (B=16 N=8192 256x256 C=3 forward call: vector 0.972 ms, matrix in
+// phases 0.876, alternating 1.03-1.13).
+// Where a row's last matrix instruction would be mostly padding the vector form stays: one channel (2 of 4 used:
+// B=4 N=8192 256x256 forward 0.251 -> 0.268 ms) and four (5 of 8: 0.343 -> 0.340); with 2, 3, 8, 12 and 16
+// channels the same shape gains 1.5, 9, 2.5, 6 and 3 %.
+#ifndef IGS_FWD_MFMA
+#define IGS_FWD_MFMA 1
+#endif
+__host__ __device__ constexpr bool fwd_mfma(int C) { return IGS_FWD_MFMA && C != 1 && C != 4; }
+typedef float fwd_v4f __attribute__((ext_vector_type(4)));
 template <int C, int P, bool kWave, bool kOne = false>
 __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_fwd_sep(const FwdArgs a) {  // (16 rows per lane: three waves per SIMD, i.e. at most 168 registers)
     static_assert(kWave || !kOne, "one-wave workgroups need a list per wave");
@@ -379,6 +437,9 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     static_assert(kSq == (P >= 8) || !IGS_FWD_SQUARE, "the completed square goes with 8 or more rows per lane");
     constexpr int RS = kSq ? frec_stride_of(C) : rec_stride_of(C), R4 = RS / 4;
     constexpr int RD = kSq ? (7 + C + 3) / 4 : R4;  // float4 of a record that every evaluation reads
+    constexpr bool kMfma = fwd_mfma(C);  // the sums on the matrix cores
+    constexpr int NM = (C + 4) / 4;      // matrix instructions per row of pixels: four of the 1 + C channels each
+    static_assert(!kMfma || kSq == kWave, "matrix form: completed-square records with a list per wave, or plain ones with a shared list");
     IGS_GATE(a);
     // Waves with lists of their own can be launched as workgroups of one wave (kOne): the four
     // waves of a tile share nothing, and a wave slot then frees as soon as its wave ends instead
@@ -423,12 +484,17 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     for (int p = 0; p < P; ++p) yv[p] = in_vgpr(yv[p]);
 
     float dsum[P], num[P][C];
+    [[maybe_unused]] fwd_v4f acc[kMfma ? P : 1][NM];  // matrix form: channel 4 m + i of row p in acc[p][m][i]
 #pragma unroll
     for (int p = 0; p < P; ++p) {
         dsum[p] = 0.0f;
 #pragma unroll
         for (int c = 0; c < C; ++c) num[p][c] = 0.0f;
     }
+#pragma unroll
+    for (int p = 0; p < (kMfma ? P : 1); ++p)
+#pragma unroll
+        for (int m = 0; m < NM; ++m) acc[p][m] = fwd_v4f{0.0f, 0.0f, 0.0f, 0.0f};
     float wylo = yv[0], wyhi = yv[0];  // y range of this wave's rows (NaN-safe: see the test below)
     bool ybad = !(yv[0] == yv[0]);
 #pragma unroll
@@ -481,12 +547,8 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     const int* list = a.lists + li * a.Np + n0;
     const float4* src = reinterpret_cast<const float4*>((kSq ? a.frecs : a.packed) + (size_t)b * a.Np * RS);
     // the exponents of the lane's P pixels for one record, and its alpha and alpha*c
-    auto exponents = [&](auto wave_skip, const float4* r, const float4* lds, float (&e)[P], float& al, float (&ac)[C]) -> bool {
-        if constexpr (kSq) {
-            const FRec<C> g = lds_frec<C>(r);
-            al = g.al;
-#pragma unroll
-            for (int c = 0; c < C; ++c) ac[c] = g.ac[c];
+    // completed-square records (px, py, sD, skD, A'', tag of `g`; `terms`: where the record's A', B2', D' are read from)
+    auto sq_exponents = [&](const FRec<C>& g, const float4* terms, float (&e)[P]) {
             const float dx = xv - g.px;
             const float pyl = g.py - yc;
             if (__ballot(g.tag <= sd_limit) != 0ull) {  // wave-uniform: both sides are
@@ -499,7 +561,7 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
                 }
             } else {  // no completed square, or its scale is too large for this wave's rows
                 float Ap, B2p, Dp;
-                lds_frec_terms<C>(RD == R4 ? r : lds, Ap, B2p, Dp);
+                lds_frec_terms<C>(terms, Ap, B2p, Dp);
                 // py - yc = pyl + lo exactly (two-sum), so that dy = y - py carries one rounding, as without
                 // the shift (the sharp Gaussians that come here need it); lo, half an ulp of pyl at most,
                 // goes into the constant and the linear coefficient of the form in dy0 = y' - pyl:
@@ -516,6 +578,27 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
                     e[p] = fmaf(t, dy, c0);
                 }
             }
+    };
+    // plain records, term by term (px, py, A', B2', D' of `g`)
+    auto plain_exponents = [&](const GRec<C>& g, float (&e)[P]) {
+        const float dx = xv - g.px;
+        const float adx = g.A * dx;
+        const float c0 = adx * dx;
+        const float c1 = g.B2 * dx;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const float dy = yv[p] - g.py;
+            const float t = fmaf(g.D, dy, c1);
+            e[p] = fmaf(t, dy, c0);
+        }
+    };
+    auto exponents = [&](auto wave_skip, const float4* r, const float4* lds, float (&e)[P], float& al, float (&ac)[C]) -> bool {
+        if constexpr (kSq) {
+            const FRec<C> g = lds_frec<C>(r);
+            al = g.al;
+#pragma unroll
+            for (int c = 0; c < C; ++c) ac[c] = g.ac[c];
+            sq_exponents(g, RD == R4 ? r : lds, e);
         } else {
             const GRec<C> g = lds_grec<C>(r);
             // A list shared by four waves of P rows each: a wave whose own rows the reach box misses
@@ -524,16 +607,7 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
             al = g.al;
 #pragma unroll
             for (int c = 0; c < C; ++c) ac[c] = g.ac[c];
-            const float dx = xv - g.px;
-            const float adx = g.A * dx;
-            const float c0 = adx * dx;
-            const float c1 = g.B2 * dx;
-#pragma unroll
-            for (int p = 0; p < P; ++p) {
-                const float dy = yv[p] - g.py;
-                const float t = fmaf(g.D, dy, c1);
-                e[p] = fmaf(t, dy, c0);
-            }
+            plain_exponents(g, e);
         }
         return true;
     };
@@ -554,7 +628,109 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
     // The per-wave test of a shared list costs a few percent when it never fires, so it is used only
     // for tiles that fewer than 7/8 of the Gaussians reach (workgroup-uniform choice of the loop):
     // there some boxes are small against the image, and those are often small against the tile too.
-    if constexpr (kWave) {
+    // Matrix form: per record one float4 and the few floats behind it that the exponents need, and per matrix
+    // instruction one float read at a lane-dependent address: channel min(4 m + lane % 4, C) of the record
+    // (channel 0 = alpha, 1 + c = alpha c_c: floats 5.. of both record layouts).  A group's exponentials
+    // first, then its matrix instructions.
+    [[maybe_unused]] const int chl = lane & 3;
+    [[maybe_unused]] auto channel_values = [&](const float4* rec, float (&cv)[NM]) {
+        const float* f = reinterpret_cast<const float*>(rec);
+#pragma unroll
+        for (int m = 0; m < NM; ++m) cv[m] = f[5 + min(4 * m + chl, C)];
+    };
+    [[maybe_unused]] auto accumulate = [&](const float (&cv)[NM], const float (&e)[P]) {
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int m = 0; m < NM; ++m) acc[p][m] = __builtin_amdgcn_mfma_f32_4x4x1f32(cv[m], e[p], acc[p][m], 0, 0, 0);
+    };
+    if constexpr (kMfma && kWave) {
+        __shared__ float4 sh0[kOne ? 1 : 4][kGaussChunk * R4];  // per wave: the two chunk buffers
+        __shared__ float4 sh1[kOne ? 1 : 4][kGaussChunk * R4];
+        struct Head {
+            float4 r0;  // px, py, sD, skD
+            float a2, tag, cv[NM];
+        };
+        stream_records_dma_f<R4, kGaussChunk, true>(
+            src, reinterpret_cast<const float4*>(a.zero_rec), n1 - n0, sh0[kOne ? 0 : wave], sh1[kOne ? 0 : wave],
+            [&](const float4* rec) {
+                const float* f = reinterpret_cast<const float*>(rec);
+                Head h;
+                h.r0 = rec[0];
+                h.a2 = f[4];
+                h.tag = f[6 + C];
+                channel_values(rec, h.cv);
+                return h;
+            },
+            [&](const Head (&h)[kStreamUnroll], const float4* lds) {
+                float e[kStreamUnroll][P];
+#pragma unroll
+                for (int u = 0; u < kStreamUnroll; ++u) {
+                    FRec<C> g;
+                    g.px = h[u].r0.x;
+                    g.py = h[u].r0.y;
+                    g.sD = h[u].r0.z;
+                    g.skD = h[u].r0.w;
+                    g.A2 = h[u].a2;
+                    g.tag = h[u].tag;
+                    sq_exponents(g, lds + u * R4, e[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < kStreamUnroll; ++u)
+#pragma unroll
+                    for (int p = 0; p < P; ++p) e[u][p] = hw_exp2(e[u][p]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < kStreamUnroll; ++u) accumulate(h[u].cv, e[u]);
+            },
+            list);
+    } else if constexpr (kMfma) {
+        __shared__ float4 sh[2 * kGaussChunk * R4];
+        struct Head {
+            float4 r0;  // px, py, A', B2'
+            float D, ylo, yhi, cv[NM];
+        };
+        auto head = [&](const float4* rec) {
+            const float* f = reinterpret_cast<const float*>(rec);
+            Head h;
+            h.r0 = rec[0];
+            h.D = f[4];
+            h.ylo = rec_has_yrange(C) ? f[6 + C] : 0.0f;
+            h.yhi = rec_has_yrange(C) ? f[7 + C] : 0.0f;
+            channel_values(rec, h.cv);
+            return h;
+        };
+        auto group = [&](auto wave_skip, const Head (&h)[kStreamUnroll]) {
+            float e[kStreamUnroll][P];
+            bool reached[kStreamUnroll];  // wave-uniform: the record's reach box meets this wave's rows
+#pragma unroll
+            for (int u = 0; u < kStreamUnroll; ++u) {
+                reached[u] = !(decltype(wave_skip)::value && __ballot(!(h[u].yhi < wylo || h[u].ylo > wyhi)) == 0ull);
+                if (reached[u]) {
+                    GRec<C> g;
+                    g.px = h[u].r0.x;
+                    g.py = h[u].r0.y;
+                    g.A = h[u].r0.z;
+                    g.B2 = h[u].r0.w;
+                    g.D = h[u].D;
+                    plain_exponents(g, e[u]);
+#pragma unroll
+                    for (int p = 0; p < P; ++p) e[u][p] = hw_exp2(e[u][p]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < kStreamUnroll; ++u)
+                if (reached[u]) accumulate(h[u].cv, e[u]);
+        };
+        // (the per-wave test of a shared list: see below)
+        if (rec_has_yrange(C) && 8L * count < 7L * a.Np)
+            stream_records_lds_f<R4, kGaussChunk, true, kThreads, true>(
+                src, n1 - n0, sh, head, [&](const Head (&h)[kStreamUnroll], const float4*) { group(std::true_type{}, h); }, list);
+        else
+            stream_records_lds_f<R4, kGaussChunk, true, kThreads, true>(
+                src, n1 - n0, sh, head, [&](const Head (&h)[kStreamUnroll], const float4*) { group(std::false_type{}, h); }, list);
+    } else if constexpr (kWave) {
         __shared__ float4 sh0[kOne ? 1 : 4][kGaussChunk * R4];  // per wave: the two chunk buffers
         __shared__ float4 sh1[kOne ? 1 : 4][kGaussChunk * R4];
         stream_records_dma<R4, kGaussChunk, RD>(
@@ -568,6 +744,14 @@ __global__ __launch_bounds__(kThreads, P >= 16 ? IGS_FWD_MIN_WAVES : 1) void k_f
         else
             stream_records_lds<R4, kGaussChunk, true, kThreads, RD>(
                 src, n1 - n0, sh, [&](const float4* r, const float4* lds) { body(std::false_type{}, r, lds); }, list);
+    }
+    if constexpr (kMfma) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            dsum[p] = acc[p][0][0];
+#pragma unroll
+            for (int c = 0; c < C; ++c) num[p][c] = acc[p][(1 + c) / 4][(1 + c) % 4];
+        }
     }
     if (col < a.W) {
 #pragma unroll
