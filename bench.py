@@ -29,15 +29,16 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 
 # Per-launch counter readings of the two hot kernels at c1, taken from the committed rocprofv3 summary
 # (profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md): wave-level instruction counts and HBM KiB.
-# executed FLOPs = (2 FMA + MUL + ADD + TRANS) x 64 lanes; HBM bytes = FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
+# executed FLOPs = (2 FMA + MUL + ADD + TRANS) x 64 lanes + 512 per 4x4x1 matrix instruction (16 blocks x 4 x 4 FMA);
+# HBM bytes = FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
 # (factors from the plain-copy calibration of the same profile run).  `csrc_sha16` names the kernel sources
 # the counters were read from (csrc_sha16() below): with other sources the instruction counts no longer
 # belong to the kernels being timed, and the fields derived from them are reported as null.
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
-    "csrc_sha16": "9fb8a21f2d84902d",
+    "csrc_sha16": "cea50b7bc4803140",
     "bwd": {"fma": 6.841e8, "mul": 1.439e8, "add": 7.404e7, "trans": 6.770e7, "fetch_kib": 55720, "write_kib": 147400},
-    "fwd": {"fma": 4.069e8, "mul": 1.268e7, "add": 8.904e6, "trans": 6.713e7, "fetch_kib": 12740, "write_kib": 131100},
+    "fwd": {"fma": 1.386e8, "mul": 1.269e7, "add": 8.919e6, "trans": 6.714e7, "mfma": 6.707e7, "fetch_kib": 12700, "write_kib": 131100},
 }
 
 
@@ -55,7 +56,7 @@ def csrc_sha16():
 
 
 def executed_flops(k):
-    return (2 * k["fma"] + k["mul"] + k["add"] + k["trans"]) * 64
+    return (2 * k["fma"] + k["mul"] + k["add"] + k["trans"]) * 64 + 512 * k.get("mfma", 0.0)
 
 
 def hbm_bytes(k):
@@ -342,12 +343,12 @@ def run(args) -> int:
                     "call's allowance, which bounds the change of every output element by 1e-7 max|colour|; frac_counting_all_pairs uses all B N H W as the metric does and can "
                     "exceed 1) / launch_ms, measured live with HIP events around igs_gs2d_backward_reduce with the tile lists "
                     "in place (IGS_OPT_LISTS_BUILT: k_bwd_sep alone; a training step builds the lists once, in its "
-                    "forward); the forward's launch_ms holds k_bin + k_fwd_sep + combine.  executed_frac: the arithmetic the hardware ran, (2 FMA + MUL + ADD + TRANS) x 64 per "
+                    "forward); the forward's launch_ms holds k_bin + k_fwd_sep + combine.  executed_frac: the arithmetic the hardware ran, (2 FMA + MUL + ADD + TRANS) x 64 + 512 per 4x4x1 matrix instruction (the forward's sums) per "
                     "launch from the rocprofv3 counters of counter_source (separable grids hoist the row/column part of "
                     "the model's operations, so it is below frac) / the live launch_ms.  traffic: HBM bytes per launch "
                     "from FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of the same summary (copy-calibrated); c1 only.  peak: "
-                    "published fp32 vector peak at 2.4 GHz; the kernels use plain fp32 VALU ops with VGPR-only operands, "
-                    "v_exp_f32 counted as 1 FLOP.",
+                    "published fp32 vector peak at 2.4 GHz; the kernels use plain fp32 VALU ops with VGPR-only operands and, for the forward's "
+                    "channel sums, fp32 v_mfma_f32_4x4x1 (same published peak); v_exp_f32 counted as 1 FLOP.",
         },
     })
 
