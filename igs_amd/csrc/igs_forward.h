@@ -793,28 +793,78 @@ __global__ __launch_bounds__(kThreads) void k_fwd_gen(const FwdArgs a) {
     const int n0 = s * a.n_per_split;
     const int n1 = min(a.Np, n0 + a.n_per_split);
     const float4* src = reinterpret_cast<const float4*>(a.packed + ((size_t)b * a.Np + n0) * RS);
-    stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r, const float4*) {
-        const GRec<C> g = lds_grec<C>(r);
-        float e[P];
+    // the weights of the lane's P pixels for a record (px, py, A', B2' in r0)
+    auto weights = [&](const float4& r0, float D, float (&e)[P]) {
 #pragma unroll
         for (int j = 0; j < P; ++j) {
-            const float dx = xv[j] - g.px;
-            const float dy = yv[j] - g.py;
-            float t = g.A * dx;
-            t = fmaf(g.B2, dy, t);
-            const float v = g.D * dy;
+            const float dx = xv[j] - r0.x;
+            const float dy = yv[j] - r0.y;
+            float t = r0.z * dx;
+            t = fmaf(r0.w, dy, t);
+            const float v = D * dy;
             float q = t * dx;
             e[j] = fmaf(v, dy, q);
         }
 #pragma unroll
         for (int j = 0; j < P; ++j) e[j] = hw_exp2(e[j]);
+    };
+    if constexpr (fwd_mfma(C)) {
+        // the sums as matrix instructions, a group's behind its vector arithmetic (see k_fwd_sep)
+        constexpr int NM = (C + 4) / 4;
+        fwd_v4f acc[P][NM];
+#pragma unroll
+        for (int j = 0; j < P; ++j)
+#pragma unroll
+            for (int m = 0; m < NM; ++m) acc[j][m] = fwd_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        const int chl = threadIdx.x & 3;
+        struct Head {
+            float4 r0;
+            float D, cv[NM];
+        };
+        stream_records_lds_f<R4, kGaussChunk, false, kThreads, true>(
+            src, n1 - n0, sh,
+            [&](const float4* rec) {
+                const float* f = reinterpret_cast<const float*>(rec);
+                Head h;
+                h.r0 = rec[0];
+                h.D = f[4];
+#pragma unroll
+                for (int m = 0; m < NM; ++m) h.cv[m] = f[5 + min(4 * m + chl, C)];
+                return h;
+            },
+            [&](const Head (&h)[kStreamUnroll], const float4*) {
+                float e[kStreamUnroll][P];
+#pragma unroll
+                for (int u = 0; u < kStreamUnroll; ++u) weights(h[u].r0, h[u].D, e[u]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < kStreamUnroll; ++u)
+#pragma unroll
+                    for (int j = 0; j < P; ++j)
+#pragma unroll
+                        for (int m = 0; m < NM; ++m)
+                            acc[j][m] = __builtin_amdgcn_mfma_f32_4x4x1f32(h[u].cv[m], e[u][j], acc[j][m], 0, 0, 0);
+            },
+            nullptr);
 #pragma unroll
         for (int j = 0; j < P; ++j) {
-            dsum[j] = fmaf(e[j], g.al, dsum[j]);
+            dsum[j] = acc[j][0][0];
 #pragma unroll
-            for (int c = 0; c < C; ++c) num[j][c] = fmaf(e[j], g.ac[c], num[j][c]);
+            for (int c = 0; c < C; ++c) num[j][c] = acc[j][(1 + c) / 4][(1 + c) % 4];
         }
-    });
+    } else {
+        stream_records_lds<R4, kGaussChunk>(src, n1 - n0, sh, [&](const float4* r, const float4*) {
+            const GRec<C> g = lds_grec<C>(r);
+            float e[P];
+            weights(r[0], g.D, e);
+#pragma unroll
+            for (int j = 0; j < P; ++j) {
+                dsum[j] = fmaf(e[j], g.al, dsum[j]);
+#pragma unroll
+                for (int c = 0; c < C; ++c) num[j][c] = fmaf(e[j], g.ac[c], num[j][c]);
+            }
+        });
+    }
 #pragma unroll
     for (int j = 0; j < P; ++j)
         if (pix[j] < HW) fwd_store<C>(a, b, s, pix[j], dsum[j], num[j]);
