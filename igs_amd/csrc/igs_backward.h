@@ -383,20 +383,17 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
                 const float dy = yv - py;
                 const float rowoff = fmaf(B2, dy, mpx);
                 const float cyy = (D * dy) * dy;
-                float R0 = 0.0f, R1 = 0.0f;
+                float R0 = 0.0f, R1 = 0.0f, RQ = 0.0f;
                 const float4* rowrec = cur + rr * ROW4;
                 // four pairs (columns i..i+3) from their u
                 auto four_pairs = [&](int i, const float (&us)[4]) {
                     // phase 1: exponents of the 4 pairs (independent chains)
-                    float vs[4], ee[4];
+                    float qs[4], ee[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        vs[j] = us[j] * us[j];
-                        ee[j] = cyy - vs[j];
-                    }
+                    for (int j = 0; j < 4; ++j) qs[j] = fmaf(-us[j], us[j], cyy);
                     // phase 2: transcendentals back to back
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) ee[j] = hw_exp2(ee[j]);
+                    for (int j = 0; j < 4; ++j) ee[j] = hw_exp2(qs[j]);
                     // phase 3: G = <g^, c> - s and the sums
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
@@ -408,7 +405,7 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
                         const float ge = Gv * ee[j];
                         R0 += ge;
                         R1 = fmaf(ge, us[j], R1);
-                        M[3] = fmaf(ge, vs[j], M[3]);
+                        RQ = fmaf(ge, qs[j], RQ);
 #pragma unroll
                         for (int c = 0; c < C; ++c) CG[c] = fmaf(ee[j], pv[c], CG[c]);
                     }
@@ -436,10 +433,11 @@ __global__ __launch_bounds__(kThreads, C > 8 ? 4 : 1) void k_bwd_sep(const BwdAr
                         four_pairs(i, us);
                     }
                 }
-                // the tile row is complete
+                // the tile row is complete; its sum of G e u^2 from that of G e q': u^2 = cyy - q'
                 M[0] += R0;
                 M[1] += R1;
                 M[2] = fmaf(dy, R0, M[2]);
+                M[3] += fmaf(cyy, R0, -RQ);
                 M[4] = fmaf(dy, R1, M[4]);
                 M[5] = fmaf(dy * dy, R0, M[5]);
             }
