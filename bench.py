@@ -36,8 +36,8 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X published fp32 vector (packed-FMA) pea
 # belong to the kernels being timed, and the fields derived from them are reported as null.
 C1_PROFILE = {
     "source": "profiles/k_fwd_sep_k_bwd_sep_c1_B16_N8192_256x256_C3.md",
-    "csrc_sha16": "cea50b7bc4803140",
-    "bwd": {"fma": 6.841e8, "mul": 1.439e8, "add": 7.404e7, "trans": 6.770e7, "fetch_kib": 55720, "write_kib": 147400},
+    "csrc_sha16": "a244c3e3a6718d95",
+    "bwd": {"fma": 6.862e8, "mul": 7.632e7, "add": 7.615e7, "trans": 6.770e7, "fetch_kib": 55720, "write_kib": 147400},
     "fwd": {"fma": 1.386e8, "mul": 1.269e7, "add": 8.919e6, "trans": 6.714e7, "mfma": 6.707e7, "fetch_kib": 12700, "write_kib": 131100},
 }
 

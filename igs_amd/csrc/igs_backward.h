@@ -211,10 +211,12 @@ constexpr int kBwdTileW = IGS_BWD_TILE_W;
 // Exponent with the square completed along the row (write_sep_records):
 //   q' = -(sA dx + skA dy)^2 + D'' dy^2 = -u^2 + cyy,   u = sA x' + (skA dy - sA px')
 // with x', px' relative to the tile's middle column, so that the hoisted row term carries no more
-// rounding than u itself.  Per pair: u (fma), u^2, cyy - u^2, exp2, G = <g^, c> - s (C fma), G e, and
-// the sums of G e {1, u, u^2} and e g^_c: 9 + 2 C instructions and one exponential.  Per row the
-// sums of G e {1, u} are folded with dy into the totals of G e {1, u, dy, u dy, dy^2}; at the end the
-// moments in (u, dy) become those in (dx, dy) (dx = (u - skA dy) / sA).  Lanes whose Gaussian has no
+// rounding than u itself.  Per pair: u, q' = fma(-u, u, cyy), exp2, G = <g^, c> - s (C fma), G e, and
+// the sums of G e {1, u, q'} and e g^_c: 8 + 2 C instructions and one exponential.  Per row the
+// sums of G e {1, u} are folded with dy into the totals of G e {1, u, dy, u dy, dy^2}, and the row's sum
+// of G e u^2 is cyy times its sum of G e less its sum of G e q' (cyy is the row's constant; where it is
+// large the row's weights are at most 2^-cyy, so the difference costs no accuracy that the total sees);
+// at the end the moments in (u, dy) become those in (dx, dy) (dx = (u - skA dy) / sA).  Lanes whose Gaussian has no
 // completed square (tag of the backward record: a form that is not positive definite, non-finite
 // values) evaluate q' = (A' dx + B2' dy) dx + D' dy^2 term by term instead; what a Gaussian's sums are
 // depends on the Gaussian only, not on which lanes share its wave.
