@@ -251,6 +251,23 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
 
 
+def test_bench_counter_constants_belong_to_the_current_kernel_sources():
+    """bench.py derives `executed_frac` and `traffic` from per-launch counter readings stored in the file, and only
+    while the kernel sources are the ones those readings were taken from: the stored hash is the current one (a
+    kernel change that leaves it behind would make the bench line report null for those fields)."""
+    import importlib.util
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("igs_bench_module", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert bench.C1_PROFILE["csrc_sha16"] == bench.csrc_sha16()
+    assert os.path.exists(os.path.join(root, bench.C1_PROFILE["source"]))
+    for leg in ("fwd", "bwd"):
+        assert bench.executed_flops(bench.C1_PROFILE[leg]) > 0 and bench.hbm_bytes(bench.C1_PROFILE[leg]) > 0
+
+
 def test_plan_invariants_over_random_shapes(lib):
     """igs_gs2d_plan over a few hundred seeded random shapes (tiny to large, square to extreme
     aspect ratios): every size positive and consistent, tiles cover the image, splits cover N."""
